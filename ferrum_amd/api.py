@@ -1,0 +1,590 @@
+"""Host-side mirror of Ferrum's quantized-matmul operator interface over the C ABI.
+
+Names, argument meaning and error behaviour follow the reference so that
+tests read like its own:
+
+* ``QuantizationFormat``, ``QuantizedMatrix.from_reader``,
+  ``QuantizedExpertMatrix.new``          src/quantization.rs:6-194
+* ``DType``, ``Tensor.from_f32`` / ``to_f32`` / ``view``   src/tensor/mod.rs
+* ``Device.project_quantized``           src/ops/transformer.rs:96-297
+* ``Device.embedding_gather_quantized``  src/ops/transformer.rs:299-360
+* ``Device.moe_route`` / ``expert_assign`` / ``expert_project_quantized`` /
+  ``expert_silu_mul`` / ``expert_combine``   src/ops/mod.rs:23-551
+* ``MoeRoutingPolicy``                   src/model/architecture.rs
+
+Everything computes on the GPU through ``libferrum_hip.so``.  There is no CPU
+path: importing this module raises if the library has not been built
+(``python -m ferrum_amd.build``).
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+import os
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libferrum_hip.so")
+
+
+class Error(Exception):
+    """ferrum::Error (src/error.rs:3-51); ``kind`` is the variant name."""
+    kind = "Error"
+
+    def __init__(self, message: str = ""):
+        super().__init__(f"{self.kind}: {message}")
+        self.message = message
+
+
+def _variant(name):
+    return type(name, (Error,), {"kind": name})
+
+
+ShapeError = _variant("Shape")
+DTypeError = _variant("DType")
+DeviceMismatch = _variant("DeviceMismatch")
+RangeError = _variant("Range")
+DispatchError = _variant("Dispatch")
+SynchronizationError = _variant("Synchronization")
+AllocationError = _variant("Allocation")
+GgufError = _variant("Gguf")
+WeightError = _variant("Weight")
+ParameterError = _variant("Parameter")
+TokenError = _variant("Token")
+ValidationError = _variant("Validation")
+
+_ERRORS = {1: ShapeError, 2: DTypeError, 3: DeviceMismatch, 4: RangeError, 5: DispatchError,
+           6: SynchronizationError, 7: AllocationError, 8: GgufError, 9: WeightError,
+           10: ParameterError, 11: TokenError, 12: ValidationError}
+
+
+class _View(ctypes.Structure):
+    _fields_ = [("buffer", ctypes.c_void_p), ("offset", ctypes.c_size_t), ("dtype", ctypes.c_uint32)]
+
+
+class _Props(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 64),
+                ("compute_units", ctypes.c_int32), ("wavefront", ctypes.c_int32),
+                ("clock_khz", ctypes.c_int32), ("memory_clock_khz", ctypes.c_int32),
+                ("memory_bus_bits", ctypes.c_int32), ("lds_bytes_per_block", ctypes.c_int32),
+                ("global_bytes", ctypes.c_uint64), ("l2_bytes", ctypes.c_uint64)]
+
+
+class _Policy(ctypes.Structure):
+    _fields_ = [("experts", ctypes.c_uint32), ("top_k", ctypes.c_uint32),
+                ("sigmoid", ctypes.c_uint32), ("normalize_top_k_prob", ctypes.c_uint32),
+                ("normalization_epsilon", ctypes.c_float), ("routed_scaling_factor", ctypes.c_float)]
+
+
+# every symbol include/ferrum_hip.h declares: (restype, argtypes)
+_P, _SZ, _U32, _U64, _I32, _I64 = (ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32,
+                                   ctypes.c_uint64, ctypes.c_int32, ctypes.c_int64)
+_VP = ctypes.POINTER(_View)
+SYMBOLS = {
+    "fh_device_create": (_I32, [_I32, ctypes.POINTER(_P)]),
+    "fh_device_destroy": (None, [_P]),
+    "fh_device_properties": (_I32, [_P, ctypes.POINTER(_Props)]),
+    "fh_synchronize": (_I32, [_P]),
+    "fh_last_error": (ctypes.c_char_p, []),
+    "fh_last_operation": (ctypes.c_char_p, [_P]),
+    "fh_device_stream": (_P, [_P]),
+    "fh_set_tuning": (_I32, [_P, ctypes.c_char_p, _I64]),
+    "fh_get_tuning": (_I32, [_P, ctypes.c_char_p, ctypes.POINTER(_I64)]),
+    "fh_buffer_alloc": (_I32, [_P, _SZ, ctypes.POINTER(_P)]),
+    "fh_buffer_free": (None, [_P]),
+    "fh_buffer_size": (_SZ, [_P]),
+    "fh_buffer_device_ptr": (_P, [_P]),
+    "fh_buffer_upload": (_I32, [_P, _SZ, _P, _SZ]),
+    "fh_buffer_download": (_I32, [_P, _SZ, _P, _SZ]),
+    "fh_buffer_fill_zero": (_I32, [_P, _SZ, _SZ]),
+    "fh_qmatrix_create": (_I32, [_P, _U32, _U64, _U64, _U64, _P, _SZ, ctypes.POINTER(_P)]),
+    "fh_qmatrix_destroy": (None, [_P]),
+    "fh_qmatrix_rows": (_U64, [_P]),
+    "fh_qmatrix_columns": (_U64, [_P]),
+    "fh_qmatrix_experts": (_U64, [_P]),
+    "fh_qmatrix_ggml_type": (_U32, [_P]),
+    "fh_qmatrix_byte_size": (_SZ, [_P]),
+    "fh_qmatrix_device_ptr": (_P, [_P]),
+    "fh_dequantize": (_I32, [_P, _P, _VP]),
+    "fh_embedding_gather_quantized": (_I32, [_P, _P, ctypes.POINTER(_U32), _SZ, _VP]),
+    "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
+    "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
+    "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
+    "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
+    "fh_expert_silu_mul": (_I32, [_P, _VP, _U32, _U32, _VP]),
+    "fh_expert_combine": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
+    "fh_event_create": (_I32, [_P, ctypes.POINTER(_P)]),
+    "fh_event_destroy": (None, [_P]),
+    "fh_event_record": (_I32, [_P]),
+    "fh_event_elapsed_ms": (_I32, [_P, _P, ctypes.POINTER(ctypes.c_float)]),
+}
+
+
+def load_library(path: str = LIB_PATH) -> ctypes.CDLL:
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python -m ferrum_amd.build` "
+                          "(there is no CPU fallback)")
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+_lib = load_library()
+
+
+def _check(status: int):
+    if status != 0:
+        message = _lib.fh_last_error().decode("utf-8", "replace")
+        raise _ERRORS.get(status, Error)(message)
+
+
+class DType(enum.IntEnum):
+    F32 = 0
+    F16 = 1
+    BF16 = 2
+
+    def size_bytes(self) -> int:
+        return 4 if self == DType.F32 else 2
+
+
+class QuantizationFormat(enum.Enum):
+    Q4_K = 12
+    Q6_K = 14
+
+    @staticmethod
+    def from_ggml_type(type_id: int) -> "QuantizationFormat":
+        try:
+            return QuantizationFormat(type_id)
+        except ValueError:
+            raise GgufError(f"unsupported quantized weight type {type_id}") from None
+
+    def ggml_type(self) -> int:
+        return self.value
+
+    def block_elements(self) -> int:
+        return 256
+
+    def block_bytes(self) -> int:
+        return 144 if self == QuantizationFormat.Q4_K else 210
+
+
+def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    bits = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = np.isnan(a)
+    if nan.any():
+        rounded[nan] = ((bits[nan] >> 16) | 0x40).astype(np.uint16)
+    return rounded
+
+
+def encode(values: np.ndarray, dtype: DType) -> np.ndarray:
+    """f32 -> storage bytes (round to nearest even), as Tensor::from_f32 does."""
+    a = np.ascontiguousarray(values, dtype=np.float32)
+    if dtype == DType.F32:
+        return a
+    if dtype == DType.F16:
+        with np.errstate(over="ignore"):
+            return a.astype(np.float16)
+    return _f32_to_bf16_bits(a)
+
+
+def decode(raw: np.ndarray, dtype: DType) -> np.ndarray:
+    if dtype == DType.F32:
+        return raw.view(np.float32).copy()
+    if dtype == DType.F16:
+        return raw.view(np.float16).astype(np.float32)
+    return (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class Buffer:
+    def __init__(self, device: "Device", nbytes: int):
+        self.device = device
+        handle = ctypes.c_void_p()
+        _check(_lib.fh_buffer_alloc(device._handle, nbytes, ctypes.byref(handle)))
+        self._handle = handle
+        self.nbytes = nbytes
+
+    def upload(self, offset: int, data: np.ndarray):
+        data = np.ascontiguousarray(data)
+        _check(_lib.fh_buffer_upload(self._handle, offset, data.ctypes.data, data.nbytes))
+
+    def download(self, offset: int, nbytes: int) -> np.ndarray:
+        out = np.empty(nbytes, dtype=np.uint8)
+        _check(_lib.fh_buffer_download(self._handle, offset, out.ctypes.data, nbytes))
+        return out
+
+    def device_ptr(self) -> int:
+        return _lib.fh_buffer_device_ptr(self._handle) or 0
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_buffer_free(h)
+
+
+class Tensor:
+    """Dense row-major tensor: a typed window on a Buffer."""
+
+    def __init__(self, buffer: Buffer, offset: int, shape, dtype: DType):
+        self.buffer, self.offset, self.dtype = buffer, offset, DType(dtype)
+        self._shape = tuple(int(d) for d in shape)
+
+    @staticmethod
+    def zeros(device: "Device", shape, dtype: DType) -> "Tensor":
+        shape = tuple(int(d) for d in shape)
+        n = int(np.prod(shape, dtype=np.int64)) if shape else 1
+        return Tensor(Buffer(device, max(n, 1) * DType(dtype).size_bytes()), 0, shape, dtype)
+
+    @staticmethod
+    def from_f32(device: "Device", shape, dtype: DType, values) -> "Tensor":
+        shape = tuple(int(d) for d in shape)
+        a = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
+        if a.size != int(np.prod(shape, dtype=np.int64)):
+            raise ShapeError("value count does not match shape")
+        t = Tensor.zeros(device, shape, dtype)
+        if a.size:
+            t.buffer.upload(0, encode(a, DType(dtype)))
+        return t
+
+    @staticmethod
+    def from_bits(device: "Device", shape, values_u32) -> "Tensor":
+        """F32-typed carrier of raw 32-bit words (the reference stores ids so)."""
+        a = np.ascontiguousarray(values_u32, dtype=np.uint32).reshape(-1)
+        t = Tensor.zeros(device, shape, DType.F32)
+        t.buffer.upload(0, a)
+        return t
+
+    def shape(self):
+        return self._shape
+
+    def numel(self) -> int:
+        return int(np.prod(self._shape, dtype=np.int64)) if self._shape else 1
+
+    def byte_size(self) -> int:
+        return self.numel() * self.dtype.size_bytes()
+
+    def view(self, element_offset: int, shape) -> "Tensor":
+        shape = tuple(int(d) for d in shape)
+        n = int(np.prod(shape, dtype=np.int64))
+        if element_offset < 0 or element_offset + n > self.numel():
+            raise RangeError("view exceeds tensor")
+        return Tensor(self.buffer, self.offset + element_offset * self.dtype.size_bytes(), shape,
+                      self.dtype)
+
+    def to_f32(self) -> np.ndarray:
+        raw = self.buffer.download(self.offset, self.byte_size())
+        return decode(raw, self.dtype).reshape(self._shape)
+
+    def raw(self) -> np.ndarray:
+        return self.buffer.download(self.offset, self.byte_size())
+
+    def _view(self) -> _View:
+        return _View(self.buffer._handle, self.offset, int(self.dtype))
+
+
+@dataclass
+class Output:
+    """src/ops/mod.rs:8-21: the result tensor plus Metrics.operation / bytes."""
+    tensor: Tensor
+    operation: str
+    bytes_read: int = 0
+    bytes_written: int = 0
+
+
+class QuantizedMatrix:
+    """Row-major [rows, columns] matrix of verbatim GGUF super-blocks."""
+
+    def __init__(self, device, handle, rows, columns, fmt):
+        self.device, self._handle = device, handle
+        self._rows, self._columns, self._format = rows, columns, fmt
+
+    @staticmethod
+    def from_reader(device: "Device", rows: int, columns: int, fmt: QuantizationFormat, fill,
+                    experts: int = 1) -> "QuantizedMatrix":
+        """``fill(destination)`` writes the packed payload into a uint8 array,
+        like the reference's FnOnce(&mut [u8]) reader."""
+        total_rows = rows * experts
+        if total_rows == 0 or columns == 0 or columns % fmt.block_elements() != 0:
+            raise ShapeError(f"{fmt.name} matrix requires nonempty rows and columns divisible by "
+                             f"block size {fmt.block_elements()}")
+        byte_len = total_rows * (columns // fmt.block_elements()) * fmt.block_bytes()
+        destination = np.zeros(byte_len, dtype=np.uint8)
+        fill(destination)
+        return QuantizedMatrix.from_bytes(device, rows, columns, fmt, destination, experts)
+
+    @staticmethod
+    def from_bytes(device, rows, columns, fmt, payload, experts: int = 1) -> "QuantizedMatrix":
+        ggml = fmt.value if isinstance(fmt, QuantizationFormat) else int(fmt)
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        handle = ctypes.c_void_p()
+        _check(_lib.fh_qmatrix_create(device._handle, ggml, rows, columns, experts,
+                                      payload.ctypes.data, payload.nbytes, ctypes.byref(handle)))
+        return QuantizedMatrix(device, handle, rows * experts, columns, QuantizationFormat(ggml))
+
+    def rows(self) -> int:
+        return self._rows
+
+    def columns(self) -> int:
+        return self._columns
+
+    def format(self) -> QuantizationFormat:
+        return self._format
+
+    def byte_size(self) -> int:
+        return int(_lib.fh_qmatrix_byte_size(self._handle))
+
+    def device_ptr(self) -> int:
+        return _lib.fh_qmatrix_device_ptr(self._handle) or 0
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_qmatrix_destroy(h)
+
+
+class QuantizedExpertMatrix:
+    """[experts, rows_per_expert, columns] stored as one packed matrix with the
+    expert axis flattened into rows."""
+
+    def __init__(self, device, handle, experts, rows_per_expert, columns, fmt):
+        self.device, self._handle = device, handle
+        self._experts, self._rows, self._columns, self._format = experts, rows_per_expert, columns, fmt
+
+    @staticmethod
+    def new(device, payload, fmt: QuantizationFormat, experts: int, rows_per_expert: int,
+            columns: int) -> "QuantizedExpertMatrix":
+        if experts == 0 or rows_per_expert == 0:
+            raise ShapeError("quantized expert matrix row geometry mismatch")
+        payload = np.ascontiguousarray(payload, dtype=np.uint8)
+        handle = ctypes.c_void_p()
+        _check(_lib.fh_qmatrix_create(device._handle, fmt.value, rows_per_expert, columns, experts,
+                                      payload.ctypes.data, payload.nbytes, ctypes.byref(handle)))
+        return QuantizedExpertMatrix(device, handle, experts, rows_per_expert, columns, fmt)
+
+    def experts(self) -> int:
+        return self._experts
+
+    def rows_per_expert(self) -> int:
+        return self._rows
+
+    def columns(self) -> int:
+        return self._columns
+
+    def format(self) -> QuantizationFormat:
+        return self._format
+
+    def byte_size(self) -> int:
+        return int(_lib.fh_qmatrix_byte_size(self._handle))
+
+    def matrix_view(self) -> QuantizedMatrix:
+        """The flattened [experts*rows, columns] matrix (shares storage; the
+        returned object does not own the handle)."""
+        m = QuantizedMatrix(self.device, None, self._experts * self._rows, self._columns, self._format)
+        m._borrowed = self._handle
+        return m
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_qmatrix_destroy(h)
+
+
+class MoeScoringFunction(enum.Enum):
+    Softmax = 0
+    Sigmoid = 1
+
+
+@dataclass
+class MoeRoutingPolicy:
+    experts: int
+    top_k: int
+    scoring_function: MoeScoringFunction = MoeScoringFunction.Softmax
+    normalize_top_k_prob: bool = True
+    normalization_epsilon: float = 0.0
+    routed_scaling_factor: float = 1.0
+    use_expert_bias: bool = False
+
+    @staticmethod
+    def softmax(experts: int, top_k: int) -> "MoeRoutingPolicy":
+        return MoeRoutingPolicy(experts, top_k)
+
+    def _c(self) -> _Policy:
+        return _Policy(self.experts, self.top_k,
+                       int(self.scoring_function == MoeScoringFunction.Sigmoid),
+                       int(self.normalize_top_k_prob), self.normalization_epsilon,
+                       self.routed_scaling_factor)
+
+
+class Event:
+    def __init__(self, device: "Device"):
+        handle = ctypes.c_void_p()
+        _check(_lib.fh_event_create(device._handle, ctypes.byref(handle)))
+        self._handle = handle
+
+    def record(self):
+        _check(_lib.fh_event_record(self._handle))
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = ctypes.c_float()
+        _check(_lib.fh_event_elapsed_ms(self._handle, stop._handle, ctypes.byref(ms)))
+        return float(ms.value)
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_event_destroy(h)
+
+
+class Device:
+    """One gfx950 GPU and its stream (the reference's MetalDevice)."""
+
+    def __init__(self, ordinal: int = 0):
+        handle = ctypes.c_void_p()
+        _check(_lib.fh_device_create(ordinal, ctypes.byref(handle)))
+        self._handle = handle
+
+    @staticmethod
+    def new(ordinal: int = 0) -> "Device":
+        return Device(ordinal)
+
+    def properties(self) -> dict:
+        p = _Props()
+        _check(_lib.fh_device_properties(self._handle, ctypes.byref(p)))
+        return {f: (getattr(p, f).decode() if isinstance(getattr(p, f), bytes) else getattr(p, f))
+                for f, _ in _Props._fields_}
+
+    def synchronize(self):
+        _check(_lib.fh_synchronize(self._handle))
+
+    def last_operation(self) -> str:
+        return _lib.fh_last_operation(self._handle).decode()
+
+    def set_tuning(self, key: str, value: int):
+        _check(_lib.fh_set_tuning(self._handle, key.encode(), value))
+
+    def get_tuning(self, key: str) -> int:
+        v = ctypes.c_int64()
+        _check(_lib.fh_get_tuning(self._handle, key.encode(), ctypes.byref(v)))
+        return int(v.value)
+
+    def set_k_quant_gemv_ksplit(self, simds: int):
+        self.set_tuning("k_quant_gemv_ksplit", simds)
+
+    def event(self) -> Event:
+        return Event(self)
+
+    # ---- operators ---------------------------------------------------------
+
+    def dequantize(self, weight, dtype: DType = DType.F32) -> Tensor:
+        rows = weight.rows() if isinstance(weight, QuantizedMatrix) else weight.experts() * weight.rows_per_expert()
+        out = Tensor.zeros(self, (rows, weight.columns()), dtype)
+        v = out._view()
+        _check(_lib.fh_dequantize(self._handle, _handle_of(weight), ctypes.byref(v)))
+        return out
+
+    def embedding_gather_quantized(self, weight: QuantizedMatrix, tokens, output_dtype: DType) -> Output:
+        ids = np.ascontiguousarray(tokens, dtype=np.uint32)
+        out = Tensor.zeros(self, (ids.size, weight.columns()), output_dtype)
+        v = out._view()
+        _check(_lib.fh_embedding_gather_quantized(
+            self._handle, _handle_of(weight), ids.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)),
+            ids.size, ctypes.byref(v)))
+        return Output(out, self.last_operation())
+
+    def project_quantized(self, a: Tensor, weight: QuantizedMatrix, out_dtype: DType | None = None,
+                          out: Tensor | None = None) -> Output:
+        dims = a.shape()
+        if len(dims) != 2 or dims[1] != weight.columns() or dims[1] > 0xFFFFFFFF - 32:
+            raise ShapeError("quantized projection requires [M,K] matching [N,K]")
+        if a.buffer.device is not self or weight.device is not self:
+            raise DeviceMismatch("tensor or weight belongs to another device")
+        m, n = dims[0], weight.rows()
+        dtype = a.dtype if out_dtype is None else DType(out_dtype)
+        if out is None:
+            out = Tensor.zeros(self, (m, n), dtype)
+        if m == 0:
+            return Output(out, "")
+        xv, yv = a._view(), out._view()
+        _check(_lib.fh_project_quantized(self._handle, _handle_of(weight), ctypes.byref(xv), m,
+                                         ctypes.byref(yv)))
+        return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
+
+    def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy) -> Tensor:
+        dims = logits.shape()
+        if len(dims) != 2 or dims[0] == 0 or dims[1] == 0 or dims[1] != policy.experts:
+            raise ShapeError("invalid sparse routing geometry")
+        if selection_bias is not None and (selection_bias.shape() != (policy.experts,)
+                                           or selection_bias.dtype != DType.F32):
+            raise ShapeError("invalid sparse routing geometry")
+        out = Tensor.zeros(self, (dims[0] * max(policy.top_k, 1), 3), DType.F32)
+        lv, ov, pc = logits._view(), out._view(), policy._c()
+        bv = selection_bias._view() if selection_bias is not None else None
+        _check(_lib.fh_moe_route(self._handle, ctypes.byref(lv), dims[0],
+                                 ctypes.byref(bv) if bv is not None else None, ctypes.byref(pc),
+                                 ctypes.byref(ov)))
+        return out
+
+    def expert_assign(self, hidden: Tensor, metadata: Tensor, top_k: int) -> Tensor:
+        x, meta = hidden.shape(), metadata.shape()
+        if (len(x) != 2 or x[0] == 0 or x[1] == 0 or len(meta) != 2 or meta[1] != 3 or top_k == 0
+                or x[0] * top_k != meta[0] or metadata.dtype != DType.F32):
+            raise ShapeError("expert assignments require [S,H] and [S*top_k,3]")
+        out = Tensor.zeros(self, (meta[0], x[1]), hidden.dtype)
+        hv, mv, ov = hidden._view(), metadata._view(), out._view()
+        _check(_lib.fh_expert_assign(self._handle, ctypes.byref(hv), x[0], x[1], ctypes.byref(mv),
+                                     top_k, ctypes.byref(ov)))
+        return out
+
+    def expert_project_quantized(self, input: Tensor, metadata: Tensor,
+                                 weight: QuantizedExpertMatrix, features: int, experts: int,
+                                 out_dtype: DType | None = None) -> Tensor:
+        x, meta = input.shape(), metadata.shape()
+        if (len(x) != 2 or x[0] == 0 or x[1] != features or meta != (x[0], 3)
+                or metadata.dtype != DType.F32 or experts == 0 or weight.experts() != experts
+                or weight.columns() != features or weight.rows_per_expert() == 0
+                or input.buffer.device is not self or metadata.buffer.device is not self
+                or weight.device is not self):
+            raise ShapeError("quantized expert projection geometry mismatch")
+        dtype = input.dtype if out_dtype is None else DType(out_dtype)
+        out = Tensor.zeros(self, (x[0], weight.rows_per_expert()), dtype)
+        xv, mv, ov = input._view(), metadata._view(), out._view()
+        _check(_lib.fh_expert_project_quantized(self._handle, weight._handle, ctypes.byref(xv), x[0],
+                                                ctypes.byref(mv), ctypes.byref(ov)))
+        return out
+
+    def expert_silu_mul(self, input: Tensor, intermediate: int) -> Tensor:
+        x = input.shape()
+        if len(x) != 2 or intermediate == 0 or intermediate * 2 != x[1]:
+            raise ShapeError("packed expert activation geometry mismatch")
+        out = Tensor.zeros(self, (x[0], intermediate), input.dtype)
+        iv, ov = input._view(), out._view()
+        _check(_lib.fh_expert_silu_mul(self._handle, ctypes.byref(iv), x[0], intermediate,
+                                       ctypes.byref(ov)))
+        return out
+
+    def expert_combine(self, input: Tensor, metadata: Tensor, tokens: int, hidden: int,
+                       top_k: int) -> Tensor:
+        x = input.shape()
+        if (top_k == 0 or hidden == 0 or x != (tokens * top_k, hidden)
+                or metadata.shape() != (x[0], 3) or metadata.dtype != DType.F32):
+            raise ShapeError("expert combine geometry mismatch")
+        out = Tensor.zeros(self, (tokens, hidden), input.dtype)
+        iv, mv, ov = input._view(), metadata._view(), out._view()
+        _check(_lib.fh_expert_combine(self._handle, ctypes.byref(iv), ctypes.byref(mv), tokens,
+                                      hidden, top_k, ctypes.byref(ov)))
+        return out
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_device_destroy(h)
+
+
+def _handle_of(weight):
+    h = getattr(weight, "_handle", None)
+    return h if h else getattr(weight, "_borrowed", None)

@@ -1,0 +1,625 @@
+// C ABI of the gfx950 backend (see include/ferrum_hip.h): objects, validation
+// and kernel selection.  Argument checks mirror the reference's operator
+// methods (src/ops/transformer.rs:96-297, src/ops/mod.rs:23-609) and its
+// binding checks (src/metal/mod.rs:840-897): shapes, ownership, bounds,
+// alignment and input/output aliasing are rejected before anything launches.
+#include <cmath>
+#include <cstdarg>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "internal.hpp"
+
+namespace fh {
+
+static thread_local std::string g_last_error;
+
+fh_status fail(fh_status code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+fh_status hip_fail(hipError_t err, const char* what) {
+    fh_status code = err == hipErrorOutOfMemory ? FH_ERR_ALLOCATION : FH_ERR_DISPATCH;
+    return fail(code, "%s: %s", what, hipGetErrorString(err));
+}
+
+namespace {
+
+#define FH_HIP(expr)                                        \
+    do {                                                    \
+        hipError_t _e = (expr);                             \
+        if (_e != hipSuccess) return hip_fail(_e, #expr);   \
+    } while (0)
+
+struct Range {
+    const uint8_t* begin;
+    size_t bytes;
+};
+
+bool overlaps(const Range& a, const Range& b) {
+    return a.begin < b.begin + b.bytes && b.begin < a.begin + a.bytes;
+}
+
+// Resolves a view to a device pointer after ownership, bounds and alignment
+// checks.  `elements` is the number of dtype-sized elements the op touches.
+fh_status resolve(const fh_device* device, const fh_view* view, uint64_t elements, const char* what,
+                  Range* out, size_t alignment = 16) {
+    if (view == nullptr || view->buffer == nullptr)
+        return fail(FH_ERR_RANGE, "%s: null view", what);
+    if (view->dtype > FH_BF16) return fail(FH_ERR_DTYPE, "%s: unknown dtype %u", what, view->dtype);
+    if (view->buffer->device != device) {
+        g_last_error = std::string(what) + ": buffer belongs to another device";
+        return FH_ERR_DEVICE_MISMATCH;
+    }
+    uint64_t bytes = elements * dtype_bytes(view->dtype);
+    if (view->offset > view->buffer->bytes || bytes > view->buffer->bytes - view->offset)
+        return fail(FH_ERR_RANGE, "%s: view [%zu, +%llu) exceeds buffer of %zu bytes", what,
+                    view->offset, (unsigned long long)bytes, view->buffer->bytes);
+    if (view->offset % alignment != 0)
+        return fail(FH_ERR_RANGE, "%s: offset %zu is not %zu-byte aligned", what, view->offset,
+                    alignment);
+    out->begin = static_cast<const uint8_t*>(view->buffer->ptr) + view->offset;
+    out->bytes = (size_t)bytes;
+    return FH_OK;
+}
+
+bool fits_u32(uint64_t v) { return v <= 0xffffffffull; }
+
+int64_t tuning(const fh_device* d, const char* key) {
+    auto it = d->tuning.find(key);
+    return it == d->tuning.end() ? 0 : it->second;
+}
+
+}  // namespace
+}  // namespace fh
+
+using namespace fh;
+
+extern "C" {
+
+const char* fh_last_error(void) { return g_last_error.c_str(); }
+
+fh_status fh_device_create(int32_t ordinal, fh_device** out) {
+    if (out == nullptr) return fail(FH_ERR_PARAMETER, "fh_device_create: null output");
+    *out = nullptr;
+    int count = 0;
+    FH_HIP(hipGetDeviceCount(&count));
+    if (ordinal < 0 || ordinal >= count)
+        return fail(FH_ERR_DISPATCH, "no HIP device %d (found %d)", ordinal, count);
+    FH_HIP(hipSetDevice(ordinal));
+    fh_device* d = new (std::nothrow) fh_device();
+    if (d == nullptr) return fail(FH_ERR_ALLOCATION, "out of host memory");
+    d->ordinal = ordinal;
+    hipError_t e = hipGetDeviceProperties(&d->props, ordinal);
+    if (e != hipSuccess) {
+        delete d;
+        return hip_fail(e, "hipGetDeviceProperties");
+    }
+    if (std::strncmp(d->props.gcnArchName, "gfx950", 6) != 0) {
+        fh_status st = fail(FH_ERR_DISPATCH, "kernels are built for gfx950 only; device %d is %s",
+                            ordinal, d->props.gcnArchName);
+        delete d;
+        return st;
+    }
+    e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete d;
+        return hip_fail(e, "hipStreamCreateWithFlags");
+    }
+    d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
+    d->tuning["gemv_rows_per_wave"] = 0;    // 0 = automatic
+    d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
+    *out = d;
+    return FH_OK;
+}
+
+void fh_device_destroy(fh_device* device) {
+    if (device == nullptr) return;
+    (void)hipSetDevice(device->ordinal);
+    if (device->stream) {
+        (void)hipStreamSynchronize(device->stream);
+        (void)hipStreamDestroy(device->stream);
+    }
+    if (device->scratch) (void)hipFree(device->scratch);
+    delete device;
+}
+
+fh_status fh_device_properties(const fh_device* device, fh_device_props* out) {
+    if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", device->props.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", device->props.gcnArchName);
+    out->compute_units = device->props.multiProcessorCount;
+    out->wavefront = device->props.warpSize;
+    out->clock_khz = device->props.clockRate;
+    out->memory_clock_khz = device->props.memoryClockRate;
+    out->memory_bus_bits = device->props.memoryBusWidth;
+    out->lds_bytes_per_block = (int32_t)device->props.sharedMemPerBlock;
+    out->global_bytes = device->props.totalGlobalMem;
+    out->l2_bytes = (uint64_t)device->props.l2CacheSize;
+    return FH_OK;
+}
+
+fh_status fh_synchronize(fh_device* device) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null device");
+    hipError_t e = hipStreamSynchronize(device->stream);
+    if (e != hipSuccess) return fail(FH_ERR_SYNCHRONIZATION, "stream: %s", hipGetErrorString(e));
+    return FH_OK;
+}
+
+const char* fh_last_operation(const fh_device* device) {
+    return device ? device->last_operation : "";
+}
+
+void* fh_device_stream(fh_device* device) { return device ? device->stream : nullptr; }
+
+fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
+    if (device == nullptr || key == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    auto it = device->tuning.find(key);
+    if (it == device->tuning.end()) return fail(FH_ERR_PARAMETER, "unknown tuning key %s", key);
+    std::string k(key);
+    bool ok = true;
+    if (k == "k_quant_gemv_ksplit") {
+        // set_k_quant_gemv_ksplit: 0 or a power of two up to 8
+        ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
+    } else if (k == "gemv_rows_per_wave") {
+        ok = value == 0 || value == 1 || value == 2 || value == 4;
+    } else if (k == "gemm_min_rows") {
+        ok = value >= 2;
+    }
+    if (!ok) return fail(FH_ERR_PARAMETER, "value %lld is out of range for %s", (long long)value, key);
+    it->second = value;
+    return FH_OK;
+}
+
+fh_status fh_get_tuning(const fh_device* device, const char* key, int64_t* value) {
+    if (device == nullptr || key == nullptr || value == nullptr)
+        return fail(FH_ERR_PARAMETER, "null argument");
+    auto it = device->tuning.find(key);
+    if (it == device->tuning.end()) return fail(FH_ERR_PARAMETER, "unknown tuning key %s", key);
+    *value = it->second;
+    return FH_OK;
+}
+
+// ---- buffers -------------------------------------------------------------------
+
+fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out) {
+    if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    *out = nullptr;
+    if (bytes == 0) return fail(FH_ERR_ALLOCATION, "zero-length buffer");
+    FH_HIP(hipSetDevice(device->ordinal));
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+    e = hipMemsetAsync(p, 0, bytes, device->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(p);
+        return hip_fail(e, "hipMemsetAsync");
+    }
+    fh_buffer* b = new (std::nothrow) fh_buffer();
+    if (b == nullptr) {
+        (void)hipFree(p);
+        return fail(FH_ERR_ALLOCATION, "out of host memory");
+    }
+    b->device = device;
+    b->ptr = p;
+    b->bytes = bytes;
+    *out = b;
+    return FH_OK;
+}
+
+void fh_buffer_free(fh_buffer* buffer) {
+    if (buffer == nullptr) return;
+    if (buffer->device) (void)hipStreamSynchronize(buffer->device->stream);
+    (void)hipFree(buffer->ptr);
+    delete buffer;
+}
+
+size_t fh_buffer_size(const fh_buffer* buffer) { return buffer ? buffer->bytes : 0; }
+void* fh_buffer_device_ptr(fh_buffer* buffer) { return buffer ? buffer->ptr : nullptr; }
+
+fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, size_t bytes) {
+    if (buffer == nullptr || (src == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
+    if (offset > buffer->bytes || bytes > buffer->bytes - offset)
+        return fail(FH_ERR_RANGE, "upload [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
+                    buffer->bytes);
+    if (bytes == 0) return FH_OK;
+    hipStream_t s = buffer->device->stream;
+    FH_HIP(hipMemcpyAsync(static_cast<uint8_t*>(buffer->ptr) + offset, src, bytes,
+                          hipMemcpyHostToDevice, s));
+    FH_HIP(hipStreamSynchronize(s));
+    return FH_OK;
+}
+
+fh_status fh_buffer_download(const fh_buffer* buffer, size_t offset, void* dst, size_t bytes) {
+    if (buffer == nullptr || (dst == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
+    if (offset > buffer->bytes || bytes > buffer->bytes - offset)
+        return fail(FH_ERR_RANGE, "download [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
+                    buffer->bytes);
+    if (bytes == 0) return FH_OK;
+    hipStream_t s = buffer->device->stream;
+    hipError_t e = hipMemcpyAsync(dst, static_cast<const uint8_t*>(buffer->ptr) + offset, bytes,
+                                  hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return hip_fail(e, "hipMemcpyAsync");
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return fail(FH_ERR_SYNCHRONIZATION, "stream: %s", hipGetErrorString(e));
+    return FH_OK;
+}
+
+fh_status fh_buffer_fill_zero(fh_buffer* buffer, size_t offset, size_t bytes) {
+    if (buffer == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (offset > buffer->bytes || bytes > buffer->bytes - offset)
+        return fail(FH_ERR_RANGE, "fill exceeds buffer");
+    if (bytes == 0) return FH_OK;
+    FH_HIP(hipMemsetAsync(static_cast<uint8_t*>(buffer->ptr) + offset, 0, bytes,
+                          buffer->device->stream));
+    return FH_OK;
+}
+
+// ---- packed weights --------------------------------------------------------------
+
+static bool f16_finite(const uint8_t* p) { return ((p[1] >> 2) & 0x1f) != 0x1f; }
+
+fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows, uint64_t cols,
+                            uint64_t experts, const void* packed, size_t packed_len,
+                            fh_qmatrix** out) {
+    if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    *out = nullptr;
+    const size_t bb = block_bytes(ggml_type);
+    if (bb == 0) return fail(FH_ERR_GGUF, "unsupported quantized weight type %u", ggml_type);
+    const char* name = ggml_type == kQ4K ? "Q4_K" : "Q6_K";
+    if (rows == 0 || cols == 0 || cols % 256 != 0)
+        return fail(FH_ERR_SHAPE, "%s matrix requires nonempty rows and columns divisible by block size 256",
+                    name);
+    if (experts == 0) return fail(FH_ERR_SHAPE, "quantized expert matrix row geometry mismatch");
+    unsigned __int128 total_rows = (unsigned __int128)rows * experts;
+    unsigned __int128 byte_len = total_rows * (cols / 256) * bb;
+    if (total_rows > 0xffffffffull || byte_len > (unsigned __int128)SIZE_MAX / 2)
+        return fail(FH_ERR_SHAPE, "packed matrix byte size overflow");
+    if (packed == nullptr) return fail(FH_ERR_PARAMETER, "null payload");
+    if (packed_len % bb != 0)
+        return fail(FH_ERR_GGUF, "tensor %s stream ended inside a block", name);
+    if ((unsigned __int128)packed_len != byte_len)
+        return fail(FH_ERR_SHAPE, "%s payload is %zu bytes, geometry needs %llu", name, packed_len,
+                    (unsigned long long)byte_len);
+    const uint8_t* p = static_cast<const uint8_t*>(packed);
+    for (size_t off = 0; off < packed_len; off += bb) {
+        bool ok = ggml_type == kQ4K ? (f16_finite(p + off) && f16_finite(p + off + 2))
+                                    : f16_finite(p + off + 208);
+        if (!ok) return fail(FH_ERR_WEIGHT, "%s scale must be finite", name);
+    }
+    FH_HIP(hipSetDevice(device->ordinal));
+    void* dptr = nullptr;
+    // 16 spare bytes keep vector loads of the last block inside the allocation
+    hipError_t e = hipMalloc(&dptr, packed_len + 16);
+    if (e != hipSuccess)
+        return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", packed_len, hipGetErrorString(e));
+    e = hipMemcpyAsync(dptr, packed, packed_len, hipMemcpyHostToDevice, device->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(static_cast<uint8_t*>(dptr) + packed_len, 0, 16, device->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(device->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(dptr);
+        return hip_fail(e, "weight upload");
+    }
+    fh_qmatrix* m = new (std::nothrow) fh_qmatrix();
+    if (m == nullptr) {
+        (void)hipFree(dptr);
+        return fail(FH_ERR_ALLOCATION, "out of host memory");
+    }
+    m->device = device;
+    m->ptr = dptr;
+    m->bytes = packed_len;
+    m->ggml_type = ggml_type;
+    m->rows = rows;
+    m->cols = cols;
+    m->experts = experts;
+    *out = m;
+    return FH_OK;
+}
+
+void fh_qmatrix_destroy(fh_qmatrix* matrix) {
+    if (matrix == nullptr) return;
+    if (matrix->device) (void)hipStreamSynchronize(matrix->device->stream);
+    (void)hipFree(matrix->ptr);
+    delete matrix;
+}
+
+uint64_t fh_qmatrix_rows(const fh_qmatrix* m) { return m ? m->rows : 0; }
+uint64_t fh_qmatrix_columns(const fh_qmatrix* m) { return m ? m->cols : 0; }
+uint64_t fh_qmatrix_experts(const fh_qmatrix* m) { return m ? m->experts : 0; }
+uint32_t fh_qmatrix_ggml_type(const fh_qmatrix* m) { return m ? m->ggml_type : 0; }
+size_t fh_qmatrix_byte_size(const fh_qmatrix* m) { return m ? m->bytes : 0; }
+void* fh_qmatrix_device_ptr(fh_qmatrix* m) { return m ? m->ptr : nullptr; }
+
+fh_status fh_dequantize(fh_device* device, const fh_qmatrix* weight, const fh_view* out) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device) return fail(FH_ERR_DEVICE_MISMATCH, "weight belongs to another device");
+    const uint64_t rows = weight->rows * weight->experts;
+    Range o;
+    fh_status st = resolve(device, out, rows * weight->cols, "dequantize output", &o);
+    if (st != FH_OK) return st;
+    device->last_operation = launch_dequantize(device->stream, weight->ggml_type, weight->ptr, rows,
+                                               weight->cols, const_cast<uint8_t*>(o.begin), out->dtype);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* weight,
+                                        const uint32_t* tokens, size_t count, const fh_view* out) {
+    if (device == nullptr || weight == nullptr || (tokens == nullptr && count))
+        return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device) return fail(FH_ERR_DEVICE_MISMATCH, "weight belongs to another device");
+    const uint64_t rows = weight->rows * weight->experts;
+    for (size_t i = 0; i < count; ++i)
+        if (tokens[i] >= rows)
+            return fail(FH_ERR_TOKEN, "token id %u is outside vocabulary of %llu", tokens[i],
+                        (unsigned long long)rows);
+    if (count == 0) return FH_OK;
+    if (!fits_u32((uint64_t)count * weight->cols)) return fail(FH_ERR_SHAPE, "gather size overflow");
+    Range o;
+    fh_status st = resolve(device, out, (uint64_t)count * weight->cols, "gather output", &o);
+    if (st != FH_OK) return st;
+    // ids travel through the device scratch (the reference carries them in a tensor)
+    size_t need = count * sizeof(uint32_t);
+    if (device->scratch_bytes < need) {
+        FH_HIP(hipStreamSynchronize(device->stream));
+        if (device->scratch) (void)hipFree(device->scratch);
+        device->scratch = nullptr;
+        device->scratch_bytes = 0;
+        size_t cap = need < (1u << 20) ? (1u << 20) : need;
+        hipError_t e = hipMalloc(&device->scratch, cap);
+        if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", cap, hipGetErrorString(e));
+        device->scratch_bytes = cap;
+    }
+    FH_HIP(hipMemcpyAsync(device->scratch, tokens, need, hipMemcpyHostToDevice, device->stream));
+    FH_HIP(hipStreamSynchronize(device->stream));
+    device->last_operation =
+        launch_embedding_gather(device->stream, weight->ggml_type, weight->ptr, weight->cols,
+                                static_cast<const uint32_t*>(device->scratch), count,
+                                const_cast<uint8_t*>(o.begin), out->dtype);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ---- dense projection --------------------------------------------------------------
+
+fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                               uint32_t m, const fh_view* y) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device) {
+        g_last_error = "weight belongs to another device";
+        return FH_ERR_DEVICE_MISMATCH;
+    }
+    const uint64_t n = weight->rows * weight->experts, k = weight->cols;
+    if (m == 0 || k > 0xffffffffull - 32)
+        return fail(FH_ERR_SHAPE, "quantized projection requires [M,K] matching [N,K]");
+    if (!fits_u32((uint64_t)m * k) || !fits_u32((uint64_t)m * n) || !fits_u32(n))
+        return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+    Range xr, yr;
+    fh_status st = resolve(device, x, (uint64_t)m * k, "projection input", &xr);
+    if (st != FH_OK) return st;
+    st = resolve(device, y, (uint64_t)m * n, "projection output", &yr);
+    if (st != FH_OK) return st;
+    if (overlaps(xr, yr)) return fail(FH_ERR_RANGE, "projection output aliases its input");
+
+    const bool tile = m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32;
+    if (tile) {
+        GemmArgs a{};
+        a.ggml_type = weight->ggml_type;
+        a.w = weight->ptr;
+        a.x = xr.begin;
+        a.y = const_cast<uint8_t*>(yr.begin);
+        a.n = (uint32_t)n;
+        a.k = (uint32_t)k;
+        a.m = m;
+        a.x_dtype = x->dtype;
+        a.y_dtype = y->dtype;
+        a.cu_count = device->props.multiProcessorCount;
+        device->last_operation = launch_gemm(device->stream, a);
+    } else {
+        GemvArgs a{};
+        a.ggml_type = weight->ggml_type;
+        a.w = weight->ptr;
+        a.x = xr.begin;
+        a.y = const_cast<uint8_t*>(yr.begin);
+        a.n = (uint32_t)n;
+        a.k = (uint32_t)k;
+        a.m = m;
+        a.x_dtype = x->dtype;
+        a.y_dtype = y->dtype;
+        a.metadata = nullptr;
+        a.experts = 1;
+        int64_t ks = tuning(device, "k_quant_gemv_ksplit");
+        a.ksplit = (int)(ks > 4 ? 4 : ks);
+        a.rows_per_wave = (int)tuning(device, "gemv_rows_per_wave");
+        a.cu_count = device->props.multiProcessorCount;
+        const char* name = launch_gemv(device->stream, a);
+        if (m > 1) name = weight->ggml_type == kQ4K ? "q4_k_gemm" : "q6_k_gemm";
+        device->last_operation = name;
+    }
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ---- mixture of experts -------------------------------------------------------------
+
+fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
+                       const fh_view* selection_bias, const fh_routing_policy* policy,
+                       const fh_view* metadata) {
+    if (device == nullptr || policy == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    const fh_routing_policy& p = *policy;
+    if (tokens == 0 || p.experts == 0 || p.top_k == 0 || p.top_k > 16 || p.top_k > p.experts ||
+        !std::isfinite(p.normalization_epsilon) || p.normalization_epsilon < 0.f ||
+        !std::isfinite(p.routed_scaling_factor) || p.routed_scaling_factor <= 0.f)
+        return fail(FH_ERR_SHAPE, "invalid sparse routing geometry");
+    if (p.experts > 1024) return fail(FH_ERR_SHAPE, "routing supports at most 1024 experts");
+    if (!fits_u32((uint64_t)tokens * p.top_k * 3) || !fits_u32((uint64_t)tokens * p.experts))
+        return fail(FH_ERR_SHAPE, "expert assignment count overflow");
+    Range lr, mr, br{nullptr, 0};
+    fh_status st = resolve(device, logits, (uint64_t)tokens * p.experts, "router logits", &lr, 4);
+    if (st != FH_OK) return st == FH_ERR_DEVICE_MISMATCH ? fail(FH_ERR_SHAPE, "invalid sparse routing geometry") : st;
+    if (selection_bias != nullptr) {
+        if (selection_bias->dtype != FH_F32) return fail(FH_ERR_SHAPE, "invalid sparse routing geometry");
+        st = resolve(device, selection_bias, p.experts, "selection bias", &br, 4);
+        if (st != FH_OK) return st == FH_ERR_DEVICE_MISMATCH ? fail(FH_ERR_SHAPE, "invalid sparse routing geometry") : st;
+    }
+    if (metadata == nullptr || metadata->dtype != FH_F32)
+        return fail(FH_ERR_DTYPE, "routing metadata must be f32");
+    st = resolve(device, metadata, (uint64_t)tokens * p.top_k * 3, "routing metadata", &mr, 4);
+    if (st != FH_OK) return st;
+    if (overlaps(lr, mr)) return fail(FH_ERR_RANGE, "routing metadata aliases the logits");
+    device->last_operation = launch_moe_route(
+        device->stream, lr.begin, logits->dtype, reinterpret_cast<const float*>(br.begin),
+        reinterpret_cast<float*>(const_cast<uint8_t*>(mr.begin)), tokens, p);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t tokens,
+                           uint32_t width, const fh_view* metadata, uint32_t top_k,
+                           const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (tokens == 0 || width == 0 || top_k == 0 || metadata == nullptr || metadata->dtype != FH_F32 ||
+        !fits_u32((uint64_t)tokens * top_k) || !fits_u32((uint64_t)tokens * top_k * width))
+        return fail(FH_ERR_SHAPE, "expert assignments require [S,H] and [S*top_k,3]");
+    const uint32_t assignments = tokens * top_k;
+    Range hr, mr, orr;
+    fh_status st = resolve(device, hidden, (uint64_t)tokens * width, "assign input", &hr);
+    if (st != FH_OK) return st;
+    st = resolve(device, metadata, (uint64_t)assignments * 3, "assign metadata", &mr, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, out, (uint64_t)assignments * width, "assign output", &orr);
+    if (st != FH_OK) return st;
+    if (out->dtype != hidden->dtype) return fail(FH_ERR_DTYPE, "assign output dtype differs from input");
+    if (overlaps(hr, orr) || overlaps(mr, orr)) return fail(FH_ERR_RANGE, "assign output aliases an input");
+    device->last_operation = launch_expert_assign(
+        device->stream, hr.begin, reinterpret_cast<const float*>(mr.begin),
+        const_cast<uint8_t*>(orr.begin), assignments, width * (uint32_t)dtype_bytes(hidden->dtype));
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weight,
+                                      const fh_view* x, uint32_t assignments,
+                                      const fh_view* metadata, const fh_view* y) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device || assignments == 0 || metadata == nullptr ||
+        metadata->dtype != FH_F32 || metadata->buffer == nullptr ||
+        metadata->buffer->device != device || x == nullptr || x->buffer == nullptr ||
+        x->buffer->device != device)
+        return fail(FH_ERR_SHAPE, "quantized expert projection geometry mismatch");
+    const uint64_t rows = weight->rows, k = weight->cols;
+    if (!fits_u32((uint64_t)assignments * rows) || !fits_u32((uint64_t)assignments * k))
+        return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+    Range xr, mr, yr;
+    fh_status st = resolve(device, x, (uint64_t)assignments * k, "expert input", &xr);
+    if (st != FH_OK) return st;
+    st = resolve(device, metadata, (uint64_t)assignments * 3, "expert metadata", &mr, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, y, (uint64_t)assignments * rows, "expert output", &yr);
+    if (st != FH_OK) return st;
+    if (overlaps(xr, yr) || overlaps(mr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    GemvArgs a{};
+    a.ggml_type = weight->ggml_type;
+    a.w = weight->ptr;
+    a.x = xr.begin;
+    a.y = const_cast<uint8_t*>(yr.begin);
+    a.n = (uint32_t)rows;
+    a.k = (uint32_t)k;
+    a.m = assignments;
+    a.x_dtype = x->dtype;
+    a.y_dtype = y->dtype;
+    a.metadata = reinterpret_cast<const float*>(mr.begin);
+    a.experts = (uint32_t)weight->experts;
+    a.ksplit = 0;
+    a.rows_per_wave = 0;
+    a.cu_count = device->props.multiProcessorCount;
+    device->last_operation = launch_gemv(device->stream, a);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assignments,
+                             uint32_t intermediate, const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (assignments == 0 || intermediate == 0 || !fits_u32((uint64_t)assignments * intermediate * 2))
+        return fail(FH_ERR_SHAPE, "packed expert activation geometry mismatch");
+    Range ir, orr;
+    fh_status st = resolve(device, in, (uint64_t)assignments * intermediate * 2, "silu_mul input", &ir, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, out, (uint64_t)assignments * intermediate, "silu_mul output", &orr, 4);
+    if (st != FH_OK) return st;
+    if (overlaps(ir, orr)) return fail(FH_ERR_RANGE, "silu_mul output aliases its input");
+    device->last_operation = launch_expert_silu_mul(device->stream, ir.begin,
+                                                    const_cast<uint8_t*>(orr.begin), assignments,
+                                                    intermediate, in->dtype, out->dtype);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
+                            uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (top_k == 0 || hidden == 0 || tokens == 0 || metadata == nullptr || metadata->dtype != FH_F32 ||
+        !fits_u32((uint64_t)tokens * top_k * hidden))
+        return fail(FH_ERR_SHAPE, "expert combine geometry mismatch");
+    Range ir, mr, orr;
+    fh_status st = resolve(device, in, (uint64_t)tokens * top_k * hidden, "combine input", &ir, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, metadata, (uint64_t)tokens * top_k * 3, "combine metadata", &mr, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, out, (uint64_t)tokens * hidden, "combine output", &orr, 4);
+    if (st != FH_OK) return st;
+    if (overlaps(ir, orr) || overlaps(mr, orr)) return fail(FH_ERR_RANGE, "combine output aliases an input");
+    device->last_operation = launch_expert_combine(
+        device->stream, ir.begin, reinterpret_cast<const float*>(mr.begin),
+        const_cast<uint8_t*>(orr.begin), tokens, hidden, top_k, in->dtype, out->dtype);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ---- timing ---------------------------------------------------------------------------
+
+fh_status fh_event_create(fh_device* device, fh_event** out) {
+    if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    *out = nullptr;
+    fh_event* ev = new (std::nothrow) fh_event();
+    if (ev == nullptr) return fail(FH_ERR_ALLOCATION, "out of host memory");
+    hipError_t e = hipEventCreate(&ev->event);
+    if (e != hipSuccess) {
+        delete ev;
+        return hip_fail(e, "hipEventCreate");
+    }
+    ev->device = device;
+    *out = ev;
+    return FH_OK;
+}
+
+void fh_event_destroy(fh_event* event) {
+    if (event == nullptr) return;
+    (void)hipEventDestroy(event->event);
+    delete event;
+}
+
+fh_status fh_event_record(fh_event* event) {
+    if (event == nullptr) return fail(FH_ERR_PARAMETER, "null event");
+    FH_HIP(hipEventRecord(event->event, event->device->stream));
+    return FH_OK;
+}
+
+fh_status fh_event_elapsed_ms(fh_event* start, fh_event* stop, float* ms) {
+    if (start == nullptr || stop == nullptr || ms == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    hipError_t e = hipEventSynchronize(stop->event);
+    if (e != hipSuccess) return fail(FH_ERR_SYNCHRONIZATION, "event: %s", hipGetErrorString(e));
+    FH_HIP(hipEventElapsedTime(ms, start->event, stop->event));
+    return FH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,118 @@
+// Whole-matrix dequantisation and embedding gather for GGUF Q4_K / Q6_K.
+//
+// Values follow the reference's per-element decoders (q4_k_weight,
+// src/metal/shaders/ops.metal:834-845; q6_k_weight, :1316-1329); the gather
+// kernels stand in for embedding_gather_q4_k / _q6_k (:1122-1127, 1486-1491).
+// One thread produces four consecutive columns, so stores are 16 bytes (f32)
+// or 8 bytes (f16 / bf16) and each 144- or 210-byte block is read by 64
+// neighbouring threads.
+#include "device_utils.hpp"
+#include "internal.hpp"
+
+namespace fh {
+namespace {
+
+template <uint32_t TYPE>
+__device__ __forceinline__ float weight_at(const uint8_t* w, size_t row, uint32_t column,
+                                           uint32_t blocks) {
+    if constexpr (TYPE == kQ4K) {
+        return q4k_weight(w, row, column, blocks);
+    } else {
+        return q6k_weight(w, row, column, blocks);
+    }
+}
+
+template <uint32_t TYPE>
+__device__ __forceinline__ void emit4(const uint8_t* w, size_t src_row, size_t dst_row,
+                                      uint32_t column, uint32_t cols, void* out, uint32_t dtype) {
+    uint32_t blocks = cols >> 8;
+    float v0 = weight_at<TYPE>(w, src_row, column, blocks);
+    float v1 = weight_at<TYPE>(w, src_row, column + 1, blocks);
+    float v2 = weight_at<TYPE>(w, src_row, column + 2, blocks);
+    float v3 = weight_at<TYPE>(w, src_row, column + 3, blocks);
+    size_t base = dst_row * cols + column;
+    if (dtype == 0) {
+        *reinterpret_cast<float4*>(static_cast<float*>(out) + base) = make_float4(v0, v1, v2, v3);
+    } else {
+        uint32_t lo, hi;
+        if (dtype == 1) {
+            lo = f32_to_f16_bits(v0) | (f32_to_f16_bits(v1) << 16);
+            hi = f32_to_f16_bits(v2) | (f32_to_f16_bits(v3) << 16);
+        } else {
+            lo = f32_to_bf16_bits(v0) | (f32_to_bf16_bits(v1) << 16);
+            hi = f32_to_bf16_bits(v2) | (f32_to_bf16_bits(v3) << 16);
+        }
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + base) = make_uint2(lo, hi);
+    }
+}
+
+template <uint32_t TYPE>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t* __restrict__ w,
+                                                         size_t rows, uint32_t cols,
+                                                         void* __restrict__ out, uint32_t dtype) {
+    uint32_t quads_per_row = cols >> 2;
+    size_t total = rows * quads_per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t row = i / quads_per_row;
+        uint32_t column = (uint32_t)(i % quads_per_row) << 2;
+        emit4<TYPE>(w, row, row, column, cols, out, dtype);
+    }
+}
+
+template <uint32_t TYPE>
+__global__ __launch_bounds__(256) void embedding_gather_kernel(const uint8_t* __restrict__ w,
+                                                               uint32_t cols,
+                                                               const uint32_t* __restrict__ ids,
+                                                               size_t count,
+                                                               void* __restrict__ out,
+                                                               uint32_t dtype) {
+    uint32_t quads_per_row = cols >> 2;
+    size_t total = count * quads_per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t token = i / quads_per_row;
+        uint32_t column = (uint32_t)(i % quads_per_row) << 2;
+        emit4<TYPE>(w, ids[token], token, column, cols, out, dtype);
+    }
+}
+
+unsigned grid_for(size_t threads) {
+    size_t blocks = (threads + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (blocks == 0) blocks = 1;
+    return (unsigned)blocks;
+}
+
+}  // namespace
+
+const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, size_t rows,
+                              size_t cols, void* out, uint32_t out_dtype) {
+    unsigned grid = grid_for(rows * (cols / 4));
+    if (ggml_type == kQ4K) {
+        hipLaunchKernelGGL(dequantize_kernel<kQ4K>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
+        return "dequantize_q4_k";
+    }
+    hipLaunchKernelGGL(dequantize_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
+    return "dequantize_q6_k";
+}
+
+const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const void* w, size_t cols,
+                                    const uint32_t* ids_dev, size_t count, void* out,
+                                    uint32_t out_dtype) {
+    unsigned grid = grid_for(count * (cols / 4));
+    if (ggml_type == kQ4K) {
+        hipLaunchKernelGGL(embedding_gather_kernel<kQ4K>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
+                           out_dtype);
+        return "embedding_gather_q4_k";
+    }
+    hipLaunchKernelGGL(embedding_gather_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
+                       static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
+                       out_dtype);
+    return "embedding_gather_q6_k";
+}
+
+}  // namespace fh

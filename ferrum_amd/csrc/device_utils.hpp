@@ -1,0 +1,179 @@
+// Device-side helpers shared by the kernels: storage dtypes, GGUF K-quant field
+// extraction and 64-lane wave reductions.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace fh {
+
+constexpr int kWave = 64;
+
+// ---- storage dtypes (0 f32, 1 f16, 2 bf16) ------------------------------------
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(bits)));
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) {
+    return __uint_as_float(bits << 16);
+}
+
+// Round to nearest even; NaN keeps its payload with the quiet bit set
+// (the reference's store(), src/metal/shaders/ops.metal:11-20).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
+    uint32_t bits = __float_as_uint(x);
+    if (x != x) return (bits >> 16) | 0x40u;
+    return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float x) {
+    return __half_as_ushort(__float2half_rn(x));
+}
+
+template <int DT>
+__device__ __forceinline__ float load_as_f32(const void* p, size_t i) {
+    if constexpr (DT == 0) {
+        return static_cast<const float*>(p)[i];
+    } else if constexpr (DT == 1) {
+        return f16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    } else {
+        return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    }
+}
+
+__device__ __forceinline__ float load_as_f32(const void* p, size_t i, uint32_t dtype) {
+    if (dtype == 0) return static_cast<const float*>(p)[i];
+    uint32_t bits = static_cast<const uint16_t*>(p)[i];
+    return dtype == 1 ? f16_bits_to_f32(bits) : bf16_bits_to_f32(bits);
+}
+
+__device__ __forceinline__ void store_from_f32(void* p, size_t i, uint32_t dtype, float v) {
+    if (dtype == 0) {
+        static_cast<float*>(p)[i] = v;
+    } else if (dtype == 1) {
+        static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_f16_bits(v));
+    } else {
+        static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    }
+}
+
+__device__ __forceinline__ float round_storage(float v, uint32_t dtype) {
+    if (dtype == 1) return f16_bits_to_f32(f32_to_f16_bits(v));
+    if (dtype == 2) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    return v;
+}
+
+// 16-byte and 2-byte loads from addresses that are only 2-byte aligned (Q6_K
+// blocks are 210 bytes); gfx950 global loads accept unaligned addresses.
+__device__ __forceinline__ uint4 load_u4_unaligned(const uint8_t* p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+__device__ __forceinline__ uint32_t load_u16_unaligned(const uint8_t* p) {
+    uint16_t v;
+    __builtin_memcpy(&v, p, 2);
+    return v;
+}
+
+// ---- Q4_K (144 B: f16 d, f16 dmin, 12 B scales, 128 B nibbles) ----------------
+
+// 6-bit scale and minimum of 32-weight group `group` (0..7).
+__device__ __forceinline__ void q4k_scale_min(const uint8_t* s, uint32_t group, uint32_t& sc,
+                                              uint32_t& mn) {
+    if (group < 4) {
+        sc = s[group] & 63u;
+        mn = s[group + 4] & 63u;
+    } else {
+        sc = (s[group + 4] & 15u) | ((uint32_t)(s[group - 4] >> 6) << 4);
+        mn = (uint32_t)(s[group + 4] >> 4) | ((uint32_t)(s[group] >> 6) << 4);
+    }
+}
+
+// Scales and minimums of the two 32-weight groups 2c and 2c+1 that share the
+// 32 quant bytes of chunk c (0..3), from the header words {bytes 4..7, 8..11,
+// 12..15 of the block}.  Groups 4..7 keep their low nibbles in bytes 8..11
+// and their top two bits in bits 6..7 of bytes 0..7.
+__device__ __forceinline__ void q4k_chunk_scales(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t c,
+                                                 float& sc_lo, float& sc_hi, float& mn_lo,
+                                                 float& mn_hi) {
+    bool upper = c >= 2;
+    uint32_t scw = upper ? ((s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)) : (s0 & 0x3f3f3f3fu);
+    uint32_t mnw = upper ? (((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u))
+                         : (s1 & 0x3f3f3f3fu);
+    uint32_t shift = (c & 1u) << 4;
+    scw >>= shift;
+    mnw >>= shift;
+    sc_lo = (float)(scw & 0xffu);
+    sc_hi = (float)((scw >> 8) & 0xffu);
+    mn_lo = (float)(mnw & 0xffu);
+    mn_hi = (float)((mnw >> 8) & 0xffu);
+}
+
+// One dequantised weight, ((d*sc)*q) - (dmin*m) with each step rounded to f32.
+// d and dmin carry 11 significant bits, so both products are exact and only
+// the subtraction rounds; the value is therefore independent of contraction.
+__device__ __forceinline__ float q4k_weight(const uint8_t* w, size_t row, uint32_t column,
+                                            uint32_t blocks) {
+    const uint8_t* block = w + (row * blocks + (column >> 8)) * 144;
+    uint32_t within = column & 255u, group = within >> 5, lane = within & 31u, chunk = within >> 6;
+    uint32_t byte = block[16 + chunk * 32 + lane];
+    uint32_t q = (group & 1u) ? (byte >> 4) : (byte & 15u);
+    float d = f16_bits_to_f32(block[0] | (block[1] << 8));
+    float dmin = f16_bits_to_f32(block[2] | (block[3] << 8));
+    uint32_t sc, mn;
+    q4k_scale_min(block + 4, group, sc, mn);
+    float a = d * (float)sc;
+    float b = a * (float)q;
+    float c = dmin * (float)mn;
+    return b - c;
+}
+
+// ---- Q6_K (210 B: ql[128], qh[64], int8 scales[16], f16 d) ---------------------
+
+__device__ __forceinline__ float q6k_weight(const uint8_t* w, size_t row, uint32_t column,
+                                            uint32_t blocks) {
+    const uint8_t* block = w + (row * blocks + (column >> 8)) * 210;
+    uint32_t within = column & 255u, group = within >> 5, lane = within & 31u;
+    uint32_t half_block = group >> 2, slice = group & 3u;
+    uint32_t byte = block[half_block * 64 + (slice & 1u) * 32 + lane];
+    uint32_t low = slice < 2 ? (byte & 15u) : (byte >> 4);
+    uint32_t high = ((uint32_t)block[128 + half_block * 32 + lane] >> (slice * 2)) & 3u;
+    int q = (int)(low | (high << 4)) - 32;
+    int scale = (int8_t)block[192 + half_block * 8 + slice * 2 + (lane >> 4)];
+    float d = f16_bits_to_f32(block[208] | (block[209] << 8));
+    float a = d * (float)scale;
+    return a * (float)q;
+}
+
+// ---- wave reductions -----------------------------------------------------------
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return v + __int_as_float(moved);
+}
+
+// Sum over the 64 lanes; every lane of the wave must be active.  The total is
+// returned in all lanes.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror: the other quad of each 8
+    v = dpp_add<0x140>(v);  // row_mirror: the other half of each 16
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+}  // namespace fh

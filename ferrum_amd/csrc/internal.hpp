@@ -1,0 +1,110 @@
+// Shared definitions of the gfx950 backend: device objects, error plumbing and
+// the host-side launchers each kernel file exports.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <string>
+
+#include "../../include/ferrum_hip.h"
+
+struct fh_device {
+    int ordinal = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t props{};
+    const char* last_operation = "";
+    std::map<std::string, int64_t> tuning;
+    // scratch owned by the device (K-split partials, MoE segment tables, ...)
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+};
+
+struct fh_buffer {
+    fh_device* device = nullptr;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+
+struct fh_qmatrix {
+    fh_device* device = nullptr;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    uint32_t ggml_type = 0;
+    uint64_t rows = 0;     // per expert
+    uint64_t cols = 0;
+    uint64_t experts = 1;
+};
+
+struct fh_event {
+    fh_device* device = nullptr;
+    hipEvent_t event = nullptr;
+};
+
+namespace fh {
+
+fh_status fail(fh_status code, const char* fmt, ...);
+fh_status hip_fail(hipError_t err, const char* what);
+
+constexpr uint32_t kQ4K = FH_GGML_Q4_K;
+constexpr uint32_t kQ6K = FH_GGML_Q6_K;
+
+inline size_t block_bytes(uint32_t ggml_type) {
+    return ggml_type == kQ4K ? 144 : ggml_type == kQ6K ? 210 : 0;
+}
+inline size_t dtype_bytes(uint32_t dtype) { return dtype == FH_F32 ? 4 : 2; }
+
+// ---- launchers (one per kernel family); each returns the kernel name ----
+
+// dequant.hip
+const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, size_t rows,
+                              size_t cols, void* out, uint32_t out_dtype);
+const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const void* w, size_t cols,
+                                    const uint32_t* ids_dev, size_t count, void* out,
+                                    uint32_t out_dtype);
+
+// gemv.hip
+struct GemvArgs {
+    uint32_t ggml_type;
+    const void* w;        // packed [n, k]
+    const void* x;        // [m, k]
+    void* y;              // [m, n]
+    uint32_t n, k, m;
+    uint32_t x_dtype, y_dtype;
+    // expert form: when metadata != nullptr, row m of x uses expert
+    // bits(metadata[3*m]) and weight rows [expert*n, expert*n + n)
+    const float* metadata;
+    uint32_t experts;
+    int ksplit;           // 0 = automatic
+    int rows_per_wave;    // 0 = automatic
+    int cu_count;
+};
+const char* launch_gemv(hipStream_t s, const GemvArgs& a);
+
+// gemm.hip
+struct GemmArgs {
+    uint32_t ggml_type;
+    const void* w;
+    const void* x;        // [m, k] f16 or bf16
+    void* y;              // [m, n]
+    uint32_t n, k, m;
+    uint32_t x_dtype, y_dtype;
+    int cu_count;
+};
+const char* launch_gemm(hipStream_t s, const GemmArgs& a);
+
+// moe.hip
+const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
+                             const float* bias, float* metadata, uint32_t tokens,
+                             const fh_routing_policy& policy);
+const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,
+                                 void* out, uint32_t assignments, uint32_t row_bytes);
+const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,
+                                   uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype);
+const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
+                                  uint32_t tokens, uint32_t hidden, uint32_t top_k,
+                                  uint32_t in_dtype, uint32_t out_dtype);
+
+}  // namespace fh

@@ -1,0 +1,251 @@
+// Mixture-of-experts helper stages on gfx950: routing, row gather, SiLU*up and
+// the weighted combine.  They stand in for moe_route, expert_assign,
+// expert_silu_mul and expert_combine of the reference
+// (src/metal/shaders/ops.metal:1894-1967, 2223-2246) and keep their rounding
+// points.  The routed projections themselves live in gemv.hip / gemm.hip.
+#include "device_utils.hpp"
+#include "internal.hpp"
+
+namespace fh {
+namespace {
+
+constexpr int kMaxPerLane = 16;  // experts <= 1024
+constexpr int kMaxTopK = 16;
+
+__device__ __forceinline__ uint32_t total_order_key(float x) {
+    uint32_t bits = __float_as_uint(x);
+    return (bits & 0x80000000u) ? ~bits : (bits ^ 0x80000000u);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t lo = __shfl_xor((uint32_t)v, off, 64);
+        uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, 64);
+        unsigned long long other = ((unsigned long long)hi << 32) | lo;
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
+// One wave per token.  Scores are computed by all lanes in parallel; the
+// softmax normaliser is then summed by one lane in expert order so it carries
+// the same f32 rounding as a sequential host loop.  Selection runs top_k
+// rounds of a wave-wide arg-max over (total-order key, lower id wins).
+__global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ logits,
+                                                       uint32_t logits_dtype,
+                                                       const float* __restrict__ bias,
+                                                       float* __restrict__ metadata,
+                                                       uint32_t tokens, uint32_t experts,
+                                                       uint32_t top_k, uint32_t sigmoid,
+                                                       uint32_t normalize, float eps,
+                                                       float scaling) {
+    extern __shared__ float scores_lds[];  // experts floats
+    const uint32_t token = blockIdx.x, lane = threadIdx.x;
+    if (token >= tokens) return;
+    const size_t base = (size_t)token * experts;
+
+    float score[kMaxPerLane];
+    float logit[kMaxPerLane];
+    float maximum = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        uint32_t e = lane + 64u * i;
+        logit[i] = e < experts ? load_as_f32(logits, base + e, logits_dtype) : -INFINITY;
+        maximum = fmaxf(maximum, logit[i]);
+    }
+    if (sigmoid) {
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) score[i] = 1.f / (1.f + expf(-logit[i]));
+    } else {
+        maximum = wave_max(maximum);
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) {
+            uint32_t e = lane + 64u * i;
+            score[i] = expf(logit[i] - maximum);
+            if (e < experts) scores_lds[e] = score[i];
+        }
+        __syncthreads();
+        float normalizer = 0.f;
+        if (lane == 0) {
+            for (uint32_t e = 0; e < experts; ++e) normalizer += scores_lds[e];
+        }
+        normalizer = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(normalizer)));
+#pragma unroll
+        for (int i = 0; i < kMaxPerLane; ++i) score[i] = score[i] / normalizer;
+    }
+
+    unsigned long long packed[kMaxPerLane];
+#pragma unroll
+    for (int i = 0; i < kMaxPerLane; ++i) {
+        uint32_t e = lane + 64u * i;
+        float selection = score[i] + (bias != nullptr && e < experts ? bias[e] : 0.f);
+        // 0 marks "not a candidate"; valid entries have low word >= 1
+        packed[i] = e < experts ? ((unsigned long long)total_order_key(selection) << 32) |
+                                      (0xffffffffu - e)
+                                : 0ull;
+    }
+
+    uint32_t sel_id[kMaxTopK];
+    float sel_score[kMaxTopK];
+#pragma unroll
+    for (int rank = 0; rank < kMaxTopK; ++rank) {
+        if ((uint32_t)rank < top_k) {
+            unsigned long long best = 0ull;
+#pragma unroll
+            for (int i = 0; i < kMaxPerLane; ++i) best = packed[i] > best ? packed[i] : best;
+            best = wave_max_u64(best);
+            uint32_t id = 0xffffffffu - (uint32_t)best;
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < kMaxPerLane; ++i) {
+                if (lane + 64u * i == id) {
+                    mine = score[i];
+                    packed[i] = 0ull;
+                }
+            }
+            // the owner lane publishes the raw score (bias excluded)
+            sel_score[rank] = __shfl(mine, id & 63u, 64);
+            sel_id[rank] = id;
+        } else {
+            sel_id[rank] = 0xffffffffu;
+            sel_score[rank] = 0.f;
+        }
+    }
+
+    float selected_sum = 0.f;
+#pragma unroll
+    for (int rank = 0; rank < kMaxTopK; ++rank)
+        if ((uint32_t)rank < top_k) selected_sum += sel_score[rank];
+    const float denominator = selected_sum + eps;
+
+    // Rows are written in expert-id order: lane r places entry r at the
+    // number of selected ids below its own.
+#pragma unroll
+    for (int rank = 0; rank < kMaxTopK; ++rank) {
+        if ((uint32_t)rank < top_k && lane == (uint32_t)rank) {
+            uint32_t position = 0;
+#pragma unroll
+            for (int other = 0; other < kMaxTopK; ++other)
+                if ((uint32_t)other < top_k && sel_id[other] < sel_id[rank]) ++position;
+            float weight = sel_score[rank];
+            if (normalize) weight = weight / denominator;
+            weight = weight * scaling;
+            float* out = metadata + ((size_t)token * top_k + position) * 3;
+            out[0] = __uint_as_float(sel_id[rank]);
+            out[1] = __uint_as_float(token);
+            out[2] = weight;
+        }
+    }
+}
+
+// out[a, :] = hidden[token(a), :]; rows are copied in pieces of sizeof(V).
+template <typename V>
+__global__ __launch_bounds__(256) void expert_assign_kernel(const V* __restrict__ hidden,
+                                                            const float* __restrict__ metadata,
+                                                            V* __restrict__ out,
+                                                            uint32_t assignments,
+                                                            uint32_t row_pieces) {
+    const uint32_t a = blockIdx.x;
+    if (a >= assignments) return;
+    const uint32_t token = __float_as_uint(metadata[3 * (size_t)a + 1]);
+    const V* src = hidden + (size_t)token * row_pieces;
+    V* dst = out + (size_t)a * row_pieces;
+    for (uint32_t i = threadIdx.x; i < row_pieces; i += blockDim.x) dst[i] = src[i];
+}
+
+__device__ __forceinline__ float silu(float gate) {
+    float s = gate >= 0.f ? 1.f / (1.f + expf(-gate)) : expf(gate) / (1.f + expf(gate));
+    return gate * s;
+}
+
+__global__ __launch_bounds__(256) void expert_silu_mul_kernel(const void* __restrict__ in,
+                                                              void* __restrict__ out,
+                                                              uint32_t assignments,
+                                                              uint32_t intermediate,
+                                                              uint32_t in_dtype,
+                                                              uint32_t out_dtype) {
+    size_t total = (size_t)assignments * intermediate;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t a = i / intermediate, column = i % intermediate;
+        size_t base = a * 2 * intermediate;
+        float gate = load_as_f32(in, base + column, in_dtype);
+        float up = load_as_f32(in, base + intermediate + column, in_dtype);
+        float activated = round_storage(silu(gate), out_dtype);
+        store_from_f32(out, i, out_dtype, activated * up);
+    }
+}
+
+__global__ __launch_bounds__(256) void expert_combine_kernel(const void* __restrict__ in,
+                                                             const float* __restrict__ metadata,
+                                                             void* __restrict__ out,
+                                                             uint32_t tokens, uint32_t hidden,
+                                                             uint32_t top_k, uint32_t in_dtype,
+                                                             uint32_t out_dtype) {
+    size_t total = (size_t)tokens * hidden;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t token = i / hidden, column = i % hidden;
+        float sum = 0.f;
+        for (uint32_t rank = 0; rank < top_k; ++rank) {
+            size_t a = token * top_k + rank;
+            float gate = round_storage(metadata[a * 3 + 2], out_dtype);
+            float value = load_as_f32(in, a * hidden + column, in_dtype);
+            sum += round_storage(gate * value, out_dtype);
+        }
+        store_from_f32(out, i, out_dtype, sum);
+    }
+}
+
+unsigned grid_for(size_t threads) {
+    size_t blocks = (threads + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (blocks == 0) blocks = 1;
+    return (unsigned)blocks;
+}
+
+}  // namespace
+
+const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
+                             const float* bias, float* metadata, uint32_t tokens,
+                             const fh_routing_policy& p) {
+    hipLaunchKernelGGL(moe_route_kernel, dim3(tokens), dim3(64), p.experts * sizeof(float), s,
+                       logits, logits_dtype, bias, metadata, tokens, p.experts, p.top_k, p.sigmoid,
+                       p.normalize_top_k_prob, p.normalization_epsilon, p.routed_scaling_factor);
+    return "moe_route";
+}
+
+const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,
+                                 void* out, uint32_t assignments, uint32_t row_bytes) {
+    if (row_bytes % 16 == 0) {
+        hipLaunchKernelGGL(expert_assign_kernel<uint4>, dim3(assignments), dim3(256), 0, s,
+                           static_cast<const uint4*>(hidden), metadata, static_cast<uint4*>(out),
+                           assignments, row_bytes / 16);
+    } else if (row_bytes % 4 == 0) {
+        hipLaunchKernelGGL(expert_assign_kernel<uint32_t>, dim3(assignments), dim3(256), 0, s,
+                           static_cast<const uint32_t*>(hidden), metadata,
+                           static_cast<uint32_t*>(out), assignments, row_bytes / 4);
+    } else {
+        hipLaunchKernelGGL(expert_assign_kernel<uint16_t>, dim3(assignments), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(hidden), metadata,
+                           static_cast<uint16_t*>(out), assignments, row_bytes / 2);
+    }
+    return "expert_assign";
+}
+
+const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,
+                                   uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype) {
+    hipLaunchKernelGGL(expert_silu_mul_kernel, dim3(grid_for((size_t)assignments * intermediate)),
+                       dim3(256), 0, s, in, out, assignments, intermediate, in_dtype, out_dtype);
+    return "expert_silu_mul";
+}
+
+const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
+                                  uint32_t tokens, uint32_t hidden, uint32_t top_k,
+                                  uint32_t in_dtype, uint32_t out_dtype) {
+    hipLaunchKernelGGL(expert_combine_kernel, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0,
+                       s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+    return "expert_combine";
+}
+
+}  // namespace fh

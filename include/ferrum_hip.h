@@ -1,0 +1,209 @@
+/*
+ * ferrum_hip.h -- C ABI of the MI355X (gfx950) backend for Ferrum's
+ * quantized-matmul operators.
+ *
+ * Each entry point names the Ferrum interface it stands in for (paths are
+ * relative to the Ferrum source tree).  A Rust `src/hip` backend would bind
+ * these with `extern "C"` and implement the `MetalDevice` operator methods of
+ * `src/ops` on top of them; GGUF super-blocks are uploaded verbatim.
+ *
+ * Conventions (the reference's, src/metal/mod.rs and src/ops/mod.rs):
+ *   - every call returns fh_status; FH_OK is 0; nothing throws or aborts on
+ *     bad input.  fh_last_error() returns a thread-local message for the most
+ *     recent failure on the calling thread.
+ *   - a device owns one HIP stream; operator calls enqueue on it and return.
+ *     Results are readable after fh_synchronize() or through
+ *     fh_buffer_download(), which waits for the stream first.
+ *   - buffers and matrices belong to the device that created them; passing a
+ *     foreign one fails with FH_ERR_DEVICE_MISMATCH.
+ *   - a device and its objects are not thread-safe (Ferrum's handles are
+ *     `Rc`, i.e. !Send + !Sync).
+ *   - tensors are dense row-major; fh_view carries {buffer, byte offset,
+ *     dtype}.  Activation and output views must be 16-byte aligned.
+ *   - all element counts and indices must fit in 32 bits (src/ops/mod.rs:991).
+ */
+#ifndef FERRUM_HIP_H
+#define FERRUM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t fh_status;
+
+/* Mirrors ferrum::Error (src/error.rs:3-51). */
+enum {
+    FH_OK = 0,
+    FH_ERR_SHAPE = 1,
+    FH_ERR_DTYPE = 2,
+    FH_ERR_DEVICE_MISMATCH = 3,
+    FH_ERR_RANGE = 4,
+    FH_ERR_DISPATCH = 5,
+    FH_ERR_SYNCHRONIZATION = 6,
+    FH_ERR_ALLOCATION = 7,
+    FH_ERR_GGUF = 8,
+    FH_ERR_WEIGHT = 9,
+    FH_ERR_PARAMETER = 10,
+    FH_ERR_TOKEN = 11,
+    FH_ERR_VALIDATION = 12
+};
+
+/* DType (src/tensor/mod.rs:5-11). */
+enum { FH_F32 = 0, FH_F16 = 1, FH_BF16 = 2 };
+
+/* GGML type ids of the supported formats (src/quantization.rs:24-49). */
+enum { FH_GGML_Q4_K = 12, FH_GGML_Q6_K = 14 };
+
+typedef struct fh_device fh_device;
+typedef struct fh_buffer fh_buffer;
+typedef struct fh_qmatrix fh_qmatrix;
+typedef struct fh_event fh_event;
+
+typedef struct fh_view {
+    fh_buffer* buffer;
+    size_t offset;  /* bytes */
+    uint32_t dtype; /* FH_F32 / FH_F16 / FH_BF16 */
+} fh_view;
+
+typedef struct fh_device_props {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t wavefront;
+    int32_t clock_khz;
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int32_t lds_bytes_per_block;
+    uint64_t global_bytes;
+    uint64_t l2_bytes;
+} fh_device_props;
+
+/* MoeRoutingPolicy (src/model/architecture.rs; consumed at src/ops/mod.rs:23-73). */
+typedef struct fh_routing_policy {
+    uint32_t experts;
+    uint32_t top_k;
+    uint32_t sigmoid;              /* 0 softmax over all experts, 1 sigmoid */
+    uint32_t normalize_top_k_prob; /* divide by (sum of selected + epsilon) */
+    float normalization_epsilon;
+    float routed_scaling_factor;
+} fh_routing_policy;
+
+/* ---- device ---------------------------------------------------------------
+ * MetalDevice::new / synchronize (src/metal/mod.rs:585-635).  Fails with
+ * FH_ERR_DISPATCH when the GPU is not gfx950. */
+fh_status fh_device_create(int32_t ordinal, fh_device** out);
+void fh_device_destroy(fh_device* device);
+fh_status fh_device_properties(const fh_device* device, fh_device_props* out);
+fh_status fh_synchronize(fh_device* device);
+const char* fh_last_error(void);
+/* Kernel the most recent operator call selected: Output.metrics.operation
+ * (src/ops/mod.rs:8-21), which the reference's tests assert on. */
+const char* fh_last_operation(const fh_device* device);
+/* Raw hipStream_t of the device, for interop and external event timing. */
+void* fh_device_stream(fh_device* device);
+
+/* Kernel-selection switches: the legacy::Tuning setters
+ * (src/metal/legacy.rs:8-111), e.g. "k_quant_gemv_ksplit" with the same value
+ * rule as set_k_quant_gemv_ksplit (0 or a power of two up to 8).  Unknown
+ * keys or out-of-range values give FH_ERR_PARAMETER. */
+fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value);
+fh_status fh_get_tuning(const fh_device* device, const char* key, int64_t* value);
+
+/* ---- buffers ----------------------------------------------------------------
+ * MetalDevice::allocate (zero-initialised, src/metal/mod.rs:727-734) and the
+ * host copies behind Tensor::from_f32 / to_f32 (src/tensor/mod.rs). */
+fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out);
+void fh_buffer_free(fh_buffer* buffer);
+size_t fh_buffer_size(const fh_buffer* buffer);
+void* fh_buffer_device_ptr(fh_buffer* buffer);
+fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, size_t bytes);
+fh_status fh_buffer_download(const fh_buffer* buffer, size_t offset, void* dst, size_t bytes);
+fh_status fh_buffer_fill_zero(fh_buffer* buffer, size_t offset, size_t bytes);
+
+/* ---- packed weights --------------------------------------------------------
+ * QuantizedMatrix::from_reader (src/quantization.rs:86-111) together with
+ * validate_gguf_quantized_payload (:212-261) and, for experts > 1,
+ * QuantizedExpertMatrix::new (:147-165): a row-major [experts*rows, cols]
+ * matrix of verbatim GGUF super-blocks.  `rows` is rows per expert.
+ * Errors: FH_ERR_SHAPE (empty, cols % 256, size overflow, length mismatch),
+ * FH_ERR_GGUF (unsupported type, payload ends inside a block),
+ * FH_ERR_WEIGHT (non-finite block scale). */
+fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows, uint64_t cols,
+                            uint64_t experts, const void* packed, size_t packed_len,
+                            fh_qmatrix** out);
+void fh_qmatrix_destroy(fh_qmatrix* matrix);
+uint64_t fh_qmatrix_rows(const fh_qmatrix* matrix);    /* rows per expert */
+uint64_t fh_qmatrix_columns(const fh_qmatrix* matrix);
+uint64_t fh_qmatrix_experts(const fh_qmatrix* matrix);
+uint32_t fh_qmatrix_ggml_type(const fh_qmatrix* matrix);
+size_t fh_qmatrix_byte_size(const fh_qmatrix* matrix);
+void* fh_qmatrix_device_ptr(fh_qmatrix* matrix);
+
+/* Whole-matrix dequantisation to [experts*rows, cols] in out.dtype.  The
+ * reference has no host decoder for these formats; its per-element GPU
+ * decoders q4_k_weight / q6_k_weight (src/metal/shaders/ops.metal:834-845,
+ * 1316-1329) define the values.  f32 output is bit-exact. */
+fh_status fh_dequantize(fh_device* device, const fh_qmatrix* weight, const fh_view* out);
+
+/* MetalDevice::embedding_gather_quantized (src/ops/transformer.rs:299-360):
+ * out[t, :] = dequantised row tokens[t], rounded to out.dtype.
+ * FH_ERR_TOKEN when an id is >= rows. */
+fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* weight,
+                                        const uint32_t* tokens, size_t count, const fh_view* out);
+
+/* ---- dense projection -------------------------------------------------------
+ * MetalDevice::project_quantized (src/ops/transformer.rs:96-297):
+ * Y[M,N] = X[M,K] * W[N,K]^T with f32 accumulation.  x is [m, K] in x.dtype,
+ * y is [m, N] in y.dtype (the reference always uses y.dtype == x.dtype).
+ * FH_ERR_SHAPE when m == 0, K exceeds u32::MAX - 32 or an index overflows;
+ * FH_ERR_RANGE when a view is out of bounds, misaligned, or y overlaps x. */
+fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                               uint32_t m, const fh_view* y);
+
+/* ---- mixture of experts -----------------------------------------------------
+ * MetalDevice::moe_route (src/ops/mod.rs:23-73; kernel ops.metal:1894-1957).
+ * logits [tokens, experts]; bias (may be NULL) [experts] f32; metadata
+ * [tokens*top_k, 3] f32 rows {expert id bits, token id bits, weight}, sorted
+ * by expert id within a token. */
+fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
+                       const fh_view* selection_bias, const fh_routing_policy* policy,
+                       const fh_view* metadata);
+
+/* MetalDevice::expert_assign (src/ops/mod.rs:75-115): out[a,:] =
+ * hidden[token(a),:]; hidden [tokens, width], out [tokens*top_k, width]. */
+fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t tokens,
+                           uint32_t width, const fh_view* metadata, uint32_t top_k,
+                           const fh_view* out);
+
+/* MetalDevice::expert_project_quantized (src/ops/mod.rs:188-333, grouped and
+ * tile forms :336-485): y[a, r] = sum_k x[a,k] * W[expert(a)*rows + r, k].
+ * x [assignments, K], metadata [assignments, 3] f32, y [assignments, rows]. */
+fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weight,
+                                      const fh_view* x, uint32_t assignments,
+                                      const fh_view* metadata, const fh_view* y);
+
+/* MetalDevice::expert_silu_mul (src/ops/mod.rs:487-508): in [A, 2*I] (gate
+ * first), out [A, I] = round(silu(gate)) * up, stored in out.dtype. */
+fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assignments,
+                             uint32_t intermediate, const fh_view* out);
+
+/* MetalDevice::expert_combine (src/ops/mod.rs:510-551): out[t,c] = sum over
+ * the token's top_k rows, in metadata order, of round(round(w) * v). */
+fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
+                            uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out);
+
+/* ---- timing ------------------------------------------------------------------
+ * Events on the device's own stream, for the per-dispatch GPU time the
+ * reference reads from its command buffers (src/metal/mod.rs:601-604). */
+fh_status fh_event_create(fh_device* device, fh_event** out);
+void fh_event_destroy(fh_event* event);
+fh_status fh_event_record(fh_event* event);
+fh_status fh_event_elapsed_ms(fh_event* start, fh_event* stop, float* ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FERRUM_HIP_H */

@@ -1,0 +1,293 @@
+"""GPU parity of the dense path (dequantize, GEMV, small-M, tile GEMM) against
+the CPU oracle, through the C ABI.
+
+The first half replays the reference's own test cases for this path
+(src/ops/transformer.rs qk_tests / q6_k_tests, src/diffusion/tests.rs:716-761)
+with its closed-form inputs and its tolerances; the second half applies the
+benchmark's bars (dequant bit-exact; max relative error 1e-3 and relative L2
+1e-5 with f32 accumulation) at the benchmark shapes on seeded synthetic blocks.
+"""
+import numpy as np
+import pytest
+
+import ferrum_fixtures as fx
+import oracle
+from helpers import assert_matmul_parity, bits, oracle_columns, rel_l2
+from ferrum_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q6_K = 12, 14
+
+
+@pytest.fixture(scope="module")
+def api():
+    from ferrum_amd import api as module
+    return module
+
+
+@pytest.fixture(scope="module")
+def d(api):
+    return api.Device.new()
+
+
+def qm(api, d, ggml, rows, cols, packed):
+    fmt = api.QuantizationFormat(ggml)
+    return api.QuantizedMatrix.from_reader(d, rows, cols, fmt, lambda dst: np.copyto(dst, packed))
+
+
+# ------------------------------------------------------------- dequantize
+
+@pytest.mark.parametrize("ggml,rows,cols", [(Q4_K, 5, 512), (Q6_K, 5, 512), (Q4_K, 133, 2560),
+                                            (Q6_K, 133, 2560)])
+def test_dequantize_is_bit_exact_on_reference_fixtures(api, d, ggml, rows, cols):
+    packed = fx.q4k_packed(rows, cols) if ggml == Q4_K else fx.q6k_packed(rows, cols)
+    w = qm(api, d, ggml, rows, cols, packed)
+    assert w.byte_size() == rows * (cols // 256) * (144 if ggml == Q4_K else 210)
+    got = d.dequantize(w).to_f32()
+    assert np.array_equal(bits(got), bits(oracle.dequantize(ggml, packed, rows, cols)))
+
+
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_dequantize_is_bit_exact_on_synthetic_blocks_in_every_dtype(api, d, ggml):
+    rows, cols = 257, 5120
+    packed = synth.matrix(ggml, rows, cols, seed=1234)
+    w = qm(api, d, ggml, rows, cols, packed)
+    want = oracle.dequantize(ggml, packed, rows, cols)
+    assert np.array_equal(bits(d.dequantize(w).to_f32()), bits(want))
+    for dtype, code in ((api.DType.F16, oracle.F16), (api.DType.BF16, oracle.BF16)):
+        got = d.dequantize(w, dtype).to_f32()
+        assert np.array_equal(bits(got), bits(oracle.round_storage(want, code).reshape(rows, cols)))
+
+
+def test_embedding_gather_decodes_selected_rows(api, d):
+    # src/ops/transformer.rs:3307-3329 and :4351-4369: bitwise after BF16 rounding
+    for ggml, packed in ((Q4_K, fx.q4k_packed(5, 512)), (Q6_K, fx.q6k_packed(5, 512))):
+        w = qm(api, d, ggml, 5, 512, packed)
+        ids = [4, 0, 3]
+        out = d.embedding_gather_quantized(w, ids, api.DType.BF16)
+        assert out.operation == ("embedding_gather_q4_k" if ggml == Q4_K else "embedding_gather_q6_k")
+        dense = oracle.dequantize(ggml, packed, 5, 512)
+        want = oracle.round_storage(dense[ids], oracle.BF16).reshape(3, 512)
+        assert np.array_equal(bits(out.tensor.to_f32()), bits(want))
+        with pytest.raises(api.TokenError):
+            d.embedding_gather_quantized(w, [5], api.DType.BF16)
+
+
+# ---------------------------------------------- the reference's GEMV / GEMM cases
+
+def test_q4_k_gemv_gemm_cover_blocks_and_batch_tails(api, d):
+    # src/ops/transformer.rs:2982-3002
+    n, k = 5, 512
+    packed = fx.q4k_packed(n, k)
+    w = qm(api, d, Q4_K, n, k, packed)
+    for m in (1, 2, 3, 4, 5, 7):
+        values = fx.q4k_input(m, k)
+        x = api.Tensor.from_f32(d, (m, k), api.DType.F32, values)
+        actual = d.project_quantized(x, w).tensor.to_f32()
+        reference = oracle.project(Q4_K, packed, n, k, values)
+        assert np.abs(actual - reference).max() <= 2.0e-4, m
+
+
+def test_q6_k_gemv_gemm_cover_superblock_and_batch_tails(api, d):
+    # src/ops/transformer.rs:4251-4269
+    n, k = 5, 512
+    packed = fx.q6k_packed(n, k)
+    w = qm(api, d, Q6_K, n, k, packed)
+    for m in (1, 2, 3, 4, 5, 7):
+        values = fx.q6k_input(m, k)
+        x = api.Tensor.from_f32(d, (m, k), api.DType.F32, values)
+        actual = d.project_quantized(x, w).tensor.to_f32()
+        reference = oracle.project(Q6_K, packed, n, k, values)
+        assert np.abs(actual - reference).max() <= 0.02, m
+        # far tighter than the reference asks: f32 parity
+        assert np.abs(actual - reference).max() <= 1e-4 * max(1.0, np.abs(reference).max())
+
+
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_gemv_ksplit_covers_row_and_block_tails(api, d, ggml):
+    # src/ops/transformer.rs:3004-3029 and :4190-4214: 133 rows leave a partial
+    # row tile; 10 and 19 super-blocks leave partial strides for every split.
+    with pytest.raises(api.ParameterError):
+        d.set_k_quant_gemv_ksplit(3)
+    try:
+        for n, k in ((133, 2560), (6, 4864)):
+            packed = fx.q4k_packed(n, k) if ggml == Q4_K else fx.q6k_packed(n, k)
+            values = fx.q4k_input(1, k) if ggml == Q4_K else fx.q6k_input(1, k)
+            w = qm(api, d, ggml, n, k, packed)
+            x = api.Tensor.from_f32(d, (1, k), api.DType.F32, values)
+            reference = oracle.project(ggml, packed, n, k, values)
+            for simds in (1, 2, 4, 8):
+                d.set_k_quant_gemv_ksplit(simds)
+                for rows_per_wave in (1, 2, 4):
+                    d.set_tuning("gemv_rows_per_wave", rows_per_wave)
+                    out = d.project_quantized(x, w)
+                    name = "q4_k" if ggml == Q4_K else "q6_k"
+                    assert out.operation == (f"{name}_gemv_ksplit" if simds > 1 else f"{name}_gemv_factored")
+                    actual = out.tensor.to_f32()
+                    assert np.all(np.abs(actual - reference) <= 1.0e-3 * np.maximum(np.abs(reference), 1.0)), \
+                        (n, k, simds, rows_per_wave)
+    finally:
+        d.set_k_quant_gemv_ksplit(0)
+        d.set_tuning("gemv_rows_per_wave", 0)
+
+
+@pytest.mark.parametrize("dtype_name", ["F16", "BF16"])
+def test_gemv_accepts_half_precision_activations(api, d, dtype_name):
+    n, k = 133, 1024
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    for ggml in (Q4_K, Q6_K):
+        packed = fx.q4k_packed(n, k) if ggml == Q4_K else fx.q6k_packed(n, k)
+        w = qm(api, d, ggml, n, k, packed)
+        values = fx.q4k_input(1, k)
+        x = api.Tensor.from_f32(d, (1, k), dtype, values)
+        rounded = x.to_f32()
+        assert np.array_equal(rounded, oracle.round_storage(values, code).reshape(1, k))
+        out = d.project_quantized(x, w)                      # output dtype = input dtype
+        want = oracle.project(ggml, packed, n, k, rounded, accumulate="f64")
+        assert np.array_equal(out.tensor.to_f32(), oracle.round_storage(out.tensor.to_f32(), code).reshape(1, n))
+        assert rel_l2(out.tensor.to_f32(), want) <= (1e-3 if dtype_name == "F16" else 6e-3)
+        out32 = d.project_quantized(x, w, out_dtype=api.DType.F32).tensor.to_f32()
+        assert_matmul_parity(out32, want, f"{dtype_name} gemv")
+
+
+def test_k_quant_gemms_match_the_cpu_dequant(api, d):
+    # src/diffusion/tests.rs:716-761: F16 activations, M=200, K=512, N=100,
+    # f64-accumulated CPU dequant, worst error <= 2e-3 * max|ref|.
+    m, k, n = 200, 512, 100
+    x = oracle.round_storage(fx.xorshift_uniform(m * k, 31), oracle.F16).reshape(m, k)
+    for ggml in (Q4_K, Q6_K):
+        packed = fx.xorshift_blocks(ggml, n * k // 256)
+        w = qm(api, d, ggml, n, k, packed)
+        xt = api.Tensor.from_f32(d, (m, k), api.DType.F16, x)
+        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        assert out.operation == ("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
+        got = out.tensor.to_f32()
+        want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
+        scale = np.abs(want).max()
+        assert scale > 0.1, "reference is vacuous"
+        assert np.abs(got - want).max() <= 2e-3 * scale
+        # against the tile-dtype oracle (weights rounded to f16 first) the
+        # result is f32-accumulation accurate
+        tile = oracle.project(ggml, packed, n, k, x, accumulate="f64", weight_round=oracle.F16)
+        assert_matmul_parity(got, tile, "f16 tile gemm")
+
+
+def test_bf16_tile_gemm_covers_row_output_and_group_tails(api, d):
+    # src/ops/transformer.rs:3115-3175: (N, K) = (65, 512), M in {4, 8, 15, 35},
+    # BF16 activations, weights rounded to BF16, result stored as BF16, abs <= 0.04.
+    n, k = 65, 512
+    for ggml, tol in ((Q4_K, 0.04), (Q6_K, 0.12)):
+        packed = fx.q4k_packed(n, k) if ggml == Q4_K else fx.q6k_packed(n, k)
+        w = qm(api, d, ggml, n, k, packed)
+        for m in (4, 8, 15, 35):
+            values = fx.q4k_input(m, k) if ggml == Q4_K else fx.q6k_input(m, k)
+            x = api.Tensor.from_f32(d, (m, k), api.DType.BF16, values)
+            rounded = x.to_f32()
+            expected = oracle.project(ggml, packed, n, k, rounded, weight_round=oracle.BF16,
+                                      out_round=oracle.BF16)
+            out = d.project_quantized(x, w)
+            assert out.operation.endswith("gemm_mfma")
+            assert np.abs(out.tensor.to_f32() - expected).max() <= tol, (ggml, m)
+
+
+# ------------------------------------------------------- benchmark shapes
+
+def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):
+    packed = synth.matrix(ggml, n, k, seed)
+    x = synth.activations(1, k, seed)
+    w = qm(api, d, ggml, n, k, packed)
+    xt = api.Tensor.from_f32(d, (1, k), api.DType.F32, x)
+    got = d.project_quantized(xt, w).tensor.to_f32()
+    want64 = oracle.project(ggml, packed, n, k, x, accumulate="f64", threads=8)
+    want32 = oracle.project(ggml, packed, n, k, x, accumulate="f32", threads=8)
+    l2, mr = assert_matmul_parity(got, want64, f"gemv {ggml} {n}x{k} vs f64", l2_tol=l2_tol)
+    # the reference's sequential-f32 answer, whose own rounding error grows with K
+    assert_matmul_parity(got, want32, f"gemv {ggml} {n}x{k} vs f32seq", l2_tol=l2_tol)
+    assert l2 <= rel_l2(want32, want64) * 1.5 + 1e-7, "GPU is less accurate than the sequential CPU sum"
+
+
+def test_config0_q4_k_gemv_4096(api, d):
+    check_gemv(api, d, Q4_K, 4096, 4096, seed=1)
+
+
+@pytest.mark.parametrize("n,k", [(5120, 5120), (17408, 5120), (5120, 17408)])
+def test_config1_q4_k_decode_shapes(api, d, n, k):
+    check_gemv(api, d, Q4_K, n, k, seed=2)
+
+
+@pytest.mark.parametrize("n,k", [(5120, 17408), (151936, 5120)])
+def test_config2_q6_k_gemv(api, d, n, k):
+    check_gemv(api, d, Q6_K, n, k, seed=3)
+
+
+@pytest.mark.parametrize("m", [8, 16, 128, 512])
+def test_config3_q4_k_gemm_5120_17408(api, d, m):
+    n, k = 17408, 5120
+    packed = synth.matrix(Q4_K, n, k, seed=4)
+    x = synth.activations(m, k, seed=4, f16=True)
+    w = qm(api, d, Q4_K, n, k, packed)
+    xt = api.Tensor.from_f32(d, (m, k), api.DType.F16, x)
+    got = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+    rows = np.sort(synth.rng(4, 77).choice(n, size=192, replace=False))
+    rows[:4] = [0, 1, 2, 3]
+    rows[-2:] = [n - 2, n - 1]
+    rows = np.unique(rows)
+    tile = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", weight_round=oracle.F16,
+                          threads=8)
+    assert_matmul_parity(got[:, rows], tile, f"gemm M={m} vs f16-tile oracle")
+    plain = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", threads=8)
+    # distance to the unrounded CPU reference: only the f16 tile rounding
+    assert rel_l2(got[:, rows], plain) <= 4e-4
+    # linearity in M: row i of the product depends only on row i of X
+    if m >= 16:
+        xt2 = api.Tensor.from_f32(d, (m // 2, k), api.DType.F16, x[: m // 2])
+        half = d.project_quantized(xt2, w, out_dtype=api.DType.F32).tensor.to_f32()
+        assert np.array_equal(half, got[: m // 2])
+
+
+# ------------------------------------------------------------ error behaviour
+
+def test_project_rejects_bad_geometry_and_foreign_buffers(api, d):
+    packed = fx.q4k_packed(5, 512)
+    w = qm(api, d, Q4_K, 5, 512, packed)
+    with pytest.raises(api.ShapeError):
+        d.project_quantized(api.Tensor.zeros(d, (1, 256), api.DType.F32), w)
+    with pytest.raises(api.ShapeError):
+        d.project_quantized(api.Tensor.zeros(d, (512,), api.DType.F32), w)
+    other = api.Device.new()
+    foreign = api.Tensor.zeros(other, (1, 512), api.DType.F32)
+    with pytest.raises(api.DeviceMismatch):
+        d.project_quantized(foreign, w)
+    x = api.Tensor.zeros(d, (2, 512), api.DType.F32)
+    with pytest.raises(api.RangeError):
+        d.project_quantized(x.view(0, (1, 512)), w, out=x.view(0, (1, 5)))     # aliasing
+    with pytest.raises(api.RangeError):
+        d.project_quantized(x.view(1, (1, 512)), w)                            # misaligned view
+
+
+def test_quantized_matrix_validation(api, d):
+    # src/quantization.rs:93-103, :212-261 and qk_tests "reject partial blocks"
+    fmt = api.QuantizationFormat.Q4_K
+    with pytest.raises(api.ShapeError):
+        api.QuantizedMatrix.from_reader(d, 3, 255, fmt, lambda dst: None)
+    with pytest.raises(api.ShapeError):
+        api.QuantizedMatrix.from_reader(d, 0, 256, fmt, lambda dst: None)
+    good = fx.q4k_packed(2, 256)
+    with pytest.raises(api.GgufError):
+        api.QuantizedMatrix.from_bytes(d, 2, 256, fmt, good[:-1])
+    with pytest.raises(api.ShapeError):
+        api.QuantizedMatrix.from_bytes(d, 3, 256, fmt, good)
+    bad = good.copy()
+    bad[146:148] = np.frombuffer(np.float16(np.nan).tobytes(), np.uint8)
+    with pytest.raises(api.WeightError):
+        api.QuantizedMatrix.from_bytes(d, 2, 256, fmt, bad)
+    bad6 = fx.q6k_packed(2, 256)
+    bad6[208:210] = np.frombuffer(np.float16(np.inf).tobytes(), np.uint8)
+    with pytest.raises(api.WeightError):
+        api.QuantizedMatrix.from_bytes(d, 2, 256, api.QuantizationFormat.Q6_K, bad6)
+    with pytest.raises(api.GgufError):
+        api.QuantizationFormat.from_ggml_type(5)
+    assert api.QuantizationFormat.from_ggml_type(12).block_bytes() == 144
+    assert api.QuantizationFormat.from_ggml_type(14).block_bytes() == 210

@@ -1,0 +1,194 @@
+"""GPU parity of the mixture-of-experts stages against the CPU oracle, through
+the C ABI.  Cases follow src/nn/moe.rs:666-819 (router), the expert
+projection tests of src/ops/transformer.rs:3331-3388 / 4371-4424, and the
+35B-A3B style configuration of the benchmark (hidden 2048, 256 experts,
+intermediate 512, top-8)."""
+import numpy as np
+import pytest
+
+import ferrum_fixtures as fx
+import oracle
+from helpers import assert_matmul_parity, bits, rel_l2
+from ferrum_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+Q4_K, Q6_K = 12, 14
+
+
+@pytest.fixture(scope="module")
+def api():
+    from ferrum_amd import api as module
+    return module
+
+
+@pytest.fixture(scope="module")
+def d(api):
+    return api.Device.new()
+
+
+def route_both(api, d, logits, policy, bias=None, dtype=None):
+    dtype = api.DType.F32 if dtype is None else dtype
+    lt = api.Tensor.from_f32(d, logits.shape, dtype, logits)
+    bt = None if bias is None else api.Tensor.from_f32(d, (policy.experts,), api.DType.F32, bias)
+    got = d.moe_route(lt, bt, policy).to_f32()
+    want = oracle.select_routes(lt.to_f32(), policy.experts, policy.top_k,
+                                sigmoid=policy.scoring_function == api.MoeScoringFunction.Sigmoid,
+                                normalize=policy.normalize_top_k_prob,
+                                eps=policy.normalization_epsilon,
+                                scaling=policy.routed_scaling_factor, bias=bias)
+    return got, want
+
+
+def assert_routes(got, want):
+    assert np.array_equal(bits(got[:, 0]), bits(want[:, 0])), "expert ids"
+    assert np.array_equal(bits(got[:, 1]), bits(want[:, 1])), "token ids"
+    assert np.abs(got[:, 2] - want[:, 2]).max() <= 2e-6, "route weights"
+
+
+def test_router_preserves_cpu_top_k_order_and_weights(api, d):
+    # src/nn/moe.rs:741-819
+    logits = np.array([[0, 0, 0, 0, 0], [2, 0.5, -1, 1.5, 0]], dtype=np.float32)
+    bias = np.array([0.1, 0.05, 0.1, -0.3, 0.1], dtype=np.float32)
+    for scoring, use_bias in ((api.MoeScoringFunction.Sigmoid, True),
+                              (api.MoeScoringFunction.Softmax, True),
+                              (api.MoeScoringFunction.Softmax, False)):
+        policy = api.MoeRoutingPolicy(5, 3, scoring, True, 1e-6, 1.25, use_bias)
+        got, want = route_both(api, d, logits, policy, bias if use_bias else None, api.DType.BF16)
+        assert_routes(got, want)
+    # expert_assign gathers the token rows named by the metadata
+    policy = api.MoeRoutingPolicy(5, 3, api.MoeScoringFunction.Softmax, True, 1e-6, 1.25)
+    lt = api.Tensor.from_f32(d, (2, 5), api.DType.BF16, logits)
+    meta = d.moe_route(lt, None, policy)
+    hidden = api.Tensor.from_f32(d, (2, 1), api.DType.BF16, [1.0, 2.0])
+    assigned = d.expert_assign(hidden, meta, 3).to_f32().reshape(-1)
+    tokens = bits(meta.to_f32()[:, 1])
+    assert np.array_equal(assigned, np.array([1.0, 2.0], dtype=np.float32)[tokens])
+
+
+def test_router_literal_cases(api, d):
+    # src/nn/moe.rs:666-739
+    policy = api.MoeRoutingPolicy(3, 2, api.MoeScoringFunction.Sigmoid, True, 1e-6, 1.5)
+    got, want = route_both(api, d, np.array([[0.0, 2.0, -2.0]], dtype=np.float32), policy)
+    assert_routes(got, want)
+    assert bits(got[:, 0]).tolist() == [0, 1] and abs(got[0, 2] + got[1, 2] - 1.5) < 2e-6
+    policy = api.MoeRoutingPolicy(3, 2, api.MoeScoringFunction.Sigmoid, True, 1e-6, 1.0, True)
+    got, want = route_both(api, d, np.array([[2.0, 1.0, 0.0]], dtype=np.float32), policy,
+                           np.array([-10.0, 0.0, 2.0], dtype=np.float32))
+    assert_routes(got, want)
+    assert bits(got[:, 0]).tolist() == [1, 2]
+
+
+@pytest.mark.parametrize("tokens", [1, 512])
+def test_router_256_experts_top8(api, d, tokens):
+    logits = synth.rng(9, tokens).standard_normal((tokens, 256)).astype(np.float32)
+    policy = api.MoeRoutingPolicy(256, 8, api.MoeScoringFunction.Softmax, True, 0.0, 1.0)
+    got, want = route_both(api, d, logits, policy)
+    assert_routes(got, want)
+    assert np.allclose(got[:, 2].reshape(tokens, 8).sum(1), 1.0, atol=1e-5)
+    # ids ascend within a token
+    ids = bits(got[:, 0]).reshape(tokens, 8).astype(np.int64)
+    assert np.all(np.diff(ids, axis=1) > 0)
+
+
+def test_router_rejects_invalid_geometry(api, d):
+    lt = api.Tensor.zeros(d, (2, 5), api.DType.F32)
+    with pytest.raises(api.ShapeError):
+        d.moe_route(lt, None, api.MoeRoutingPolicy(5, 0))
+    with pytest.raises(api.ShapeError):
+        d.moe_route(lt, None, api.MoeRoutingPolicy(5, 6))
+    with pytest.raises(api.ShapeError):
+        d.moe_route(lt, None, api.MoeRoutingPolicy(4, 2))
+    with pytest.raises(api.ShapeError):
+        d.moe_route(lt, None, api.MoeRoutingPolicy(5, 17))
+    with pytest.raises(api.ShapeError):
+        d.moe_route(lt, None, api.MoeRoutingPolicy(5, 2, routed_scaling_factor=0.0))
+
+
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_expert_projection_uses_assignment_metadata(api, d, ggml):
+    # src/ops/transformer.rs:3331-3388: 3 experts x 5 rows, ids [2, 1, 2, 0],
+    # BF16 activations and outputs, abs <= 0.06 (Q4_K) / 0.12 (Q6_K)
+    experts, rows, cols = 3, 5, 512
+    expert_ids = [2, 1, 2, 0]
+    packed = fx.q4k_packed(experts * rows, cols) if ggml == Q4_K else fx.q6k_packed(experts * rows, cols)
+    fmt = api.QuantizationFormat(ggml)
+    w = api.QuantizedExpertMatrix.new(d, packed, fmt, experts, rows, cols)
+    values = fx.q4k_input(len(expert_ids), cols)
+    x = api.Tensor.from_f32(d, (len(expert_ids), cols), api.DType.BF16, values)
+    meta_bits = np.zeros((len(expert_ids), 3), dtype=np.uint32)
+    meta_bits[:, 0] = expert_ids
+    meta_bits[:, 1] = np.arange(len(expert_ids))
+    meta_bits[:, 2] = np.float32(1.0).view(np.uint32)
+    meta = api.Tensor.from_bits(d, (len(expert_ids), 3), meta_bits)
+    actual = d.expert_project_quantized(x, meta, w, cols, experts).to_f32()
+    expected = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), meta.to_f32(),
+                                     out_round=oracle.BF16)
+    assert np.abs(actual - expected).max() <= (0.06 if ggml == Q4_K else 0.12)
+    exact = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32).to_f32()
+    want64 = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), meta.to_f32(),
+                                   accumulate="f64")
+    assert_matmul_parity(exact, want64, "expert projection")
+    with pytest.raises(api.ShapeError):
+        d.expert_project_quantized(x, meta, w, cols, experts + 1)
+
+
+def test_silu_mul_and_combine_keep_the_storage_rounding_points(api, d):
+    rng = synth.rng(21)
+    a, inter, tokens, top_k, hidden = 24, 96, 6, 4, 64
+    for dtype, code in ((api.DType.F32, oracle.F32), (api.DType.F16, oracle.F16),
+                        (api.DType.BF16, oracle.BF16)):
+        packed_rows = (rng.standard_normal((a, 2 * inter)) * 2).astype(np.float32)
+        t = api.Tensor.from_f32(d, packed_rows.shape, dtype, packed_rows)
+        got = d.expert_silu_mul(t, inter).to_f32()
+        want = oracle.expert_silu_mul(t.to_f32(), inter, code)
+        if dtype == api.DType.F32:
+            assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+        else:
+            # expf may differ in the last ulp between libm and the GPU; after
+            # storage rounding at most a rare one-step difference remains
+            step = 2.0 ** (-10 if dtype == api.DType.F16 else -7)
+            assert np.all(np.abs(got - want) <= step * np.maximum(np.abs(want), 1e-3))
+            assert np.mean(got != want) < 0.01
+
+        values = rng.standard_normal((tokens * top_k, hidden)).astype(np.float32)
+        logits = rng.standard_normal((tokens, 16)).astype(np.float32)
+        meta_np = oracle.select_routes(logits, 16, top_k)
+        vt = api.Tensor.from_f32(d, values.shape, dtype, values)
+        mt = api.Tensor.from_bits(d, meta_np.shape, meta_np.view(np.uint32))
+        got = d.expert_combine(vt, mt, tokens, hidden, top_k).to_f32()
+        want = oracle.expert_combine(vt.to_f32(), meta_np, tokens, hidden, top_k, code)
+        assert np.array_equal(bits(got), bits(want))
+
+
+@pytest.mark.parametrize("tokens", [1, 48])
+def test_routed_ffn_pipeline_matches_the_oracle(api, d, tokens):
+    # hidden 2048, intermediate 512, top-8; 16 experts keep the CPU side quick
+    hidden, inter, experts, top_k = 2048, 512, 16, 8
+    w_in = synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=31)
+    w_out = synth.matrix(Q4_K, experts * hidden, inter, seed=32)
+    x = synth.activations(tokens, hidden, seed=33, f16=True)
+    logits = synth.rng(34).standard_normal((tokens, experts)).astype(np.float32)
+    fmt = api.QuantizationFormat.Q4_K
+    win = api.QuantizedExpertMatrix.new(d, w_in, fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, w_out, fmt, experts, hidden, inter)
+    policy = api.MoeRoutingPolicy(experts, top_k)
+
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F32, x)
+    meta = d.moe_route(api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits), None, policy)
+    assigned = d.expert_assign(xt, meta, top_k)
+    up = d.expert_project_quantized(assigned, meta, win, hidden, experts)
+    act = d.expert_silu_mul(up, inter)
+    down = d.expert_project_quantized(act, meta, wout, inter, experts)
+    got = d.expert_combine(down, meta, tokens, hidden, top_k).to_f32()
+
+    m = oracle.select_routes(logits, experts, top_k)
+    assert np.array_equal(bits(meta.to_f32()[:, :2]), bits(m[:, :2]))
+    o_assigned = oracle.expert_assign(x, m)
+    o_up = oracle.expert_project(Q4_K, w_in, experts, 2 * inter, hidden, o_assigned, m, accumulate="f64")
+    o_act = oracle.expert_silu_mul(o_up, inter)
+    o_down = oracle.expert_project(Q4_K, w_out, experts, hidden, inter, o_act, m, accumulate="f64")
+    want = oracle.expert_combine(o_down, m, tokens, hidden, top_k)
+    assert np.abs(want).max() > 1e-2
+    assert rel_l2(got, want) <= 2e-5
+    assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max()) * 8

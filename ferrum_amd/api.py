@@ -115,6 +115,10 @@ SYMBOLS = {
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
     "fh_expert_silu_mul": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_expert_combine": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
+    "fh_execution_begin": (_I32, [_P]),
+    "fh_execution_end": (_I32, [_P, ctypes.POINTER(_P)]),
+    "fh_graph_launch": (_I32, [_P]),
+    "fh_graph_destroy": (None, [_P]),
     "fh_event_create": (_I32, [_P, ctypes.POINTER(_P)]),
     "fh_event_destroy": (None, [_P]),
     "fh_event_record": (_I32, [_P]),
@@ -440,6 +444,43 @@ class Event:
             _lib.fh_event_destroy(h)
 
 
+class Graph:
+    """A recorded batch of operator calls (the reference's Execution scope),
+    replayable with launch()."""
+
+    def __init__(self, device: "Device", handle):
+        self.device, self._handle = device, handle
+
+    def launch(self):
+        _check(_lib.fh_graph_launch(self._handle))
+
+    def __del__(self):
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            _lib.fh_graph_destroy(h)
+
+
+class Execution:
+    """with device.execution() as e: ...ops with preallocated outputs...; e.graph.launch()"""
+
+    def __init__(self, device: "Device"):
+        self.device, self.graph = device, None
+
+    def __enter__(self):
+        _check(_lib.fh_execution_begin(self.device._handle))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        handle = ctypes.c_void_p()
+        status = _lib.fh_execution_end(self.device._handle, ctypes.byref(handle))
+        if exc_type is None:
+            _check(status)
+            self.graph = Graph(self.device, handle)
+        elif handle:
+            _lib.fh_graph_destroy(handle)
+        return False
+
+
 class Device:
     """One gfx950 GPU and its stream (the reference's MetalDevice)."""
 
@@ -477,6 +518,9 @@ class Device:
 
     def event(self) -> Event:
         return Event(self)
+
+    def execution(self) -> Execution:
+        return Execution(self)
 
     # ---- operators ---------------------------------------------------------
 

@@ -72,6 +72,45 @@ fh_status resolve(const fh_device* device, const fh_view* view, uint64_t element
 
 bool fits_u32(uint64_t v) { return v <= 0xffffffffull; }
 
+// Device scratch: kCounterWords zeroed counter words followed by a data area
+// of at least `data_bytes`.  Growing it waits for the stream first.
+fh_status ensure_scratch(fh_device* d, size_t data_bytes) {
+    const size_t counter_bytes = fh_device::kCounterWords * sizeof(uint32_t);
+    if (d->scratch != nullptr && d->scratch_bytes >= counter_bytes + data_bytes) return FH_OK;
+    if (d->capturing)
+        return fail(FH_ERR_SYNCHRONIZATION, "device scratch must grow: run the operator once before recording it");
+    FH_HIP(hipStreamSynchronize(d->stream));
+    if (d->scratch) (void)hipFree(d->scratch);
+    d->scratch = nullptr;
+    d->scratch_bytes = 0;
+    size_t cap = counter_bytes + (data_bytes < (16u << 20) ? (16u << 20) : data_bytes);
+    hipError_t e = hipMalloc(&d->scratch, cap);
+    if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", cap, hipGetErrorString(e));
+    d->scratch_bytes = cap;
+    FH_HIP(hipMemsetAsync(d->scratch, 0, counter_bytes, d->stream));
+    return FH_OK;
+}
+uint32_t* scratch_counters(fh_device* d) { return static_cast<uint32_t*>(d->scratch); }
+uint8_t* scratch_data(fh_device* d) {
+    return static_cast<uint8_t*>(d->scratch) + fh_device::kCounterWords * sizeof(uint32_t);
+}
+
+// Points a GEMV launch that cuts K into segments at the device scratch
+// (partial sums and one zeroed counter word per row tile and batch row).
+fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
+    GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    if (plan.segments > 1) {
+        if ((uint64_t)plan.tiles * a.m > fh_device::kCounterWords)
+            return fail(FH_ERR_SHAPE, "projection needs %llu row tiles, more than the K-split scratch holds",
+                        (unsigned long long)plan.tiles * a.m);
+        fh_status st = ensure_scratch(d, (size_t)plan.segments * a.m * a.n * sizeof(float));
+        if (st != FH_OK) return st;
+        a.partials = reinterpret_cast<float*>(scratch_data(d));
+        a.counters = scratch_counters(d);
+    }
+    return FH_OK;
+}
+
 int64_t tuning(const fh_device* d, const char* key) {
     auto it = d->tuning.find(key);
     return it == d->tuning.end() ? 0 : it->second;
@@ -114,8 +153,13 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
         return hip_fail(e, "hipStreamCreateWithFlags");
     }
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
-    d->tuning["gemv_rows_per_wave"] = 0;    // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
+    fh_status st = ensure_scratch(d, 0);
+    if (st != FH_OK) {
+        (void)hipStreamDestroy(d->stream);
+        delete d;
+        return st;
+    }
     *out = d;
     return FH_OK;
 }
@@ -148,6 +192,7 @@ fh_status fh_device_properties(const fh_device* device, fh_device_props* out) {
 }
 
 fh_status fh_synchronize(fh_device* device) {
+    if (device && device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (device == nullptr) return fail(FH_ERR_PARAMETER, "null device");
     hipError_t e = hipStreamSynchronize(device->stream);
     if (e != hipSuccess) return fail(FH_ERR_SYNCHRONIZATION, "stream: %s", hipGetErrorString(e));
@@ -169,8 +214,6 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
     if (k == "k_quant_gemv_ksplit") {
         // set_k_quant_gemv_ksplit: 0 or a power of two up to 8
         ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
-    } else if (k == "gemv_rows_per_wave") {
-        ok = value == 0 || value == 1 || value == 2 || value == 4;
     } else if (k == "gemm_min_rows") {
         ok = value >= 2;
     }
@@ -191,6 +234,7 @@ fh_status fh_get_tuning(const fh_device* device, const char* key, int64_t* value
 // ---- buffers -------------------------------------------------------------------
 
 fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out) {
+    if (device && device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     *out = nullptr;
     if (bytes == 0) return fail(FH_ERR_ALLOCATION, "zero-length buffer");
@@ -226,6 +270,7 @@ size_t fh_buffer_size(const fh_buffer* buffer) { return buffer ? buffer->bytes :
 void* fh_buffer_device_ptr(fh_buffer* buffer) { return buffer ? buffer->ptr : nullptr; }
 
 fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, size_t bytes) {
+    if (buffer && buffer->device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (buffer == nullptr || (src == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
     if (offset > buffer->bytes || bytes > buffer->bytes - offset)
         return fail(FH_ERR_RANGE, "upload [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
@@ -239,6 +284,7 @@ fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, si
 }
 
 fh_status fh_buffer_download(const fh_buffer* buffer, size_t offset, void* dst, size_t bytes) {
+    if (buffer && buffer->device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (buffer == nullptr || (dst == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
     if (offset > buffer->bytes || bytes > buffer->bytes - offset)
         return fail(FH_ERR_RANGE, "download [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
@@ -254,6 +300,7 @@ fh_status fh_buffer_download(const fh_buffer* buffer, size_t offset, void* dst, 
 }
 
 fh_status fh_buffer_fill_zero(fh_buffer* buffer, size_t offset, size_t bytes) {
+    if (buffer && buffer->device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (buffer == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (offset > buffer->bytes || bytes > buffer->bytes - offset)
         return fail(FH_ERR_RANGE, "fill exceeds buffer");
@@ -270,6 +317,7 @@ static bool f16_finite(const uint8_t* p) { return ((p[1] >> 2) & 0x1f) != 0x1f; 
 fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows, uint64_t cols,
                             uint64_t experts, const void* packed, size_t packed_len,
                             fh_qmatrix** out) {
+    if (device && device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     *out = nullptr;
     const size_t bb = block_bytes(ggml_type);
@@ -353,6 +401,7 @@ fh_status fh_dequantize(fh_device* device, const fh_qmatrix* weight, const fh_vi
 
 fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* weight,
                                         const uint32_t* tokens, size_t count, const fh_view* out) {
+    if (device && device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (device == nullptr || weight == nullptr || (tokens == nullptr && count))
         return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device) return fail(FH_ERR_DEVICE_MISMATCH, "weight belongs to another device");
@@ -368,21 +417,13 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
     if (st != FH_OK) return st;
     // ids travel through the device scratch (the reference carries them in a tensor)
     size_t need = count * sizeof(uint32_t);
-    if (device->scratch_bytes < need) {
-        FH_HIP(hipStreamSynchronize(device->stream));
-        if (device->scratch) (void)hipFree(device->scratch);
-        device->scratch = nullptr;
-        device->scratch_bytes = 0;
-        size_t cap = need < (1u << 20) ? (1u << 20) : need;
-        hipError_t e = hipMalloc(&device->scratch, cap);
-        if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", cap, hipGetErrorString(e));
-        device->scratch_bytes = cap;
-    }
-    FH_HIP(hipMemcpyAsync(device->scratch, tokens, need, hipMemcpyHostToDevice, device->stream));
+    fh_status sst = ensure_scratch(device, need);
+    if (sst != FH_OK) return sst;
+    FH_HIP(hipMemcpyAsync(scratch_data(device), tokens, need, hipMemcpyHostToDevice, device->stream));
     FH_HIP(hipStreamSynchronize(device->stream));
     device->last_operation =
         launch_embedding_gather(device->stream, weight->ggml_type, weight->ptr, weight->cols,
-                                static_cast<const uint32_t*>(device->scratch), count,
+                                reinterpret_cast<const uint32_t*>(scratch_data(device)), count,
                                 const_cast<uint8_t*>(o.begin), out->dtype);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -421,7 +462,6 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
         a.m = m;
         a.x_dtype = x->dtype;
         a.y_dtype = y->dtype;
-        a.cu_count = device->props.multiProcessorCount;
         device->last_operation = launch_gemm(device->stream, a);
     } else {
         GemvArgs a{};
@@ -436,10 +476,9 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
         a.y_dtype = y->dtype;
         a.metadata = nullptr;
         a.experts = 1;
-        int64_t ks = tuning(device, "k_quant_gemv_ksplit");
-        a.ksplit = (int)(ks > 4 ? 4 : ks);
-        a.rows_per_wave = (int)tuning(device, "gemv_rows_per_wave");
-        a.cu_count = device->props.multiProcessorCount;
+        a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
+        st = prepare_gemv(device, a);
+        if (st != FH_OK) return st;
         const char* name = launch_gemv(device->stream, a);
         if (m > 1) name = weight->ggml_type == kQ4K ? "q4_k_gemm" : "q6_k_gemm";
         device->last_operation = name;
@@ -539,8 +578,8 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
     a.metadata = reinterpret_cast<const float*>(mr.begin);
     a.experts = (uint32_t)weight->experts;
     a.ksplit = 0;
-    a.rows_per_wave = 0;
-    a.cu_count = device->props.multiProcessorCount;
+    st = prepare_gemv(device, a);
+    if (st != FH_OK) return st;
     device->last_operation = launch_gemv(device->stream, a);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -583,6 +622,57 @@ fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view*
         const_cast<uint8_t*>(orr.begin), tokens, hidden, top_k, in->dtype, out->dtype);
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+// ---- batched execution ---------------------------------------------------------------
+
+fh_status fh_execution_begin(fh_device* device) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null device");
+    if (device->capturing) return fail(FH_ERR_DISPATCH, "nested executions are not supported");
+    FH_HIP(hipStreamBeginCapture(device->stream, hipStreamCaptureModeThreadLocal));
+    device->capturing = true;
+    return FH_OK;
+}
+
+fh_status fh_execution_end(fh_device* device, fh_graph** out) {
+    if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    *out = nullptr;
+    if (!device->capturing) return fail(FH_ERR_DISPATCH, "no execution is being recorded");
+    device->capturing = false;
+    hipGraph_t graph = nullptr;
+    FH_HIP(hipStreamEndCapture(device->stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return hip_fail(e, "hipGraphInstantiate");
+    }
+    fh_graph* g = new (std::nothrow) fh_graph();
+    if (g == nullptr) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return fail(FH_ERR_ALLOCATION, "out of host memory");
+    }
+    g->device = device;
+    g->graph = graph;
+    g->exec = exec;
+    *out = g;
+    return FH_OK;
+}
+
+fh_status fh_graph_launch(fh_graph* graph) {
+    if (graph == nullptr) return fail(FH_ERR_PARAMETER, "null graph");
+    if (graph->device->capturing) return fail(FH_ERR_DISPATCH, "cannot replay while recording");
+    FH_HIP(hipGraphLaunch(graph->exec, graph->device->stream));
+    return FH_OK;
+}
+
+void fh_graph_destroy(fh_graph* graph) {
+    if (graph == nullptr) return;
+    (void)hipStreamSynchronize(graph->device->stream);
+    (void)hipGraphExecDestroy(graph->exec);
+    (void)hipGraphDestroy(graph->graph);
+    delete graph;
 }
 
 // ---- timing ---------------------------------------------------------------------------

@@ -2,346 +2,374 @@
 //
 // Stands in for the reference's M = 1 kernels q4_k_gemv_ksplit / _factored
 // (src/metal/shaders/ops.metal:983-1070) and q6_k_gemv_ksplit / _factored
-// (:1331-1439), and, with a metadata pointer, for the per-assignment expert
-// form expert_project_q4_k_factored / _q6_k_factored (:1088-1101, 1452-1465).
-// Like those it uses the factored arithmetic: per 16-weight run the integer
-// quants are dotted with the activations and the block scale (and, for Q4_K,
-// the minimum times the activation sum) is applied once.
+// (:1331-1439), for the f32 small-batch kernels q4_k_gemm / q6_k_gemm
+// (:1102-1121, 1466-1485; one grid slice per batch row) and, with a metadata
+// pointer, for the per-assignment expert form expert_project_q4_k_factored /
+// _q6_k_factored (:1088-1101, 1452-1465).  Like those it uses the factored
+// arithmetic: integer quants are dotted with the activations per run of
+// equal scale, and the scale (and the minimum times the activation sum) is
+// applied once per run.
 //
-// Wave64 mapping.  Eight lanes own one 256-weight super-block: lane `sub`
-// loads 16 bytes of 4-bit quants (32 weights: a run of 16 in their low
-// nibbles and a run of 16 in their high nibbles).  A wave therefore streams
-// eight consecutive super-blocks of a row per step with 128-bit loads, and
-// keeps the 32 activations it needs in registers across R rows.
+// Wave64 mapping.  Four lanes own one 256-weight super-block, 64 weights
+// each; a wave covers RS rows x BS consecutive super-blocks per step
+// (RS * BS = 16) and takes IT steps, so every 128-bit weight load of the wave
+// is issued before anything is consumed.  The 4*BS lanes of a row are
+// contiguous, so row sums are DPP reductions inside 16-lane rows.
 //
-// Activations are staged once per workgroup in LDS as f32, permuted so that
-// the eight float4 reads of a lane are conflict free: float4 number
-// (4*seg + jj)*8 + sub of a block holds the jj-th float4 of lane `sub`'s
-// low-nibble (seg 0) or high-nibble (seg 1) run.
+// Integer quants reach the FMA without a conversion instruction: a nibble
+// masked in place inside a 16-bit half is the f16 subnormal q * 2^-24 (or
+// q * 2^-20 four bits up), which v_fma_mix_f32 widens exactly; the power of
+// two is folded into the run scale.
 //
-// KS waves of a workgroup may share the same rows and interleave super-blocks
-// (the reference's K-split); partial sums meet in LDS in a fixed order, so
-// results do not depend on scheduling.
+// Activations are requested first (loads return in order, so they arrive
+// before the weights queued behind them), widened to f32 and staged in LDS in
+// lane order: float4 number u*4 + c of a block is the u-th float4 of lane c.
+// Rows of a wave read the same LDS words (broadcast).  Sums of 16 consecutive
+// activations are formed during the fill with DPP adds.
+//
+// Long rows are cut into K segments across workgroups (grid.y); each writes
+// its partial sums to a scratch buffer and the last to arrive (a counter per
+// row tile) adds them in segment order, so results are deterministic.
 #include "device_utils.hpp"
 #include "internal.hpp"
 
 namespace fh {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / kWave;
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kXStride = 68;  // float4 per block in LDS: 64 + 4, so neighbouring blocks use the other bank half
+constexpr int kMaxIt = 3;
 
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
-// ---- activation permutation ------------------------------------------------------
+// exact widening of an f16 (sub)normal held in one half of a dword
+__device__ __forceinline__ float lo_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).x; }
+__device__ __forceinline__ float hi_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).y; }
 
-// float4 index q (0..63) inside a super-block -> LDS float4 slot.
+// float4 index q (0..63) inside a super-block -> LDS slot u*4 + c (lane c, position u)
 template <uint32_t TYPE>
 __device__ __forceinline__ uint32_t x_slot(uint32_t q) {
-    uint32_t jj = q & 3u;
     if constexpr (TYPE == kQ4K) {
-        // element e = 64c + 32seg + 16h + 4jj + t
-        uint32_t c = q >> 4, seg = (q >> 3) & 1u, h = (q >> 2) & 1u;
-        return (4u * seg + jj) * 8u + (2u * c + h);
+        // element 64c + 32hi + 4u' : lane c, float4 u = 8hi + u'
+        return (q & 15u) * 4u + (q >> 4);
     } else {
-        // element e = 128half + 32slice + 16hh + 4jj + t; low nibbles hold
-        // slices 0/1, high nibbles slices 2/3
-        uint32_t half = q >> 5, slice = (q >> 3) & 3u, hh = (q >> 2) & 1u;
-        return (4u * (slice >> 1) + jj) * 8u + (4u * half + 2u * (slice & 1u) + hh);
+        // element 128h + 64hi + 32o + 4u' : lane c = 2h + o, float4 u = 8hi + u'
+        uint32_t c = 2u * (q >> 5) + ((q >> 3) & 1u);
+        uint32_t u = 8u * ((q >> 4) & 1u) + (q & 7u);
+        return u * 4u + c;
     }
 }
-
-// ---- per-format fragments ---------------------------------------------------------
 
 template <uint32_t TYPE>
 struct Frag;
 
+// Q4_K: lane c owns chunk c: 32 quant bytes = groups 2c (low nibbles) and 2c+1 (high).
 template <>
 struct Frag<kQ4K> {
-    uint4 hdr;  // d, dmin, 12 scale bytes
-    uint4 qs;   // this lane's 32 nibbles
-
-    __device__ __forceinline__ void load(const uint8_t* block, uint32_t sub) {
+    uint4 hdr, qa, qb;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c) {
         hdr = *reinterpret_cast<const uint4*>(block);
-        qs = *reinterpret_cast<const uint4*>(block + 16 + 16 * sub);
+        qa = *reinterpret_cast<const uint4*>(block + 16 + 32 * c);
+        qb = *reinterpret_cast<const uint4*>(block + 32 + 32 * c);
     }
-
-    // dot of this lane's 32 weights with xv; sums are the activation sums of
-    // the low- and high-nibble runs.
-    __device__ __forceinline__ float dot(const float4 (&xv)[8], float sum_lo, float sum_hi,
-                                         uint32_t sub) const {
-        float d = f16_bits_to_f32(hdr.x & 0xffffu);
-        float dmin = f16_bits_to_f32(hdr.x >> 16);
+    // xc: this lane's 16 float4 (stride 4 float4); s: sums of its four 16-runs
+    __device__ __forceinline__ float dot(const float4* xc, float4 s, uint32_t c) const {
+        float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
         float sc_lo, sc_hi, mn_lo, mn_hi;
-        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, sub >> 1, sc_lo, sc_hi, mn_lo, mn_hi);
-        float a_lo = 0.f, a_hi = 0.f;
-        const uint32_t q[4] = {qs.x, qs.y, qs.z, qs.w};
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, c, sc_lo, sc_hi, mn_lo, mn_hi);
+        float a_lo = 0.f, a_hi = 0.f, b_lo = 0.f, b_hi = 0.f;
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            uint32_t lo = q[t] & 0x0f0f0f0fu;
-            uint32_t hi = (q[t] >> 4) & 0x0f0f0f0fu;
-            a_lo = fmaf(xv[t].x, (float)(lo & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].y, (float)((lo >> 8) & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].z, (float)((lo >> 16) & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].w, (float)(lo >> 24), a_lo);
-            a_hi = fmaf(xv[4 + t].x, (float)(hi & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].y, (float)((hi >> 8) & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].z, (float)((hi >> 16) & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].w, (float)(hi >> 24), a_hi);
+        for (int t = 0; t < 8; ++t) {
+            float4 xl = xc[t * 4], xh = xc[(8 + t) * 4];
+            uint32_t w0 = q[t], w1 = q[t] >> 8;
+            uint32_t l02 = w0 & 0x000f000fu, h02 = w0 & 0x00f000f0u;  // bytes 0, 2
+            uint32_t l13 = w1 & 0x000f000fu, h13 = w1 & 0x00f000f0u;  // bytes 1, 3
+            a_lo = fmaf(lo_half(l02), xl.x, a_lo);
+            b_lo = fmaf(lo_half(l13), xl.y, b_lo);
+            a_lo = fmaf(hi_half(l02), xl.z, a_lo);
+            b_lo = fmaf(hi_half(l13), xl.w, b_lo);
+            a_hi = fmaf(lo_half(h02), xh.x, a_hi);
+            b_hi = fmaf(lo_half(h13), xh.y, b_hi);
+            a_hi = fmaf(hi_half(h02), xh.z, a_hi);
+            b_hi = fmaf(hi_half(h13), xh.w, b_hi);
         }
-        float scaled = fmaf(sc_lo, a_lo, sc_hi * a_hi);
-        float offset = fmaf(mn_lo, sum_lo, mn_hi * sum_hi);
+        a_lo += b_lo;
+        a_hi += b_hi;
+        // low nibbles were q * 2^-24, high nibbles 16q * 2^-24
+        float scaled = fmaf(sc_lo * 16777216.f, a_lo, (sc_hi * 1048576.f) * a_hi);
+        float offset = fmaf(mn_lo, s.x + s.y, mn_hi * (s.z + s.w));
         return fmaf(d, scaled, -(dmin * offset));
     }
 };
 
+// Q6_K: lane c = 2h + o owns ql bytes [64h + 32o, +32): slice o in the low
+// nibbles and slice o + 2 in the high nibbles, with the 2-bit planes 2o and
+// 2o + 4 of qh bytes [32h, +32).  Four runs of 16 weights, one int8 scale each.
 template <>
 struct Frag<kQ6K> {
-    uint4 ql;      // 16 bytes: low nibbles slice s, high nibbles slice s+2
-    uint4 qh;      // 16 bytes of 2-bit planes for the same 16 positions
-    uint32_t tail; // {scale of the low run, scale of the high run} << 16 | f16 d
-
-    __device__ __forceinline__ void load(const uint8_t* block, uint32_t sub) {
-        uint32_t half = sub >> 2, hh = sub & 1u, sl = (sub >> 1) & 1u;
-        ql = load_u4_unaligned(block + 16 * sub);
-        qh = load_u4_unaligned(block + 128 + 32 * half + 16 * hh);
-        uint32_t si = 192 + 8 * half + 2 * sl + hh;
-        uint32_t lo = block[si], hi = block[si + 4];
-        uint32_t d = load_u16_unaligned(block + 208);
-        tail = d | (lo << 16) | (hi << 24);
+    uint4 la, lb, ha, hb;
+    uint32_t scales;  // bytes: low run 0..15, low run 16..31, high run 0..15, high run 16..31
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c) {
+        uint32_t h = c >> 1, o = c & 1u;
+        la = load_u4_unaligned(block + 64 * h + 32 * o);
+        lb = load_u4_unaligned(block + 64 * h + 32 * o + 16);
+        ha = load_u4_unaligned(block + 128 + 32 * h);
+        hb = load_u4_unaligned(block + 128 + 32 * h + 16);
+        uint32_t si = 192 + 8 * h + 2 * o;
+        scales = load_u16_unaligned(block + si) | (load_u16_unaligned(block + si + 4) << 16);
+        d = load_u16_unaligned(block + 208);
     }
-
-    __device__ __forceinline__ float dot(const float4 (&xv)[8], float sum_lo, float sum_hi,
-                                         uint32_t sub) const {
-        float d = f16_bits_to_f32(tail & 0xffffu);
-        float sc_lo = (float)(int)(int8_t)(tail >> 16);
-        float sc_hi = (float)(int)(int8_t)(tail >> 24);
-        uint32_t shift = (sub & 2u);  // slice&1 -> 2-bit plane 0/1 for low, +4 for high
-        float a_lo = 0.f, a_hi = 0.f;
-        const uint32_t l[4] = {ql.x, ql.y, ql.z, ql.w};
-        const uint32_t h[4] = {qh.x, qh.y, qh.z, qh.w};
+    __device__ __forceinline__ float dot(const float4* xc, float4 s, uint32_t c) const {
+        const uint32_t shift = (c & 1u) * 2u;
+        const uint32_t l[8] = {la.x, la.y, la.z, la.w, lb.x, lb.y, lb.z, lb.w};
+        const uint32_t p[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};  // low 0..15, low 16..31, high 0..15, high 16..31
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            uint32_t hb = h[t] >> shift;
-            uint32_t lo = (l[t] & 0x0f0f0f0fu) | ((hb & 0x03030303u) << 4);
-            uint32_t hi = ((l[t] >> 4) & 0x0f0f0f0fu) | (((hb >> 4) & 0x03030303u) << 4);
-            a_lo = fmaf(xv[t].x, (float)(lo & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].y, (float)((lo >> 8) & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].z, (float)((lo >> 16) & 0xffu), a_lo);
-            a_lo = fmaf(xv[t].w, (float)(lo >> 24), a_lo);
-            a_hi = fmaf(xv[4 + t].x, (float)(hi & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].y, (float)((hi >> 8) & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].z, (float)((hi >> 16) & 0xffu), a_hi);
-            a_hi = fmaf(xv[4 + t].w, (float)(hi >> 24), a_hi);
+        for (int t = 0; t < 8; ++t) {
+            float4 xl = xc[t * 4], xh = xc[(8 + t) * 4];
+            uint32_t w0 = l[t], w1 = l[t] >> 8;
+            uint32_t p0 = p[t] >> shift, p1 = p0 >> 8;
+            // low slice: nibble | plane bits 0..1 << 4, read as q * 2^-24
+            uint32_t l02 = (w0 & 0x000f000fu) | ((p0 & 0x00030003u) << 4);
+            uint32_t l13 = (w1 & 0x000f000fu) | ((p1 & 0x00030003u) << 4);
+            // high slice: nibble in bits 4..7 | plane bits 4..5 << 4, read as 16q * 2^-24
+            uint32_t h02 = (w0 & 0x00f000f0u) | ((p0 & 0x00300030u) << 4);
+            uint32_t h13 = (w1 & 0x00f000f0u) | ((p1 & 0x00300030u) << 4);
+            float& al = acc[t >> 2];
+            float& ah = acc[2 + (t >> 2)];
+            al = fmaf(lo_half(l02), xl.x, al);
+            al = fmaf(lo_half(l13), xl.y, al);
+            al = fmaf(hi_half(l02), xl.z, al);
+            al = fmaf(hi_half(l13), xl.w, al);
+            ah = fmaf(lo_half(h02), xh.x, ah);
+            ah = fmaf(lo_half(h13), xh.y, ah);
+            ah = fmaf(hi_half(h02), xh.z, ah);
+            ah = fmaf(hi_half(h13), xh.w, ah);
         }
+        float s0 = (float)(int)(int8_t)scales, s1 = (float)(int)(int8_t)(scales >> 8);
+        float s2 = (float)(int)(int8_t)(scales >> 16), s3 = (float)(int)(int8_t)(scales >> 24);
         // stored quants are weight + 32
-        a_lo = fmaf(-32.f, sum_lo, a_lo);
-        a_hi = fmaf(-32.f, sum_hi, a_hi);
-        return d * fmaf(sc_lo, a_lo, sc_hi * a_hi);
+        float r0 = fmaf(acc[0], 16777216.f, -32.f * s.x), r1 = fmaf(acc[1], 16777216.f, -32.f * s.y);
+        float r2 = fmaf(acc[2], 1048576.f, -32.f * s.z), r3 = fmaf(acc[3], 1048576.f, -32.f * s.w);
+        float total = fmaf(s0, r0, s1 * r1) + fmaf(s2, r2, s3 * r3);
+        return f16_bits_to_f32(d) * total;
     }
 };
 
-// ---- kernel -----------------------------------------------------------------------
-
-template <int XDT>
-__device__ __forceinline__ float4 load_x4(const void* x, size_t quad) {
-    if constexpr (XDT == 0) {
-        return static_cast<const float4*>(x)[quad];
-    } else {
-        uint2 raw = static_cast<const uint2*>(x)[quad];
-        if constexpr (XDT == 1) {
-            return make_float4(f16_bits_to_f32(raw.x & 0xffffu), f16_bits_to_f32(raw.x >> 16),
-                               f16_bits_to_f32(raw.y & 0xffffu), f16_bits_to_f32(raw.y >> 16));
-        } else {
-            return make_float4(bf16_bits_to_f32(raw.x & 0xffffu), bf16_bits_to_f32(raw.x >> 16),
-                               bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
-        }
-    }
+__device__ __forceinline__ float4 load_x4(const void* x, uint32_t dtype, size_t quad) {
+    if (dtype == FH_F32) return static_cast<const float4*>(x)[quad];
+    uint2 raw = static_cast<const uint2*>(x)[quad];
+    if (dtype == FH_F16)
+        return make_float4(f16_bits_to_f32(raw.x & 0xffffu), f16_bits_to_f32(raw.x >> 16),
+                           f16_bits_to_f32(raw.y & 0xffffu), f16_bits_to_f32(raw.y >> 16));
+    return make_float4(bf16_bits_to_f32(raw.x & 0xffffu), bf16_bits_to_f32(raw.x >> 16),
+                       bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
 }
 
-// grid: (ceil(n / rows_per_group / groups), m).  chunk_blocks super-blocks of x
-// fit the dynamic LDS allocation; longer rows take several passes.
-template <uint32_t TYPE, int R, int KS, int XDT>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(
-    const uint8_t* __restrict__ w, const void* __restrict__ x, void* __restrict__ y, uint32_t n,
-    uint32_t nb, uint32_t y_dtype, uint32_t chunk_blocks, const float* __restrict__ metadata,
-    uint32_t experts) {
-    extern __shared__ float4 xs[];
-    __shared__ float partial[kWaves][R];
-    constexpr int kGroups = kWaves / KS;  // row groups per workgroup
+struct Params {
+    const uint8_t* w;
+    const void* x;
+    void* y;
+    const float* metadata;
+    float* partials;     // [segments][m][n] when segments > 1
+    uint32_t* counters;  // one per (row tile, m), zero between launches
+    uint32_t n, nb, m;
+    uint32_t seg_len;    // super-blocks per K segment
+    uint32_t segments;
+    uint32_t x_dtype, y_dtype, experts;
+};
+
+// grid: (row tiles, K segments, m)
+template <uint32_t TYPE, int BS, int IT>
+__global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
+    constexpr int RS = 16 / BS;
     constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
+    extern __shared__ float4 xs[];  // seg_len * kXStride float4, then seg_len * 16 run sums
+    __shared__ uint32_t last_flag;
+    float* rsum = reinterpret_cast<float*>(xs + (size_t)p.seg_len * kXStride);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t group = wave / KS, ks = wave % KS;
-    const uint32_t slot = lane >> 3, sub = lane & 7u;
-    const uint32_t m = blockIdx.y;
-    const uint32_t k = nb << 8;
+    const uint32_t c = lane & 3u, bs = (lane >> 2) % BS, rs = lane / (4 * BS);
+    const uint32_t seg = blockIdx.y, m = blockIdx.z;
+    const uint32_t b0 = seg * p.seg_len;
+    const uint32_t cb = p.nb - b0 < p.seg_len ? p.nb - b0 : p.seg_len;  // blocks in this segment
 
     size_t row_base = 0;
     bool live = true;
-    if (metadata != nullptr) {
-        uint32_t expert = __float_as_uint(metadata[3 * (size_t)m]);
-        live = expert < experts;
-        row_base = live ? (size_t)expert * n : 0;
+    if (p.metadata != nullptr) {
+        uint32_t expert = __float_as_uint(p.metadata[3 * (size_t)m]);
+        live = expert < p.experts;
+        row_base = live ? (size_t)expert * p.n : 0;
     }
-    const uint32_t r0 = (blockIdx.x * kGroups + group) * R;
-    const uint8_t* rows[R];
+    const uint32_t row = (blockIdx.x * kWaves + wave) * RS + rs;
+    const uint8_t* rp = p.w + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
+
+    // 1. activations of this segment (requested first, consumed first)
+    const size_t xbase = ((size_t)m * p.nb + b0) * 64;  // float4 index of the segment start
+    const uint32_t xq = cb * 64;
+    constexpr int kXPer = 6;
+    float4 xr[kXPer];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        uint32_t row = r0 + r < n ? r0 + r : n - 1;
-        rows[r] = w + (row_base + row) * (size_t)nb * kBlockBytes;
+    for (int i = 0; i < kXPer; ++i) {
+        uint32_t q = tid + i * kThreads;
+        xr[i] = q < xq ? load_x4(p.x, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    const void* xrow = static_cast<const uint8_t*>(x) + (size_t)m * k * (XDT == 0 ? 4 : 2);
+    asm volatile("" ::: "memory");
 
-    float acc[R];
+    // 2. every weight fragment of this wave
+    Frag<TYPE> frag[IT];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
-
-    for (uint32_t c0 = 0; c0 < nb; c0 += chunk_blocks) {
-        const uint32_t cb = nb - c0 < chunk_blocks ? nb - c0 : chunk_blocks;
-        // first fragments of this pass are requested before the LDS fill
-        Frag<TYPE> cur[R];
-        uint32_t bl = ks * 8 + slot;
-        {
-            uint32_t b = c0 + (bl < cb ? bl : cb - 1);
-#pragma unroll
-            for (int r = 0; r < R; ++r) cur[r].load(rows[r] + (size_t)b * kBlockBytes, sub);
-        }
-        if (c0) __syncthreads();
-        for (uint32_t q = tid; q < cb * 64; q += kThreads) {
-            float4 v = load_x4<XDT>(xrow, (size_t)c0 * 64 + q);
-            xs[(q & ~63u) + x_slot<TYPE>(q & 63u)] = v;
-        }
-        __syncthreads();
-
-        for (; bl - slot < cb; bl += 8 * KS) {   // uniform trip count per wave
-            const bool valid = bl < cb;
-            Frag<TYPE> nxt[R];
-            {
-                uint32_t nb_l = bl + 8 * KS;
-                uint32_t b = c0 + (nb_l < cb ? nb_l : cb - 1);
-#pragma unroll
-                for (int r = 0; r < R; ++r) nxt[r].load(rows[r] + (size_t)b * kBlockBytes, sub);
-            }
-            float4 xv[8];
-            const float4* xb = xs + (size_t)(valid ? bl : 0) * 64 + sub;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) xv[j] = xb[j * 8];
-            float sum_lo = 0.f, sum_hi = 0.f;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                sum_lo += (xv[j].x + xv[j].y) + (xv[j].z + xv[j].w);
-                sum_hi += (xv[4 + j].x + xv[4 + j].y) + (xv[4 + j].z + xv[4 + j].w);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                float v = cur[r].dot(xv, sum_lo, sum_hi, sub);
-                acc[r] += valid ? v : 0.f;
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) cur[r] = nxt[r];
-        }
+    for (int it = 0; it < IT; ++it) {
+        uint32_t b = it * BS + bs;
+        frag[it].load(rp + (size_t)(b < cb ? b : cb - 1) * kBlockBytes, c);
     }
+    asm volatile("" ::: "memory");
 
+    // 3. stage activations and the sums of their 16-runs
+    auto stage = [&](uint32_t q, float4 v) {
+        const uint32_t slot = x_slot<TYPE>(q & 63u);
+        xs[(q >> 6) * kXStride + slot] = v;
+        // four consecutive float4 (one quad of lanes) are one 16-run of one lane
+        float s = (v.x + v.y) + (v.z + v.w);
+        s = dpp_add<0xB1>(s);
+        s = dpp_add<0x4E>(s);
+        if ((q & 3u) == 0) rsum[(q >> 6) * 16 + (slot & 3u) * 4 + (slot >> 4)] = s;
+    };
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+    for (int i = 0; i < kXPer; ++i) {
+        uint32_t q = tid + i * kThreads;
+        if (q < xq) stage(q, xr[i]);
+    }
+    for (uint32_t q = tid + kXPer * kThreads; q < xq; q += kThreads)
+        stage(q, load_x4(p.x, p.x_dtype, xbase + q));
+    __syncthreads();
 
-    if constexpr (KS == 1) {
-        if (lane == 0) {
+    // 4. consume, one step at a time
+    float acc = 0.f;
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                if (r0 + r < n)
-                    store_from_f32(y, (size_t)m * n + r0 + r, y_dtype, live ? acc[r] : 0.f);
-        }
-    } else {
-        if (lane == 0) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) partial[wave][r] = acc[r];
-        }
-        __syncthreads();
-        if (tid < kGroups * R) {
-            uint32_t g = tid / R, r = tid % R;
+    for (int it = 0; it < IT; ++it) {
+        uint32_t b = it * BS + bs;
+        bool valid = b < cb;
+        uint32_t bb = valid ? b : 0;
+        float4 s = *reinterpret_cast<const float4*>(rsum + bb * 16 + c * 4);
+        float v = frag[it].dot(xs + bb * kXStride + c, s, c);
+        acc += valid ? v : 0.f;
+        asm volatile("" : "+v"(acc)::"memory");
+    }
+    acc = dpp_add<0xB1>(acc);
+    acc = dpp_add<0x4E>(acc);
+    if (BS >= 2) acc = dpp_add<0x141>(acc);
+    if (BS >= 4) acc = dpp_add<0x140>(acc);
+    if (BS >= 8) acc += __shfl_xor(acc, 16, 64);
+    const bool writer = (lane & (4 * BS - 1)) == 0 && row < p.n;
+    if (!live) acc = 0.f;
+
+    if (p.segments == 1) {
+        if (writer) store_from_f32(p.y, (size_t)m * p.n + row, p.y_dtype, acc);
+        return;
+    }
+    // 5. K segments meet in the scratch buffer; the last workgroup of a tile adds
+    // them.  Partials and the counter use device-scope atomic accesses, which
+    // are coherent across the chip's L2 slices without cache-wide flushes.
+    if (writer)
+        __hip_atomic_store(&p.partials[((size_t)seg * p.m + m) * p.n + row], acc, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stores above have completed
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t* counter = p.counters + (size_t)m * gridDim.x + blockIdx.x;
+        uint32_t ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t last = ticket == p.segments - 1 ? 1u : 0u;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = last;
+    }
+    __syncthreads();
+    if (last_flag == 0) return;
+    if (tid < kWaves * RS) {
+        uint32_t r = blockIdx.x * (kWaves * RS) + tid;
+        if (r < p.n) {
             float total = 0.f;
-#pragma unroll
-            for (int s = 0; s < KS; ++s) total += partial[g * KS + s][r];
-            uint32_t row = (blockIdx.x * kGroups + g) * R + r;
-            if (row < n) store_from_f32(y, (size_t)m * n + row, y_dtype, live ? total : 0.f);
+            for (uint32_t s = 0; s < p.segments; ++s)
+                total += __hip_atomic_load(&p.partials[((size_t)s * p.m + m) * p.n + r], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+            store_from_f32(p.y, (size_t)m * p.n + r, p.y_dtype, total);
         }
     }
 }
 
-struct Launch {
-    void (*set_lds)(size_t);
-    void (*run)(dim3, size_t, hipStream_t, const GemvArgs&, uint32_t nb, uint32_t chunk);
-};
+typedef void (*LaunchFn)(dim3, size_t, hipStream_t, const Params&);
 
-template <uint32_t TYPE, int R, int KS, int XDT>
-void set_lds_impl(size_t bytes) {
-    static size_t configured = 0;
-    if (bytes > configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<TYPE, R, KS, XDT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-        configured = bytes;
-    }
-}
-
-template <uint32_t TYPE, int R, int KS, int XDT>
-void run_impl(dim3 grid, size_t lds, hipStream_t s, const GemvArgs& a, uint32_t nb,
-              uint32_t chunk) {
-    hipLaunchKernelGGL((gemv_kernel<TYPE, R, KS, XDT>), grid, dim3(kThreads), lds, s,
-                       static_cast<const uint8_t*>(a.w), a.x, a.y, a.n, nb, a.y_dtype, chunk,
-                       a.metadata, a.experts);
-}
-
-template <uint32_t TYPE, int R, int KS>
-Launch pick_dtype(uint32_t x_dtype) {
-    switch (x_dtype) {
-        case FH_F32: return {set_lds_impl<TYPE, R, KS, 0>, run_impl<TYPE, R, KS, 0>};
-        case FH_F16: return {set_lds_impl<TYPE, R, KS, 1>, run_impl<TYPE, R, KS, 1>};
-        default: return {set_lds_impl<TYPE, R, KS, 2>, run_impl<TYPE, R, KS, 2>};
-    }
+template <uint32_t TYPE, int BS, int IT>
+void launch_impl(dim3 grid, size_t lds, hipStream_t s, const Params& p) {
+    hipLaunchKernelGGL((gemv_kernel<TYPE, BS, IT>), grid, dim3(kThreads), lds, s, p);
 }
 
 template <uint32_t TYPE>
-Launch pick(int r, int ks, uint32_t x_dtype) {
-#define FH_CASE(RR, KK) \
-    if (r == RR && ks == KK) return pick_dtype<TYPE, RR, KK>(x_dtype);
-    FH_CASE(1, 1) FH_CASE(1, 2) FH_CASE(1, 4)
-    FH_CASE(2, 1) FH_CASE(2, 2) FH_CASE(2, 4)
-    FH_CASE(4, 1) FH_CASE(4, 2) FH_CASE(4, 4)
+LaunchFn pick(int bs, int it) {
+#define FH_CASE(B, I) \
+    if (bs == B && it == I) return launch_impl<TYPE, B, I>;
+    FH_CASE(8, 1) FH_CASE(8, 2) FH_CASE(8, 3)
+    FH_CASE(4, 1) FH_CASE(4, 2) FH_CASE(4, 3)
+    FH_CASE(2, 1) FH_CASE(2, 2) FH_CASE(2, 3)
+    FH_CASE(1, 1) FH_CASE(1, 2) FH_CASE(1, 3)
 #undef FH_CASE
-    return pick_dtype<TYPE, 2, 1>(x_dtype);
+    return nullptr;
 }
 
 }  // namespace
 
-const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
-    const uint32_t nb = a.k / 256;
-    // Automatic geometry: enough workgroups to cover the chip several times,
-    // K-split when rows alone cannot (the reference's rule of thumb,
-    // src/ops/transformer.rs:262-270, re-derived for 256 CUs).
-    int r = a.rows_per_wave, ks = a.ksplit;
-    const uint64_t total_rows = (uint64_t)a.n * a.m;
-    if (r == 0) r = total_rows >= 16384 ? 4 : total_rows >= 4096 ? 2 : 1;
-    if (ks == 0) {
-        ks = 1;
-        uint64_t waves = total_rows / r;
-        while (ks < 4 && waves * ks < (uint64_t)a.cu_count * 8 && nb >= (uint32_t)(16 * ks)) ks *= 2;
+GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
+    GemvPlan plan{};
+    const uint32_t nb = k / 256;
+    // widest block-slot count the row length fills
+    const int bs = nb >= 8 ? 8 : nb >= 4 ? 4 : nb >= 2 ? 2 : 1;
+    uint32_t segments = (nb + bs * kMaxIt - 1) / (bs * kMaxIt);
+    if (forced_segments > 0) {
+        // the reference's K-split switch: at least that many segments, as far
+        // as the row length allows
+        uint32_t want = (uint32_t)forced_segments;
+        const uint32_t most = (nb + bs - 1) / bs;
+        if (want > most) want = most;
+        if (want > segments) segments = want;
     }
-    if (r != 1 && r != 2 && r != 4) r = 2;
-    if (ks != 1 && ks != 2 && ks != 4) ks = 1;
+    const uint32_t seg_len = (nb + segments - 1) / segments;
+    plan.bs = bs;
+    plan.it = (int)((seg_len + bs - 1) / bs);
+    plan.segments = (nb + seg_len - 1) / seg_len;
+    plan.seg_len = seg_len;
+    plan.rows_per_wg = (uint32_t)(kWaves * (16 / bs));
+    plan.tiles = (n + plan.rows_per_wg - 1) / plan.rows_per_wg;
+    (void)m;
+    return plan;
+}
 
-    const uint32_t max_chunk = 144;  // 144 KiB of the 160 KiB LDS
-    const uint32_t chunk = nb < max_chunk ? nb : max_chunk;
-    const size_t lds = (size_t)chunk * 1024;
-    const uint32_t rows_per_wg = (uint32_t)(r * (kWaves / ks));
-    dim3 grid((a.n + rows_per_wg - 1) / rows_per_wg, a.m);
-
-    Launch l = a.ggml_type == kQ4K ? pick<kQ4K>(r, ks, a.x_dtype) : pick<kQ6K>(r, ks, a.x_dtype);
-    if (lds > 48 * 1024) l.set_lds(lds);
-    l.run(grid, lds, s, a, nb, chunk);
+const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
+    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    Params p{};
+    p.w = static_cast<const uint8_t*>(a.w);
+    p.x = a.x;
+    p.y = a.y;
+    p.metadata = a.metadata;
+    p.partials = a.partials;
+    p.counters = a.counters;
+    p.n = a.n;
+    p.nb = a.k / 256;
+    p.m = a.m;
+    p.seg_len = plan.seg_len;
+    p.segments = plan.segments;
+    p.x_dtype = a.x_dtype;
+    p.y_dtype = a.y_dtype;
+    p.experts = a.experts;
+    const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
+    dim3 grid(plan.tiles, plan.segments, a.m);
+    LaunchFn fn = a.ggml_type == kQ4K ? pick<kQ4K>(plan.bs, plan.it) : pick<kQ6K>(plan.bs, plan.it);
+    fn(grid, lds, s, p);
     if (a.metadata != nullptr)
         return a.ggml_type == kQ4K ? "expert_project_q4_k_factored" : "expert_project_q6_k_factored";
-    if (ks > 1) return a.ggml_type == kQ4K ? "q4_k_gemv_ksplit" : "q6_k_gemv_ksplit";
+    if (plan.segments > 1) return a.ggml_type == kQ4K ? "q4_k_gemv_ksplit" : "q6_k_gemv_ksplit";
     return a.ggml_type == kQ4K ? "q4_k_gemv_factored" : "q6_k_gemv_factored";
 }
 

@@ -16,10 +16,12 @@ struct fh_device {
     hipStream_t stream = nullptr;
     hipDeviceProp_t props{};
     const char* last_operation = "";
+    bool capturing = false;
     std::map<std::string, int64_t> tuning;
-    // scratch owned by the device (K-split partials, MoE segment tables, ...)
+    // scratch owned by the device: [counter words | floats / ids]
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    static constexpr size_t kCounterWords = 1u << 16;
 };
 
 struct fh_buffer {
@@ -36,6 +38,12 @@ struct fh_qmatrix {
     uint64_t rows = 0;     // per expert
     uint64_t cols = 0;
     uint64_t experts = 1;
+};
+
+struct fh_graph {
+    fh_device* device = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
 };
 
 struct fh_event {
@@ -68,7 +76,7 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
 // gemv.hip
 struct GemvArgs {
     uint32_t ggml_type;
-    const void* w;        // packed [n, k]
+    const void* w;        // packed [n, k] (per expert when metadata is set)
     const void* x;        // [m, k]
     void* y;              // [m, n]
     uint32_t n, k, m;
@@ -77,10 +85,15 @@ struct GemvArgs {
     // bits(metadata[3*m]) and weight rows [expert*n, expert*n + n)
     const float* metadata;
     uint32_t experts;
-    int ksplit;           // 0 = automatic
-    int rows_per_wave;    // 0 = automatic
-    int cu_count;
+    int ksplit;           // 0 = automatic, else at least this many K segments
+    float* partials;      // scratch for K segments (gemv_plan says how much)
+    uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
 };
+struct GemvPlan {
+    int bs, it;           // block slots per wave step, steps
+    uint32_t segments, seg_len, rows_per_wg, tiles;
+};
+GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments);
 const char* launch_gemv(hipStream_t s, const GemvArgs& a);
 
 // gemm.hip
@@ -91,7 +104,6 @@ struct GemmArgs {
     void* y;              // [m, n]
     uint32_t n, k, m;
     uint32_t x_dtype, y_dtype;
-    int cu_count;
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

@@ -61,6 +61,7 @@ typedef struct fh_device fh_device;
 typedef struct fh_buffer fh_buffer;
 typedef struct fh_qmatrix fh_qmatrix;
 typedef struct fh_event fh_event;
+typedef struct fh_graph fh_graph;
 
 typedef struct fh_view {
     fh_buffer* buffer;
@@ -194,6 +195,20 @@ fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assi
  * the token's top_k rows, in metadata order, of round(round(w) * v). */
 fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
                             uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out);
+
+/* ---- batched execution ---------------------------------------------------------
+ * MetalDevice::execution_with_shared_encoder / Execution::finish
+ * (src/metal/mod.rs:263-278, 563-572): operator calls between begin and end
+ * are recorded instead of run (up to the reference's batch of 1,024
+ * dispatches and beyond) and replayed as one HIP graph by fh_graph_launch.
+ * While recording, calls that must wait for the GPU or allocate (buffer and
+ * matrix creation, upload, download, embedding gather) fail with
+ * FH_ERR_SYNCHRONIZATION; size the outputs before.  A nested begin is an
+ * error, like a nested execution. */
+fh_status fh_execution_begin(fh_device* device);
+fh_status fh_execution_end(fh_device* device, fh_graph** out);
+fh_status fh_graph_launch(fh_graph* graph);
+void fh_graph_destroy(fh_graph* graph);
 
 /* ---- timing ------------------------------------------------------------------
  * Events on the device's own stream, for the per-dispatch GPU time the

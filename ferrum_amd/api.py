@@ -26,7 +26,7 @@ from dataclasses import dataclass
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libferrum_hip.so")
+LIB_PATH = os.environ.get("FERRUM_HIP_LIB") or os.path.join(_HERE, "lib", "libferrum_hip.so")
 
 
 class Error(Exception):

@@ -50,19 +50,20 @@ def _compile(src: str, extra: list[str]) -> str:
     return obj
 
 
-def build(extra_flags: list[str] | None = None, jobs: int = 5) -> str:
+def build(extra_flags: list[str] | None = None, jobs: int = 5, output: str | None = None) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     extra = list(extra_flags or [])
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(lambda s: _compile(s, extra), SOURCES))
-    tmp = LIB_PATH + ".tmp"
+    target = output or LIB_PATH
+    tmp = target + ".tmp"
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, target)
+    return target
 
 
 if __name__ == "__main__":

@@ -230,9 +230,478 @@ __global__ __launch_bounds__(kThreads) void gemm_tile_kernel(const uint8_t* __re
         }
 }
 
+
+// ---- wide tile: 256 (M) x 16*NT (N) x 64 (K) ---------------------------------------
+//
+// For prefill-sized M.  One workgroup owns `cols` (<= 16*NT) output columns and
+// 256 rows, so the grid can be sized to the chip (e.g. 17408 columns = 128
+// tiles of 136, times two M tiles = 256 workgroups on 256 CUs) and every
+// weight is decoded once per 256 rows.  Eight waves: four consumers, each 64
+// rows x 16*NT columns as 4 x NT MFMA 16x16x32 tiles with their activation
+// fragments loaded straight from global memory, and four producers that
+// decode the weight slab into LDS.  A SIMD therefore
+// holds one wave issuing MFMAs and one issuing VALU / memory work, which the
+// hardware overlaps.  LDS is double buffered: while slab s feeds the matrix
+// cores, slab s+1 is decoded into the other buffer and the global loads of
+// slabs s+2 and s+3 are in flight; one barrier per slab.
+//
+// Workgroup ids are mapped so that the M tiles of one weight tile sit on the
+// same XCD (ids that are equal mod 8) and share it through that XCD's L2.
+constexpr int kWM = 256;
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ float4v mfma16(uint4 a, uint4 b, float4v c) {
+    if constexpr (DT == 1) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a),
+                                                      __builtin_bit_cast(half8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+template <uint32_t TYPE, int DT>
+__device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c, uint32_t h,
+                                              uint16_t* wrow_lds) {
+    uint32_t lo[8], hi[8];
+    if constexpr (TYPE == kQ4K) {
+        raw.template decode<DT>(c, lo, hi);
+    } else {
+        raw.template decode<DT>(c, lo, hi, h);
+    }
+    // Q4_K: lo -> k 16h.., hi -> k 32+16h..;  Q6_K: lo -> k 32h.., hi -> k 32h+16..
+    const uint32_t k_lo = TYPE == kQ4K ? 16 * h : 32 * h;
+    const uint32_t k_hi = TYPE == kQ4K ? 32 + 16 * h : 32 * h + 16;
+    uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + k_lo);
+    uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + k_hi);
+    dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    dst_lo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+    dst_hi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    dst_hi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+}
+
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// exact widening of an f16 (sub)normal held in one half of a dword
+__device__ __forceinline__ float lo_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).x; }
+__device__ __forceinline__ float hi_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).y; }
+
+// Two tile values fma(q, scale, offset), each rounded once to the tile dtype,
+// packed into a dword.  q arrives as an f16 subnormal (an integer quant masked
+// in place, i.e. q * 2^-24 or 16q * 2^-24) and `scale` carries the inverse
+// power of two, so the f32 product is the exact integer multiple and the
+// result has the bits of the reference's (d*sc)*q - dmin*m.  For f16 the
+// compiler emits v_fma_mixlo/mixhi_f16: no conversion or pack instructions.
+template <int DT>
+__device__ __forceinline__ uint32_t fma_pair(float qa, float qb, float scale, float offset) {
+    if constexpr (DT == 1) {
+        half2v r;
+        r.x = (_Float16)fmaf(qa, scale, offset);
+        r.y = (_Float16)fmaf(qb, scale, offset);
+        return __builtin_bit_cast(uint32_t, r);
+    } else {
+        return f32_to_bf16_bits(fmaf(qa, scale, offset)) | (f32_to_bf16_bits(fmaf(qb, scale, offset)) << 16);
+    }
+}
+
+// Raw bytes one producer thread needs from a whole super-block: its half h of
+// each of the four 64-weight K slabs.  Loading by block (not by slab) issues
+// the global loads four slabs or more ahead of their use.  decode() turns one
+// input dword (4 quant bytes) of slab c into tile values: Q4_K gives two
+// dwords for k = 16h + 4t .. (low nibbles) and two for k = 32 + 16h + 4t ..
+// (high nibbles); Q6_K gives two dwords for k = 32h + 4t ...
+template <uint32_t TYPE>
+struct BlockW;
+
+template <>
+struct BlockW<kQ4K> {
+    static constexpr int kDwords = 4;    // input dwords per (slab, half)
+    uint4 hdr, q[4];
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q[c] = *reinterpret_cast<const uint4*>(block + 16 + 32 * c + 16 * h);
+    }
+    struct Scales {
+        float a_lo, a_hi, b_lo, b_hi;
+    };
+    __device__ __forceinline__ Scales scales(int c, uint32_t) const {
+        float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc0, sc1, mn0, mn1;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, (uint32_t)c, sc0, sc1, mn0, mn1);
+        // d*sc and dmin*m are exact in f32; the powers of two undo the subnormal encoding
+        return {(d * sc0) * 16777216.f, (d * sc1) * 1048576.f, -(dmin * mn0), -(dmin * mn1)};
+    }
+    __device__ __forceinline__ uint32_t dword(int c, int t) const {
+        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
+        return v[t];
+    }
+    // out[0..1]: low-nibble pair dwords, out[2..3]: high-nibble pair dwords
+    template <int DT>
+    __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
+        const uint32_t w0 = dword(c, t), w1 = w0 >> 8;
+        const uint32_t l02 = w0 & 0x000f000fu, h02 = w0 & 0x00f000f0u;
+        const uint32_t l13 = w1 & 0x000f000fu, h13 = w1 & 0x00f000f0u;
+        out[0] = fma_pair<DT>(lo_half(l02), lo_half(l13), s.a_lo, s.b_lo);
+        out[1] = fma_pair<DT>(hi_half(l02), hi_half(l13), s.a_lo, s.b_lo);
+        out[2] = fma_pair<DT>(lo_half(h02), lo_half(h13), s.a_hi, s.b_hi);
+        out[3] = fma_pair<DT>(hi_half(h02), hi_half(h13), s.a_hi, s.b_hi);
+    }
+};
+
+template <>
+struct BlockW<kQ6K> {
+    static constexpr int kDwords = 8;
+    uint4 l[2][2], p[2][2], sc;  // ql / qh of both halves, the 16 scales
+    uint32_t d;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            l[half][0] = load_u4_unaligned(block + 64 * half + 32 * h);
+            l[half][1] = load_u4_unaligned(block + 64 * half + 32 * h + 16);
+            p[half][0] = load_u4_unaligned(block + 128 + 32 * half);
+            p[half][1] = load_u4_unaligned(block + 128 + 32 * half + 16);
+        }
+        sc = load_u4_unaligned(block + 192);
+        d = load_u16_unaligned(block + 208);
+    }
+    struct Scales {
+        float s[2], off[2];   // scale (with the power of two) and -32*scale of positions 0..15 / 16..31
+        uint32_t plane_shift;
+    };
+    __device__ __forceinline__ Scales scales(int c, uint32_t h) const {
+        const int half = c >> 1;
+        // scales 8*half + 2*slice (+1), slice = 2(c&1) + h: a 16-bit pair of word 2*half + (c&1)
+        const uint32_t words[4] = {sc.x, sc.y, sc.z, sc.w};
+        const uint32_t pair = words[2 * half + (c & 1)] >> (16 * h);
+        const float df = f16_bits_to_f32(d);
+        const float s0 = df * (float)(int)(int8_t)pair, s1 = df * (float)(int)(int8_t)(pair >> 8);
+        const float pow2 = (c & 1) ? 1048576.f : 16777216.f;  // high nibbles sit four bits up
+        return {{s0 * pow2, s1 * pow2}, {-32.f * s0, -32.f * s1}, 2u * (2u * (c & 1) + h)};
+    }
+    // out[0..1]: the two pair dwords of positions 4t .. 4t+3
+    template <int DT>
+    __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
+        const int half = c >> 1;
+        const uint32_t lw[8] = {l[half][0].x, l[half][0].y, l[half][0].z, l[half][0].w,
+                                l[half][1].x, l[half][1].y, l[half][1].z, l[half][1].w};
+        const uint32_t pw[8] = {p[half][0].x, p[half][0].y, p[half][0].z, p[half][0].w,
+                                p[half][1].x, p[half][1].y, p[half][1].z, p[half][1].w};
+        const uint32_t w0 = lw[t], w1 = w0 >> 8;
+        const uint32_t p0 = pw[t] >> s.plane_shift, p1 = p0 >> 8;
+        uint32_t q02, q13;
+        if ((c & 1) == 0) {   // low nibbles | plane bits << 4 : q * 2^-24
+            q02 = (w0 & 0x000f000fu) | ((p0 & 0x00030003u) << 4);
+            q13 = (w1 & 0x000f000fu) | ((p1 & 0x00030003u) << 4);
+        } else {              // high nibbles in place | plane bits << 8 : 16q * 2^-24
+            q02 = (w0 & 0x00f000f0u) | ((p0 & 0x00030003u) << 8);
+            q13 = (w1 & 0x00f000f0u) | ((p1 & 0x00030003u) << 8);
+        }
+        const float sv = s.s[t >> 2], ov = s.off[t >> 2];
+        out[0] = fma_pair<DT>(lo_half(q02), lo_half(q13), sv, ov);
+        out[1] = fma_pair<DT>(hi_half(q02), hi_half(q13), sv, ov);
+        out[2] = 0;
+        out[3] = 0;
+    }
+};
+
+// Decode one (slab c, half h) task of a row into its LDS row.
+template <uint32_t TYPE, int DT>
+__device__ __forceinline__ void decode_block_slab(const BlockW<TYPE>& blk, int c, uint32_t h,
+                                                  uint16_t* wrow_lds) {
+    const auto s = blk.scales(c, h);
+    if constexpr (TYPE == kQ4K) {
+        uint32_t lo[8], hi[8];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            uint32_t out[4];
+            blk.template decode<DT>(c, h, t, s, out);
+            lo[2 * t] = out[0];
+            lo[2 * t + 1] = out[1];
+            hi[2 * t] = out[2];
+            hi[2 * t + 1] = out[3];
+        }
+        uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + 16 * h);        // k = 16h ..
+        uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + 32 + 16 * h);   // k = 32 + 16h ..
+        dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        dst_lo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        dst_hi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        dst_hi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+    } else {
+        uint32_t v[16];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            uint32_t out[4];
+            blk.template decode<DT>(c, h, t, s, out);
+            v[2 * t] = out[0];
+            v[2 * t + 1] = out[1];
+        }
+        uint4* dst = reinterpret_cast<uint4*>(wrow_lds + 32 * h);           // k = 32h ..
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[i] = make_uint4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
+    }
+}
+
+// A quarter of a task: input dword t of Q4_K, or dwords t and t + 4 of Q6_K.
+template <uint32_t TYPE, int DT>
+__device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int c, uint32_t h, int t,
+                                                   uint16_t* wrow_lds) {
+    const auto s = blk.scales(c, h);
+    if constexpr (TYPE == kQ4K) {
+        uint32_t out[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+            if (tt == t) blk.template decode<DT>(c, h, tt, s, out);
+        *reinterpret_cast<uint2*>(wrow_lds + 16 * h + 4 * t) = make_uint2(out[0], out[1]);
+        *reinterpret_cast<uint2*>(wrow_lds + 32 + 16 * h + 4 * t) = make_uint2(out[2], out[3]);
+    } else {
+        uint32_t a[4] = {0, 0, 0, 0}, b[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+            if (tt == t) {
+                blk.template decode<DT>(c, h, tt, s, a);
+                blk.template decode<DT>(c, h, tt + 4, s, b);
+            }
+        *reinterpret_cast<uint2*>(wrow_lds + 32 * h + 4 * t) = make_uint2(a[0], a[1]);
+        *reinterpret_cast<uint2*>(wrow_lds + 32 * h + 16 + 4 * t) = make_uint2(b[0], b[1]);
+    }
+}
+
+constexpr int kWideThreads = 512;
+
+template <uint32_t TYPE, int DT, int NT>
+__global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* __restrict__ w,
+                                                                 const uint16_t* __restrict__ x,
+                                                                 void* __restrict__ y, uint32_t m,
+                                                                 uint32_t n, uint32_t nb,
+                                                                 uint32_t y_dtype, uint32_t cols,
+                                                                 uint32_t tiles_m, uint32_t tiles_n) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
+    constexpr uint32_t kRowsW = 16 * NT;
+    constexpr uint32_t kStage = kRowsW * kLd;  // halfs per buffer
+    constexpr bool kExtra = NT > 8;                    // rows 128.. need a second decode task
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    // XCD-aware tile order: ids r, r+8, r+16, .. of a group share the XCD (id mod 8)
+    uint32_t tile_m, tile_n;
+    {
+        const uint32_t group_ids = 8 * tiles_m, id = blockIdx.x;
+        const uint32_t g = id / group_ids, r = id % group_ids;
+        tile_n = g * 8 + (r & 7u);
+        tile_m = r >> 3;
+        if (tile_n >= tiles_n) return;
+    }
+    const uint32_t n0 = tile_n * cols, m0 = tile_m * kWM;
+    const uint32_t ncols = n - n0 < cols ? n - n0 : cols;
+    const uint32_t k = nb << 8;
+    const uint32_t steps = nb * 4;
+
+    if (wave >= 4) {
+        // ---- producers: global -> registers -> (decode) -> LDS, two slabs ahead ----
+        const uint32_t pt = tid - 256, pw = wave - 4;
+        const uint32_t wr = pt >> 1, wh = pt & 1u;
+        const uint8_t* wsrc = w + (size_t)(n0 + (wr < ncols ? wr : ncols - 1)) * nb * kBlockBytes;
+        // rows 128.. of a 136-column tile: 8 rows x 2 halves x 4 quarter pieces, one per lane
+        const uint32_t er = 128 + (lane >> 3), eh = (lane >> 2) & 1u, et = lane & 3u;
+        const uint8_t* esrc = w + (size_t)(n0 + (er < ncols ? er : ncols - 1)) * nb * kBlockBytes;
+        // register sets: the block being decoded and the next one or two in flight
+        constexpr bool kDeep = TYPE == kQ4K;   // Q6_K sets are twice as large: one block ahead
+        BlockW<TYPE> cur, n1, n2, ecur, en1, en2;
+        auto load_block = [&](BlockW<TYPE>& main, BlockW<TYPE>& extra, uint32_t b) {
+            main.load(wsrc + (size_t)b * kBlockBytes, wh);
+            if (kExtra) extra.load(esrc + (size_t)b * kBlockBytes, eh);
+        };
+        auto store_slab = [&](int c) {
+            uint16_t* ws = lds + (c & 1) * kStage;
+            decode_block_slab<TYPE, DT>(cur, c, wh, ws + wr * kLd);
+            if (kExtra && pw == (uint32_t)c && er < ncols)
+                decode_block_piece<TYPE, DT>(ecur, c, eh, (int)et, ws + er * kLd);
+        };
+        load_block(cur, ecur, 0);
+        if (nb > 1) load_block(n1, en1, 1);
+        if (kDeep && nb > 2) load_block(n2, en2, 2);
+        store_slab(0);
+        for (uint32_t b = 0; b < nb; ++b) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                __syncthreads();  // slab 4b + c is visible; the other buffer is free
+                if (c < 3) {
+                    store_slab(c + 1);
+                } else if (b + 1 < nb) {
+                    cur = n1;
+                    ecur = en1;
+                    if (kDeep) {
+                        n1 = n2;
+                        en1 = en2;
+                        if (b + 3 < nb) load_block(n2, en2, b + 3);
+                    } else if (b + 2 < nb) {
+                        load_block(n1, en1, b + 2);
+                    }
+                    store_slab(0);
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- consumers: LDS fragments -> MFMA ----
+    float4v acc[4][NT];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    // A fragments come straight from global memory (the activation tile is
+    // L2 resident and each wave owns its 64 rows): lane (row = lane & 15,
+    // g = lane >> 4) holds k = 8g .. 8g+7 of a 32-wide K half.  They run
+    // through a ring of three register sets, loaded two K halves ahead.
+    const uint32_t g = lane >> 4;
+    // rows past m are clamped: they only feed outputs that are never stored
+    const uint16_t* asrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t row = m0 + wave * 64 + 16 * i + (lane & 15u);
+        asrc[i] = x + (size_t)(row < m ? row : m - 1) * k + 8 * g;
+    }
+    auto load_a = [&](uint4 (&a)[4], uint32_t u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const uint4*>(asrc[i] + (size_t)u * 32);
+    };
+    const uint32_t frag_off = (lane & 15u) * kLd + 8 * g;
+    auto mma_half = [&](const uint4 (&a)[4], uint32_t u) {
+        const uint16_t* ws = lds + ((u >> 1) & 1u) * kStage + frag_off + (u & 1u) * 32;
+        // B fragments through a ring of four so three LDS reads stay in flight
+        uint4 b[4];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) b[j] = *reinterpret_cast<const uint4*>(ws + 16 * j * kLd);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            if (j + 3 < NT) b[(j + 3) % 4] = *reinterpret_cast<const uint4*>(ws + 16 * (j + 3) * kLd);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i][j] = mfma16<DT>(a[i], b[j % 4], acc[i][j]);
+        }
+        // issue order for the scheduler (0x100 = DS read, 0x008 = MFMA)
+        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+        for (int j = 0; j < NT - 3; ++j) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 12, 0);
+    };
+    const uint32_t halves = steps * 2;
+    constexpr int kRing = 4;               // A register sets: loads run kRing - 1 halves ahead
+    static_assert(kRing % 2 == 0, "the slab barrier falls on even halves of the ring");
+    uint4 a[kRing][4];
+#pragma unroll
+    for (int i = 0; i < kRing - 1; ++i)
+        if ((uint32_t)i < halves) load_a(a[i], i);
+    __builtin_amdgcn_s_setprio(2);  // the MFMA wave goes first when both waves of a SIMD can issue
+    // Main loop: kRing K halves of straight-line code, so the outstanding-load
+    // counts are exact and the A loads stay ahead; the last halves run through
+    // a guarded tail.
+    uint32_t u = 0;
+    for (; u + 2 * kRing - 1 <= halves; u += kRing) {
+#pragma unroll
+        for (int ph = 0; ph < kRing; ++ph) {
+            if ((ph & 1) == 0) __syncthreads();  // a new slab
+            load_a(a[(ph + kRing - 1) % kRing], u + ph + kRing - 1);
+            mma_half(a[ph], u + ph);
+        }
+    }
+    for (; u < halves; u += kRing) {
+#pragma unroll
+        for (int ph = 0; ph < kRing; ++ph) {
+            const uint32_t uu = u + ph;
+            if (uu < halves) {
+                if ((uu & 1u) == 0) __syncthreads();  // a new slab
+                if (uu + kRing - 1 < halves) load_a(a[(ph + kRing - 1) % kRing], uu + kRing - 1);
+                mma_half(a[ph], uu);
+            }
+        }
+    }
+    __builtin_amdgcn_s_setprio(0);
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const uint32_t lc = 16 * j + (lane & 15u);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t row = m0 + wave * 64 + 16 * i + 4 * (lane >> 4) + v;
+                if (row < m && lc < ncols)
+                    store_from_f32(y, (size_t)row * n + n0 + lc, y_dtype, acc[i][j][v]);
+            }
+        }
+}
+
+struct WidePlan {
+    int nt;
+    uint32_t cols, tiles_m, tiles_n;
+};
+
+// Columns per workgroup: 128, 136 or 144, whichever wastes the least of the
+// chip's `cus` compute units (whole rounds of workgroups) and of the MFMA tile.
+WidePlan wide_plan(uint32_t m, uint32_t n, int cus) {
+    WidePlan best{};
+    double best_cost = 1e300;
+    const uint32_t tiles_m = (m + kWM - 1) / kWM;
+    for (uint32_t cols : {128u, 136u, 144u}) {
+        const int nt = cols > 128 ? 9 : 8;
+        const uint32_t tiles_n = (n + cols - 1) / cols;
+        const uint64_t wgs = (uint64_t)tiles_m * tiles_n;
+        const uint64_t rounds = (wgs + cus - 1) / cus;
+        const double cost = (double)rounds * nt;   // time ~ rounds x MFMA tiles per slab
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = {nt, cols, tiles_m, tiles_n};
+        }
+    }
+    return best;
+}
+
+template <uint32_t TYPE, int DT, int NT>
+void launch_wide(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
+    const size_t lds = 2 * (size_t)(16 * NT) * kLd * sizeof(uint16_t);
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wide_kernel<TYPE, DT, NT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        configured = true;
+    }
+    const uint32_t groups = (plan.tiles_n + 7) / 8;
+    dim3 grid(groups * 8 * plan.tiles_m);
+    hipLaunchKernelGGL((gemm_wide_kernel<TYPE, DT, NT>), grid, dim3(kWideThreads), lds, s,
+                       static_cast<const uint8_t*>(a.w), static_cast<const uint16_t*>(a.x), a.y, a.m, a.n,
+                       a.k / 256, a.y_dtype, plan.cols, plan.tiles_m, plan.tiles_n);
+}
+
+template <uint32_t TYPE, int DT>
+void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
+    if (plan.nt == 9) {
+        launch_wide<TYPE, DT, 9>(s, a, plan);
+    } else {
+        launch_wide<TYPE, DT, 8>(s, a, plan);
+    }
+}
+
 }  // namespace
 
 const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
+    if (a.m >= (uint32_t)a.wide_min_rows) {
+        const WidePlan plan = wide_plan(a.m, a.n, a.cu_count);
+        if (a.ggml_type == kQ4K) {
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan); else launch_wide_nt<kQ4K, 2>(s, a, plan);
+            return "q4_k_gemm_mfma_m256";
+        }
+        if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
+        return "q6_k_gemm_mfma_m256";
+    }
     dim3 grid((a.n + kBN - 1) / kBN, (a.m + kBM - 1) / kBM);
     const uint32_t nb = a.k / 256;
     const uint8_t* w = static_cast<const uint8_t*>(a.w);

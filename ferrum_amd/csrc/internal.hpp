@@ -104,6 +104,8 @@ struct GemmArgs {
     void* y;              // [m, n]
     uint32_t n, k, m;
     uint32_t x_dtype, y_dtype;
+    int cu_count;
+    int wide_min_rows;   // smallest M that takes the 256-row tile
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

@@ -164,7 +164,7 @@ def test_k_quant_gemms_match_the_cpu_dequant(api, d):
         w = qm(api, d, ggml, n, k, packed)
         xt = api.Tensor.from_f32(d, (m, k), api.DType.F16, x)
         out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
-        assert out.operation == ("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
+        assert out.operation.startswith("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
         got = out.tensor.to_f32()
         want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
         scale = np.abs(want).max()
@@ -190,7 +190,7 @@ def test_bf16_tile_gemm_covers_row_output_and_group_tails(api, d):
             expected = oracle.project(ggml, packed, n, k, rounded, weight_round=oracle.BF16,
                                       out_round=oracle.BF16)
             out = d.project_quantized(x, w)
-            assert out.operation.endswith("gemm_mfma")
+            assert "gemm_mfma" in out.operation
             assert np.abs(out.tensor.to_f32() - expected).max() <= tol, (ggml, m)
 
 

@@ -1,0 +1,259 @@
+"""Throughput of the quantized-matmul hot path on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` prints one JSON line.  A step
+is one Q4_K GEMV, y[17408] = W[17408, 5120] . x[5120] with fp32 activations (the
+FFN gate/up projection of a 27B-class decode layer).  Twelve distinct copies of
+the weight matrix (600 MB) are visited in turn so every step streams its 50 MB
+from HBM rather than from the 256 MB last-level cache.  The K steps are
+recorded once into a HIP graph and replayed, so the timed region holds kernel
+launches only; HIP events on the library's own stream bracket it.
+
+``value`` is algorithmic bytes per step / time per step.  ``roofline`` prices the
+GEMV kernel against the 8 TB/s HBM peak.  ``cases`` carries the other shapes of
+the dense-decode, Q6_K, small-M / prefill GEMM workloads (GB/s and TFLOP/s
+against both peaks), and ``cpu_baseline`` is the CPU oracle's sequential-fp32
+GEMV on the host's cores over a bounded number of repeats of the same step.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
+Q4_K, Q6_K = 12, 14
+BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
+
+# HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
+# FETCH_SIZE 24691.6 KiB x 1.94486 + WRITE_SIZE 68.0 KiB x 1.0, the factors being
+# known bytes / counter reading for the row-copy kernel of `--cases copy`.
+MEASURED_TRAFFIC_BYTES = 49243760
+
+
+def algorithmic_bytes(ggml, n, k, m, x_size, y_size):
+    return n * (k // 256) * BLOCK_BYTES[ggml] + m * k * x_size + m * n * y_size
+
+
+class Case:
+    """One projection shape with its rotating weight copies resident in HBM."""
+
+    def __init__(self, api, synth, dev, ggml, n, k, m, x_dtype, label, copies=None):
+        self.api, self.dev = api, dev
+        self.ggml, self.n, self.k, self.m, self.label = ggml, n, k, m, label
+        wbytes = n * (k // 256) * BLOCK_BYTES[ggml]
+        if copies is None:
+            copies = max(2, min(24, -(-ROTATE_BYTES // wbytes)))
+        base = synth.matrix(ggml, n, k, seed=1).reshape(n, -1)
+        self.packed = base
+        fmt = api.QuantizationFormat.from_ggml_type(ggml)
+        self.weights = [
+            api.QuantizedMatrix.from_bytes(dev, n, k, fmt, np.roll(base, i, axis=0).reshape(-1))
+            for i in range(copies)
+        ]
+        half = x_dtype != api.DType.F32
+        self.x_host = synth.activations(m, k, seed=3, f16=half)
+        self.x = api.Tensor.from_f32(dev, (m, k), x_dtype, self.x_host)
+        self.y = api.Tensor.zeros(dev, (m, n), api.DType.F32)
+        self.bytes = algorithmic_bytes(ggml, n, k, m, x_dtype.size_bytes(), 4)
+        self.weight_bytes = wbytes
+        self.flops = 2 * m * n * k
+        self.operation = ""
+
+    def enqueue(self, i):
+        self.dev.project_quantized(self.x, self.weights[i % len(self.weights)], out=self.y)
+
+
+def run_graph(dev, enqueue, steps, warmup):
+    """Replays `steps` recorded launches; returns (wall seconds, event seconds)."""
+    for i in range(max(warmup, 1)):
+        enqueue(i)
+    dev.synchronize()
+    with dev.execution() as ex:
+        for i in range(steps):
+            enqueue(i)
+    graph = ex.graph
+    graph.launch()  # first replay uploads the graph; untimed
+    dev.synchronize()
+    start, stop = dev.event(), dev.event()
+    t0 = time.perf_counter()
+    start.record()
+    graph.launch()
+    stop.record()
+    dev.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, start.elapsed_ms(stop) * 1e-3
+
+
+def measure(dev, case, steps, warmup, repeats=3):
+    best_wall, best_event = float("inf"), float("inf")
+    for _ in range(repeats):
+        wall, event = run_graph(dev, case.enqueue, steps, warmup)
+        best_wall, best_event = min(best_wall, wall), min(best_event, event)
+    case.operation = dev.last_operation()
+    return best_wall, best_event
+
+
+def report(case, seconds_per_step):
+    gbs = case.bytes / seconds_per_step / 1e9
+    tf = case.flops / seconds_per_step / 1e12
+    return {
+        "workload": case.label,
+        "operation": case.operation,
+        "us": round(seconds_per_step * 1e6, 3),
+        "GB/s": round(gbs, 1),
+        "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+        "TFLOP/s": round(tf, 2),
+        "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+        "weight_copies": len(case.weights),
+    }
+
+
+def cpu_baseline(case, budget_seconds=12.0):
+    """The CPU oracle's sequential-fp32 GEMV on the same tensors, all host threads."""
+    import oracle
+    threads = max(1, min(16, os.cpu_count() or 1))
+    packed = case.packed.reshape(-1)
+    x = case.x_host
+    oracle.project(case.ggml, packed, case.n, case.k, x, threads=threads)  # page in
+    runs, spent = 0, 0.0
+    while spent < budget_seconds and runs < 20000:
+        t0 = time.perf_counter()
+        oracle.project(case.ggml, packed, case.n, case.k, x, threads=threads)
+        spent += time.perf_counter() - t0
+        runs += 1
+    per = spent / runs
+    return {
+        "value": round(case.bytes / per / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{runs} repeats of the same {case.label} step ({per * 1e3:.1f} ms each), "
+                  f"dequant + sequential fp32 dot, rows split over {threads} threads",
+    }
+
+
+def copy_calibration(api, dev, rows=65536, width=1024, launches=10):
+    """Launches expert_assign with identity routing: a row copy that reads and
+    writes rows*width*4 bytes each, the known size the HBM counters are scaled by."""
+    hidden = api.Tensor.from_f32(dev, (rows, width), api.DType.F32,
+                                 np.arange(rows * width, dtype=np.float32) % 251.0)
+    meta = np.zeros((rows, 3), dtype=np.uint32)
+    meta[:, 0] = 0
+    meta[:, 1] = np.arange(rows, dtype=np.uint32)
+    meta[:, 2] = np.float32(1.0).view(np.uint32)
+    metadata = api.Tensor.from_bits(dev, (rows, 3), meta)
+    out = None
+    for _ in range(launches):
+        out = dev.expert_assign(hidden, metadata, 1)
+    dev.synchronize()
+    same = np.array_equal(out.to_f32(), hidden.to_f32())
+    print(json.dumps({"copy_kernel": dev.last_operation(), "launches": launches,
+                      "read_bytes": rows * width * 4 + rows * 12, "write_bytes": rows * width * 4,
+                      "copied_correctly": bool(same)}), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2400)
+    ap.add_argument("--warmup", type=int, default=240)
+    ap.add_argument("--cases", choices=["headline", "all", "copy"], default="all",
+                    help="'headline' times only the metric's GEMV; 'all' adds the other shapes; "
+                         "'copy' launches a plain row copy of known size (counter calibration)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; every box has one and no multi-GPU "
+                 f"path exists (asked for --gpus {args.gpus})")
+
+    from ferrum_amd import api, synth
+    dev = api.Device.new(0)
+    props = dev.properties()
+    f32, f16 = api.DType.F32, api.DType.F16
+    if args.cases == "copy":
+        return copy_calibration(api, dev)
+
+    head = Case(api, synth, dev, Q4_K, 17408, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=17408 f32 x")
+    wall, event = measure(dev, head, args.steps, args.warmup)
+    step_wall, step_event = wall / args.steps, event / args.steps
+    gbs = head.bytes / step_wall / 1e9
+    kernel_gbs = head.bytes / step_event / 1e9
+    head_report = report(head, step_event)
+    cpu = None if args.no_cpu else cpu_baseline(head)
+
+    cases = [head_report]
+    gemm = None
+    if args.cases == "all":
+        def timed(ggml, n, k, m, xd, label, steps, copies=None):
+            c = Case(api, synth, dev, ggml, n, k, m, xd, label, copies)
+            _, ev = measure(dev, c, steps, min(args.warmup, len(c.weights)), repeats=2)
+            r = report(c, ev / steps)
+            cases.append(r)
+            del c
+            return r
+
+        timed(Q4_K, 4096, 4096, 1, f32, "Q4_K GEMV M=1 K=4096 N=4096", 1200)
+        timed(Q4_K, 5120, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=5120", 1200)
+        timed(Q4_K, 5120, 17408, 1, f32, "Q4_K GEMV M=1 K=17408 N=5120", 1200)
+        timed(Q6_K, 5120, 17408, 1, f32, "Q6_K GEMV M=1 K=17408 N=5120", 600)
+        timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
+        for m in (8, 16, 128):
+            timed(Q4_K, 17408, 5120, m, f16, f"Q4_K GEMM M={m} K=5120 N=17408 f16 x", 240)
+        gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
+
+    line = {
+        "metric": "Q4_K GEMV GB/s at M=1, K=5120, N=17408",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_wall * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": head.label,
+            "weights": "Q4_K super-blocks, seeded (d=|N|*0.01, dmin=|N|*0.005, 6-bit scales/mins, nibbles)",
+            "weight_copies_rotated": len(head.weights),
+            "bytes_per_step": head.bytes,
+            "device": props.get("name") or props.get("arch"),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(kernel_gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(kernel_gbs / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES,
+            "kernel": head.operation,
+            "kernel_us": round(step_event * 1e6, 3),
+        },
+        "cpu_baseline": cpu,
+        "gemm_m512": None if gemm is None else {
+            "metric": "Q4_K GEMM TFLOP/s at M=512, K=5120, N=17408, f16 activations, f32 output",
+            "value": gemm["TFLOP/s"],
+            "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": gemm["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": gemm["frac_mfma_f16"], "traffic": None,
+                         "kernel": gemm["operation"], "kernel_us": gemm["us"]},
+        },
+        "cases": cases,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

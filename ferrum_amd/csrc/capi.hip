@@ -155,6 +155,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
     d->tuning["gemm_wide_min_rows"] = 192;  // smallest M that takes the 256-row tile
+    d->tuning["gemm_skinny_max_rows"] = 32; // largest M that takes the register-dequant MFMA kernel (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
         (void)hipStreamDestroy(d->stream);
@@ -219,6 +220,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 2;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
+    } else if (k == "gemm_skinny_max_rows") {
+        ok = value >= 0 && value <= 32;
     }
     if (!ok) return fail(FH_ERR_PARAMETER, "value %lld is out of range for %s", (long long)value, key);
     it->second = value;
@@ -467,6 +470,7 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
         a.y_dtype = y->dtype;
         a.cu_count = device->props.multiProcessorCount;
         a.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
+        a.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         device->last_operation = launch_gemm(device->stream, a);
     } else {
         GemvArgs a{};

@@ -100,10 +100,12 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t* s, uint32_t group, 
 __device__ __forceinline__ void q4k_chunk_scales(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t c,
                                                  float& sc_lo, float& sc_hi, float& mn_lo,
                                                  float& mn_hi) {
-    bool upper = c >= 2;
-    uint32_t scw = upper ? ((s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)) : (s0 & 0x3f3f3f3fu);
-    uint32_t mnw = upper ? (((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u))
-                         : (s1 & 0x3f3f3f3fu);
+    // blended with a mask rather than selected: c differs between lanes and a
+    // select of two computed values tends to come back as a divergent branch
+    const uint32_t upper = 0u - (c >> 1);
+    uint32_t scw = (((s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u)) & upper) | (s0 & 0x3f3f3f3fu & ~upper);
+    uint32_t mnw = ((((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u)) & upper) |
+                   (s1 & 0x3f3f3f3fu & ~upper);
     uint32_t shift = (c & 1u) << 4;
     scw >>= shift;
     mnw >>= shift;

@@ -12,13 +12,12 @@
 // 2 x 2 arrangement, each owning 64 x 64 outputs as 2 x 2 MFMA 32x32x16 tiles.
 // LDS rows are padded to 72 halfs so 128-bit fragment reads are conflict free.
 #include "device_utils.hpp"
+#include "tile_decode.hpp"
 #include "internal.hpp"
 
 namespace fh {
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 64;
@@ -249,19 +248,6 @@ __global__ __launch_bounds__(kThreads) void gemm_tile_kernel(const uint8_t* __re
 // same XCD (ids that are equal mod 8) and share it through that XCD's L2.
 constexpr int kWM = 256;
 
-typedef float float4v __attribute__((ext_vector_type(4)));
-
-template <int DT>
-__device__ __forceinline__ float4v mfma16(uint4 a, uint4 b, float4v c) {
-    if constexpr (DT == 1) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a),
-                                                      __builtin_bit_cast(half8, b), c, 0, 0, 0);
-    } else {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-}
-
 template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c, uint32_t h,
                                               uint16_t* wrow_lds) {
@@ -282,30 +268,6 @@ __device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c,
     dst_hi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
 }
 
-
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-
-// exact widening of an f16 (sub)normal held in one half of a dword
-__device__ __forceinline__ float lo_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).x; }
-__device__ __forceinline__ float hi_half(uint32_t v) { return (float)__builtin_bit_cast(half2v, v).y; }
-
-// Two tile values fma(q, scale, offset), each rounded once to the tile dtype,
-// packed into a dword.  q arrives as an f16 subnormal (an integer quant masked
-// in place, i.e. q * 2^-24 or 16q * 2^-24) and `scale` carries the inverse
-// power of two, so the f32 product is the exact integer multiple and the
-// result has the bits of the reference's (d*sc)*q - dmin*m.  For f16 the
-// compiler emits v_fma_mixlo/mixhi_f16: no conversion or pack instructions.
-template <int DT>
-__device__ __forceinline__ uint32_t fma_pair(float qa, float qb, float scale, float offset) {
-    if constexpr (DT == 1) {
-        half2v r;
-        r.x = (_Float16)fmaf(qa, scale, offset);
-        r.y = (_Float16)fmaf(qb, scale, offset);
-        return __builtin_bit_cast(uint32_t, r);
-    } else {
-        return f32_to_bf16_bits(fmaf(qa, scale, offset)) | (f32_to_bf16_bits(fmaf(qb, scale, offset)) << 16);
-    }
-}
 
 // Raw bytes one producer thread needs from a whole super-block: its half h of
 // each of the four 64-weight K slabs.  Loading by block (not by slab) issues
@@ -693,6 +655,7 @@ void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
 }  // namespace
 
 const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
+    if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
     if (a.m >= (uint32_t)a.wide_min_rows) {
         const WidePlan plan = wide_plan(a.m, a.n, a.cu_count);
         if (a.ggml_type == kQ4K) {

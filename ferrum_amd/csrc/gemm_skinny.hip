@@ -1,0 +1,288 @@
+// Skinny-M projection (2 <= M <= 32 tokens, f16 / bf16 activations) on the
+// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q6_K weights.
+//
+// With this few tokens the job is a weight stream (HBM bound), so nothing of
+// the weights goes through LDS.  A wave owns 16 weight rows.  Its 64 lanes are
+// 16 rows x 4 lane groups, and a lane group owns one quarter of every
+// super-block of its row (Q4_K: one 64-weight chunk, 32 contiguous bytes;
+// Q6_K: 16 positions of one 128-weight half).  The lane decodes its 64 weights
+// in registers straight into eight A operands of v_mfma_f32_16x16x32 (rows =
+// weight rows): an MFMA only needs A and B to agree on which 32 K indices a
+// step covers, so step s simply takes "the s-th run of 8 weights of every lane
+// group's quarter", and the activations are read from LDS in the same order.
+// Decoding is the one-rounding fma of tile_decode.hpp, so tile values carry the
+// bits of the reference's dequantisation rounded once to the tile type.
+//
+// The four waves of a workgroup cover 64 rows and share the activation slab
+// (16*TT tokens x 256 K) of the current super-block through a double-buffered
+// LDS tile; one barrier per super-block.  Every lane keeps kRing super-blocks
+// and kRing activation slabs in flight in registers: loads return in order, so
+// both rings must run equally far ahead or the nearer one would drain the
+// farther.
+#include <hip/hip_runtime.h>
+
+#include "device_utils.hpp"
+#include "tile_decode.hpp"
+#include "internal.hpp"
+
+namespace fh {
+namespace {
+
+constexpr int kSkThreads = 256;
+constexpr int kSkRows = 64;         // weight rows per workgroup
+constexpr int kSlabLd = 256 + 8;    // halfs per token row of the LDS slab (16-byte skew)
+constexpr int kRing = 5;
+
+// One lane's quarter of a super-block, raw, and its decode into 8 A operands.
+// klocal(g, s): K offset inside the super-block of the 8 weights of operand s.
+template <uint32_t TYPE>
+struct Quarter;
+
+template <>
+struct Quarter<kQ4K> {
+    static constexpr uint32_t kBlockBytes = 144;
+    uint4 hdr, qa, qb;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t g) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+        qa = *reinterpret_cast<const uint4*>(block + 16 + 32 * g);
+        qb = *reinterpret_cast<const uint4*>(block + 32 + 32 * g);
+    }
+    // operands 0..3: low nibbles (weights 64g + 8s ..), 4..7: high nibbles (64g + 32 + 8(s-4) ..)
+    static __device__ __forceinline__ uint32_t klocal(uint32_t g, int s) { return 64 * g + 8 * s; }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t g, uint4 (&a)[8]) const {
+        const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc0, sc1, mn0, mn1;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, g, sc0, sc1, mn0, mn1);
+        // d*sc and dmin*m are exact in f32; the powers of two undo the subnormal encoding
+        const float a_lo = (d * sc0) * 16777216.f, a_hi = (d * sc1) * 1048576.f;
+        const float b_lo = -(dmin * mn0), b_hi = -(dmin * mn1);
+        const uint32_t v[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        uint32_t lo[16], hi[16];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t w0 = v[t], w1 = w0 >> 8;
+            const uint32_t l02 = w0 & 0x000f000fu, h02 = w0 & 0x00f000f0u;
+            const uint32_t l13 = w1 & 0x000f000fu, h13 = w1 & 0x00f000f0u;
+            lo[2 * t] = fma_pair<DT>(lo_half(l02), lo_half(l13), a_lo, b_lo);
+            lo[2 * t + 1] = fma_pair<DT>(hi_half(l02), hi_half(l13), a_lo, b_lo);
+            hi[2 * t] = fma_pair<DT>(lo_half(h02), lo_half(h13), a_hi, b_hi);
+            hi[2 * t + 1] = fma_pair<DT>(hi_half(h02), hi_half(h13), a_hi, b_hi);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            a[s] = make_uint4(lo[4 * s], lo[4 * s + 1], lo[4 * s + 2], lo[4 * s + 3]);
+            a[4 + s] = make_uint4(hi[4 * s], hi[4 * s + 1], hi[4 * s + 2], hi[4 * s + 3]);
+        }
+    }
+};
+
+template <>
+struct Quarter<kQ6K> {
+    static constexpr uint32_t kBlockBytes = 210;
+    uint4 la, lb, ph, sc;
+    uint32_t d;
+    // lane group g: half h = g / 2 of the block, positions j0 = 16 (g & 1) .. j0 + 15
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t g) {
+        const uint32_t h = g >> 1, j0 = (g & 1u) * 16;
+        la = load_u4_unaligned(block + 64 * h + j0);
+        lb = load_u4_unaligned(block + 64 * h + 32 + j0);
+        ph = load_u4_unaligned(block + 128 + 32 * h + j0);
+        sc = load_u4_unaligned(block + 192);
+        d = load_u16_unaligned(block + 208);
+    }
+    // operand s: slice s / 2 (32 weights each), positions j0 + 8 (s & 1) ..
+    static __device__ __forceinline__ uint32_t klocal(uint32_t g, int s) {
+        return 128 * (g >> 1) + 32 * (s >> 1) + 16 * (g & 1u) + 8 * (s & 1);
+    }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t g, uint4 (&a)[8]) const {
+        const float df = f16_bits_to_f32(d);
+        const uint32_t h = g >> 1;
+        const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+        const uint32_t lav[4] = {la.x, la.y, la.z, la.w}, lbv[4] = {lb.x, lb.y, lb.z, lb.w};
+        const uint32_t phv[4] = {ph.x, ph.y, ph.z, ph.w};
+        // scales 8h + 2*slice + (g & 1): slices 0,1 in word 2h, slices 2,3 in word 2h + 1
+        const uint32_t w_lo = (h ? scw[2] : scw[0]) >> (8 * (g & 1u));
+        const uint32_t w_hi = (h ? scw[3] : scw[1]) >> (8 * (g & 1u));
+#pragma unroll
+        for (int slice = 0; slice < 4; ++slice) {
+            const uint32_t word = slice < 2 ? w_lo : w_hi;
+            const float s = df * (float)(int)(int8_t)(word >> (16 * (slice & 1)));
+            const float scale = s * ((slice < 2) ? 16777216.f : 1048576.f);  // high nibbles sit 4 bits up
+            const float offset = -32.f * s;
+            uint32_t out[8];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t w0 = (slice & 1) ? lbv[t] : lav[t], w1 = w0 >> 8;
+                const uint32_t p0 = phv[t] >> (2 * slice), p1 = p0 >> 8;
+                uint32_t q02, q13;
+                if (slice < 2) {  // low nibble | plane bits << 4 : q * 2^-24
+                    q02 = (w0 & 0x000f000fu) | ((p0 & 0x00030003u) << 4);
+                    q13 = (w1 & 0x000f000fu) | ((p1 & 0x00030003u) << 4);
+                } else {          // high nibble in place | plane bits << 8 : 16 q * 2^-24
+                    q02 = (w0 & 0x00f000f0u) | ((p0 & 0x00030003u) << 8);
+                    q13 = (w1 & 0x00f000f0u) | ((p1 & 0x00030003u) << 8);
+                }
+                out[2 * t] = fma_pair<DT>(lo_half(q02), lo_half(q13), scale, offset);
+                out[2 * t + 1] = fma_pair<DT>(hi_half(q02), hi_half(q13), scale, offset);
+            }
+            a[2 * slice] = make_uint4(out[0], out[1], out[2], out[3]);
+            a[2 * slice + 1] = make_uint4(out[4], out[5], out[6], out[7]);
+        }
+    }
+};
+
+// One thread's share of an activation slab (16*TT tokens x 256 K) on its way
+// from global memory to LDS.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // a native vector: copies stay in registers
+
+template <int XP>
+struct SlabRegs {
+    u32x4 v[XP];
+    __device__ __forceinline__ void load(const uint16_t* x, uint32_t tok0, uint32_t m, size_t k, size_t col) {
+#pragma unroll
+        for (int p = 0; p < XP; ++p)
+            v[p] = *reinterpret_cast<const u32x4*>(x + (size_t)min(tok0 + 8 * p, m - 1) * k + col);
+    }
+    __device__ __forceinline__ void store(uint16_t* dst) const {
+#pragma unroll
+        for (int p = 0; p < XP; ++p) *reinterpret_cast<u32x4*>(dst + p * 8 * kSlabLd) = v[p];
+    }
+};
+
+template <uint32_t TYPE, int DT, int TT>
+__global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* __restrict__ w,
+                                                                 const uint16_t* __restrict__ x,
+                                                                 void* __restrict__ y, uint32_t m,
+                                                                 uint32_t n, uint32_t nb,
+                                                                 uint32_t y_dtype) {
+    constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
+    constexpr int kTokens = 16 * TT;
+    constexpr int kSlab = kTokens * kSlabLd;      // halfs per LDS buffer
+    constexpr int kXP = 2 * TT;                   // 16-byte pieces of a slab per thread
+    __shared__ __attribute__((aligned(16))) uint16_t slab[2 * kSlab];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t row0 = blockIdx.x * kSkRows + wave * 16;
+    const uint32_t row = min(row0 + r, n - 1);
+    const uint8_t* wrow = w + (size_t)row * nb * kBB;
+    const size_t k = (size_t)nb * 256;
+
+    // activation slab pieces of this thread: piece p covers token 8p + tid / 32, halfs
+    // 8 (tid % 32) ..; tokens past m repeat token m - 1 (their output columns are never
+    // stored), which keeps the loop free of branches
+    const uint32_t xtok = tid >> 5, xcol = 8 * (tid & 31u);
+    const uint32_t xdst = xtok * kSlabLd + xcol;
+    SlabRegs<kXP> xr[kRing];
+    Quarter<TYPE> ring[kRing];
+    // ring[i] holds super-block j with j % kRing == i; xr[i] holds activation slab j + 1
+    {
+        SlabRegs<kXP> first;
+        first.load(x, xtok, m, k, xcol);
+#pragma unroll
+        for (int i = 0; i < kRing; ++i) {
+            ring[i].load(wrow + (size_t)min((uint32_t)i, nb - 1) * kBB, g);
+            xr[i].load(x, xtok, m, k, xcol + 256 * (size_t)min((uint32_t)i + 1, nb - 1));
+        }
+        first.store(slab + xdst);
+    }
+
+    float4v acc[TT];
+#pragma unroll
+    for (int t = 0; t < TT; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    // B operand address of (token r of tile tt, step s) inside a slab
+    uint32_t boff[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) boff[s] = r * kSlabLd + Quarter<TYPE>::klocal(g, s);
+
+    auto multiply = [&](const uint4 (&a)[8], uint32_t buf) {
+        const uint16_t* sl = slab + buf * kSlab;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                const uint4 bfrag = *reinterpret_cast<const uint4*>(sl + boff[s] + t * 16 * kSlabLd);
+                acc[t] = mfma16<DT>(a[s], bfrag, acc[t]);
+            }
+        }
+    };
+
+    uint32_t b = 0;
+    // Full rings, straight-line: a load that would run past the row re-reads the
+    // last super-block / slab instead (a cache hit that is never used), so the
+    // loop body has no branch and the outstanding-load counts stay exact.
+    const uint32_t last = nb - 1;
+    for (; b + kRing <= nb; b += kRing) {
+#pragma unroll
+        for (int i = 0; i < kRing; ++i) {
+            const uint32_t j = b + i;
+            __syncthreads();
+            xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
+            xr[i].load(x, xtok, m, k, xcol + 256 * (size_t)min(j + 1 + kRing, last));
+            uint4 a[8];
+            ring[i].template decode<DT>(g, a);
+            ring[i].load(wrow + (size_t)min(j + kRing, last) * kBB, g);
+            multiply(a, j & 1u);
+        }
+    }
+    // the nb % kRing super-blocks left over are already in registers
+#pragma unroll
+    for (int i = 0; i < kRing - 1; ++i) {
+        const uint32_t j = b + i;
+        if (j < nb) {
+            __syncthreads();
+            xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
+            uint4 a[8];
+            ring[i].template decode<DT>(g, a);
+            multiply(a, j & 1u);
+        }
+    }
+
+    // C layout of 16x16x32: acc[t][v] = (weight row 4g + v, token 16t + r)
+    const uint32_t out_row = row0 + 4 * g;
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+        const uint32_t tok = 16 * t + r;
+        if (tok >= m) continue;
+        const size_t base = (size_t)tok * n + out_row;
+        if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
+            *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
+                make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (out_row + v < n) store_from_f32(y, base + v, y_dtype, acc[t][v]);
+        }
+    }
+}
+
+template <uint32_t TYPE, int DT>
+void launch_tt(hipStream_t s, const GemmArgs& a) {
+    const dim3 grid((a.n + kSkRows - 1) / kSkRows);
+    const uint8_t* w = static_cast<const uint8_t*>(a.w);
+    const uint16_t* x = static_cast<const uint16_t*>(a.x);
+    const uint32_t nb = a.k / 256;
+    if (a.m <= 16) {
+        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1>), grid, dim3(kSkThreads), 0, s, w, x, a.y, a.m,
+                           a.n, nb, a.y_dtype);
+    } else {
+        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 2>), grid, dim3(kSkThreads), 0, s, w, x, a.y, a.m,
+                           a.n, nb, a.y_dtype);
+    }
+}
+
+}  // namespace
+
+const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
+    if (a.ggml_type == kQ4K) {
+        if (a.x_dtype == FH_F16) launch_tt<kQ4K, 1>(s, a); else launch_tt<kQ4K, 2>(s, a);
+        return "q4_k_gemm_mfma_skinny";
+    }
+    if (a.x_dtype == FH_F16) launch_tt<kQ6K, 1>(s, a); else launch_tt<kQ6K, 2>(s, a);
+    return "q6_k_gemm_mfma_skinny";
+}
+
+}  // namespace fh

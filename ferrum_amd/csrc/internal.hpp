@@ -106,8 +106,12 @@ struct GemmArgs {
     uint32_t x_dtype, y_dtype;
     int cu_count;
     int wide_min_rows;   // smallest M that takes the 256-row tile
+    int skinny_max_rows; // largest M that takes the register-dequant kernel
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
+
+// gemm_skinny.hip
+const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a);
 
 // moe.hip
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,

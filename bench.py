@@ -142,6 +142,64 @@ def cpu_baseline(case, budget_seconds=12.0):
     }
 
 
+def moe_case(api, synth, dev, tokens, steps):
+    """A3B-style routed FFN: hidden 2048, 256 experts x intermediate 512 in Q4_K,
+    top-8 softmax routing with renormalised weights, plus one shared expert;
+    f16 activations.  One step = route, gather, gate|up, SiLU*up, down, combine
+    and the shared expert's two projections.  Distinct router logits per step
+    move the set of experts that are hit."""
+    hidden, inter, experts, top_k = 2048, 512, 256, 8
+    fmt = api.QuantizationFormat.Q4_K
+    f16, f32 = api.DType.F16, api.DType.F32
+    eight_in = synth.matrix(Q4_K, 8 * 2 * inter, hidden, seed=11).reshape(8, -1)
+    eight_out = synth.matrix(Q4_K, 8 * hidden, inter, seed=12).reshape(8, -1)
+    win = api.QuantizedExpertMatrix.new(dev, np.tile(eight_in, (experts // 8, 1)).reshape(-1), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(dev, np.tile(eight_out, (experts // 8, 1)).reshape(-1), fmt,
+                                         experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(dev, 2 * inter, hidden, fmt, synth.matrix(Q4_K, 2 * inter, hidden, seed=13))
+    sout = api.QuantizedMatrix.from_bytes(dev, hidden, inter, fmt, synth.matrix(Q4_K, hidden, inter, seed=14))
+    moe = api.SparseMoe(dev, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    moe.workspace(tokens, f16)
+    x = api.Tensor.from_f32(dev, (tokens, hidden), f16,
+                            synth.activations(tokens, hidden, seed=15, f16=True) * np.float32(2.0 ** -6))
+    variants = 16
+    logit_sets, hit = [], []
+    for i in range(variants):
+        values = synth.rng(16, i).standard_normal((tokens, experts)).astype(np.float32)
+        logit_sets.append(api.Tensor.from_f32(dev, values.shape, f32, values))
+        hit.append(len(np.unique(np.argsort(-values, axis=1)[:, :top_k])))
+    s_up = api.Tensor.zeros(dev, (tokens, 2 * inter), f16)
+    s_act = api.Tensor.zeros(dev, (tokens, inter), f16)
+    s_out = api.Tensor.zeros(dev, (tokens, hidden), f16)
+    names = []
+
+    def enqueue(i):
+        moe.forward(x, logit_sets[i % variants])
+        names.append(dev.last_operation())
+        dev.project_quantized(x, sin, out=s_up)
+        dev.expert_silu_mul(s_up, inter, out=s_act)
+        dev.project_quantized(s_act, sout, out=s_out)
+
+    best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(2)) / steps
+    per_expert = (2 * inter * hidden + hidden * inter) // 256 * BLOCK_BYTES[Q4_K]
+    mean_hit = float(np.mean(hit))
+    act_bytes = tokens * hidden * 2 * 2 + tokens * experts * 4
+    nbytes = mean_hit * per_expert + per_expert + act_bytes
+    flops = 2 * tokens * (top_k + 1) * (2 * inter * hidden + hidden * inter)
+    return {
+        "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
+        "operation": "moe_route + expert_assign + 2 x expert_project + silu_mul + combine + shared FFN",
+        "us": round(best * 1e6, 2),
+        "GB/s": round(nbytes / best / 1e9, 1),
+        "frac_hbm": round(nbytes / best / 1e9 / HBM_PEAK_GBS, 4),
+        "TFLOP/s": round(flops / best / 1e12, 2),
+        "frac_mfma_f16": round(flops / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+        "experts_hit_mean": mean_hit,
+        "algorithmic_bytes": int(nbytes),
+    }
+
+
 def copy_calibration(api, dev, rows=65536, width=1024, launches=10):
     """Launches expert_assign with identity routing: a row copy that reads and
     writes rows*width*4 bytes each, the known size the HBM counters are scaled by."""
@@ -210,6 +268,8 @@ def main():
         for m in (8, 16, 128):
             timed(Q4_K, 17408, 5120, m, f16, f"Q4_K GEMM M={m} K=5120 N=17408 f16 x", 240)
         gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
+        cases.append(moe_case(api, synth, dev, 1, 200))
+        cases.append(moe_case(api, synth, dev, 512, 20))
 
     line = {
         "metric": "Q4_K GEMV GB/s at M=1, K=5120, N=17408",

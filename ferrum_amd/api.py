@@ -54,6 +54,7 @@ WeightError = _variant("Weight")
 ParameterError = _variant("Parameter")
 TokenError = _variant("Token")
 ValidationError = _variant("Validation")
+ConfigError = _variant("Config")   # host-side only (src/error.rs: Error::Config)
 
 _ERRORS = {1: ShapeError, 2: DTypeError, 3: DeviceMismatch, 4: RangeError, 5: DispatchError,
            6: SynchronizationError, 7: AllocationError, 8: GgufError, 9: WeightError,
@@ -558,14 +559,16 @@ class Device:
                                          ctypes.byref(yv)))
         return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
 
-    def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy) -> Tensor:
+    def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy,
+                  out: Tensor | None = None) -> Tensor:
         dims = logits.shape()
         if len(dims) != 2 or dims[0] == 0 or dims[1] == 0 or dims[1] != policy.experts:
             raise ShapeError("invalid sparse routing geometry")
         if selection_bias is not None and (selection_bias.shape() != (policy.experts,)
                                            or selection_bias.dtype != DType.F32):
             raise ShapeError("invalid sparse routing geometry")
-        out = Tensor.zeros(self, (dims[0] * max(policy.top_k, 1), 3), DType.F32)
+        if out is None:
+            out = Tensor.zeros(self, (dims[0] * max(policy.top_k, 1), 3), DType.F32)
         lv, ov, pc = logits._view(), out._view(), policy._c()
         bv = selection_bias._view() if selection_bias is not None else None
         _check(_lib.fh_moe_route(self._handle, ctypes.byref(lv), dims[0],
@@ -573,12 +576,14 @@ class Device:
                                  ctypes.byref(ov)))
         return out
 
-    def expert_assign(self, hidden: Tensor, metadata: Tensor, top_k: int) -> Tensor:
+    def expert_assign(self, hidden: Tensor, metadata: Tensor, top_k: int,
+                      out: Tensor | None = None) -> Tensor:
         x, meta = hidden.shape(), metadata.shape()
         if (len(x) != 2 or x[0] == 0 or x[1] == 0 or len(meta) != 2 or meta[1] != 3 or top_k == 0
                 or x[0] * top_k != meta[0] or metadata.dtype != DType.F32):
             raise ShapeError("expert assignments require [S,H] and [S*top_k,3]")
-        out = Tensor.zeros(self, (meta[0], x[1]), hidden.dtype)
+        if out is None:
+            out = Tensor.zeros(self, (meta[0], x[1]), hidden.dtype)
         hv, mv, ov = hidden._view(), metadata._view(), out._view()
         _check(_lib.fh_expert_assign(self._handle, ctypes.byref(hv), x[0], x[1], ctypes.byref(mv),
                                      top_k, ctypes.byref(ov)))
@@ -586,7 +591,7 @@ class Device:
 
     def expert_project_quantized(self, input: Tensor, metadata: Tensor,
                                  weight: QuantizedExpertMatrix, features: int, experts: int,
-                                 out_dtype: DType | None = None) -> Tensor:
+                                 out_dtype: DType | None = None, out: Tensor | None = None) -> Tensor:
         x, meta = input.shape(), metadata.shape()
         if (len(x) != 2 or x[0] == 0 or x[1] != features or meta != (x[0], 3)
                 or metadata.dtype != DType.F32 or experts == 0 or weight.experts() != experts
@@ -595,29 +600,32 @@ class Device:
                 or weight.device is not self):
             raise ShapeError("quantized expert projection geometry mismatch")
         dtype = input.dtype if out_dtype is None else DType(out_dtype)
-        out = Tensor.zeros(self, (x[0], weight.rows_per_expert()), dtype)
+        if out is None:
+            out = Tensor.zeros(self, (x[0], weight.rows_per_expert()), dtype)
         xv, mv, ov = input._view(), metadata._view(), out._view()
         _check(_lib.fh_expert_project_quantized(self._handle, weight._handle, ctypes.byref(xv), x[0],
                                                 ctypes.byref(mv), ctypes.byref(ov)))
         return out
 
-    def expert_silu_mul(self, input: Tensor, intermediate: int) -> Tensor:
+    def expert_silu_mul(self, input: Tensor, intermediate: int, out: Tensor | None = None) -> Tensor:
         x = input.shape()
         if len(x) != 2 or intermediate == 0 or intermediate * 2 != x[1]:
             raise ShapeError("packed expert activation geometry mismatch")
-        out = Tensor.zeros(self, (x[0], intermediate), input.dtype)
+        if out is None:
+            out = Tensor.zeros(self, (x[0], intermediate), input.dtype)
         iv, ov = input._view(), out._view()
         _check(_lib.fh_expert_silu_mul(self._handle, ctypes.byref(iv), x[0], intermediate,
                                        ctypes.byref(ov)))
         return out
 
     def expert_combine(self, input: Tensor, metadata: Tensor, tokens: int, hidden: int,
-                       top_k: int) -> Tensor:
+                       top_k: int, out: Tensor | None = None) -> Tensor:
         x = input.shape()
         if (top_k == 0 or hidden == 0 or x != (tokens * top_k, hidden)
                 or metadata.shape() != (x[0], 3) or metadata.dtype != DType.F32):
             raise ShapeError("expert combine geometry mismatch")
-        out = Tensor.zeros(self, (tokens, hidden), input.dtype)
+        if out is None:
+            out = Tensor.zeros(self, (tokens, hidden), input.dtype)
         iv, mv, ov = input._view(), metadata._view(), out._view()
         _check(_lib.fh_expert_combine(self._handle, ctypes.byref(iv), ctypes.byref(mv), tokens,
                                       hidden, top_k, ctypes.byref(ov)))
@@ -627,6 +635,62 @@ class Device:
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_device_destroy(h)
+
+
+class SparseMoe:
+    """Routed expert FFN, the orchestration of SparseMoe::forward
+    (src/nn/moe.rs:222-390): route -> assign -> gate|up projection -> SiLU*up ->
+    down projection -> weighted combine.  The reference computes the router
+    logits with a dense linear layer of its own; that layer is not part of the
+    quantized path, so `forward` takes the logits.  With `workspace(tokens)`
+    every intermediate is allocated ahead, which lets a forward pass be
+    recorded into an execution."""
+
+    def __init__(self, device: "Device", input_experts: QuantizedExpertMatrix,
+                 output_experts: QuantizedExpertMatrix, routing: MoeRoutingPolicy,
+                 selection_bias: Tensor | None = None):
+        e, two_i, h = input_experts.experts(), input_experts.rows_per_expert(), input_experts.columns()
+        if (two_i == 0 or two_i % 2 or output_experts.experts() != e
+                or output_experts.rows_per_expert() != h or output_experts.columns() * 2 != two_i
+                or routing.experts != e or routing.top_k == 0 or routing.top_k > e
+                or routing.use_expert_bias != (selection_bias is not None)
+                or input_experts.device is not device or output_experts.device is not device):
+            raise ConfigError("invalid sparse expert weight geometry")
+        self.device, self.routing, self.selection_bias = device, routing, selection_bias
+        self.input_experts, self.output_experts = input_experts, output_experts
+        self.expert_count, self.hidden_size, self.intermediate_size = e, h, two_i // 2
+        self._ws = None
+
+    def workspace(self, tokens: int, dtype: DType):
+        a, h, i = tokens * self.routing.top_k, self.hidden_size, self.intermediate_size
+        d = self.device
+        self._ws = {"tokens": tokens, "dtype": dtype,
+                    "metadata": Tensor.zeros(d, (a, 3), DType.F32),
+                    "assigned": Tensor.zeros(d, (a, h), dtype),
+                    "projected": Tensor.zeros(d, (a, 2 * i), dtype),
+                    "activated": Tensor.zeros(d, (a, i), dtype),
+                    "expert_output": Tensor.zeros(d, (a, h), dtype),
+                    "combined": Tensor.zeros(d, (tokens, h), dtype)}
+        return self._ws
+
+    def forward(self, hidden: Tensor, router_logits: Tensor) -> Tensor:
+        dims = hidden.shape()
+        if len(dims) != 2 or dims[1] != self.hidden_size or dims[0] == 0:
+            raise ShapeError("sparse expert input requires [tokens,hidden]")
+        if hidden.buffer.device is not self.device:
+            raise DeviceMismatch("tensor belongs to another device")
+        d, k = self.device, self.routing.top_k
+        ws = self._ws if self._ws and self._ws["tokens"] == dims[0] and self._ws["dtype"] == hidden.dtype else {}
+        metadata = d.moe_route(router_logits, self.selection_bias, self.routing, out=ws.get("metadata"))
+        assigned = d.expert_assign(hidden, metadata, k, out=ws.get("assigned"))
+        projected = d.expert_project_quantized(assigned, metadata, self.input_experts, self.hidden_size,
+                                               self.expert_count, out=ws.get("projected"))
+        activated = d.expert_silu_mul(projected, self.intermediate_size, out=ws.get("activated"))
+        expert_output = d.expert_project_quantized(activated, metadata, self.output_experts,
+                                                   self.intermediate_size, self.expert_count,
+                                                   out=ws.get("expert_output"))
+        return d.expert_combine(expert_output, metadata, dims[0], self.hidden_size, k,
+                                out=ws.get("combined"))
 
 
 def _handle_of(weight):

@@ -156,6 +156,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
     d->tuning["gemm_wide_min_rows"] = 192;  // smallest M that takes the 256-row tile
     d->tuning["gemm_skinny_max_rows"] = 32; // largest M that takes the register-dequant MFMA kernel (0 = never)
+    d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
         (void)hipStreamDestroy(d->stream);
@@ -222,6 +223,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {
         ok = value >= 0 && value <= 32;
+    } else if (k == "expert_grouped_min_assignments") {
+        ok = value >= 0;
     }
     if (!ok) return fail(FH_ERR_PARAMETER, "value %lld is out of range for %s", (long long)value, key);
     it->second = value;
@@ -574,6 +577,36 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
     st = resolve(device, y, (uint64_t)assignments * rows, "expert output", &yr);
     if (st != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(mr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    const int64_t grouped_min = tuning(device, "expert_grouped_min_assignments");
+    if (x->dtype != FH_F32 && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
+        weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
+        // grouped form: every expert's weights are streamed once for all of its assignments
+        const size_t words = (size_t)weight->experts + 1 + assignments;
+        st = ensure_scratch(device, words * sizeof(uint32_t));
+        if (st != FH_OK) return st;
+        uint32_t* offsets = reinterpret_cast<uint32_t*>(scratch_data(device));
+        uint32_t* order = offsets + weight->experts + 1;
+        launch_expert_group(device->stream, reinterpret_cast<const float*>(mr.begin), assignments,
+                            (uint32_t)weight->experts, offsets, order, const_cast<uint8_t*>(yr.begin),
+                            (uint32_t)(rows * dtype_bytes(y->dtype)));
+        GemmArgs g{};
+        g.ggml_type = weight->ggml_type;
+        g.w = weight->ptr;
+        g.x = xr.begin;
+        g.y = const_cast<uint8_t*>(yr.begin);
+        g.n = (uint32_t)rows;
+        g.k = (uint32_t)k;
+        g.m = assignments;
+        g.x_dtype = x->dtype;
+        g.y_dtype = y->dtype;
+        g.cu_count = device->props.multiProcessorCount;
+        g.experts = (uint32_t)weight->experts;
+        g.expert_offsets = offsets;
+        g.expert_order = order;
+        device->last_operation = launch_gemm_skinny(device->stream, g);
+        FH_HIP(hipGetLastError());
+        return FH_OK;
+    }
     GemvArgs a{};
     a.ggml_type = weight->ggml_type;
     a.w = weight->ptr;

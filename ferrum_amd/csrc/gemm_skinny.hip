@@ -138,12 +138,16 @@ struct Quarter<kQ6K> {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // a native vector: copies stay in registers
 
 template <int XP>
+struct SlabRows {
+    const uint16_t* row[XP];  // activation row of the token each piece belongs to, at this thread's column
+};
+
+template <int XP>
 struct SlabRegs {
     u32x4 v[XP];
-    __device__ __forceinline__ void load(const uint16_t* x, uint32_t tok0, uint32_t m, size_t k, size_t col) {
+    __device__ __forceinline__ void load(const SlabRows<XP>& rows, size_t col) {
 #pragma unroll
-        for (int p = 0; p < XP; ++p)
-            v[p] = *reinterpret_cast<const u32x4*>(x + (size_t)min(tok0 + 8 * p, m - 1) * k + col);
+        for (int p = 0; p < XP; ++p) v[p] = *reinterpret_cast<const u32x4*>(rows.row[p] + col);
     }
     __device__ __forceinline__ void store(uint16_t* dst) const {
 #pragma unroll
@@ -151,12 +155,20 @@ struct SlabRegs {
     }
 };
 
-template <uint32_t TYPE, int DT, int TT>
+// GROUPED = false: the dense projection, tokens 0 .. m-1 of x, one weight matrix.
+// GROUPED = true: the routed-expert projection.  blockIdx.y is an expert; its
+// tokens are the assignments order[offsets[e]] .. order[offsets[e+1] - 1] (rows
+// of x and of y), its weights rows [e*n, e*n + n), and the workgroup makes as
+// many passes of 16*TT tokens as the expert's count needs (the weights of the
+// later passes come from L2).
+template <uint32_t TYPE, int DT, int TT, bool GROUPED>
 __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* __restrict__ w,
                                                                  const uint16_t* __restrict__ x,
                                                                  void* __restrict__ y, uint32_t m,
                                                                  uint32_t n, uint32_t nb,
-                                                                 uint32_t y_dtype) {
+                                                                 uint32_t y_dtype,
+                                                                 const uint32_t* __restrict__ offsets,
+                                                                 const uint32_t* __restrict__ order) {
     constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
     constexpr int kTokens = 16 * TT;
     constexpr int kSlab = kTokens * kSlabLd;      // halfs per LDS buffer
@@ -167,122 +179,163 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
     const uint32_t r = lane & 15u, g = lane >> 4;
     const uint32_t row0 = blockIdx.x * kSkRows + wave * 16;
     const uint32_t row = min(row0 + r, n - 1);
-    const uint8_t* wrow = w + (size_t)row * nb * kBB;
     const size_t k = (size_t)nb * 256;
 
+    uint32_t first_token = 0, count = m;
+    size_t expert_row = 0;
+    if constexpr (GROUPED) {
+        first_token = offsets[blockIdx.y];
+        count = offsets[blockIdx.y + 1] - first_token;
+        expert_row = (size_t)blockIdx.y * n;
+    }
+    const uint8_t* wrow = w + (expert_row + row) * nb * kBB;
+
     // activation slab pieces of this thread: piece p covers token 8p + tid / 32, halfs
-    // 8 (tid % 32) ..; tokens past m repeat token m - 1 (their output columns are never
-    // stored), which keeps the loop free of branches
+    // 8 (tid % 32) ..
     const uint32_t xtok = tid >> 5, xcol = 8 * (tid & 31u);
     const uint32_t xdst = xtok * kSlabLd + xcol;
-    SlabRegs<kXP> xr[kRing];
-    Quarter<TYPE> ring[kRing];
-    // ring[i] holds super-block j with j % kRing == i; xr[i] holds activation slab j + 1
-    {
-        SlabRegs<kXP> first;
-        first.load(x, xtok, m, k, xcol);
-#pragma unroll
-        for (int i = 0; i < kRing; ++i) {
-            ring[i].load(wrow + (size_t)min((uint32_t)i, nb - 1) * kBB, g);
-            xr[i].load(x, xtok, m, k, xcol + 256 * (size_t)min((uint32_t)i + 1, nb - 1));
-        }
-        first.store(slab + xdst);
-    }
-
-    float4v acc[TT];
-#pragma unroll
-    for (int t = 0; t < TT; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
 
     // B operand address of (token r of tile tt, step s) inside a slab
     uint32_t boff[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) boff[s] = r * kSlabLd + Quarter<TYPE>::klocal(g, s);
+    const uint32_t last = nb - 1;
 
-    auto multiply = [&](const uint4 (&a)[8], uint32_t buf) {
-        const uint16_t* sl = slab + buf * kSlab;
+    for (uint32_t t0 = 0; t0 < count; t0 += kTokens) {
+        const uint32_t mt = min((uint32_t)kTokens, count - t0);
+        if (t0 != 0) __syncthreads();  // the previous pass is done with the slabs
+        // tokens past the count repeat the last one (their output columns are never
+        // stored), which keeps the loop free of branches
+        SlabRows<kXP> rows;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int p = 0; p < kXP; ++p) {
+            uint32_t token = first_token + t0 + min(xtok + 8 * p, mt - 1);
+            if constexpr (GROUPED) token = order[token];
+            rows.row[p] = x + (size_t)token * k + xcol;
+        }
+
+        SlabRegs<kXP> xr[kRing];
+        Quarter<TYPE> ring[kRing];
+        // ring[i] holds super-block j with j % kRing == i; xr[i] holds activation slab j + 1
+        {
+            SlabRegs<kXP> first;
+            first.load(rows, 0);
 #pragma unroll
-            for (int t = 0; t < TT; ++t) {
-                const uint4 bfrag = *reinterpret_cast<const uint4*>(sl + boff[s] + t * 16 * kSlabLd);
-                acc[t] = mfma16<DT>(a[s], bfrag, acc[t]);
+            for (int i = 0; i < kRing; ++i) {
+                ring[i].load(wrow + (size_t)min((uint32_t)i, last) * kBB, g);
+                xr[i].load(rows, 256 * (size_t)min((uint32_t)i + 1, last));
+                // issue order matters: the loop waits by count, oldest first
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            first.store(slab + xdst);
+        }
+
+        float4v acc[TT];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+        auto multiply = [&](const uint4 (&a)[8], uint32_t buf) {
+            const uint16_t* sl = slab + buf * kSlab;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const uint4 bfrag = *reinterpret_cast<const uint4*>(sl + boff[s] + t * 16 * kSlabLd);
+                    acc[t] = mfma16<DT>(a[s], bfrag, acc[t]);
+                }
+            }
+        };
+
+        uint32_t b = 0;
+        // Full rings, straight-line: a load that would run past the row re-reads the
+        // last super-block / slab instead (a cache hit that is never used), so the
+        // loop body has no branch and the outstanding-load counts stay exact.
+        for (; b + kRing <= nb; b += kRing) {
+#pragma unroll
+            for (int i = 0; i < kRing; ++i) {
+                const uint32_t j = b + i;
+                __syncthreads();
+                // keep the scheduler from pulling a later super-block's decode up to here:
+                // it would have to wait for that block's loads and drain the ring
+                __builtin_amdgcn_sched_barrier(0);
+                xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
+                xr[i].load(rows, 256 * (size_t)min(j + 1 + kRing, last));
+                uint4 a[8];
+                ring[i].template decode<DT>(g, a);
+                ring[i].load(wrow + (size_t)min(j + kRing, last) * kBB, g);
+                multiply(a, j & 1u);
             }
         }
-    };
-
-    uint32_t b = 0;
-    // Full rings, straight-line: a load that would run past the row re-reads the
-    // last super-block / slab instead (a cache hit that is never used), so the
-    // loop body has no branch and the outstanding-load counts stay exact.
-    const uint32_t last = nb - 1;
-    for (; b + kRing <= nb; b += kRing) {
+        // the nb % kRing super-blocks left over are already in registers
 #pragma unroll
-        for (int i = 0; i < kRing; ++i) {
+        for (int i = 0; i < kRing - 1; ++i) {
             const uint32_t j = b + i;
-            __syncthreads();
-            xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
-            xr[i].load(x, xtok, m, k, xcol + 256 * (size_t)min(j + 1 + kRing, last));
-            uint4 a[8];
-            ring[i].template decode<DT>(g, a);
-            ring[i].load(wrow + (size_t)min(j + kRing, last) * kBB, g);
-            multiply(a, j & 1u);
+            if (j < nb) {
+                __syncthreads();
+                xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
+                uint4 a[8];
+                ring[i].template decode<DT>(g, a);
+                multiply(a, j & 1u);
+            }
         }
-    }
-    // the nb % kRing super-blocks left over are already in registers
-#pragma unroll
-    for (int i = 0; i < kRing - 1; ++i) {
-        const uint32_t j = b + i;
-        if (j < nb) {
-            __syncthreads();
-            xr[i].store(slab + ((j + 1) & 1u) * kSlab + xdst);
-            uint4 a[8];
-            ring[i].template decode<DT>(g, a);
-            multiply(a, j & 1u);
-        }
-    }
 
-    // C layout of 16x16x32: acc[t][v] = (weight row 4g + v, token 16t + r)
-    const uint32_t out_row = row0 + 4 * g;
+        // C layout of 16x16x32: acc[t][v] = (weight row 4g + v, token 16t + r)
+        const uint32_t out_row = row0 + 4 * g;
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-        const uint32_t tok = 16 * t + r;
-        if (tok >= m) continue;
-        const size_t base = (size_t)tok * n + out_row;
-        if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
-            *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
-                make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-        } else {
+        for (int t = 0; t < TT; ++t) {
+            const uint32_t tok = 16 * t + r;
+            if (tok >= mt) continue;
+            uint32_t token = first_token + t0 + tok;
+            if constexpr (GROUPED) token = order[token];
+            const size_t base = (size_t)token * n + out_row;
+            if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
+                *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
+                    make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+            } else {
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (out_row + v < n) store_from_f32(y, base + v, y_dtype, acc[t][v]);
+                for (int v = 0; v < 4; ++v)
+                    if (out_row + v < n) store_from_f32(y, base + v, y_dtype, acc[t][v]);
+            }
         }
     }
 }
 
 template <uint32_t TYPE, int DT>
 void launch_tt(hipStream_t s, const GemmArgs& a) {
-    const dim3 grid((a.n + kSkRows - 1) / kSkRows);
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
     const uint32_t nb = a.k / 256;
+    if (a.expert_offsets != nullptr) {
+        const dim3 grid((a.n + kSkRows - 1) / kSkRows, a.experts);
+        if (a.m <= 8 * a.experts) {   // mean tokens per expert <= 8
+            hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1, true>), grid, dim3(kSkThreads), 0, s, w, x,
+                               a.y, a.m, a.n, nb, a.y_dtype, a.expert_offsets, a.expert_order);
+        } else {
+            hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 2, true>), grid, dim3(kSkThreads), 0, s, w, x,
+                               a.y, a.m, a.n, nb, a.y_dtype, a.expert_offsets, a.expert_order);
+        }
+        return;
+    }
+    const dim3 grid((a.n + kSkRows - 1) / kSkRows);
     if (a.m <= 16) {
-        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1>), grid, dim3(kSkThreads), 0, s, w, x, a.y, a.m,
-                           a.n, nb, a.y_dtype);
+        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1, false>), grid, dim3(kSkThreads), 0, s, w, x, a.y,
+                           a.m, a.n, nb, a.y_dtype, nullptr, nullptr);
     } else {
-        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 2>), grid, dim3(kSkThreads), 0, s, w, x, a.y, a.m,
-                           a.n, nb, a.y_dtype);
+        hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 2, false>), grid, dim3(kSkThreads), 0, s, w, x, a.y,
+                           a.m, a.n, nb, a.y_dtype, nullptr, nullptr);
     }
 }
 
 }  // namespace
 
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
+    const bool grouped = a.expert_offsets != nullptr;
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) launch_tt<kQ4K, 1>(s, a); else launch_tt<kQ4K, 2>(s, a);
-        return "q4_k_gemm_mfma_skinny";
+        return grouped ? "expert_project_q4_k_grouped_mfma" : "q4_k_gemm_mfma_skinny";
     }
     if (a.x_dtype == FH_F16) launch_tt<kQ6K, 1>(s, a); else launch_tt<kQ6K, 2>(s, a);
-    return "q6_k_gemm_mfma_skinny";
+    return grouped ? "expert_project_q6_k_grouped_mfma" : "q6_k_gemm_mfma_skinny";
 }
 
 }  // namespace fh

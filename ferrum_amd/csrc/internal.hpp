@@ -107,6 +107,12 @@ struct GemmArgs {
     int cu_count;
     int wide_min_rows;   // smallest M that takes the 256-row tile
     int skinny_max_rows; // largest M that takes the register-dequant kernel
+    // routed-expert form of the register-dequant kernel: w is [experts, n, k],
+    // x and y rows are assignments, m is their count; tokens of expert e are
+    // expert_order[expert_offsets[e] .. expert_offsets[e + 1])
+    uint32_t experts;
+    const uint32_t* expert_offsets;
+    const uint32_t* expert_order;
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 
@@ -117,6 +123,9 @@ const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a);
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
                              const float* bias, float* metadata, uint32_t tokens,
                              const fh_routing_policy& policy);
+const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t assignments,
+                                uint32_t experts, uint32_t* offsets, uint32_t* order, void* y,
+                                uint32_t row_bytes);
 const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,
                                  void* out, uint32_t assignments, uint32_t row_bytes);
 const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,

@@ -204,6 +204,56 @@ unsigned grid_for(size_t threads) {
     return (unsigned)blocks;
 }
 
+// Groups assignments by expert for the grouped projection: offsets[e] is the
+// first slot of expert e in `order` (offsets[experts] = number of valid
+// assignments) and order[] lists assignment ids expert by expert.  The order
+// inside an expert is whatever the LDS atomics give; every output row depends
+// on its own assignment only, so results do not depend on it.  Rows whose
+// expert id is out of range are zero-filled here, as the per-assignment form
+// leaves them.  One workgroup; experts <= 1024.
+constexpr int kGroupThreads = 1024;
+
+__global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float* __restrict__ metadata,
+                                                                     uint32_t assignments, uint32_t experts,
+                                                                     uint32_t* __restrict__ offsets,
+                                                                     uint32_t* __restrict__ order,
+                                                                     uint32_t* __restrict__ y_words,
+                                                                     uint32_t row_words) {
+    __shared__ uint32_t count[kGroupThreads];
+    __shared__ uint32_t scan[kGroupThreads];
+    const uint32_t tid = threadIdx.x;
+    count[tid] = 0;
+    __syncthreads();
+    for (uint32_t a = tid; a < assignments; a += kGroupThreads) {
+        const uint32_t e = __float_as_uint(metadata[3 * (size_t)a]);
+        if (e < experts) atomicAdd(&count[e], 1u);
+    }
+    __syncthreads();
+    // inclusive scan over the expert counts
+    uint32_t v = count[tid];
+    scan[tid] = v;
+    __syncthreads();
+    for (uint32_t step = 1; step < kGroupThreads; step <<= 1) {
+        const uint32_t add = tid >= step ? scan[tid - step] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    const uint32_t first = scan[tid] - v;
+    if (tid < experts) offsets[tid] = first;
+    if (tid == experts - 1) offsets[experts] = scan[tid];
+    count[tid] = first;  // now the next free slot of each expert
+    __syncthreads();
+    for (uint32_t a = tid; a < assignments; a += kGroupThreads) {
+        const uint32_t e = __float_as_uint(metadata[3 * (size_t)a]);
+        if (e < experts) {
+            order[atomicAdd(&count[e], 1u)] = a;
+        } else {
+            for (uint32_t i = 0; i < row_words; ++i) y_words[(size_t)a * row_words + i] = 0u;
+        }
+    }
+}
+
 }  // namespace
 
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
@@ -213,6 +263,14 @@ const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_
                        logits, logits_dtype, bias, metadata, tokens, p.experts, p.top_k, p.sigmoid,
                        p.normalize_top_k_prob, p.normalization_epsilon, p.routed_scaling_factor);
     return "moe_route";
+}
+
+const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t assignments,
+                                uint32_t experts, uint32_t* offsets, uint32_t* order, void* y,
+                                uint32_t row_bytes) {
+    hipLaunchKernelGGL(expert_group_kernel, dim3(1), dim3(kGroupThreads), 0, s, metadata, assignments,
+                       experts, offsets, order, static_cast<uint32_t*>(y), row_bytes / 4);
+    return "expert_group";
 }
 
 const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,

@@ -192,3 +192,129 @@ def test_routed_ffn_pipeline_matches_the_oracle(api, d, tokens):
     assert np.abs(want).max() > 1e-2
     assert rel_l2(got, want) <= 2e-5
     assert np.abs(got - want).max() <= 2e-5 * max(1.0, np.abs(want).max()) * 8
+
+
+def _routing_rows(expert_ids):
+    meta = np.zeros((len(expert_ids), 3), dtype=np.uint32)
+    meta[:, 0] = expert_ids
+    meta[:, 1] = np.arange(len(expert_ids))
+    meta[:, 2] = np.float32(1.0).view(np.uint32)
+    return meta
+
+
+@pytest.mark.parametrize("ggml,dtype", [(Q4_K, "F16"), (Q4_K, "BF16"), (Q6_K, "F16")])
+def test_grouped_expert_projection_matches_the_oracle_and_the_direct_form(api, d, ggml, dtype):
+    # 6 experts x 72 rows (a ragged last row tile), K = 768.  Expert 3 gets no
+    # assignment, expert 1 gets 37 (more than one pass of 32 tokens), expert 5
+    # a single one, and two assignments carry an expert id that does not exist.
+    experts, rows, cols = 6, 72, 768
+    rng = synth.rng(51)
+    ids = np.concatenate([np.full(37, 1), np.full(9, 0), np.full(17, 2), np.full(12, 4), [5], [9, 77]])
+    rng.shuffle(ids)
+    packed = synth.matrix(ggml, experts * rows, cols, seed=52)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(ggml), experts, rows, cols)
+    dt = getattr(api.DType, dtype)
+    code = oracle.F16 if dtype == "F16" else oracle.BF16
+    x = api.Tensor.from_f32(d, (len(ids), cols), dt, synth.activations(len(ids), cols, seed=53))
+    meta = api.Tensor.from_bits(d, (len(ids), 3), _routing_rows(ids))
+    valid = ids < experts
+
+    got = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32)
+    assert d.last_operation() == ("expert_project_q4_k_grouped_mfma" if ggml == Q4_K
+                                  else "expert_project_q6_k_grouped_mfma")
+    got = got.to_f32()
+    safe = _routing_rows(np.where(valid, ids, 0)).view(np.float32)
+    tile = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), safe,
+                                 weight_round=code, accumulate="f64")
+    full = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), safe, accumulate="f64")
+    assert np.all(got[~valid] == 0), "rows of unknown experts are zero"
+    assert_matmul_parity(got[valid], tile[valid], "grouped expert projection (tile-rounded weights)")
+    assert rel_l2(got[valid], full[valid]) <= (6e-4 if dtype == "F16" else 5e-3)
+
+    d.set_tuning("expert_grouped_min_assignments", 0)
+    try:
+        direct = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32)
+        assert d.last_operation().endswith("_factored")
+        direct = direct.to_f32()
+    finally:
+        d.set_tuning("expert_grouped_min_assignments", 32)
+    assert_matmul_parity(direct[valid], full[valid], "direct expert projection")
+    assert np.all(direct[~valid] == 0)
+
+    half = d.expert_project_quantized(x, meta, w, cols, experts).to_f32()   # output in the input dtype
+    assert np.array_equal(bits(half), bits(oracle.round_storage(got, code)))
+
+
+@pytest.mark.parametrize("tokens", [1, 512])
+def test_a3b_style_ffn_with_shared_expert(api, d, tokens):
+    # hidden 2048, 256 experts of intermediate 512, top-8 after softmax with
+    # renormalised weights, plus one always-on shared expert; f16 activations.
+    hidden, inter, experts, top_k = 2048, 512, 256, 8
+    fmt = api.QuantizationFormat.Q4_K
+    # 256 distinct experts would take the CPU side minutes: 8 distinct weight
+    # sets are tiled 32 times, which leaves routing, grouping and addressing
+    # at full size while the oracle evaluates 8 experts' worth of rows
+    distinct = 8
+    w_in8 = synth.matrix(Q4_K, distinct * 2 * inter, hidden, seed=61).reshape(distinct, -1)
+    w_out8 = synth.matrix(Q4_K, distinct * hidden, inter, seed=62).reshape(distinct, -1)
+    w_in = np.tile(w_in8, (experts // distinct, 1)).reshape(-1)
+    w_out = np.tile(w_out8, (experts // distinct, 1)).reshape(-1)
+    s_in = synth.matrix(Q4_K, 2 * inter, hidden, seed=63)
+    s_out = synth.matrix(Q4_K, hidden, inter, seed=64)
+    # the synthetic weights are O(1), so unit activations would overflow f16 after two
+    # chained projections; 2^-6 keeps every stage inside the f16 range
+    x = synth.activations(tokens, hidden, seed=65, f16=True) * np.float32(2.0 ** -6)
+    logits = synth.rng(66).standard_normal((tokens, experts)).astype(np.float32)
+
+    win = api.QuantizedExpertMatrix.new(d, w_in, fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, w_out, fmt, experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, s_in)
+    sout = api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, s_out)
+    policy = api.MoeRoutingPolicy(experts, top_k)
+    f16, f32 = api.DType.F16, api.DType.F32
+
+    xt = api.Tensor.from_f32(d, x.shape, f16, x)
+    meta = d.moe_route(api.Tensor.from_f32(d, logits.shape, f32, logits), None, policy)
+    assigned = d.expert_assign(xt, meta, top_k)
+    up = d.expert_project_quantized(assigned, meta, win, hidden, experts)
+    assert d.last_operation() == ("expert_project_q4_k_grouped_mfma" if tokens > 1
+                                  else "expert_project_q4_k_factored")
+    act = d.expert_silu_mul(up, inter)
+    down = d.expert_project_quantized(act, meta, wout, inter, experts)
+    routed = d.expert_combine(down, meta, tokens, hidden, top_k).to_f32()
+    s_up = d.project_quantized(xt, sin).tensor
+    s_act = d.expert_silu_mul(s_up, inter)
+    shared = d.project_quantized(s_act, sout).tensor.to_f32()
+    got = routed + shared
+
+    m = oracle.select_routes(logits, experts, top_k)
+    assert np.array_equal(bits(meta.to_f32()[:, :2]), bits(m[:, :2]))
+    # a token's output depends on its own eight routes only: the oracle follows
+    # every token at T = 1 and a sample of 24 tokens at T = 512
+    picked = np.arange(tokens) if tokens <= 24 else np.sort(synth.rng(67).choice(tokens, 24, replace=False))
+    m = m.reshape(tokens, top_k, 3)[picked].reshape(-1, 3).copy()
+    m[:, 1] = np.repeat(np.arange(len(picked), dtype=np.uint32), top_k).view(np.float32)
+    x, got, tokens = x[picked], got[picked], len(picked)
+    folded = m.copy()
+    folded_ids = m[:, 0].view(np.uint32) % distinct
+    folded[:, 0] = folded_ids.astype(np.uint32).view(np.float32)
+    tile = oracle.F16 if tokens > 1 else 0     # one token runs the f32-weight GEMV form
+    o_up = oracle.expert_project(Q4_K, w_in8.reshape(-1), distinct, 2 * inter, hidden,
+                                 oracle.expert_assign(x, m), folded, weight_round=tile,
+                                 out_round=oracle.F16, accumulate="f64")
+    o_act = oracle.expert_silu_mul(o_up, inter, oracle.F16)
+    o_down = oracle.expert_project(Q4_K, w_out8.reshape(-1), distinct, hidden, inter, o_act, folded,
+                                   weight_round=tile, out_round=oracle.F16, accumulate="f64")
+    o_routed = oracle.expert_combine(o_down, m, tokens, hidden, top_k, oracle.F16)
+    stile = oracle.F16 if tokens > 1 else 0
+    o_sup = oracle.round_storage(oracle.project(Q4_K, s_in, 2 * inter, hidden, x, accumulate="f64",
+                                                weight_round=stile), oracle.F16)
+    o_sact = oracle.expert_silu_mul(o_sup, inter, oracle.F16)
+    o_shared = oracle.round_storage(oracle.project(Q4_K, s_out, hidden, inter, o_sact, accumulate="f64",
+                                                   weight_round=stile), oracle.F16)
+    want = o_routed + o_shared
+    assert np.abs(want).max() > 1e-2
+    # every stage stores f16, so a last-place difference in an intermediate moves
+    # the result by about one f16 step of that stage
+    assert rel_l2(got, want) <= 2e-3
+    assert np.abs(got - want).max() <= 4e-3 * np.abs(want).max()

@@ -656,7 +656,9 @@ void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
 
 const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
-    if (a.m >= (uint32_t)a.wide_min_rows) {
+    // the 256-row tile pays off only when its workgroups cover at least half the chip
+    const uint64_t wide_wgs = (uint64_t)((a.m + kWM - 1) / kWM) * ((a.n + 127) / 128);
+    if (a.m >= (uint32_t)a.wide_min_rows && wide_wgs * 2 >= (uint64_t)a.cu_count) {
         const WidePlan plan = wide_plan(a.m, a.n, a.cu_count);
         if (a.ggml_type == kQ4K) {
             if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan); else launch_wide_nt<kQ4K, 2>(s, a, plan);

@@ -300,14 +300,190 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
     }
 }
 
+// Routed-expert projection with the expert's activations resident in LDS.
+// When an expert's tokens (16*TT of them at a time) fit LDS for the whole K, a
+// workgroup gathers them once and then streams weight rows past them with no
+// further barrier: wave w takes row tiles w, w+4, ... of the workgroup's share
+// and walks (tile, super-block) units through a register ring, so the prefetch
+// runs across tile boundaries.  blockIdx.y = expert, blockIdx.x = which share
+// of the expert's rows.  Dynamic LDS: 16*TT rows of (K + 8) halfs.
+constexpr int kResRing = 6;
+
+template <uint32_t TYPE, int DT, int TT>
+__global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8_t* __restrict__ w,
+                                                                     const uint16_t* __restrict__ x,
+                                                                     void* __restrict__ y, uint32_t n,
+                                                                     uint32_t nb, uint32_t y_dtype,
+                                                                     const uint32_t* __restrict__ offsets,
+                                                                     const uint32_t* __restrict__ order,
+                                                                     uint32_t tiles_per_wg) {
+    constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
+    constexpr int kTokens = 16 * TT;
+    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t k = nb * 256, ld = k + 8;
+    const uint32_t first_token = offsets[blockIdx.y];
+    const uint32_t count = offsets[blockIdx.y + 1] - first_token;
+    const uint32_t tiles = (n + 15) / 16;
+    const uint32_t tile_begin = blockIdx.x * tiles_per_wg + wave;
+    const uint32_t tile_end = min(tiles, (blockIdx.x + 1) * tiles_per_wg);
+    const uint8_t* wexpert = w + (size_t)blockIdx.y * n * nb * kBB;
+    const uint32_t pieces = k / 8;  // 16-byte pieces per activation row
+
+    for (uint32_t t0 = 0; t0 < count; t0 += kTokens) {
+        const uint32_t mt = min((uint32_t)kTokens, count - t0);
+        if (t0 != 0) __syncthreads();  // the previous pass is done with the rows
+        // gather the expert's rows, eight 16-byte pieces per thread in flight at a time
+        const uint32_t total = mt * pieces;
+        for (uint32_t base = 0; base < total; base += 8 * kSkThreads) {
+            u32x4 v[8];
+            uint32_t dst[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t idx = min(base + j * kSkThreads + tid, total - 1);
+                const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
+                dst[j] = tok * ld + 8 * pc;
+                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)order[first_token + t0 + tok] * k + 8 * pc);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
+        }
+        __syncthreads();
+        if (tile_begin >= tile_end) continue;  // uniform per wave; no barrier follows in this pass
+
+        // B operand rows: token 16t + r, clamped (columns past mt are never stored)
+        uint32_t boff[TT];
+        uint32_t out_token[TT];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+            const uint32_t tok = min(16u * t + r, mt - 1);
+            boff[t] = tok * ld;
+            out_token[t] = order[first_token + t0 + tok];
+        }
+        uint32_t kl[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) kl[s] = Quarter<TYPE>::klocal(g, s);
+
+        // units = (tile, super-block) pairs of this wave, in order
+        const uint32_t my_tiles = (tile_end - tile_begin + 3) / 4;
+        const uint32_t units = my_tiles * nb;
+        auto unit_ptr = [&](uint32_t tile, uint32_t b) {
+            const uint32_t row = min(tile * 16 + r, n - 1);
+            return wexpert + ((size_t)row * nb + b) * kBB;
+        };
+        Quarter<TYPE> ring[kResRing];
+        uint32_t ptile = tile_begin, pb = 0;  // next unit to prefetch
+        auto prefetch = [&](Quarter<TYPE>& slot) {
+            slot.load(unit_ptr(min(ptile, tile_end - 1), pb), g);
+            if (++pb == nb) {
+                pb = 0;
+                ptile += 4;
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < kResRing; ++i) {
+            prefetch(ring[i]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        float4v acc[TT];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+        uint32_t tile = tile_begin, b = 0;
+        auto consume = [&](Quarter<TYPE>& slot) {
+            uint4 a[8];
+            slot.template decode<DT>(g, a);
+            prefetch(slot);
+            const uint16_t* xb = xs + 256 * b;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    const uint4 bfrag = *reinterpret_cast<const uint4*>(xb + boff[t] + kl[s]);
+                    acc[t] = mfma16<DT>(a[s], bfrag, acc[t]);
+                }
+            }
+            if (++b == nb) {
+                // C layout of 16x16x32: acc[t][v] = (weight row 4g + v, token 16t + r)
+                const uint32_t out_row = tile * 16 + 4 * g;
+#pragma unroll
+                for (int t = 0; t < TT; ++t) {
+                    if (16u * t + r < mt) {
+                        const size_t base = (size_t)out_token[t] * n + out_row;
+                        if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
+                            *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
+                                make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+                        } else if (y_dtype != FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
+                            uint2 packed;
+                            if (y_dtype == FH_F16) {
+                                packed.x = f32_to_f16_bits(acc[t][0]) | (f32_to_f16_bits(acc[t][1]) << 16);
+                                packed.y = f32_to_f16_bits(acc[t][2]) | (f32_to_f16_bits(acc[t][3]) << 16);
+                            } else {
+                                packed.x = f32_to_bf16_bits(acc[t][0]) | (f32_to_bf16_bits(acc[t][1]) << 16);
+                                packed.y = f32_to_bf16_bits(acc[t][2]) | (f32_to_bf16_bits(acc[t][3]) << 16);
+                            }
+                            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + base) = packed;
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v)
+                                if (out_row + v < n) store_from_f32(y, base + v, y_dtype, acc[t][v]);
+                        }
+                    }
+                    acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+                }
+                b = 0;
+                tile += 4;
+            }
+        };
+        uint32_t u = 0;
+        for (; u + kResRing <= units; u += kResRing) {
+#pragma unroll
+            for (int i = 0; i < kResRing; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                consume(ring[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kResRing - 1; ++i)
+            if (u + i < units) consume(ring[i]);
+    }
+}
+
 template <uint32_t TYPE, int DT>
 void launch_tt(hipStream_t s, const GemmArgs& a) {
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
     const uint32_t nb = a.k / 256;
     if (a.expert_offsets != nullptr) {
+        const bool wide = a.m > 8 * a.experts;   // mean tokens per expert > 8: 32 tokens a pass
+        const size_t lds = (size_t)(wide ? 32 : 16) * (a.k + 8) * 2;
+        if (lds <= 150u * 1024) {
+            // the expert's rows are cut into shares so that about 1024 workgroups exist
+            const uint32_t tiles = (a.n + 15) / 16;
+            uint32_t shares = (1024 + a.experts - 1) / a.experts;
+            shares = shares < 1 ? 1 : shares;
+            uint32_t tiles_per_wg = (tiles + shares - 1) / shares;
+            tiles_per_wg = (tiles_per_wg + 3) / 4 * 4;
+            const dim3 rgrid((tiles + tiles_per_wg - 1) / tiles_per_wg, a.experts);
+            if (wide) {
+                auto kernel = expert_resident_kernel<TYPE, DT, 2>;
+                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                hipLaunchKernelGGL(kernel, rgrid, dim3(kSkThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
+                                   a.expert_offsets, a.expert_order, tiles_per_wg);
+            } else {
+                auto kernel = expert_resident_kernel<TYPE, DT, 1>;
+                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                hipLaunchKernelGGL(kernel, rgrid, dim3(kSkThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
+                                   a.expert_offsets, a.expert_order, tiles_per_wg);
+            }
+            return;
+        }
         const dim3 grid((a.n + kSkRows - 1) / kSkRows, a.experts);
-        if (a.m <= 8 * a.experts) {   // mean tokens per expert <= 8
+        if (!wide) {
             hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1, true>), grid, dim3(kSkThreads), 0, s, w, x,
                                a.y, a.m, a.n, nb, a.y_dtype, a.expert_offsets, a.expert_order);
         } else {

@@ -66,5 +66,21 @@ def build(extra_flags: list[str] | None = None, jobs: int = 5, output: str | Non
     return target
 
 
+def build_host_test() -> str:
+    """Compiles the C++ host-side test (g++, no HIP headers needed) against the
+    built library and the CPU oracle; the GPU test suite runs the binary."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "host_mirror_test.cpp")
+    out = os.path.join(root, "tests", "cpp", "host_mirror_test")
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-I" + os.path.join(root, "include"), src, "-o", out,
+           "-L" + LIB_DIR, "-lferrum_hip", "-L" + os.path.join(root, "oracle"), "-lferrum_oracle",
+           "-Wl,-rpath,$ORIGIN/../../ferrum_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle",
+           "-Wl,-rpath,/opt/rocm/lib"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"g++ failed for the host test:\n{proc.stdout}\n{proc.stderr}")
+    return out
+
+
 if __name__ == "__main__":
     print(build(sys.argv[1:]))

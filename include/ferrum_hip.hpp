@@ -1,0 +1,444 @@
+// ferrum_hip.hpp -- C++17 host side over the C ABI of ferrum_hip.h.
+//
+// It mirrors the operator interface of the reference's device type for the
+// quantized-matmul path: the same names, argument meaning and error variants
+// as MetalDevice::project_quantized (src/ops/transformer.rs:96-297), the
+// routed-expert operators (src/ops/mod.rs:23-551), QuantizedMatrix /
+// QuantizedExpertMatrix (src/quantization.rs:76-194), Tensor and DType
+// (src/tensor/mod.rs), Execution (src/metal/mod.rs:263-278) and
+// SparseMoe::forward (src/nn/moe.rs:222-390).  Header only; link
+// libferrum_hip.so.  Errors are thrown as ferrum::Error carrying the variant
+// of src/error.rs:3-51.  Like the reference's Rc handles, nothing here is
+// thread-safe.
+#ifndef FERRUM_HIP_HPP
+#define FERRUM_HIP_HPP
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <functional>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "ferrum_hip.h"
+
+namespace ferrum {
+
+enum class ErrorKind {
+    Shape = FH_ERR_SHAPE, DType = FH_ERR_DTYPE, DeviceMismatch = FH_ERR_DEVICE_MISMATCH,
+    Range = FH_ERR_RANGE, Dispatch = FH_ERR_DISPATCH, Synchronization = FH_ERR_SYNCHRONIZATION,
+    Allocation = FH_ERR_ALLOCATION, Gguf = FH_ERR_GGUF, Weight = FH_ERR_WEIGHT,
+    Parameter = FH_ERR_PARAMETER, Token = FH_ERR_TOKEN, Validation = FH_ERR_VALIDATION,
+    Config = 100  // host-side only
+};
+
+class Error : public std::runtime_error {
+public:
+    Error(ErrorKind kind, const std::string& message) : std::runtime_error(message), kind_(kind) {}
+    ErrorKind kind() const { return kind_; }
+private:
+    ErrorKind kind_;
+};
+
+inline void check(fh_status status) {
+    if (status != FH_OK) throw Error(static_cast<ErrorKind>(status), fh_last_error());
+}
+
+enum class DType : uint32_t { F32 = FH_F32, F16 = FH_F16, BF16 = FH_BF16 };
+inline size_t size_bytes(DType d) { return d == DType::F32 ? 4 : 2; }
+
+// ---- storage rounding, as DType::round / Tensor::from_f32 (src/tensor/mod.rs:19-25) ----
+inline uint16_t f32_to_bf16_bits(float v) {
+    uint32_t u;
+    std::memcpy(&u, &v, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+inline float bf16_bits_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float v;
+    std::memcpy(&v, &u, 4);
+    return v;
+}
+inline uint16_t f32_to_f16_bits(float v) {
+    uint32_t u;
+    std::memcpy(&u, &v, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    u &= 0x7fffffffu;
+    if (u > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((u >> 13) & 0x1ffu));
+    if (u >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);  // >= 65536 (or inf)
+    if (u < 0x33000001u) return (uint16_t)sign;                // rounds to zero
+    int32_t exp = (int32_t)(u >> 23) - 127;
+    uint32_t man = (u & 0x7fffffu) | 0x800000u;
+    int shift = exp < -14 ? 13 + (-14 - exp) : 13;              // subnormal results lose more bits
+    uint32_t half = man >> shift, rest = man & ((1u << shift) - 1), mid = 1u << (shift - 1);
+    if (rest > mid || (rest == mid && (half & 1u))) ++half;
+    uint32_t bits = exp < -14 ? half : ((uint32_t)(exp + 15) << 10) + (half - 0x400u);
+    if (bits >= 0x7c00u) bits = 0x7c00u;
+    return (uint16_t)(sign | bits);
+}
+inline float f16_bits_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 31u, man = h & 0x3ffu;
+    float v;
+    if (exp == 0) {
+        v = std::ldexp((float)man, -24);
+    } else if (exp == 31) {
+        uint32_t u = 0x7f800000u | (man << 13);
+        std::memcpy(&v, &u, 4);
+    } else {
+        v = std::ldexp((float)(man | 0x400u), (int)exp - 25);
+    }
+    uint32_t u;
+    std::memcpy(&u, &v, 4);
+    u |= sign;
+    std::memcpy(&v, &u, 4);
+    return v;
+}
+
+enum class QuantizationFormat : uint32_t { Q4_K = FH_GGML_Q4_K, Q6_K = FH_GGML_Q6_K };
+inline size_t block_elements(QuantizationFormat) { return 256; }
+inline size_t block_bytes(QuantizationFormat f) { return f == QuantizationFormat::Q4_K ? 144 : 210; }
+inline QuantizationFormat format_from_ggml_type(uint32_t id) {
+    if (id == FH_GGML_Q4_K) return QuantizationFormat::Q4_K;
+    if (id == FH_GGML_Q6_K) return QuantizationFormat::Q6_K;
+    throw Error(ErrorKind::Gguf, "unsupported GGML type " + std::to_string(id));
+}
+
+class Device;
+
+namespace detail {
+struct DeviceHandle {
+    fh_device* raw = nullptr;
+    ~DeviceHandle() { if (raw) fh_device_destroy(raw); }
+};
+struct BufferHandle {
+    fh_buffer* raw = nullptr;
+    std::shared_ptr<DeviceHandle> owner;
+    size_t bytes = 0;
+    ~BufferHandle() { if (raw) fh_buffer_free(raw); }
+};
+struct MatrixHandle {
+    fh_qmatrix* raw = nullptr;
+    std::shared_ptr<DeviceHandle> owner;
+    ~MatrixHandle() { if (raw) fh_qmatrix_destroy(raw); }
+};
+}  // namespace detail
+
+// A dense row-major view into a device buffer (src/tensor/mod.rs).
+class Tensor {
+public:
+    Tensor() = default;
+    const std::vector<size_t>& shape() const { return shape_; }
+    DType dtype() const { return dtype_; }
+    size_t numel() const {
+        size_t n = 1;
+        for (size_t d : shape_) n *= d;
+        return n;
+    }
+    size_t byte_size() const { return numel() * size_bytes(dtype_); }
+    Tensor view(size_t element_offset, std::vector<size_t> shape) const {
+        Tensor t = *this;
+        t.shape_ = std::move(shape);
+        t.offset_ = offset_ + element_offset * size_bytes(dtype_);
+        if (t.offset_ + t.byte_size() > buffer_->bytes) throw Error(ErrorKind::Range, "tensor view is out of range");
+        return t;
+    }
+    // Waits for the device, then widens to f32.
+    std::vector<float> to_f32() const {
+        const size_t n = numel();
+        std::vector<float> out(n);
+        if (dtype_ == DType::F32) {
+            check(fh_buffer_download(buffer_->raw, offset_, out.data(), n * 4));
+            return out;
+        }
+        std::vector<uint16_t> raw(n);
+        check(fh_buffer_download(buffer_->raw, offset_, raw.data(), n * 2));
+        for (size_t i = 0; i < n; ++i)
+            out[i] = dtype_ == DType::F16 ? f16_bits_to_f32(raw[i]) : bf16_bits_to_f32(raw[i]);
+        return out;
+    }
+    fh_view c_view() const { return fh_view{buffer_->raw, offset_, static_cast<uint32_t>(dtype_)}; }
+    const std::shared_ptr<detail::DeviceHandle>& owner() const { return buffer_->owner; }
+
+private:
+    friend class Device;
+    std::shared_ptr<detail::BufferHandle> buffer_;
+    size_t offset_ = 0;
+    std::vector<size_t> shape_;
+    DType dtype_ = DType::F32;
+};
+
+struct Metrics {
+    std::string operation;
+    size_t bytes_read = 0, bytes_written = 0;
+};
+struct Output {
+    Tensor tensor;
+    Metrics metrics;
+};
+
+class QuantizedMatrix {
+public:
+    size_t rows() const { return rows_; }
+    size_t columns() const { return columns_; }
+    QuantizationFormat format() const { return format_; }
+    size_t byte_size() const { return fh_qmatrix_byte_size(handle_->raw); }
+    fh_qmatrix* raw() const { return handle_->raw; }
+    const std::shared_ptr<detail::DeviceHandle>& owner() const { return handle_->owner; }
+
+private:
+    friend class Device;
+    friend class QuantizedExpertMatrix;
+    std::shared_ptr<detail::MatrixHandle> handle_;
+    size_t rows_ = 0, columns_ = 0;
+    QuantizationFormat format_ = QuantizationFormat::Q4_K;
+};
+
+class QuantizedExpertMatrix {
+public:
+    size_t experts() const { return experts_; }
+    size_t rows_per_expert() const { return matrix_.rows_ / experts_; }
+    size_t columns() const { return matrix_.columns_; }
+    QuantizationFormat format() const { return matrix_.format_; }
+    size_t byte_size() const { return matrix_.byte_size(); }
+    const QuantizedMatrix& matrix() const { return matrix_; }
+
+private:
+    friend class Device;
+    QuantizedMatrix matrix_;
+    size_t experts_ = 0;
+};
+
+enum class MoeScoringFunction { Softmax, Sigmoid };
+struct MoeRoutingPolicy {
+    size_t experts = 0, top_k = 0;
+    MoeScoringFunction scoring_function = MoeScoringFunction::Softmax;
+    bool normalize_top_k_prob = true;
+    float normalization_epsilon = 0.f;
+    float routed_scaling_factor = 1.f;
+    bool use_expert_bias = false;
+    fh_routing_policy c() const {
+        return fh_routing_policy{(uint32_t)experts, (uint32_t)top_k,
+                                 scoring_function == MoeScoringFunction::Sigmoid ? 1u : 0u,
+                                 normalize_top_k_prob ? 1u : 0u, normalization_epsilon, routed_scaling_factor};
+    }
+};
+
+// Recorded operator calls, replayed as one HIP graph (Execution of the reference).
+class Graph {
+public:
+    explicit Graph(fh_graph* raw) : raw_(raw, fh_graph_destroy) {}
+    void launch() const { check(fh_graph_launch(raw_.get())); }
+private:
+    std::shared_ptr<fh_graph> raw_;
+};
+
+class Device {
+public:
+    explicit Device(int ordinal = 0) : handle_(std::make_shared<detail::DeviceHandle>()) {
+        check(fh_device_create(ordinal, &handle_->raw));
+    }
+    fh_device* raw() const { return handle_->raw; }
+    void synchronize() const { check(fh_synchronize(handle_->raw)); }
+    std::string last_operation() const { return fh_last_operation(handle_->raw); }
+    void set_k_quant_gemv_ksplit(int64_t simds) const { check(fh_set_tuning(handle_->raw, "k_quant_gemv_ksplit", simds)); }
+    void set_tuning(const char* key, int64_t value) const { check(fh_set_tuning(handle_->raw, key, value)); }
+    bool owns(const Tensor& t) const { return t.buffer_ && t.buffer_->owner == handle_; }
+
+    // ---- tensors ----
+    Tensor zeros(std::vector<size_t> shape, DType dtype) const {
+        Tensor t;
+        t.shape_ = std::move(shape);
+        t.dtype_ = dtype;
+        auto buffer = std::make_shared<detail::BufferHandle>();
+        buffer->owner = handle_;
+        buffer->bytes = t.byte_size() ? t.byte_size() : 1;
+        check(fh_buffer_alloc(handle_->raw, buffer->bytes, &buffer->raw));
+        t.buffer_ = std::move(buffer);
+        return t;
+    }
+    Tensor from_f32(std::vector<size_t> shape, DType dtype, const std::vector<float>& values) const {
+        Tensor t = zeros(std::move(shape), dtype);
+        if (values.size() != t.numel()) throw Error(ErrorKind::Shape, "value count does not match the shape");
+        if (dtype == DType::F32) {
+            check(fh_buffer_upload(t.buffer_->raw, 0, values.data(), values.size() * 4));
+        } else {
+            std::vector<uint16_t> raw(values.size());
+            for (size_t i = 0; i < raw.size(); ++i)
+                raw[i] = dtype == DType::F16 ? f32_to_f16_bits(values[i]) : f32_to_bf16_bits(values[i]);
+            check(fh_buffer_upload(t.buffer_->raw, 0, raw.data(), raw.size() * 2));
+        }
+        return t;
+    }
+    Tensor from_bits(std::vector<size_t> shape, const std::vector<uint32_t>& words) const {
+        Tensor t = zeros(std::move(shape), DType::F32);
+        if (words.size() != t.numel()) throw Error(ErrorKind::Shape, "value count does not match the shape");
+        check(fh_buffer_upload(t.buffer_->raw, 0, words.data(), words.size() * 4));
+        return t;
+    }
+
+    // ---- weights ----
+    // QuantizedMatrix::from_reader: `fill` writes the packed GGUF bytes.
+    QuantizedMatrix quantized_matrix(size_t rows, size_t columns, QuantizationFormat format,
+                                     const std::function<void(uint8_t*, size_t)>& fill,
+                                     size_t experts = 1) const {
+        if (rows == 0 || columns == 0 || columns % block_elements(format) != 0 || experts == 0 || rows % experts)
+            throw Error(ErrorKind::Shape, "quantized matrix requires nonempty rows and whole blocks");
+        std::vector<uint8_t> host(rows * (columns / 256) * block_bytes(format));
+        fill(host.data(), host.size());
+        QuantizedMatrix m;
+        m.handle_ = std::make_shared<detail::MatrixHandle>();
+        m.handle_->owner = handle_;
+        check(fh_qmatrix_create(handle_->raw, static_cast<uint32_t>(format), rows / experts, columns, experts,
+                                host.data(), host.size(), &m.handle_->raw));
+        m.rows_ = rows;
+        m.columns_ = columns;
+        m.format_ = format;
+        return m;
+    }
+    QuantizedExpertMatrix quantized_expert_matrix(size_t experts, size_t rows_per_expert, size_t columns,
+                                                  QuantizationFormat format,
+                                                  const std::function<void(uint8_t*, size_t)>& fill) const {
+        if (experts == 0 || rows_per_expert == 0) throw Error(ErrorKind::Shape, "invalid quantized expert geometry");
+        QuantizedExpertMatrix e;
+        e.matrix_ = quantized_matrix(experts * rows_per_expert, columns, format, fill, experts);
+        e.experts_ = experts;
+        return e;
+    }
+
+    // ---- operators ----
+    Tensor dequantize(const QuantizedMatrix& w, DType dtype = DType::F32) const {
+        Tensor out = zeros({w.rows(), w.columns()}, dtype);
+        fh_view v = out.c_view();
+        check(fh_dequantize(handle_->raw, w.raw(), &v));
+        return out;
+    }
+    Output embedding_gather_quantized(const QuantizedMatrix& w, const std::vector<uint32_t>& tokens,
+                                      DType dtype) const {
+        if (tokens.empty()) throw Error(ErrorKind::Shape, "embedding gather requires tokens");
+        Tensor out = zeros({tokens.size(), w.columns()}, dtype);
+        fh_view v = out.c_view();
+        check(fh_embedding_gather_quantized(handle_->raw, w.raw(), tokens.data(), tokens.size(), &v));
+        return {out, {last_operation(), 0, out.byte_size()}};
+    }
+    // Y[M,N] = X[M,K] . W[N,K]^T; the output takes the activation dtype unless told otherwise.
+    Output project_quantized(const Tensor& a, const QuantizedMatrix& w, const Tensor* out = nullptr,
+                             const DType* out_dtype = nullptr) const {
+        const auto& dims = a.shape();
+        if (dims.size() != 2 || dims[1] != w.columns() || dims[0] == 0)
+            throw Error(ErrorKind::Shape, "quantized projection requires [M,K] matching [N,K]");
+        if (!owns(a) || w.owner() != handle_) throw Error(ErrorKind::DeviceMismatch, "tensor or weight belongs to another device");
+        Tensor y = out ? *out : zeros({dims[0], w.rows()}, out_dtype ? *out_dtype : a.dtype());
+        fh_view xv = a.c_view(), yv = y.c_view();
+        check(fh_project_quantized(handle_->raw, w.raw(), &xv, (uint32_t)dims[0], &yv));
+        return {y, {last_operation(), a.byte_size() + w.byte_size(), y.byte_size()}};
+    }
+    Tensor moe_route(const Tensor& logits, const Tensor* selection_bias, const MoeRoutingPolicy& policy,
+                     const Tensor* out = nullptr) const {
+        const auto& dims = logits.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != policy.experts)
+            throw Error(ErrorKind::Shape, "invalid sparse routing geometry");
+        Tensor meta = out ? *out : zeros({dims[0] * policy.top_k, 3}, DType::F32);
+        fh_view lv = logits.c_view(), mv = meta.c_view(), bv{};
+        if (selection_bias) bv = selection_bias->c_view();
+        fh_routing_policy pc = policy.c();
+        check(fh_moe_route(handle_->raw, &lv, (uint32_t)dims[0], selection_bias ? &bv : nullptr, &pc, &mv));
+        return meta;
+    }
+    Tensor expert_assign(const Tensor& hidden, const Tensor& metadata, size_t top_k, const Tensor* out = nullptr) const {
+        const auto& x = hidden.shape();
+        const auto& m = metadata.shape();
+        if (x.size() != 2 || m.size() != 2 || m[1] != 3 || top_k == 0 || x[0] * top_k != m[0])
+            throw Error(ErrorKind::Shape, "expert assignments require [S,H] and [S*top_k,3]");
+        Tensor y = out ? *out : zeros({m[0], x[1]}, hidden.dtype());
+        fh_view hv = hidden.c_view(), mv = metadata.c_view(), yv = y.c_view();
+        check(fh_expert_assign(handle_->raw, &hv, (uint32_t)x[0], (uint32_t)x[1], &mv, (uint32_t)top_k, &yv));
+        return y;
+    }
+    Tensor expert_project_quantized(const Tensor& input, const Tensor& metadata, const QuantizedExpertMatrix& w,
+                                    size_t features, size_t experts, const Tensor* out = nullptr) const {
+        const auto& x = input.shape();
+        if (x.size() != 2 || x[0] == 0 || x[1] != features || metadata.shape() != std::vector<size_t>{x[0], 3} ||
+            w.experts() != experts || w.columns() != features)
+            throw Error(ErrorKind::Shape, "quantized expert projection geometry mismatch");
+        Tensor y = out ? *out : zeros({x[0], w.rows_per_expert()}, input.dtype());
+        fh_view xv = input.c_view(), mv = metadata.c_view(), yv = y.c_view();
+        check(fh_expert_project_quantized(handle_->raw, w.matrix().raw(), &xv, (uint32_t)x[0], &mv, &yv));
+        return y;
+    }
+    Tensor expert_silu_mul(const Tensor& input, size_t intermediate, const Tensor* out = nullptr) const {
+        const auto& x = input.shape();
+        if (x.size() != 2 || intermediate == 0 || intermediate * 2 != x[1])
+            throw Error(ErrorKind::Shape, "packed expert activation geometry mismatch");
+        Tensor y = out ? *out : zeros({x[0], intermediate}, input.dtype());
+        fh_view iv = input.c_view(), yv = y.c_view();
+        check(fh_expert_silu_mul(handle_->raw, &iv, (uint32_t)x[0], (uint32_t)intermediate, &yv));
+        return y;
+    }
+    Tensor expert_combine(const Tensor& input, const Tensor& metadata, size_t tokens, size_t hidden, size_t top_k,
+                          const Tensor* out = nullptr) const {
+        if (top_k == 0 || hidden == 0 || input.shape() != std::vector<size_t>{tokens * top_k, hidden})
+            throw Error(ErrorKind::Shape, "expert combine geometry mismatch");
+        Tensor y = out ? *out : zeros({tokens, hidden}, input.dtype());
+        fh_view iv = input.c_view(), mv = metadata.c_view(), yv = y.c_view();
+        check(fh_expert_combine(handle_->raw, &iv, &mv, (uint32_t)tokens, (uint32_t)hidden, (uint32_t)top_k, &yv));
+        return y;
+    }
+
+    // Records the operator calls made by `body` and returns them as a graph.
+    Graph execution(const std::function<void()>& body) const {
+        check(fh_execution_begin(handle_->raw));
+        fh_graph* raw = nullptr;
+        try {
+            body();
+        } catch (...) {
+            (void)fh_execution_end(handle_->raw, &raw);
+            if (raw) fh_graph_destroy(raw);
+            throw;
+        }
+        check(fh_execution_end(handle_->raw, &raw));
+        return Graph(raw);
+    }
+
+private:
+    std::shared_ptr<detail::DeviceHandle> handle_;
+};
+
+// SparseMoe::forward without the router's own dense layer: the caller passes
+// the router logits (that layer is outside the quantized path).
+class SparseMoe {
+public:
+    SparseMoe(const Device& device, QuantizedExpertMatrix input_experts, QuantizedExpertMatrix output_experts,
+              MoeRoutingPolicy routing)
+        : device_(device), input_(std::move(input_experts)), output_(std::move(output_experts)), routing_(routing) {
+        const size_t two_i = input_.rows_per_expert();
+        if (two_i == 0 || two_i % 2 || output_.experts() != input_.experts() ||
+            output_.rows_per_expert() != input_.columns() || output_.columns() * 2 != two_i ||
+            routing_.experts != input_.experts() || routing_.top_k == 0 || routing_.top_k > routing_.experts)
+            throw Error(ErrorKind::Config, "invalid sparse expert weight geometry");
+    }
+    Tensor forward(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias = nullptr) const {
+        const auto& dims = hidden.shape();
+        const size_t h = input_.columns(), i = input_.rows_per_expert() / 2, e = input_.experts();
+        if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
+            throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
+        Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
+        Tensor assigned = device_.expert_assign(hidden, meta, routing_.top_k);
+        Tensor projected = device_.expert_project_quantized(assigned, meta, input_, h, e);
+        Tensor activated = device_.expert_silu_mul(projected, i);
+        Tensor expert_output = device_.expert_project_quantized(activated, meta, output_, i, e);
+        return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
+    }
+
+private:
+    const Device& device_;
+    QuantizedExpertMatrix input_, output_;
+    MoeRoutingPolicy routing_;
+};
+
+}  // namespace ferrum
+
+#endif  // FERRUM_HIP_HPP

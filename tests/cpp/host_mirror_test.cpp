@@ -1,0 +1,205 @@
+// Exercises the C++ host side (include/ferrum_hip.hpp) on the GPU and checks
+// it against the CPU oracle.  The cases follow the reference's operator tests:
+// embedding gather bitwise (src/ops/transformer.rs:3307-3329), GEMV / GEMM
+// against the CPU dequant (src/diffusion/tests.rs:718-761), shape and ownership
+// errors (src/ops/mod.rs:553-609), and the routed FFN against a host evaluation
+// (src/nn/moe.rs:602-651).  Prints one line per case; exit status 0 = all passed.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "ferrum_hip.hpp"
+
+extern "C" {
+int fo_dequantize(uint32_t ggml_type, const uint8_t* packed, size_t rows, size_t cols, float* out);
+int fo_project_f64(uint32_t ggml_type, const uint8_t* packed, size_t n, size_t k, const float* x,
+                   size_t m, float* y, int weight_round, int threads);
+int fo_select_routes(const float* logits, size_t tokens, size_t experts, size_t top_k, int sigmoid,
+                     int normalize, float eps, float scaling, const float* bias, float* metadata);
+void fo_expert_assign(const float* hidden, const float* metadata, size_t assignments, size_t width, float* out);
+int fo_expert_project(uint32_t ggml_type, const uint8_t* packed, size_t experts, size_t rows, size_t k,
+                      const float* x, const float* metadata, size_t assignments, float* y, int weight_round,
+                      int out_round, int f64);
+void fo_expert_silu_mul(const float* in, size_t assignments, size_t intermediate, uint32_t dtype, float* out);
+void fo_expert_combine(const float* in, const float* metadata, size_t tokens, size_t hidden, size_t top_k,
+                       uint32_t dtype, float* out);
+void fo_round_storage_array(const float* in, size_t n, uint32_t dtype, float* out);
+}
+
+using namespace ferrum;
+
+static int failures = 0;
+static void report(const char* name, bool ok, double figure = 0) {
+    std::printf("%-58s %s  %.3g\n", name, ok ? "ok" : "FAILED", figure);
+    std::fflush(stdout);
+    if (!ok) ++failures;
+}
+
+struct Rng {  // splitmix64
+    uint64_t s;
+    uint64_t next() {
+        uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+    }
+    double uniform() { return (double)(next() >> 11) / 9007199254740992.0; }
+    float normal() { return (float)(std::sqrt(-2.0 * std::log(uniform() + 1e-300)) * std::cos(6.283185307179586 * uniform())); }
+};
+
+// Random super-blocks with small finite f16 scales.
+static std::vector<uint8_t> blocks(QuantizationFormat f, size_t rows, size_t cols, uint64_t seed) {
+    Rng rng{seed};
+    const size_t bb = block_bytes(f), n = rows * (cols / 256);
+    std::vector<uint8_t> out(n * bb);
+    for (auto& b : out) b = (uint8_t)rng.next();
+    for (size_t i = 0; i < n; ++i) {
+        uint8_t* blk = out.data() + i * bb;
+        const uint16_t d = f32_to_f16_bits((float)(std::fabs(rng.normal()) * (f == QuantizationFormat::Q4_K ? 0.01 : 0.002)));
+        if (f == QuantizationFormat::Q4_K) {
+            const uint16_t dmin = f32_to_f16_bits((float)(std::fabs(rng.normal()) * 0.005));
+            std::memcpy(blk, &d, 2);
+            std::memcpy(blk + 2, &dmin, 2);
+        } else {
+            std::memcpy(blk + 208, &d, 2);
+        }
+    }
+    return out;
+}
+
+static double rel_l2(const std::vector<float>& a, const std::vector<float>& b) {
+    double num = 0, den = 0;
+    for (size_t i = 0; i < a.size(); ++i) {
+        num += ((double)a[i] - b[i]) * ((double)a[i] - b[i]);
+        den += (double)b[i] * b[i];
+    }
+    return std::sqrt(num / den);
+}
+
+static QuantizedMatrix upload(const Device& d, QuantizationFormat f, size_t rows, size_t cols,
+                              const std::vector<uint8_t>& bytes) {
+    return d.quantized_matrix(rows, cols, f, [&](uint8_t* dst, size_t n) { std::memcpy(dst, bytes.data(), n); });
+}
+
+int main() {
+    Device d(0);
+    const uint32_t kF16 = 1;
+    for (QuantizationFormat f : {QuantizationFormat::Q4_K, QuantizationFormat::Q6_K}) {
+        const uint32_t type = static_cast<uint32_t>(f);
+        const size_t n = 200, k = 1024;
+        const auto packed = blocks(f, n, k, 11 + type);
+        QuantizedMatrix w = upload(d, f, n, k, packed);
+
+        std::vector<float> want(n * k);
+        fo_dequantize(type, packed.data(), n, k, want.data());
+        const auto dense = d.dequantize(w).to_f32();
+        report(f == QuantizationFormat::Q4_K ? "q4_k dequantize is bit-exact" : "q6_k dequantize is bit-exact",
+               std::memcmp(dense.data(), want.data(), want.size() * 4) == 0);
+
+        const std::vector<uint32_t> tokens = {3, 0, 199, 3};
+        const auto gathered = d.embedding_gather_quantized(w, tokens, DType::BF16).tensor.to_f32();
+        bool same = true;
+        for (size_t t = 0; t < tokens.size(); ++t)
+            for (size_t c = 0; c < k; ++c)
+                same &= gathered[t * k + c] == bf16_bits_to_f32(f32_to_bf16_bits(want[tokens[t] * k + c]));
+        report("embedding gather matches the rounded dequant bitwise", same);
+
+        Rng rng{5};
+        std::vector<float> x(k);
+        for (auto& v : x) v = rng.normal();
+        std::vector<float> ref(n);
+        fo_project_f64(type, packed.data(), n, k, x.data(), 1, ref.data(), 0, 4);
+        Output y = d.project_quantized(d.from_f32({1, k}, DType::F32, x), w);
+        report(("gemv vs f64 oracle: " + y.metrics.operation).c_str(), rel_l2(y.tensor.to_f32(), ref) <= 1e-5,
+               rel_l2(y.tensor.to_f32(), ref));
+
+        const size_t m = 8;
+        std::vector<float> xm(m * k);
+        for (auto& v : xm) v = f16_bits_to_f32(f32_to_f16_bits(rng.normal()));
+        std::vector<float> refm(m * n);
+        fo_project_f64(type, packed.data(), n, k, xm.data(), m, refm.data(), kF16, 4);
+        const DType f32 = DType::F32;
+        Output ym = d.project_quantized(d.from_f32({m, k}, DType::F16, xm), w, nullptr, &f32);
+        report(("small-M gemm vs f16-tile oracle: " + ym.metrics.operation).c_str(),
+               rel_l2(ym.tensor.to_f32(), refm) <= 1e-5, rel_l2(ym.tensor.to_f32(), refm));
+
+        bool threw = false;
+        try {
+            d.project_quantized(d.from_f32({1, k / 2}, DType::F32, std::vector<float>(k / 2, 1.f)), w);
+        } catch (const Error& e) {
+            threw = e.kind() == ErrorKind::Shape;
+        }
+        report("mismatched K is Error::Shape", threw);
+    }
+    {
+        bool threw = false;
+        try {
+            d.quantized_matrix(4, 256, QuantizationFormat::Q4_K, [](uint8_t* dst, size_t n) {
+                std::memset(dst, 0, n);
+                dst[1] = 0x7c;  // d = +inf
+            });
+        } catch (const Error& e) {
+            threw = e.kind() == ErrorKind::Weight;
+        }
+        report("non-finite block scale is Error::Weight", threw);
+    }
+    {
+        // routed FFN: 8 experts, hidden 512, intermediate 256, top-2, 40 tokens, f32 activations
+        const size_t experts = 8, hidden = 512, inter = 256, top_k = 2, tokens = 40;
+        const auto win = blocks(QuantizationFormat::Q4_K, experts * 2 * inter, hidden, 21);
+        const auto wout = blocks(QuantizationFormat::Q4_K, experts * hidden, inter, 22);
+        Rng rng{23};
+        std::vector<float> x(tokens * hidden), logits(tokens * experts);
+        for (auto& v : x) v = rng.normal();
+        for (auto& v : logits) v = rng.normal();
+        auto copy_from = [](const std::vector<uint8_t>& src) {
+            return [&src](uint8_t* dst, size_t n) { std::memcpy(dst, src.data(), n); };
+        };
+        SparseMoe moe(d, d.quantized_expert_matrix(experts, 2 * inter, hidden, QuantizationFormat::Q4_K, copy_from(win)),
+                      d.quantized_expert_matrix(experts, hidden, inter, QuantizationFormat::Q4_K, copy_from(wout)),
+                      MoeRoutingPolicy{experts, top_k});
+        const auto got = moe.forward(d.from_f32({tokens, hidden}, DType::F32, x),
+                                     d.from_f32({tokens, experts}, DType::F32, logits)).to_f32();
+        const size_t a = tokens * top_k;
+        std::vector<float> meta(a * 3), assigned(a * hidden), up(a * 2 * inter), act(a * inter), down(a * hidden),
+            want(tokens * hidden);
+        fo_select_routes(logits.data(), tokens, experts, top_k, 0, 1, 0.f, 1.f, nullptr, meta.data());
+        fo_expert_assign(x.data(), meta.data(), a, hidden, assigned.data());
+        fo_expert_project(FH_GGML_Q4_K, win.data(), experts, 2 * inter, hidden, assigned.data(), meta.data(), a,
+                          up.data(), 0, 0, 1);
+        fo_expert_silu_mul(up.data(), a, inter, 0, act.data());
+        fo_expert_project(FH_GGML_Q4_K, wout.data(), experts, hidden, inter, act.data(), meta.data(), a, down.data(),
+                          0, 0, 1);
+        fo_expert_combine(down.data(), meta.data(), tokens, hidden, top_k, 0, want.data());
+        report("SparseMoe::forward vs host evaluation", rel_l2(got, want) <= 2e-5, rel_l2(got, want));
+
+        Device other(0);
+        bool threw = false;
+        try {
+            d.project_quantized(other.from_f32({1, 256}, DType::F32, std::vector<float>(256, 1.f)),
+                                upload(d, QuantizationFormat::Q4_K, 4, 256, blocks(QuantizationFormat::Q4_K, 4, 256, 3)));
+        } catch (const Error& e) {
+            threw = e.kind() == ErrorKind::DeviceMismatch;
+        }
+        report("a tensor of another device is Error::DeviceMismatch", threw);
+    }
+    {
+        // an execution records the calls and replays them
+        const size_t n = 256, k = 512;
+        const auto packed = blocks(QuantizationFormat::Q4_K, n, k, 31);
+        QuantizedMatrix w = upload(d, QuantizationFormat::Q4_K, n, k, packed);
+        Tensor x = d.from_f32({1, k}, DType::F32, std::vector<float>(k, 0.5f));
+        Tensor y = d.zeros({1, n}, DType::F32);
+        const auto eager = d.project_quantized(x, w).tensor.to_f32();
+        Graph graph = d.execution([&] { d.project_quantized(x, w, &y); });
+        graph.launch();
+        graph.launch();
+        const auto replayed = y.to_f32();
+        report("a recorded execution replays the projection bitwise",
+               std::memcmp(eager.data(), replayed.data(), eager.size() * 4) == 0);
+    }
+    std::printf("%d failure(s)\n", failures);
+    return failures ? 1 : 0;
+}

@@ -154,7 +154,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     }
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
-    d->tuning["gemm_wide_min_rows"] = 192;  // smallest M that takes the 256-row tile
+    d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 32; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     fh_status st = ensure_scratch(d, 0);

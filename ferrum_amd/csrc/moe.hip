@@ -31,6 +31,7 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
 // softmax normaliser is then summed by one lane in expert order so it carries
 // the same f32 rounding as a sequential host loop.  Selection runs top_k
 // rounds of a wave-wide arg-max over (total-order key, lower id wins).
+template <int kPerLane>   // experts <= 64 * kPerLane
 __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ logits,
                                                        uint32_t logits_dtype,
                                                        const float* __restrict__ bias,
@@ -44,39 +45,46 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
     if (token >= tokens) return;
     const size_t base = (size_t)token * experts;
 
-    float score[kMaxPerLane];
-    float logit[kMaxPerLane];
+    float score[kPerLane];
+    float logit[kPerLane];
     float maximum = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
         uint32_t e = lane + 64u * i;
         logit[i] = e < experts ? load_as_f32(logits, base + e, logits_dtype) : -INFINITY;
         maximum = fmaxf(maximum, logit[i]);
     }
     if (sigmoid) {
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) score[i] = 1.f / (1.f + expf(-logit[i]));
+        for (int i = 0; i < kPerLane; ++i) score[i] = 1.f / (1.f + expf(-logit[i]));
     } else {
         maximum = wave_max(maximum);
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) {
+        for (int i = 0; i < kPerLane; ++i) {
             uint32_t e = lane + 64u * i;
             score[i] = expf(logit[i] - maximum);
-            if (e < experts) scores_lds[e] = score[i];
+            if (e < ((experts + 3u) & ~3u)) scores_lds[e] = e < experts ? score[i] : 0.f;
         }
         __syncthreads();
         float normalizer = 0.f;
         if (lane == 0) {
-            for (uint32_t e = 0; e < experts; ++e) normalizer += scores_lds[e];
+            // expert order, four per LDS read; the zero padding does not change the sum
+            for (uint32_t e = 0; e < experts; e += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(scores_lds + e);
+                normalizer += v.x;
+                normalizer += v.y;
+                normalizer += v.z;
+                normalizer += v.w;
+            }
         }
         normalizer = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(normalizer)));
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) score[i] = score[i] / normalizer;
+        for (int i = 0; i < kPerLane; ++i) score[i] = score[i] / normalizer;
     }
 
-    unsigned long long packed[kMaxPerLane];
+    unsigned long long packed[kPerLane];
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < kPerLane; ++i) {
         uint32_t e = lane + 64u * i;
         float selection = score[i] + (bias != nullptr && e < experts ? bias[e] : 0.f);
         // 0 marks "not a candidate"; valid entries have low word >= 1
@@ -92,12 +100,12 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
         if ((uint32_t)rank < top_k) {
             unsigned long long best = 0ull;
 #pragma unroll
-            for (int i = 0; i < kMaxPerLane; ++i) best = packed[i] > best ? packed[i] : best;
+            for (int i = 0; i < kPerLane; ++i) best = packed[i] > best ? packed[i] : best;
             best = wave_max_u64(best);
             uint32_t id = 0xffffffffu - (uint32_t)best;
             float mine = 0.f;
 #pragma unroll
-            for (int i = 0; i < kMaxPerLane; ++i) {
+            for (int i = 0; i < kPerLane; ++i) {
                 if (lane + 64u * i == id) {
                     mine = score[i];
                     packed[i] = 0ull;
@@ -197,6 +205,76 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(const void* __restr
     }
 }
 
+// Eight consecutive elements of a row at a time (one 128-bit access for the
+// 16-bit types), for rows whose length is a multiple of 8 and 16-byte aligned.
+__device__ __forceinline__ void load8(const void* p, size_t i, uint32_t dtype, float (&v)[8]) {
+    if (dtype == FH_F32) {
+        const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i);
+        const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(p) + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(p) + i);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[2 * j] = dtype == FH_F16 ? f16_bits_to_f32(w[j] & 0xffffu) : bf16_bits_to_f32(w[j] & 0xffffu);
+            v[2 * j + 1] = dtype == FH_F16 ? f16_bits_to_f32(w[j] >> 16) : bf16_bits_to_f32(w[j] >> 16);
+        }
+    }
+}
+__device__ __forceinline__ void store8(void* p, size_t i, uint32_t dtype, const float (&v)[8]) {
+    if (dtype == FH_F32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(p) + i) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>(static_cast<float*>(p) + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            w[j] = dtype == FH_F16 ? (f32_to_f16_bits(v[2 * j]) | (f32_to_f16_bits(v[2 * j + 1]) << 16))
+                                   : (f32_to_bf16_bits(v[2 * j]) | (f32_to_bf16_bits(v[2 * j + 1]) << 16));
+        *reinterpret_cast<uint4*>(static_cast<uint16_t*>(p) + i) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+__global__ __launch_bounds__(256) void expert_silu_mul8_kernel(const void* __restrict__ in,
+                                                               void* __restrict__ out,
+                                                               uint32_t assignments, uint32_t intermediate,
+                                                               uint32_t in_dtype, uint32_t out_dtype) {
+    const size_t total = (size_t)assignments * intermediate / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const size_t a = (i * 8) / intermediate, column = (i * 8) % intermediate;
+        float gate[8], up[8], result[8];
+        load8(in, a * 2 * intermediate + column, in_dtype, gate);
+        load8(in, a * 2 * intermediate + intermediate + column, in_dtype, up);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) result[j] = round_storage(silu(gate[j]), out_dtype) * up[j];
+        store8(out, i * 8, out_dtype, result);
+    }
+}
+
+__global__ __launch_bounds__(256) void expert_combine8_kernel(const void* __restrict__ in,
+                                                              const float* __restrict__ metadata,
+                                                              void* __restrict__ out, uint32_t tokens,
+                                                              uint32_t hidden, uint32_t top_k,
+                                                              uint32_t in_dtype, uint32_t out_dtype) {
+    const size_t total = (size_t)tokens * hidden / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const size_t token = (i * 8) / hidden, column = (i * 8) % hidden;
+        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (uint32_t rank = 0; rank < top_k; ++rank) {
+            const size_t a = token * top_k + rank;
+            const float gate = round_storage(metadata[a * 3 + 2], out_dtype);
+            float value[8];
+            load8(in, a * hidden + column, in_dtype, value);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum[j] += round_storage(gate * value[j], out_dtype);
+        }
+        store8(out, i * 8, out_dtype, sum);
+    }
+}
+
 unsigned grid_for(size_t threads) {
     size_t blocks = (threads + 255) / 256;
     if (blocks > 16384) blocks = 16384;
@@ -259,9 +337,17 @@ __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
                              const float* bias, float* metadata, uint32_t tokens,
                              const fh_routing_policy& p) {
-    hipLaunchKernelGGL(moe_route_kernel, dim3(tokens), dim3(64), p.experts * sizeof(float), s,
-                       logits, logits_dtype, bias, metadata, tokens, p.experts, p.top_k, p.sigmoid,
-                       p.normalize_top_k_prob, p.normalization_epsilon, p.routed_scaling_factor);
+    const size_t lds = ((p.experts + 3u) & ~3u) * sizeof(float);
+#define FH_ROUTE(PL)                                                                                   \
+    hipLaunchKernelGGL(moe_route_kernel<PL>, dim3(tokens), dim3(64), lds, s, logits, logits_dtype, bias, \
+                       metadata, tokens, p.experts, p.top_k, p.sigmoid, p.normalize_top_k_prob,         \
+                       p.normalization_epsilon, p.routed_scaling_factor)
+    if (p.experts <= 64) FH_ROUTE(1);
+    else if (p.experts <= 128) FH_ROUTE(2);
+    else if (p.experts <= 256) FH_ROUTE(4);
+    else if (p.experts <= 512) FH_ROUTE(8);
+    else FH_ROUTE(kMaxPerLane);
+#undef FH_ROUTE
     return "moe_route";
 }
 
@@ -293,16 +379,28 @@ const char* launch_expert_assign(hipStream_t s, const void* hidden, const float*
 
 const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,
                                    uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype) {
-    hipLaunchKernelGGL(expert_silu_mul_kernel, dim3(grid_for((size_t)assignments * intermediate)),
-                       dim3(256), 0, s, in, out, assignments, intermediate, in_dtype, out_dtype);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (intermediate % 8 == 0 && aligned) {
+        hipLaunchKernelGGL(expert_silu_mul8_kernel, dim3(grid_for((size_t)assignments * intermediate / 8)),
+                           dim3(256), 0, s, in, out, assignments, intermediate, in_dtype, out_dtype);
+    } else {
+        hipLaunchKernelGGL(expert_silu_mul_kernel, dim3(grid_for((size_t)assignments * intermediate)),
+                           dim3(256), 0, s, in, out, assignments, intermediate, in_dtype, out_dtype);
+    }
     return "expert_silu_mul";
 }
 
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
                                   uint32_t tokens, uint32_t hidden, uint32_t top_k,
                                   uint32_t in_dtype, uint32_t out_dtype) {
-    hipLaunchKernelGGL(expert_combine_kernel, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0,
-                       s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (hidden % 8 == 0 && aligned) {
+        hipLaunchKernelGGL(expert_combine8_kernel, dim3(grid_for((size_t)tokens * hidden / 8)), dim3(256), 0,
+                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+    } else {
+        hipLaunchKernelGGL(expert_combine_kernel, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0,
+                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+    }
     return "expert_combine";
 }
 

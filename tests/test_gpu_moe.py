@@ -135,9 +135,11 @@ def test_expert_projection_uses_assignment_metadata(api, d, ggml):
 
 def test_silu_mul_and_combine_keep_the_storage_rounding_points(api, d):
     rng = synth.rng(21)
-    a, inter, tokens, top_k, hidden = 24, 96, 6, 4, 64
-    for dtype, code in ((api.DType.F32, oracle.F32), (api.DType.F16, oracle.F16),
-                        (api.DType.BF16, oracle.BF16)):
+    # 96 / 64 columns take the eight-wide kernels, 10 / 6 the element-wise ones
+    cases = [(24, 96, 6, 4, 64, dt) for dt in ((api.DType.F32, oracle.F32), (api.DType.F16, oracle.F16),
+                                               (api.DType.BF16, oracle.BF16))]
+    cases += [(12, 10, 4, 3, 6, dt) for dt in ((api.DType.F32, oracle.F32), (api.DType.BF16, oracle.BF16))]
+    for a, inter, tokens, top_k, hidden, (dtype, code) in cases:
         packed_rows = (rng.standard_normal((a, 2 * inter)) * 2).astype(np.float32)
         t = api.Tensor.from_f32(d, packed_rows.shape, dtype, packed_rows)
         got = d.expert_silu_mul(t, inter).to_f32()

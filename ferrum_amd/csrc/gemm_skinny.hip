@@ -308,9 +308,11 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
 // runs across tile boundaries.  blockIdx.y = expert, blockIdx.x = which share
 // of the expert's rows.  Dynamic LDS: 16*TT rows of (K + 8) halfs.
 constexpr int kResRing = 6;
+constexpr int kResWaves = 8;                    // two waves per SIMD hide each other's decode and MFMA waits
+constexpr int kResThreads = 64 * kResWaves;
 
 template <uint32_t TYPE, int DT, int TT>
-__global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8_t* __restrict__ w,
+__global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint8_t* __restrict__ w,
                                                                      const uint16_t* __restrict__ x,
                                                                      void* __restrict__ y, uint32_t n,
                                                                      uint32_t nb, uint32_t y_dtype,
@@ -337,12 +339,12 @@ __global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8
         if (t0 != 0) __syncthreads();  // the previous pass is done with the rows
         // gather the expert's rows, eight 16-byte pieces per thread in flight at a time
         const uint32_t total = mt * pieces;
-        for (uint32_t base = 0; base < total; base += 8 * kSkThreads) {
+        for (uint32_t base = 0; base < total; base += 8 * kResThreads) {
             u32x4 v[8];
             uint32_t dst[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const uint32_t idx = min(base + j * kSkThreads + tid, total - 1);
+                const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
                 const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
                 dst[j] = tok * ld + 8 * pc;
                 v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)order[first_token + t0 + tok] * k + 8 * pc);
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8
         for (int s = 0; s < 8; ++s) kl[s] = Quarter<TYPE>::klocal(g, s);
 
         // units = (tile, super-block) pairs of this wave, in order
-        const uint32_t my_tiles = (tile_end - tile_begin + 3) / 4;
+        const uint32_t my_tiles = (tile_end - tile_begin + kResWaves - 1) / kResWaves;
         const uint32_t units = my_tiles * nb;
         auto unit_ptr = [&](uint32_t tile, uint32_t b) {
             const uint32_t row = min(tile * 16 + r, n - 1);
@@ -379,7 +381,7 @@ __global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8
             slot.load(unit_ptr(min(ptile, tile_end - 1), pb), g);
             if (++pb == nb) {
                 pb = 0;
-                ptile += 4;
+                ptile += kResWaves;
             }
         };
 #pragma unroll
@@ -434,7 +436,7 @@ __global__ __launch_bounds__(kSkThreads) void expert_resident_kernel(const uint8
                     acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
                 }
                 b = 0;
-                tile += 4;
+                tile += kResWaves;
             }
         };
         uint32_t u = 0;
@@ -465,19 +467,19 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
             uint32_t shares = (1024 + a.experts - 1) / a.experts;
             shares = shares < 1 ? 1 : shares;
             uint32_t tiles_per_wg = (tiles + shares - 1) / shares;
-            tiles_per_wg = (tiles_per_wg + 3) / 4 * 4;
+            tiles_per_wg = (tiles_per_wg + kResWaves - 1) / kResWaves * kResWaves;
             const dim3 rgrid((tiles + tiles_per_wg - 1) / tiles_per_wg, a.experts);
             if (wide) {
                 auto kernel = expert_resident_kernel<TYPE, DT, 2>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                hipLaunchKernelGGL(kernel, rgrid, dim3(kSkThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
+                hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
                                    a.expert_offsets, a.expert_order, tiles_per_wg);
             } else {
                 auto kernel = expert_resident_kernel<TYPE, DT, 1>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                hipLaunchKernelGGL(kernel, rgrid, dim3(kSkThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
+                hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
                                    a.expert_offsets, a.expert_order, tiles_per_wg);
             }
             return;

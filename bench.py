@@ -142,6 +142,44 @@ def cpu_baseline(case, budget_seconds=12.0):
     }
 
 
+def layer_case(api, synth, dev, steps, layers=4):
+    """One dense decode layer's four Q4_K GEMVs back to back (attention
+    projection 5120x5120, FFN gate and up 17408x5120, FFN down 5120x17408;
+    165 MB), over `layers` distinct sets of weights so nothing is cache resident."""
+    fmt = api.QuantizationFormat.Q4_K
+    f32 = api.DType.F32
+    shapes = [(5120, 5120), (17408, 5120), (17408, 5120), (5120, 17408)]
+    bases = {shape: synth.matrix(Q4_K, shape[0], shape[1], seed=21).reshape(shape[0], -1) for shape in set(shapes)}
+    sets = []
+    for layer in range(layers):
+        sets.append([api.QuantizedMatrix.from_bytes(dev, n, k, fmt, np.roll(bases[(n, k)], 4 * layer + i, axis=0).reshape(-1))
+                     for i, (n, k) in enumerate(shapes)])
+    x5 = api.Tensor.from_f32(dev, (1, 5120), f32, synth.activations(1, 5120, seed=22))
+    x17 = api.Tensor.from_f32(dev, (1, 17408), f32, synth.activations(1, 17408, seed=23))
+    outs = [api.Tensor.zeros(dev, (1, n), f32) for n, _ in shapes]
+
+    def enqueue(i):
+        mats = sets[i % layers]
+        dev.project_quantized(x5, mats[0], out=outs[0])
+        dev.project_quantized(x5, mats[1], out=outs[1])
+        dev.project_quantized(x5, mats[2], out=outs[2])
+        dev.project_quantized(x17, mats[3], out=outs[3])
+
+    best = min(run_graph(dev, enqueue, steps, layers)[1] for _ in range(2)) / steps
+    nbytes = sum(algorithmic_bytes(Q4_K, n, k, 1, 4, 4) for n, k in shapes)
+    flops = sum(2 * n * k for n, k in shapes)
+    return {
+        "workload": "Q4_K decode layer: attn 5120x5120 + gate/up 2 x (17408x5120) + down 5120x17408, M=1",
+        "operation": "4 x q4_k_gemv",
+        "us": round(best * 1e6, 2),
+        "GB/s": round(nbytes / best / 1e9, 1),
+        "frac_hbm": round(nbytes / best / 1e9 / HBM_PEAK_GBS, 4),
+        "TFLOP/s": round(flops / best / 1e12, 2),
+        "frac_mfma_f16": round(flops / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+        "weight_copies": layers,
+    }
+
+
 def moe_case(api, synth, dev, tokens, steps):
     """A3B-style routed FFN: hidden 2048, 256 experts x intermediate 512 in Q4_K,
     top-8 softmax routing with renormalised weights, plus one shared expert;
@@ -263,6 +301,7 @@ def main():
         timed(Q4_K, 4096, 4096, 1, f32, "Q4_K GEMV M=1 K=4096 N=4096", 1200)
         timed(Q4_K, 5120, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=5120", 1200)
         timed(Q4_K, 5120, 17408, 1, f32, "Q4_K GEMV M=1 K=17408 N=5120", 1200)
+        cases.append(layer_case(api, synth, dev, 400))
         timed(Q6_K, 5120, 17408, 1, f32, "Q6_K GEMV M=1 K=17408 N=5120", 600)
         timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
         for m in (8, 16, 128):

@@ -73,11 +73,23 @@ class Case:
         self.dev.project_quantized(self.x, self.weights[i % len(self.weights)], out=self.y)
 
 
+EAGER = False   # --eager: launch step by step instead of replaying a recording (for profilers)
+
+
 def run_graph(dev, enqueue, steps, warmup):
     """Replays `steps` recorded launches; returns (wall seconds, event seconds)."""
     for i in range(max(warmup, 1)):
         enqueue(i)
     dev.synchronize()
+    if EAGER:
+        start, stop = dev.event(), dev.event()
+        t0 = time.perf_counter()
+        start.record()
+        for i in range(steps):
+            enqueue(i)
+        stop.record()
+        dev.synchronize()
+        return time.perf_counter() - t0, start.elapsed_ms(stop) * 1e-3
     with dev.execution() as ex:
         for i in range(steps):
             enqueue(i)
@@ -267,7 +279,13 @@ def main():
                     help="'headline' times only the metric's GEMV; 'all' adds the other shapes; "
                          "'copy' launches a plain row copy of known size (counter calibration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="with --cases all: run only the cases whose label contains this text")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every step from the host instead of replaying a HIP graph (timings then "
+                         "include launch gaps; meant for kernel traces)")
     args = ap.parse_args()
+    global EAGER
+    EAGER = args.eager
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; every box has one and no multi-GPU "
                  f"path exists (asked for --gpus {args.gpus})")
@@ -291,6 +309,8 @@ def main():
     gemm = None
     if args.cases == "all":
         def timed(ggml, n, k, m, xd, label, steps, copies=None):
+            if args.only and args.only not in label:
+                return None
             c = Case(api, synth, dev, ggml, n, k, m, xd, label, copies)
             _, ev = measure(dev, c, steps, min(args.warmup, len(c.weights)), repeats=2)
             r = report(c, ev / steps)
@@ -301,14 +321,17 @@ def main():
         timed(Q4_K, 4096, 4096, 1, f32, "Q4_K GEMV M=1 K=4096 N=4096", 1200)
         timed(Q4_K, 5120, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=5120", 1200)
         timed(Q4_K, 5120, 17408, 1, f32, "Q4_K GEMV M=1 K=17408 N=5120", 1200)
-        cases.append(layer_case(api, synth, dev, 400))
+        if not args.only or args.only in "decode layer":
+            cases.append(layer_case(api, synth, dev, 400))
         timed(Q6_K, 5120, 17408, 1, f32, "Q6_K GEMV M=1 K=17408 N=5120", 600)
         timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
         for m in (8, 16, 128):
             timed(Q4_K, 17408, 5120, m, f16, f"Q4_K GEMM M={m} K=5120 N=17408 f16 x", 240)
         gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
-        cases.append(moe_case(api, synth, dev, 1, 200))
-        cases.append(moe_case(api, synth, dev, 512, 20))
+        if not args.only or args.only in "MoE FFN T=1":
+            cases.append(moe_case(api, synth, dev, 1, 200))
+        if not args.only or args.only in "MoE FFN T=512":
+            cases.append(moe_case(api, synth, dev, 512, 20))
 
     line = {
         "metric": "Q4_K GEMV GB/s at M=1, K=5120, N=17408",

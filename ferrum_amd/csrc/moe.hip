@@ -17,14 +17,29 @@ __device__ __forceinline__ uint32_t total_order_key(float x) {
     return (bits & 0x80000000u) ? ~bits : (bits ^ 0x80000000u);
 }
 
+template <int CTRL>
+__device__ __forceinline__ unsigned long long dpp_max_u64(unsigned long long v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, 0xf, 0xf, false);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, 0xf, 0xf, false);
+    const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+    return other > v ? other : v;
+}
+
+// Maximum over the 64 lanes, returned in all lanes; every lane must be active.
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-    for (int off = 32; off > 0; off >>= 1) {
-        uint32_t lo = __shfl_xor((uint32_t)v, off, 64);
-        uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, 64);
-        unsigned long long other = ((unsigned long long)hi << 32) | lo;
-        v = other > v ? other : v;
+    v = dpp_max_u64<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_u64<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_u64<0x141>(v);  // row_half_mirror
+    v = dpp_max_u64<0x140>(v);  // row_mirror: every lane now holds its row's maximum
+    unsigned long long best = 0ull;
+#pragma unroll
+    for (int row = 0; row < 4; ++row) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 16 * row);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 16 * row);
+        const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+        best = other > best ? other : best;
     }
-    return v;
+    return best;
 }
 
 // One wave per token.  Scores are computed by all lanes in parallel; the
@@ -112,7 +127,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
                 }
             }
             // the owner lane publishes the raw score (bias excluded)
-            sel_score[rank] = __shfl(mine, id & 63u, 64);
+            sel_score[rank] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), id & 63u));
             sel_id[rank] = id;
         } else {
             sel_id[rank] = 0xffffffffu;

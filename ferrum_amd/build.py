@@ -82,5 +82,18 @@ def build_host_test() -> str:
     return out
 
 
+def build_gguf_probe() -> str:
+    """Compiles tests/cpp/gguf_probe.cpp (the C++ GGUF reader's CPU test
+    program; host code only, nothing to link)."""
+    root = os.path.dirname(HERE)
+    out = os.path.join(root, "tests", "cpp", "gguf_probe")
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Werror", "-I" + os.path.join(root, "include"),
+           os.path.join(root, "tests", "cpp", "gguf_probe.cpp"), "-o", out]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"g++ failed for the GGUF probe:\n{proc.stdout}\n{proc.stderr}")
+    return out
+
+
 if __name__ == "__main__":
     print(build(sys.argv[1:]))

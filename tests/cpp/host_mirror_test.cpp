@@ -10,6 +10,7 @@
 #include <cstring>
 #include <vector>
 
+#include "ferrum_gguf.hpp"
 #include "ferrum_hip.hpp"
 
 extern "C" {
@@ -81,6 +82,44 @@ static double rel_l2(const std::vector<float>& a, const std::vector<float>& b) {
 static QuantizedMatrix upload(const Device& d, QuantizationFormat f, size_t rows, size_t cols,
                               const std::vector<uint8_t>& bytes) {
     return d.quantized_matrix(rows, cols, f, [&](uint8_t* dst, size_t n) { std::memcpy(dst, bytes.data(), n); });
+}
+
+// A GGUF v3 file holding the given K-quant tensors back to back at 32-byte
+// aligned offsets (the layout src/loader/gguf.rs:709-748 builds for its tests).
+struct FileTensor {
+    std::string name;
+    std::vector<uint64_t> dims;
+    uint32_t type;
+    const std::vector<uint8_t>* payload;
+};
+static std::string gguf_file(const std::vector<FileTensor>& tensors) {
+    std::string out("GGUF");
+    auto put = [&out](const void* p, size_t n) { out.append(static_cast<const char*>(p), n); };
+    auto u32 = [&](uint32_t v) { put(&v, 4); };
+    auto u64 = [&](uint64_t v) { put(&v, 8); };
+    auto str = [&](const std::string& v) { u64(v.size()); out += v; };
+    u32(3);
+    u64(tensors.size());
+    u64(2);
+    str("general.architecture"); u32(8); str("qwen3moe");
+    str("general.quantization_version"); u32(4); u32(2);
+    uint64_t cursor = 0;
+    std::vector<uint64_t> offsets;
+    for (const auto& t : tensors) {
+        str(t.name);
+        u32((uint32_t)t.dims.size());
+        for (uint64_t dim : t.dims) u64(dim);
+        u32(t.type);
+        u64(cursor);
+        offsets.push_back(cursor);
+        cursor = (cursor + t.payload->size() + 31) / 32 * 32;
+    }
+    out.resize((out.size() + 31) / 32 * 32, '\0');
+    const size_t base = out.size();
+    out.resize(base + cursor, '\0');
+    for (size_t i = 0; i < tensors.size(); ++i)
+        std::memcpy(&out[base + offsets[i]], tensors[i].payload->data(), tensors[i].payload->size());
+    return out;
 }
 
 int main() {
@@ -199,6 +238,41 @@ int main() {
         const auto replayed = y.to_f32();
         report("a recorded execution replays the projection bitwise",
                std::memcmp(eager.data(), replayed.data(), eager.size() * 4) == 0);
+    }
+    {
+        // tensors read from a GGUF stream reach the device unchanged
+        const size_t n = 96, k = 768, experts = 3, rows = 32;
+        const auto q4 = blocks(QuantizationFormat::Q4_K, n, k, 41);
+        const auto q6 = blocks(QuantizationFormat::Q6_K, n, k, 42);
+        const auto ex = blocks(QuantizationFormat::Q4_K, experts * rows, k, 43);
+        std::istringstream stream(gguf_file({{"blk.0.attn_q.weight", {k, n}, FH_GGML_Q4_K, &q4},
+                                             {"output.weight", {k, n}, FH_GGML_Q6_K, &q6},
+                                             {"blk.0.ffn_down_exps.weight", {k, rows, experts}, FH_GGML_Q4_K, &ex}}));
+        gguf::Reader file(stream);
+        bool exact = true;
+        for (const auto& [name, packed] : {std::pair<const char*, const std::vector<uint8_t>*>{"blk.0.attn_q.weight", &q4},
+                                           {"output.weight", &q6}}) {
+            QuantizedMatrix w = gguf::load_quantized_matrix(d, file, name);
+            std::vector<float> want(n * k);
+            fo_dequantize(static_cast<uint32_t>(w.format()), packed->data(), n, k, want.data());
+            const auto dense = d.dequantize(w).to_f32();
+            exact &= w.rows() == n && w.columns() == k && std::memcmp(dense.data(), want.data(), want.size() * 4) == 0;
+        }
+        report("matrices loaded from GGUF dequantize bit-exactly", exact);
+        QuantizedExpertMatrix e = gguf::load_quantized_expert_matrix(d, file, "blk.0.ffn_down_exps.weight");
+        std::vector<float> want(experts * rows * k);
+        fo_dequantize(FH_GGML_Q4_K, ex.data(), experts * rows, k, want.data());
+        const auto dense = d.dequantize(e.matrix()).to_f32();
+        report("expert tensor loaded from GGUF keeps [experts, rows, columns]",
+               e.experts() == experts && e.rows_per_expert() == rows && e.columns() == k &&
+                   std::memcmp(dense.data(), want.data(), want.size() * 4) == 0);
+        bool threw = false;
+        try {
+            gguf::load_quantized_matrix(d, file, "blk.0.ffn_down_exps.weight");
+        } catch (const Error& err) {
+            threw = err.kind() == ErrorKind::Gguf;
+        }
+        report("a rank-3 tensor is not a matrix: Error::Gguf", threw);
     }
     std::printf("%d failure(s)\n", failures);
     return failures ? 1 : 0;

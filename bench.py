@@ -228,8 +228,11 @@ def moe_case(api, synth, dev, tokens, steps):
         moe.forward(x, logit_sets[i % variants])
         names.append(dev.last_operation())
         dev.project_quantized(x, sin, out=s_up)
-        dev.expert_silu_mul(s_up, inter, out=s_act)
-        dev.project_quantized(s_act, sout, out=s_out)
+        if tokens * top_k <= moe.fused_max_assignments:
+            dev.project_quantized(s_up, sout, out=s_out, silu_mul=True)   # decode: SiLU*up rides in the projection
+        else:
+            dev.expert_silu_mul(s_up, inter, out=s_act)
+            dev.project_quantized(s_act, sout, out=s_out)
 
     best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(2)) / steps
     per_expert = (2 * inter * hidden + hidden * inter) // 256 * BLOCK_BYTES[Q4_K]

@@ -114,6 +114,8 @@ SYMBOLS = {
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
     "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
+    "fh_expert_project_fused": (_I32, [_P, _P, _VP, _U32, _U32, _U32, _VP, _VP]),
+    "fh_project_silu_mul_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_expert_silu_mul": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_expert_combine": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_execution_begin": (_I32, [_P]),
@@ -542,9 +544,12 @@ class Device:
         return Output(out, self.last_operation())
 
     def project_quantized(self, a: Tensor, weight: QuantizedMatrix, out_dtype: DType | None = None,
-                          out: Tensor | None = None) -> Output:
+                          out: Tensor | None = None, silu_mul: bool = False) -> Output:
+        """``silu_mul=True`` takes ``a`` as [M, 2K] (gate first) and projects
+        round(round(silu(gate)) * up), as expert_silu_mul followed by this call would."""
         dims = a.shape()
-        if len(dims) != 2 or dims[1] != weight.columns() or dims[1] > 0xFFFFFFFF - 32:
+        if (len(dims) != 2 or dims[1] != weight.columns() * (2 if silu_mul else 1)
+                or dims[1] > 0xFFFFFFFF - 32):
             raise ShapeError("quantized projection requires [M,K] matching [N,K]")
         if a.buffer.device is not self or weight.device is not self:
             raise DeviceMismatch("tensor or weight belongs to another device")
@@ -555,8 +560,8 @@ class Device:
         if m == 0:
             return Output(out, "")
         xv, yv = a._view(), out._view()
-        _check(_lib.fh_project_quantized(self._handle, _handle_of(weight), ctypes.byref(xv), m,
-                                         ctypes.byref(yv)))
+        call = _lib.fh_project_silu_mul_quantized if silu_mul else _lib.fh_project_quantized
+        _check(call(self._handle, _handle_of(weight), ctypes.byref(xv), m, ctypes.byref(yv)))
         return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
 
     def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy,
@@ -591,9 +596,16 @@ class Device:
 
     def expert_project_quantized(self, input: Tensor, metadata: Tensor,
                                  weight: QuantizedExpertMatrix, features: int, experts: int,
-                                 out_dtype: DType | None = None, out: Tensor | None = None) -> Tensor:
+                                 out_dtype: DType | None = None, out: Tensor | None = None,
+                                 form: str = "rows") -> Tensor:
+        """``form``: "rows" reads input [A, K]; "gather" reads input as hidden
+        [tokens, K] and uses row token(a) (expert_assign folded in); "silu_mul"
+        reads input [A, 2K] and applies expert_silu_mul on the way in."""
         x, meta = input.shape(), metadata.shape()
-        if (len(x) != 2 or x[0] == 0 or x[1] != features or meta != (x[0], 3)
+        code = {"rows": 0, "gather": 1, "silu_mul": 2}[form]
+        width = features * (2 if code == 2 else 1)
+        if (len(x) != 2 or x[0] == 0 or x[1] != width or len(meta) != 2 or meta[1] != 3 or meta[0] == 0
+                or (code != 1 and meta[0] != x[0])
                 or metadata.dtype != DType.F32 or experts == 0 or weight.experts() != experts
                 or weight.columns() != features or weight.rows_per_expert() == 0
                 or input.buffer.device is not self or metadata.buffer.device is not self
@@ -601,10 +613,14 @@ class Device:
             raise ShapeError("quantized expert projection geometry mismatch")
         dtype = input.dtype if out_dtype is None else DType(out_dtype)
         if out is None:
-            out = Tensor.zeros(self, (x[0], weight.rows_per_expert()), dtype)
+            out = Tensor.zeros(self, (meta[0], weight.rows_per_expert()), dtype)
         xv, mv, ov = input._view(), metadata._view(), out._view()
-        _check(_lib.fh_expert_project_quantized(self._handle, weight._handle, ctypes.byref(xv), x[0],
-                                                ctypes.byref(mv), ctypes.byref(ov)))
+        if code == 0:
+            _check(_lib.fh_expert_project_quantized(self._handle, weight._handle, ctypes.byref(xv), x[0],
+                                                    ctypes.byref(mv), ctypes.byref(ov)))
+        else:
+            _check(_lib.fh_expert_project_fused(self._handle, weight._handle, ctypes.byref(xv), x[0], code,
+                                                meta[0], ctypes.byref(mv), ctypes.byref(ov)))
         return out
 
     def expert_silu_mul(self, input: Tensor, intermediate: int, out: Tensor | None = None) -> Tensor:
@@ -660,6 +676,9 @@ class SparseMoe:
         self.input_experts, self.output_experts = input_experts, output_experts
         self.expert_count, self.hidden_size, self.intermediate_size = e, h, two_i // 2
         self._ws = None
+        # most assignments that take the fused per-assignment kernels; above it the
+        # separate steps run (and group by expert from 32 assignments on)
+        self.fused_max_assignments = 31
 
     def workspace(self, tokens: int, dtype: DType):
         a, h, i = tokens * self.routing.top_k, self.hidden_size, self.intermediate_size
@@ -682,13 +701,21 @@ class SparseMoe:
         d, k = self.device, self.routing.top_k
         ws = self._ws if self._ws and self._ws["tokens"] == dims[0] and self._ws["dtype"] == hidden.dtype else {}
         metadata = d.moe_route(router_logits, self.selection_bias, self.routing, out=ws.get("metadata"))
-        assigned = d.expert_assign(hidden, metadata, k, out=ws.get("assigned"))
-        projected = d.expert_project_quantized(assigned, metadata, self.input_experts, self.hidden_size,
-                                               self.expert_count, out=ws.get("projected"))
-        activated = d.expert_silu_mul(projected, self.intermediate_size, out=ws.get("activated"))
-        expert_output = d.expert_project_quantized(activated, metadata, self.output_experts,
-                                                   self.intermediate_size, self.expert_count,
-                                                   out=ws.get("expert_output"))
+        if dims[0] * k <= self.fused_max_assignments:
+            # decode: the copy and the activation ride inside the projections
+            projected = d.expert_project_quantized(hidden, metadata, self.input_experts, self.hidden_size,
+                                                   self.expert_count, out=ws.get("projected"), form="gather")
+            expert_output = d.expert_project_quantized(projected, metadata, self.output_experts,
+                                                       self.intermediate_size, self.expert_count,
+                                                       out=ws.get("expert_output"), form="silu_mul")
+        else:
+            assigned = d.expert_assign(hidden, metadata, k, out=ws.get("assigned"))
+            projected = d.expert_project_quantized(assigned, metadata, self.input_experts, self.hidden_size,
+                                                   self.expert_count, out=ws.get("projected"))
+            activated = d.expert_silu_mul(projected, self.intermediate_size, out=ws.get("activated"))
+            expert_output = d.expert_project_quantized(activated, metadata, self.output_experts,
+                                                       self.intermediate_size, self.expert_count,
+                                                       out=ws.get("expert_output"))
         return d.expert_combine(expert_output, metadata, dims[0], self.hidden_size, k,
                                 out=ws.get("combined"))
 

@@ -121,6 +121,9 @@ int64_t tuning(const fh_device* d, const char* key) {
 
 using namespace fh;
 
+static_assert(kXPlain == FH_INPUT_ROWS && kXGather == FH_INPUT_GATHER && kXSiluMul == FH_INPUT_SILU_MUL,
+              "the kernel's input modes are the ABI's input forms");
+
 extern "C" {
 
 const char* fh_last_error(void) { return g_last_error.c_str(); }
@@ -440,8 +443,10 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
 
 // ---- dense projection --------------------------------------------------------------
 
-fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
-                               uint32_t m, const fh_view* y) {
+namespace {
+
+fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t m,
+                  const fh_view* y, bool silu_mul) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device) {
         g_last_error = "weight belongs to another device";
@@ -450,16 +455,17 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
     const uint64_t n = weight->rows * weight->experts, k = weight->cols;
     if (m == 0 || k > 0xffffffffull - 32)
         return fail(FH_ERR_SHAPE, "quantized projection requires [M,K] matching [N,K]");
-    if (!fits_u32((uint64_t)m * k) || !fits_u32((uint64_t)m * n) || !fits_u32(n))
+    const uint64_t x_elements = (uint64_t)m * k * (silu_mul ? 2 : 1);
+    if (!fits_u32(x_elements) || !fits_u32((uint64_t)m * n) || !fits_u32(n))
         return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
     Range xr, yr;
-    fh_status st = resolve(device, x, (uint64_t)m * k, "projection input", &xr);
+    fh_status st = resolve(device, x, x_elements, "projection input", &xr);
     if (st != FH_OK) return st;
     st = resolve(device, y, (uint64_t)m * n, "projection output", &yr);
     if (st != FH_OK) return st;
     if (overlaps(xr, yr)) return fail(FH_ERR_RANGE, "projection output aliases its input");
 
-    const bool tile = m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32;
+    const bool tile = !silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32;
     if (tile) {
         GemmArgs a{};
         a.ggml_type = weight->ggml_type;
@@ -489,6 +495,8 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
         a.metadata = nullptr;
         a.experts = 1;
         a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
+        a.x_mode = silu_mul ? kXSiluMul : kXPlain;
+        a.x_rows = m;
         st = prepare_gemv(device, a);
         if (st != FH_OK) return st;
         const char* name = launch_gemv(device->stream, a);
@@ -497,6 +505,18 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
     }
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                               uint32_t m, const fh_view* y) {
+    return project(device, weight, x, m, y, false);
+}
+
+fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* packed,
+                                        uint32_t m, const fh_view* y) {
+    return project(device, weight, packed, m, y, true);
 }
 
 // ---- mixture of experts -------------------------------------------------------------
@@ -557,20 +577,26 @@ fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t to
     return FH_OK;
 }
 
-fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weight,
-                                      const fh_view* x, uint32_t assignments,
-                                      const fh_view* metadata, const fh_view* y) {
+namespace {
+
+fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t x_rows,
+                         uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (form > FH_INPUT_SILU_MUL) return fail(FH_ERR_PARAMETER, "unknown input form %u", form);
+    if (form == FH_INPUT_GATHER && x_rows == 0) return fail(FH_ERR_SHAPE, "gathered expert projection needs tokens");
     if (weight->device != device || assignments == 0 || metadata == nullptr ||
         metadata->dtype != FH_F32 || metadata->buffer == nullptr ||
         metadata->buffer->device != device || x == nullptr || x->buffer == nullptr ||
         x->buffer->device != device)
         return fail(FH_ERR_SHAPE, "quantized expert projection geometry mismatch");
     const uint64_t rows = weight->rows, k = weight->cols;
-    if (!fits_u32((uint64_t)assignments * rows) || !fits_u32((uint64_t)assignments * k))
+    // elements the input view must hold: [A,K], [tokens,K] or [A,2K]
+    const uint64_t x_elements = form == FH_INPUT_GATHER ? (uint64_t)x_rows * k
+                                : (uint64_t)assignments * k * (form == FH_INPUT_SILU_MUL ? 2 : 1);
+    if (!fits_u32((uint64_t)assignments * rows) || !fits_u32(x_elements))
         return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
     Range xr, mr, yr;
-    fh_status st = resolve(device, x, (uint64_t)assignments * k, "expert input", &xr);
+    fh_status st = resolve(device, x, x_elements, "expert input", &xr);
     if (st != FH_OK) return st;
     st = resolve(device, metadata, (uint64_t)assignments * 3, "expert metadata", &mr, 4);
     if (st != FH_OK) return st;
@@ -578,7 +604,7 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
     if (st != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(mr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
     const int64_t grouped_min = tuning(device, "expert_grouped_min_assignments");
-    if (x->dtype != FH_F32 && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
+    if (form == FH_INPUT_ROWS && x->dtype != FH_F32 && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
         weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
         // grouped form: every expert's weights are streamed once for all of its assignments
         const size_t words = (size_t)weight->experts + 1 + assignments;
@@ -620,11 +646,27 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
     a.metadata = reinterpret_cast<const float*>(mr.begin);
     a.experts = (uint32_t)weight->experts;
     a.ksplit = 0;
+    a.x_mode = form;
+    a.x_rows = form == FH_INPUT_GATHER ? x_rows : assignments;
     st = prepare_gemv(device, a);
     if (st != FH_OK) return st;
     device->last_operation = launch_gemv(device->stream, a);
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weight,
+                                      const fh_view* x, uint32_t assignments,
+                                      const fh_view* metadata, const fh_view* y) {
+    return expert_project(device, weight, x, assignments, FH_INPUT_ROWS, assignments, metadata, y);
+}
+
+fh_status fh_expert_project_fused(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                  uint32_t x_rows, uint32_t input_form, uint32_t assignments,
+                                  const fh_view* metadata, const fh_view* y) {
+    return expert_project(device, weight, x, x_rows, input_form, assignments, metadata, y);
 }
 
 fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assignments,

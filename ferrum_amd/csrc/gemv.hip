@@ -39,7 +39,8 @@ namespace {
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kXStride = 68;  // float4 per block in LDS: 64 + 4, so neighbouring blocks use the other bank half
-constexpr int kMaxIt = 3;
+// most steps per wave: bounded by the registers that hold the weight fragments
+constexpr int max_steps(int bs) { return bs >= 8 ? 3 : 5; }
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
@@ -169,6 +170,21 @@ __device__ __forceinline__ float4 load_x4(const void* x, uint32_t dtype, size_t 
                        bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
 }
 
+// SiLU in the branch-stable form of expert_silu_mul (src/metal/shaders/ops.metal:2223-2232)
+__device__ __forceinline__ float gemv_silu(float gate) {
+    float s = gate >= 0.f ? 1.f / (1.f + expf(-gate)) : expf(gate) / (1.f + expf(gate));
+    return gate * s;
+}
+
+// What expert_silu_mul would have stored for four columns, rounded to the
+// activation dtype at the same two points.
+__device__ __forceinline__ float4 silu_mul4(float4 g, float4 u, uint32_t dtype) {
+    return make_float4(round_storage(round_storage(gemv_silu(g.x), dtype) * u.x, dtype),
+                       round_storage(round_storage(gemv_silu(g.y), dtype) * u.y, dtype),
+                       round_storage(round_storage(gemv_silu(g.z), dtype) * u.z, dtype),
+                       round_storage(round_storage(gemv_silu(g.w), dtype) * u.w, dtype));
+}
+
 struct Params {
     const uint8_t* w;
     const void* x;
@@ -180,6 +196,8 @@ struct Params {
     uint32_t seg_len;    // super-blocks per K segment
     uint32_t segments;
     uint32_t x_dtype, y_dtype, experts;
+    uint32_t x_rows;     // rows of x, for kXGather
+    uint32_t x_mode;     // kXPlain, kXGather (row = token of the assignment) or kXSiluMul (x = silu(gate) * up)
 };
 
 // grid: (row tiles, K segments, m)
@@ -208,14 +226,28 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     const uint8_t* rp = p.w + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
 
     // 1. activations of this segment (requested first, consumed first)
-    const size_t xbase = ((size_t)m * p.nb + b0) * 64;  // float4 index of the segment start
+    // float4 index of the segment start in the row this batch entry reads
+    size_t xrow = m;
+    if (p.x_mode == kXGather) {
+        const uint32_t token = __float_as_uint(p.metadata[3 * (size_t)m + 1]);
+        xrow = token < p.x_rows ? token : p.x_rows - 1;
+    }
+    const size_t xbase = (xrow * (p.x_mode == kXSiluMul ? 2 : 1) * p.nb + b0) * 64;
+    // the SiLU form computes on what it loads, so it fetches after the weight
+    // loads are queued instead of ahead of them
+    const bool early = p.x_mode != kXSiluMul;
+    auto fetch = [&](uint32_t q) {
+        float4 v = load_x4(p.x, p.x_dtype, xbase + q);
+        if (p.x_mode == kXSiluMul) v = silu_mul4(v, load_x4(p.x, p.x_dtype, xbase + (size_t)p.nb * 64 + q), p.x_dtype);
+        return v;
+    };
     const uint32_t xq = cb * 64;
-    constexpr int kXPer = 6;
+    constexpr int kXPer = (BS * IT + 3) / 4;  // float4 per thread that cover the longest segment
     float4 xr[kXPer];
 #pragma unroll
     for (int i = 0; i < kXPer; ++i) {
         uint32_t q = tid + i * kThreads;
-        xr[i] = q < xq ? load_x4(p.x, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
+        xr[i] = q < xq && early ? load_x4(p.x, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     asm volatile("" ::: "memory");
 
@@ -241,10 +273,10 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
 #pragma unroll
     for (int i = 0; i < kXPer; ++i) {
         uint32_t q = tid + i * kThreads;
-        if (q < xq) stage(q, xr[i]);
+        if (q < xq && early) stage(q, xr[i]);
     }
-    for (uint32_t q = tid + kXPer * kThreads; q < xq; q += kThreads)
-        stage(q, load_x4(p.x, p.x_dtype, xbase + q));
+    for (uint32_t q = tid + (early ? kXPer * kThreads : 0); q < xq; q += kThreads)
+        stage(q, fetch(q));
     __syncthreads();
 
     // 4. consume, one step at a time
@@ -312,7 +344,7 @@ LaunchFn pick(int bs, int it) {
 #define FH_CASE(B, I) \
     if (bs == B && it == I) return launch_impl<TYPE, B, I>;
     FH_CASE(8, 1) FH_CASE(8, 2) FH_CASE(8, 3)
-    FH_CASE(4, 1) FH_CASE(4, 2) FH_CASE(4, 3)
+    FH_CASE(4, 1) FH_CASE(4, 2) FH_CASE(4, 3) FH_CASE(4, 4) FH_CASE(4, 5)
     FH_CASE(2, 1) FH_CASE(2, 2) FH_CASE(2, 3)
     FH_CASE(1, 1) FH_CASE(1, 2) FH_CASE(1, 3)
 #undef FH_CASE
@@ -321,12 +353,13 @@ LaunchFn pick(int bs, int it) {
 
 }  // namespace
 
-GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
+namespace {
+
+// Segments, segment length and steps for a block-slot count.
+GemvPlan plan_for(uint32_t nb, int bs, int forced_segments) {
     GemvPlan plan{};
-    const uint32_t nb = k / 256;
-    // widest block-slot count the row length fills
-    const int bs = nb >= 8 ? 8 : nb >= 4 ? 4 : nb >= 2 ? 2 : 1;
-    uint32_t segments = (nb + bs * kMaxIt - 1) / (bs * kMaxIt);
+    const uint32_t span = (uint32_t)(bs * max_steps(bs));
+    uint32_t segments = (nb + span - 1) / span;
     if (forced_segments > 0) {
         // the reference's K-split switch: at least that many segments, as far
         // as the row length allows
@@ -340,7 +373,26 @@ GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
     plan.it = (int)((seg_len + bs - 1) / bs);
     plan.segments = (nb + seg_len - 1) / seg_len;
     plan.seg_len = seg_len;
-    plan.rows_per_wg = (uint32_t)(kWaves * (16 / bs));
+    return plan;
+}
+
+}  // namespace
+
+GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
+    const uint32_t nb = k / 256;
+    // widest block-slot count the row length fills ...
+    const int bs = nb >= 8 ? 8 : nb >= 4 ? 4 : nb >= 2 ? 2 : 1;
+    GemvPlan plan = plan_for(nb, bs, forced_segments);
+    if (bs == 8 && n >= 16384) {
+        // ... unless four slots and more steps leave fewer idle slot-steps (20
+        // blocks: 4 x 5 covers them exactly, 8 x 3 idles a sixth of the wave)
+        // and the matrix still makes a thousand 16-row workgroups
+        const GemvPlan narrow = plan_for(nb, 4, forced_segments);
+        const uint32_t idle_wide = plan.segments * (uint32_t)(plan.bs * plan.it) - nb;
+        const uint32_t idle_narrow = narrow.segments * (uint32_t)(narrow.bs * narrow.it) - nb;
+        if (idle_narrow < idle_wide && narrow.segments <= plan.segments) plan = narrow;
+    }
+    plan.rows_per_wg = (uint32_t)(kWaves * (16 / plan.bs));
     plan.tiles = (n + plan.rows_per_wg - 1) / plan.rows_per_wg;
     (void)m;
     return plan;
@@ -363,6 +415,8 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     p.x_dtype = a.x_dtype;
     p.y_dtype = a.y_dtype;
     p.experts = a.experts;
+    p.x_mode = a.x_mode;
+    p.x_rows = a.x_rows;
     const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
     dim3 grid(plan.tiles, plan.segments, a.m);
     LaunchFn fn = a.ggml_type == kQ4K ? pick<kQ4K>(plan.bs, plan.it) : pick<kQ6K>(plan.bs, plan.it);

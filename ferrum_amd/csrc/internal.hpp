@@ -74,6 +74,13 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                                     uint32_t out_dtype);
 
 // gemv.hip
+// how a GEMV launch reads its activations
+enum : uint32_t {
+    kXPlain = 0,    // row m of x
+    kXGather = 1,   // row token(m) of x, the token id from the routing metadata (expert_assign fused)
+    kXSiluMul = 2,  // x is [m, 2K]: silu(x[:, :K]) * x[:, K:] with expert_silu_mul's rounding
+};
+
 struct GemvArgs {
     uint32_t ggml_type;
     const void* w;        // packed [n, k] (per expert when metadata is set)
@@ -86,6 +93,8 @@ struct GemvArgs {
     const float* metadata;
     uint32_t experts;
     int ksplit;           // 0 = automatic, else at least this many K segments
+    uint32_t x_mode;      // kXPlain, kXGather or kXSiluMul
+    uint32_t x_rows;      // rows of x (kXGather clamps the token id to it)
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
 };

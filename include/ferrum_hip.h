@@ -186,6 +186,29 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
                                       const fh_view* x, uint32_t assignments,
                                       const fh_view* metadata, const fh_view* y);
 
+/* Decode-sized fusions.  SparseMoe::forward (src/nn/moe.rs:222-390) encodes
+ * expert_assign, the gate|up projection, expert_silu_mul and the down
+ * projection back to back; with a handful of assignments each of them is a
+ * launch that lasts microseconds.  These two entry points fold the copy or the
+ * activation into the projection that follows and give the same bits as the
+ * separate calls.  They always take the per-assignment (per-row) kernel, so
+ * callers keep the separate calls for prefill-sized batches.
+ *
+ * fh_expert_project_fused: input_form FH_INPUT_ROWS is
+ * fh_expert_project_quantized; FH_INPUT_GATHER reads x as hidden [x_rows, K]
+ * and row a uses hidden[token(a), :] (expert_assign, src/ops/mod.rs:75-115,
+ * folded in); FH_INPUT_SILU_MUL reads x as [assignments, 2K], gate first, and
+ * multiplies by round(round(silu(gate)) * up) in x's dtype (expert_silu_mul,
+ * src/ops/mod.rs:487-508, folded in).
+ * fh_project_silu_mul_quantized: the dense projection of FH_INPUT_SILU_MUL,
+ * packed [m, 2K] -> y [m, N] (a shared expert's down projection). */
+enum { FH_INPUT_ROWS = 0, FH_INPUT_GATHER = 1, FH_INPUT_SILU_MUL = 2 };
+fh_status fh_expert_project_fused(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                  uint32_t x_rows, uint32_t input_form, uint32_t assignments,
+                                  const fh_view* metadata, const fh_view* y);
+fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* weight,
+                                        const fh_view* packed, uint32_t m, const fh_view* y);
+
 /* MetalDevice::expert_silu_mul (src/ops/mod.rs:487-508): in [A, 2*I] (gate
  * first), out [A, I] = round(silu(gate)) * up, stored in out.dtype. */
 fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assignments,

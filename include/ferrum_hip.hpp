@@ -369,6 +369,27 @@ public:
         check(fh_expert_project_quantized(handle_->raw, w.matrix().raw(), &xv, (uint32_t)x[0], &mv, &yv));
         return y;
     }
+    // Decode-sized fusions (see ferrum_hip.h): the same bits as the separate calls in one launch.
+    // Gather: input is hidden [tokens, K], row a uses hidden[token(a), :].
+    Tensor expert_project_gathered(const Tensor& hidden, const Tensor& metadata, const QuantizedExpertMatrix& w,
+                                   const Tensor* out = nullptr) const {
+        return expert_project_fused(hidden, metadata, w, FH_INPUT_GATHER, out);
+    }
+    // SiLU: input is [A, 2K], gate first; expert_silu_mul is applied on the way in.
+    Tensor expert_project_silu_mul(const Tensor& packed, const Tensor& metadata, const QuantizedExpertMatrix& w,
+                                   const Tensor* out = nullptr) const {
+        return expert_project_fused(packed, metadata, w, FH_INPUT_SILU_MUL, out);
+    }
+    Output project_silu_mul_quantized(const Tensor& packed, const QuantizedMatrix& w, const Tensor* out = nullptr) const {
+        const auto& dims = packed.shape();
+        if (dims.size() != 2 || dims[1] != 2 * w.columns() || dims[0] == 0)
+            throw Error(ErrorKind::Shape, "quantized projection requires [M,2K] matching [N,K]");
+        if (!owns(packed) || w.owner() != handle_) throw Error(ErrorKind::DeviceMismatch, "tensor or weight belongs to another device");
+        Tensor y = out ? *out : zeros({dims[0], w.rows()}, packed.dtype());
+        fh_view xv = packed.c_view(), yv = y.c_view();
+        check(fh_project_silu_mul_quantized(handle_->raw, w.raw(), &xv, (uint32_t)dims[0], &yv));
+        return {y, {last_operation(), packed.byte_size() + w.byte_size(), y.byte_size()}};
+    }
     Tensor expert_silu_mul(const Tensor& input, size_t intermediate, const Tensor* out = nullptr) const {
         const auto& x = input.shape();
         if (x.size() != 2 || intermediate == 0 || intermediate * 2 != x[1])
@@ -404,6 +425,19 @@ public:
     }
 
 private:
+    Tensor expert_project_fused(const Tensor& input, const Tensor& metadata, const QuantizedExpertMatrix& w,
+                                uint32_t form, const Tensor* out) const {
+        const auto& x = input.shape();
+        const auto& m = metadata.shape();
+        const size_t width = w.columns() * (form == FH_INPUT_SILU_MUL ? 2 : 1);
+        if (x.size() != 2 || x[0] == 0 || x[1] != width || m.size() != 2 || m[0] == 0 || m[1] != 3 ||
+            (form != FH_INPUT_GATHER && m[0] != x[0]))
+            throw Error(ErrorKind::Shape, "quantized expert projection geometry mismatch");
+        Tensor y = out ? *out : zeros({m[0], w.rows_per_expert()}, input.dtype());
+        fh_view xv = input.c_view(), mv = metadata.c_view(), yv = y.c_view();
+        check(fh_expert_project_fused(handle_->raw, w.matrix().raw(), &xv, (uint32_t)x[0], form, (uint32_t)m[0], &mv, &yv));
+        return y;
+    }
     std::shared_ptr<detail::DeviceHandle> handle_;
 };
 
@@ -426,12 +460,21 @@ public:
         if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
             throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
         Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
+        if (dims[0] * routing_.top_k <= fused_max_assignments) {
+            // decode: the copy and the activation ride inside the projections
+            Tensor projected = device_.expert_project_gathered(hidden, meta, input_);
+            Tensor expert_output = device_.expert_project_silu_mul(projected, meta, output_);
+            return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
+        }
         Tensor assigned = device_.expert_assign(hidden, meta, routing_.top_k);
         Tensor projected = device_.expert_project_quantized(assigned, meta, input_, h, e);
         Tensor activated = device_.expert_silu_mul(projected, i);
         Tensor expert_output = device_.expert_project_quantized(activated, meta, output_, i, e);
         return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
     }
+
+    // most assignments that take the fused per-assignment kernels
+    size_t fused_max_assignments = 31;
 
 private:
     const Device& device_;

@@ -214,6 +214,16 @@ int main() {
         fo_expert_combine(down.data(), meta.data(), tokens, hidden, top_k, 0, want.data());
         report("SparseMoe::forward vs host evaluation", rel_l2(got, want) <= 2e-5, rel_l2(got, want));
 
+        // decode-sized batch: the fused projections give the bits of the separate steps
+        const size_t few = 3;
+        Tensor xs = d.from_f32({few, hidden}, DType::F16, std::vector<float>(x.begin(), x.begin() + few * hidden));
+        Tensor ls = d.from_f32({few, experts}, DType::F32, std::vector<float>(logits.begin(), logits.begin() + few * experts));
+        const auto fused = moe.forward(xs, ls).to_f32();
+        moe.fused_max_assignments = 0;
+        const auto separate = moe.forward(xs, ls).to_f32();
+        report("SparseMoe::forward decode path equals the separate steps bitwise",
+               std::memcmp(fused.data(), separate.data(), fused.size() * 4) == 0);
+
         Device other(0);
         bool threw = false;
         try {

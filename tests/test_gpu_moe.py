@@ -320,3 +320,89 @@ def test_a3b_style_ffn_with_shared_expert(api, d, tokens):
     # the result by about one f16 step of that stage
     assert rel_l2(got, want) <= 2e-3
     assert np.abs(got - want).max() <= 4e-3 * np.abs(want).max()
+
+
+# ------------------------------------------------------- decode-sized fusions
+
+@pytest.mark.parametrize("ggml,dtype", [(Q4_K, "F32"), (Q4_K, "F16"), (Q4_K, "BF16"), (Q6_K, "F16"), (Q6_K, "F32")])
+def test_fused_expert_projections_give_the_bits_of_the_separate_calls(api, d, ggml, dtype):
+    # 3 tokens x top-2 over 5 experts; hidden 768 -> 2 x 256 -> 768
+    experts, hidden, inter, tokens, top_k = 5, 768, 256, 3, 2
+    dt = getattr(api.DType, dtype)
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
+    w_in = synth.matrix(ggml, experts * 2 * inter, hidden, seed=61)
+    w_out = synth.matrix(ggml, experts * hidden, inter, seed=62)
+    fmt = api.QuantizationFormat(ggml)
+    win = api.QuantizedExpertMatrix.new(d, w_in, fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, w_out, fmt, experts, hidden, inter)
+    meta = np.zeros((tokens * top_k, 3), dtype=np.uint32)
+    meta[:, 0] = [1, 4, 0, 1, 2, 3]
+    meta[:, 1] = [0, 0, 1, 1, 2, 2]
+    meta[:, 2] = np.float32(0.5).view(np.uint32)
+    mt = api.Tensor.from_bits(d, meta.shape, meta)
+    x = oracle.round_storage(synth.activations(tokens, hidden, seed=63) * np.float32(2.0 ** -10), code).reshape(tokens, hidden)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+
+    assigned = d.expert_assign(xt, mt, top_k)
+    up = d.expert_project_quantized(assigned, mt, win, hidden, experts)
+    fused_up = d.expert_project_quantized(xt, mt, win, hidden, experts, form="gather")
+    assert d.last_operation().endswith("_factored")
+    assert np.array_equal(up.raw(), fused_up.raw())
+
+    act = d.expert_silu_mul(up, inter)
+    down = d.expert_project_quantized(act, mt, wout, inter, experts)
+    fused_down = d.expert_project_quantized(up, mt, wout, inter, experts, form="silu_mul")
+    assert np.array_equal(down.raw(), fused_down.raw())
+
+    # and against the oracle end to end (f64 accumulation, storage rounding at the same points)
+    m = meta.view(np.float32)
+    o_up = oracle.round_storage(oracle.expert_project(ggml, w_in, experts, 2 * inter, hidden,
+                                                      oracle.expert_assign(x, m), m, accumulate="f64"), code)
+    o_up = o_up.reshape(tokens * top_k, 2 * inter)
+    assert rel_l2(fused_up.to_f32(), o_up) <= (1e-5 if dtype == "F32" else 2e-3)
+    o_act = oracle.expert_silu_mul(fused_up.to_f32(), inter, code)
+    o_down = oracle.expert_project(ggml, w_out, experts, hidden, inter, o_act, m, accumulate="f64")
+    assert rel_l2(fused_down.to_f32(), o_down) <= (1e-5 if dtype == "F32" else 2e-3)
+
+    with pytest.raises(api.ShapeError):
+        d.expert_project_quantized(xt, mt, wout, inter, experts, form="gather")      # K mismatch
+    with pytest.raises(api.ShapeError):
+        d.expert_project_quantized(assigned, mt, wout, inter, experts, form="silu_mul")
+
+
+@pytest.mark.parametrize("dtype,m", [("F32", 1), ("F32", 3), ("F16", 1), ("BF16", 1)])
+def test_dense_projection_with_silu_mul_input_matches_the_two_calls(api, d, dtype, m):
+    n, k = 520, 1024
+    dt = getattr(api.DType, dtype)
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
+    packed = synth.matrix(Q4_K, n, k, seed=71)
+    w = api.QuantizedMatrix.from_bytes(d, n, k, api.QuantizationFormat(Q4_K), packed)
+    gate_up = oracle.round_storage(synth.activations(m, 2 * k, seed=72), code).reshape(m, 2 * k)
+    t = api.Tensor.from_f32(d, gate_up.shape, dt, gate_up)
+    two = d.project_quantized(d.expert_silu_mul(t, k), w).tensor
+    one = d.project_quantized(t, w, silu_mul=True).tensor
+    assert np.array_equal(one.raw(), two.raw())
+    want = oracle.project(Q4_K, packed, n, k, oracle.expert_silu_mul(gate_up, k, code), accumulate="f64")
+    assert rel_l2(one.to_f32(), want) <= (1e-5 if dtype == "F32" else 2e-3)
+    with pytest.raises(api.ShapeError):
+        d.project_quantized(api.Tensor.zeros(d, (m, k), dt), w, silu_mul=True)
+
+
+@pytest.mark.parametrize("tokens", [1, 3])
+def test_sparse_moe_decode_path_matches_the_separate_steps(api, d, tokens):
+    experts, hidden, inter, top_k = 16, 512, 256, 4
+    fmt = api.QuantizationFormat(Q4_K)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=81), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * hidden, inter, seed=82), fmt,
+                                         experts, hidden, inter)
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    x = synth.activations(tokens, hidden, seed=83, f16=True) * np.float32(2.0 ** -4)
+    logits = synth.rng(84).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    fused = moe.forward(xt, lt)
+    moe.fused_max_assignments = 0
+    separate = moe.forward(xt, lt)
+    assert np.array_equal(fused.raw(), separate.raw())
+    assert np.abs(fused.to_f32()).max() > 1e-3

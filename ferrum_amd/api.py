@@ -21,6 +21,7 @@ from __future__ import annotations
 import ctypes
 import enum
 import os
+import sys
 from dataclasses import dataclass
 
 import numpy as np
@@ -229,6 +230,8 @@ class Buffer:
         return _lib.fh_buffer_device_ptr(self._handle) or 0
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_buffer_free(h)
@@ -349,6 +352,8 @@ class QuantizedMatrix:
         return _lib.fh_qmatrix_device_ptr(self._handle) or 0
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_qmatrix_destroy(h)
@@ -396,6 +401,8 @@ class QuantizedExpertMatrix:
         return m
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_qmatrix_destroy(h)
@@ -442,6 +449,8 @@ class Event:
         return float(ms.value)
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_event_destroy(h)
@@ -458,6 +467,8 @@ class Graph:
         _check(_lib.fh_graph_launch(self._handle))
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_graph_destroy(h)
@@ -648,6 +659,8 @@ class Device:
         return out
 
     def __del__(self):
+        if sys.is_finalizing():   # the HIP runtime may already be gone at interpreter exit
+            return
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             _lib.fh_device_destroy(h)

@@ -22,7 +22,6 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 64;
 constexpr int kLd = kBK + 8;  // halfs per LDS row
-constexpr int kThreads = 256;
 
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
@@ -130,18 +129,21 @@ __device__ __forceinline__ float16v mfma(uint4 a, uint4 b, float16v c) {
     }
 }
 
-template <uint32_t TYPE, int DT>
-__global__ __launch_bounds__(kThreads) void gemm_tile_kernel(const uint8_t* __restrict__ w,
+// TS = 128: four waves, 64 x 64 each; TS = 64: two waves, 32 x 64 each (four times the
+// workgroups, for matrices too small to fill the chip with 128 x 128 tiles).
+template <uint32_t TYPE, int DT, int TS>
+__global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __restrict__ w,
                                                              const uint16_t* __restrict__ x,
                                                              void* __restrict__ y, uint32_t m,
                                                              uint32_t n, uint32_t nb,
                                                              uint32_t y_dtype) {
-    __shared__ __attribute__((aligned(16))) uint16_t xs[kBM * kLd];
-    __shared__ __attribute__((aligned(16))) uint16_t ws[kBN * kLd];
+    constexpr int WI = TS / 64;  // 32-row tiles per wave
+    __shared__ __attribute__((aligned(16))) uint16_t xs[TS * kLd];
+    __shared__ __attribute__((aligned(16))) uint16_t ws[TS * kLd];
     constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t n0 = blockIdx.x * kBN, m0 = blockIdx.y * kBM;
+    const uint32_t n0 = blockIdx.x * TS, m0 = blockIdx.y * TS;
     const uint32_t k = nb << 8;
 
     // loader roles: one tile row per thread pair
@@ -151,10 +153,10 @@ __global__ __launch_bounds__(kThreads) void gemm_tile_kernel(const uint8_t* __re
     const bool xlive = m0 + lrow < m;
     const uint16_t* xsrc = x + (size_t)(xlive ? m0 + lrow : 0) * k + 32 * lh;
 
-    const uint32_t wm = (wave >> 1) * 64, wn = (wave & 1u) * 64;
-    float16v acc[2][2];
+    const uint32_t wm = TS == 128 ? (wave >> 1) * 64 : wave * 32, wn = TS == 128 ? (wave & 1u) * 64 : 0;
+    float16v acc[WI][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -202,22 +204,22 @@ __global__ __launch_bounds__(kThreads) void gemm_tile_kernel(const uint8_t* __re
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             uint32_t koff = kk * 16 + 8 * (lane >> 5);
-            uint4 a[2], b[2];
+            uint4 a[WI], b[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < WI; ++i)
                 a[i] = *reinterpret_cast<const uint4*>(&xs[(wm + 32 * i + (lane & 31u)) * kLd + koff]);
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 b[j] = *reinterpret_cast<const uint4*>(&ws[(wn + 32 * j + (lane & 31u)) * kLd + koff]);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < WI; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = mfma<DT>(a[i], b[j], acc[i][j]);
         }
     }
 
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WI; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             uint32_t col = n0 + wn + 32 * j + (lane & 31u);
@@ -667,26 +669,33 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
         if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
         return "q6_k_gemm_mfma_m256";
     }
-    dim3 grid((a.n + kBN - 1) / kBN, (a.m + kBM - 1) / kBM);
+    // 128 x 128 tiles, or 64 x 64 when those would leave most of the chip idle
+    const uint64_t big_wgs = (uint64_t)((a.n + kBN - 1) / kBN) * ((a.m + kBM - 1) / kBM);
+    const bool small = big_wgs * 2 < (uint64_t)a.cu_count;
+    const uint32_t ts = small ? 64 : 128;
+    dim3 grid((a.n + ts - 1) / ts, (a.m + ts - 1) / ts);
     const uint32_t nb = a.k / 256;
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
+    auto run = [&](auto big, auto little) {
+        if (small) {
+            hipLaunchKernelGGL(little, grid, dim3(128), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype);
+        } else {
+            hipLaunchKernelGGL(big, grid, dim3(256), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype);
+        }
+    };
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) {
-            hipLaunchKernelGGL((gemm_tile_kernel<kQ4K, 1>), grid, dim3(kThreads), 0, s, w, x, a.y, a.m,
-                               a.n, nb, a.y_dtype);
+            run(gemm_tile_kernel<kQ4K, 1, 128>, gemm_tile_kernel<kQ4K, 1, 64>);
         } else {
-            hipLaunchKernelGGL((gemm_tile_kernel<kQ4K, 2>), grid, dim3(kThreads), 0, s, w, x, a.y, a.m,
-                               a.n, nb, a.y_dtype);
+            run(gemm_tile_kernel<kQ4K, 2, 128>, gemm_tile_kernel<kQ4K, 2, 64>);
         }
         return "q4_k_gemm_mfma";
     }
     if (a.x_dtype == FH_F16) {
-        hipLaunchKernelGGL((gemm_tile_kernel<kQ6K, 1>), grid, dim3(kThreads), 0, s, w, x, a.y, a.m, a.n,
-                           nb, a.y_dtype);
+        run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>);
     } else {
-        hipLaunchKernelGGL((gemm_tile_kernel<kQ6K, 2>), grid, dim3(kThreads), 0, s, w, x, a.y, a.m, a.n,
-                           nb, a.y_dtype);
+        run(gemm_tile_kernel<kQ6K, 2, 128>, gemm_tile_kernel<kQ6K, 2, 64>);
     }
     return "q6_k_gemm_mfma";
 }

@@ -194,6 +194,27 @@ def test_bf16_tile_gemm_covers_row_output_and_group_tails(api, d):
             assert np.abs(out.tensor.to_f32() - expected).max() <= tol, (ggml, m)
 
 
+@pytest.mark.parametrize("ggml,dtype_name", [(Q4_K, "F16"), (Q6_K, "BF16")])
+def test_tile_gemm_both_tile_sizes_match_the_f16_tile_oracle(api, d, ggml, dtype_name):
+    # M = 130 rows: N = 16000 takes 128 x 128 tiles (250 workgroups), N = 1000 takes
+    # 64 x 64 tiles; both have ragged last tiles in M and N.  Oracle on sampled columns.
+    k, m = 512, 130
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    x = oracle.round_storage(synth.activations(m, k, seed=91), code).reshape(m, k)
+    xt = api.Tensor.from_f32(d, x.shape, dtype, x)
+    for n in (16000, 1000):
+        packed = synth.matrix(ggml, n, k, seed=92 + n)
+        w = qm(api, d, ggml, n, k, packed)
+        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        assert out.operation == ("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
+        got = out.tensor.to_f32()
+        rows = np.unique(np.concatenate([np.arange(0, 130), np.arange(n - 70, n),
+                                         synth.rng(93).integers(0, n, 64)]))
+        want = oracle_columns(ggml, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+        assert_matmul_parity(got[:, rows], want, f"tile gemm n={n}")
+
+
 # ------------------------------------------------------- benchmark shapes
 
 def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):

@@ -111,6 +111,29 @@ fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
     return FH_OK;
 }
 
+// Frees device memory now, or after the recording in progress has ended.
+void release_memory(fh_device* d, void* ptr) {
+    if (ptr == nullptr) return;
+    if (d != nullptr && d->capturing) {
+        d->deferred_frees.push_back(ptr);
+        return;
+    }
+    if (d != nullptr) (void)hipStreamSynchronize(d->stream);
+    (void)hipFree(ptr);
+}
+
+void drain_deferred(fh_device* d) {
+    if (d->deferred_frees.empty() && d->deferred_graphs.empty()) return;
+    (void)hipStreamSynchronize(d->stream);
+    for (void* ptr : d->deferred_frees) (void)hipFree(ptr);
+    for (auto& g : d->deferred_graphs) {
+        (void)hipGraphExecDestroy(g.first);
+        (void)hipGraphDestroy(g.second);
+    }
+    d->deferred_frees.clear();
+    d->deferred_graphs.clear();
+}
+
 int64_t tuning(const fh_device* d, const char* key) {
     auto it = d->tuning.find(key);
     return it == d->tuning.end() ? 0 : it->second;
@@ -177,6 +200,7 @@ void fh_device_destroy(fh_device* device) {
         (void)hipStreamSynchronize(device->stream);
         (void)hipStreamDestroy(device->stream);
     }
+    drain_deferred(device);
     if (device->scratch) (void)hipFree(device->scratch);
     delete device;
 }
@@ -273,8 +297,7 @@ fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out) {
 
 void fh_buffer_free(fh_buffer* buffer) {
     if (buffer == nullptr) return;
-    if (buffer->device) (void)hipStreamSynchronize(buffer->device->stream);
-    (void)hipFree(buffer->ptr);
+    release_memory(buffer->device, buffer->ptr);
     delete buffer;
 }
 
@@ -386,8 +409,7 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
 
 void fh_qmatrix_destroy(fh_qmatrix* matrix) {
     if (matrix == nullptr) return;
-    if (matrix->device) (void)hipStreamSynchronize(matrix->device->stream);
-    (void)hipFree(matrix->ptr);
+    release_memory(matrix->device, matrix->ptr);
     delete matrix;
 }
 
@@ -724,7 +746,9 @@ fh_status fh_execution_end(fh_device* device, fh_graph** out) {
     if (!device->capturing) return fail(FH_ERR_DISPATCH, "no execution is being recorded");
     device->capturing = false;
     hipGraph_t graph = nullptr;
-    FH_HIP(hipStreamEndCapture(device->stream, &graph));
+    const hipError_t ended = hipStreamEndCapture(device->stream, &graph);
+    drain_deferred(device);
+    if (ended != hipSuccess) return hip_fail(ended, "hipStreamEndCapture");
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
@@ -753,9 +777,13 @@ fh_status fh_graph_launch(fh_graph* graph) {
 
 void fh_graph_destroy(fh_graph* graph) {
     if (graph == nullptr) return;
-    (void)hipStreamSynchronize(graph->device->stream);
-    (void)hipGraphExecDestroy(graph->exec);
-    (void)hipGraphDestroy(graph->graph);
+    if (graph->device->capturing) {
+        graph->device->deferred_graphs.emplace_back(graph->exec, graph->graph);
+    } else {
+        (void)hipStreamSynchronize(graph->device->stream);
+        (void)hipGraphExecDestroy(graph->exec);
+        (void)hipGraphDestroy(graph->graph);
+    }
     delete graph;
 }
 

@@ -7,6 +7,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <map>
+#include <utility>
+#include <vector>
 #include <string>
 
 #include "../../include/ferrum_hip.h"
@@ -22,6 +24,10 @@ struct fh_device {
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
     static constexpr size_t kCounterWords = 1u << 16;
+    // Releases asked for while an execution is being recorded wait for its end:
+    // freeing or synchronizing inside a stream capture would invalidate it.
+    std::vector<void*> deferred_frees;
+    std::vector<std::pair<hipGraphExec_t, hipGraph_t>> deferred_graphs;
 };
 
 struct fh_buffer {

@@ -84,8 +84,24 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
         float normalizer = 0.f;
         if (lane == 0) {
             // expert order, four per LDS read; the zero padding does not change the sum
-            for (uint32_t e = 0; e < experts; e += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(scores_lds + e);
+            // the reads of a batch are issued together; the additions stay in expert order
+            const float4* in = reinterpret_cast<const float4*>(scores_lds);
+            const uint32_t quads = (experts + 3u) / 4u;
+            uint32_t q = 0;
+            for (; q + 8 <= quads; q += 8) {
+                float4 v[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = in[q + i];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    normalizer += v[i].x;
+                    normalizer += v[i].y;
+                    normalizer += v[i].z;
+                    normalizer += v[i].w;
+                }
+            }
+            for (; q < quads; ++q) {
+                const float4 v = in[q];
                 normalizer += v.x;
                 normalizer += v.y;
                 normalizer += v.z;

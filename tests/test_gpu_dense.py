@@ -314,3 +314,54 @@ def test_quantized_matrix_validation(api, d):
         api.QuantizationFormat.from_ggml_type(5)
     assert api.QuantizationFormat.from_ggml_type(12).block_bytes() == 144
     assert api.QuantizationFormat.from_ggml_type(14).block_bytes() == 210
+
+
+# ------------------------------------------------------------ executions
+
+def test_recorded_execution_replays_bitwise_with_eager_work_in_between(api, d):
+    # Execution (src/metal/mod.rs:263-278): calls recorded once, replayed many times
+    n, k = 1024, 2048
+    w = qm(api, d, Q4_K, n, k, synth.matrix(Q4_K, n, k, seed=101))
+    x = api.Tensor.from_f32(d, (1, k), api.DType.F32, synth.activations(1, k, seed=102))
+    x8 = api.Tensor.from_f32(d, (8, k), api.DType.F16, synth.activations(8, k, seed=103, f16=True))
+    y, y8 = api.Tensor.zeros(d, (1, n), api.DType.F32), api.Tensor.zeros(d, (8, n), api.DType.F32)
+    eager = d.project_quantized(x, w).tensor.raw()
+    eager8 = d.project_quantized(x8, w, out_dtype=api.DType.F32).tensor.raw()
+    with d.execution() as ex:
+        d.project_quantized(x, w, out=y)
+        d.project_quantized(x8, w, out=y8)
+        with pytest.raises(api.Error):
+            api.Tensor.zeros(d, (4,), api.DType.F32)          # allocation is refused while recording
+        with pytest.raises(api.Error):
+            y.to_f32()                                         # so is a download
+    for _ in range(3):
+        ex.graph.launch()
+        assert np.array_equal(y.raw(), eager) and np.array_equal(y8.raw(), eager8)
+        y.buffer.upload(0, np.zeros(n, np.float32))            # eager work between the replays
+        d.project_quantized(x8, w)
+        d.synchronize()
+
+
+def test_releases_asked_for_while_recording_wait_for_its_end(api, d):
+    import gc
+    n, k = 512, 1024
+    packed = synth.matrix(Q4_K, n, k, seed=111)
+    w = qm(api, d, Q4_K, n, k, packed)
+    x = api.Tensor.from_f32(d, (1, k), api.DType.F32, synth.activations(1, k, seed=112))
+    y = api.Tensor.zeros(d, (1, n), api.DType.F32)
+    want = d.project_quantized(x, w).tensor.raw()
+    with d.execution() as old:
+        d.project_quantized(x, w, out=y)
+    old.graph.launch()
+    spare_w = qm(api, d, Q4_K, n, k, packed)
+    spare_t = api.Tensor.zeros(d, (64, 64), api.DType.F32)
+    with d.execution() as ex:
+        d.project_quantized(x, w, out=y)
+        # dropping a graph, a matrix and a tensor here must not disturb the recording
+        del old, spare_w, spare_t
+        gc.collect()
+        d.project_quantized(x, w, out=y)
+    y.buffer.upload(0, np.zeros(n, np.float32))
+    ex.graph.launch()
+    assert np.array_equal(y.raw(), want)
+    assert np.array_equal(d.project_quantized(x, w).tensor.raw(), want)

@@ -35,9 +35,9 @@ BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
 ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
 
 # HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
-# FETCH_SIZE 24691.6 KiB x 1.94486 + WRITE_SIZE 68.0 KiB x 1.0, the factors being
+# FETCH_SIZE 24723.1 KiB x 1.94485 + WRITE_SIZE 68.0 KiB x 1.0, the factors being
 # known bytes / counter reading for the row-copy kernel of `--cases copy`.
-MEASURED_TRAFFIC_BYTES = 49243760
+MEASURED_TRAFFIC_BYTES = 49306489
 
 
 def algorithmic_bytes(ggml, n, k, m, x_size, y_size):

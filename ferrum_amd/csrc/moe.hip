@@ -294,13 +294,25 @@ __global__ __launch_bounds__(256) void expert_combine8_kernel(const void* __rest
          i += (size_t)gridDim.x * blockDim.x) {
         const size_t token = (i * 8) / hidden, column = (i * 8) % hidden;
         float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (uint32_t rank = 0; rank < top_k; ++rank) {
-            const size_t a = token * top_k + rank;
-            const float gate = round_storage(metadata[a * 3 + 2], out_dtype);
-            float value[8];
-            load8(in, a * hidden + column, in_dtype, value);
+        // eight ranks at a time: their loads are issued together (one memory
+        // latency instead of eight), the additions stay in rank order
+        for (uint32_t rank0 = 0; rank0 < top_k; rank0 += 8) {
+            float gate[8], value[8][8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) sum[j] += round_storage(gate * value[j], out_dtype);
+            for (int r = 0; r < 8; ++r) {
+                const uint32_t rank = rank0 + r < top_k ? rank0 + r : top_k - 1;
+                const size_t a = token * top_k + rank;
+                gate[r] = metadata[a * 3 + 2];
+                load8(in, a * hidden + column, in_dtype, value[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                if (rank0 + r < top_k) {
+                    const float weight = round_storage(gate[r], out_dtype);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) sum[j] += round_storage(weight * value[r][j], out_dtype);
+                }
+            }
         }
         store8(out, i * 8, out_dtype, sum);
     }

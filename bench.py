@@ -331,6 +331,10 @@ def main():
         for m in (8, 16, 128):
             timed(Q4_K, 17408, 5120, m, f16, f"Q4_K GEMM M={m} K=5120 N=17408 f16 x", 240)
         gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
+        if not args.only or args.only in "Q4_K GEMM M=512 K=5120 N=17408 f32 x":
+            dev.set_tuning("gemm_f32_min_rows", 5)   # the hybrid engine's tiering: f16 tiles from 5 rows on
+            timed(Q4_K, 17408, 5120, 512, f32, "Q4_K GEMM M=512 K=5120 N=17408 f32 x (rounded to f16 for the tiles)", 120)
+            dev.set_tuning("gemm_f32_min_rows", 0)
         if not args.only or args.only in "MoE FFN T=1":
             cases.append(moe_case(api, synth, dev, 1, 200))
         if not args.only or args.only in "MoE FFN T=512":

@@ -183,6 +183,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 32; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
+    d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
         (void)hipStreamDestroy(d->stream);
@@ -252,6 +253,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 0 && value <= 32;
     } else if (k == "expert_grouped_min_assignments") {
         ok = value >= 0;
+    } else if (k == "gemm_f32_min_rows") {
+        ok = value == 0 || value >= 2;
     }
     if (!ok) return fail(FH_ERR_PARAMETER, "value %lld is out of range for %s", (long long)value, key);
     it->second = value;
@@ -487,17 +490,32 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
     if (st != FH_OK) return st;
     if (overlaps(xr, yr)) return fail(FH_ERR_RANGE, "projection output aliases its input");
 
-    const bool tile = !silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32;
+    // f32 activations stay on exact f32 weights (the GEMV kernel, once per row) unless the
+    // caller asks for the tile kernels from some row count on, as the reference's hybrid
+    // engine does from 5 rows (HybridModel::project, src/hybrid/engine.rs:3407-3500): the
+    // activations are then rounded to f16 into the device scratch first.
+    const int64_t f32_tile_rows = tuning(device, "gemm_f32_min_rows");
+    const bool f32_tile = !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
+                          ((uintptr_t)xr.begin & 15u) == 0;
+    const void* tile_x = xr.begin;
+    if (f32_tile) {
+        st = ensure_scratch(device, (size_t)m * k * sizeof(uint16_t));
+        if (st != FH_OK) return st;
+        launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin),
+                            reinterpret_cast<uint16_t*>(scratch_data(device)), (size_t)m * k);
+        tile_x = scratch_data(device);
+    }
+    const bool tile = f32_tile || (!silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32);
     if (tile) {
         GemmArgs a{};
         a.ggml_type = weight->ggml_type;
         a.w = weight->ptr;
-        a.x = xr.begin;
+        a.x = tile_x;
         a.y = const_cast<uint8_t*>(yr.begin);
         a.n = (uint32_t)n;
         a.k = (uint32_t)k;
         a.m = m;
-        a.x_dtype = x->dtype;
+        a.x_dtype = f32_tile ? FH_F16 : x->dtype;
         a.y_dtype = y->dtype;
         a.cu_count = device->props.multiProcessorCount;
         a.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");

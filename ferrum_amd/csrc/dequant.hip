@@ -115,4 +115,31 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
     return "embedding_gather_q6_k";
 }
 
+namespace {
+
+__global__ __launch_bounds__(256) void round_to_f16_kernel(const float4* __restrict__ in, uint4* __restrict__ out,
+                                                           size_t groups) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < groups;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const float4 a = in[2 * i], b = in[2 * i + 1];
+        uint4 v;
+        v.x = f32_to_f16_bits(a.x) | (f32_to_f16_bits(a.y) << 16);
+        v.y = f32_to_f16_bits(a.z) | (f32_to_f16_bits(a.w) << 16);
+        v.z = f32_to_f16_bits(b.x) | (f32_to_f16_bits(b.y) << 16);
+        v.w = f32_to_f16_bits(b.z) | (f32_to_f16_bits(b.w) << 16);
+        out[i] = v;
+    }
+}
+
+}  // namespace
+
+void launch_round_to_f16(hipStream_t s, const float* in, uint16_t* out, size_t count) {
+    const size_t groups = count / 8;
+    size_t blocks = (groups + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(round_to_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                       reinterpret_cast<const float4*>(in), reinterpret_cast<uint4*>(out), groups);
+}
+
 }  // namespace fh

@@ -73,6 +73,8 @@ inline size_t dtype_bytes(uint32_t dtype) { return dtype == FH_F32 ? 4 : 2; }
 // ---- launchers (one per kernel family); each returns the kernel name ----
 
 // dequant.hip
+// f32 -> f16 (round to nearest even), `count` a multiple of 8: activations on their way to the tile kernels
+void launch_round_to_f16(hipStream_t s, const float* in, uint16_t* out, size_t count);
 const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, size_t rows,
                               size_t cols, void* out, uint32_t out_dtype);
 const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const void* w, size_t cols,

@@ -215,6 +215,38 @@ def test_tile_gemm_both_tile_sizes_match_the_f16_tile_oracle(api, d, ggml, dtype
         assert_matmul_parity(got[:, rows], want, f"tile gemm n={n}")
 
 
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_f32_activations_take_the_tile_kernels_from_a_chosen_row_count(api, d, ggml):
+    # HybridModel::project (src/hybrid/engine.rs:3407-3500) sends f32 activations to f16
+    # tiles from 5 rows on; here that is opt-in, and below the threshold (or with the key at
+    # 0) every row keeps exact f32 weights.
+    n, k = 1100, 1024
+    packed = synth.matrix(ggml, n, k, seed=121)
+    w = qm(api, d, ggml, n, k, packed)
+    d.set_tuning("gemm_f32_min_rows", 5)
+    try:
+        for m in (4, 5, 16, 40, 130):
+            x = synth.activations(m, k, seed=122 + m)
+            out = d.project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x), w)
+            assert out.tensor.dtype == api.DType.F32
+            if m < 5:
+                assert out.operation.endswith("_gemm") and "mfma" not in out.operation
+                want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
+            else:
+                assert "gemm_mfma" in out.operation
+                want = oracle.project(ggml, packed, n, k, oracle.round_storage(x, oracle.F16).reshape(m, k),
+                                      weight_round=oracle.F16, accumulate="f64")
+            assert_matmul_parity(out.tensor.to_f32(), want, f"f32 activations m={m}")
+    finally:
+        d.set_tuning("gemm_f32_min_rows", 0)
+    x = synth.activations(16, k, seed=123)
+    exact = d.project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x), w)
+    assert "mfma" not in exact.operation
+    assert_matmul_parity(exact.tensor.to_f32(), oracle.project(ggml, packed, n, k, x, accumulate="f64"), "exact f32")
+    with pytest.raises(api.ParameterError):
+        d.set_tuning("gemm_f32_min_rows", 1)
+
+
 # ------------------------------------------------------- benchmark shapes
 
 def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):

@@ -112,6 +112,7 @@ SYMBOLS = {
     "fh_dequantize": (_I32, [_P, _P, _VP]),
     "fh_embedding_gather_quantized": (_I32, [_P, _P, ctypes.POINTER(_U32), _SZ, _VP]),
     "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
+    "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
     "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
@@ -574,6 +575,19 @@ class Device:
         call = _lib.fh_project_silu_mul_quantized if silu_mul else _lib.fh_project_quantized
         _check(call(self._handle, _handle_of(weight), ctypes.byref(xv), m, ctypes.byref(yv)))
         return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
+
+    def argmax_rows(self, logits: Tensor) -> Tensor:
+        """[rows, 2] F32 carrier of u32 bits: first maximal index and a non-finite flag
+        (MetalDevice::argmax_rows, src/ops/transformer.rs:768-792)."""
+        dims = logits.shape()
+        if len(dims) != 2 or 0 in dims or dims[1] > 0xFFFFFFFF:
+            raise ShapeError("argmax requires nonempty [rows,width]")
+        if logits.buffer.device is not self:
+            raise DeviceMismatch("tensor belongs to another device")
+        out = Tensor.zeros(self, (dims[0], 2), DType.F32)
+        lv, ov = logits._view(), out._view()
+        _check(_lib.fh_argmax_rows(self._handle, ctypes.byref(lv), dims[0], dims[1], ctypes.byref(ov)))
+        return out
 
     def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy,
                   out: Tensor | None = None) -> Tensor:

@@ -561,6 +561,24 @@ fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* wei
 
 // ---- mixture of experts -------------------------------------------------------------
 
+fh_status fh_argmax_rows(fh_device* device, const fh_view* logits, uint32_t rows, uint32_t width,
+                         const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (rows == 0 || width == 0 || !fits_u32((uint64_t)rows * width))
+        return fail(FH_ERR_SHAPE, "argmax requires nonempty [rows,width]");
+    if (out == nullptr || out->dtype != FH_F32) return fail(FH_ERR_DTYPE, "argmax output is an f32 carrier of [rows,2]");
+    Range lr, orr;
+    fh_status st = resolve(device, logits, (uint64_t)rows * width, "argmax input", &lr);
+    if (st != FH_OK) return st;
+    st = resolve(device, out, (uint64_t)rows * 2, "argmax output", &orr, 4);
+    if (st != FH_OK) return st;
+    if (overlaps(lr, orr)) return fail(FH_ERR_RANGE, "argmax output aliases its input");
+    device->last_operation = launch_argmax_rows(device->stream, lr.begin, logits->dtype, rows, width,
+                                                reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(orr.begin)));
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
                        const fh_view* selection_bias, const fh_routing_policy* policy,
                        const fh_view* metadata) {

@@ -133,6 +133,64 @@ __global__ __launch_bounds__(256) void round_to_f16_kernel(const float4* __restr
 
 }  // namespace
 
+namespace {
+
+// argmax_rows (src/metal/shaders/ops.metal:2438-2464) with the reference's own
+// schedule, so rows that hold NaN report the same (flagged) index: 1024
+// threads per row scan columns tid, tid + 1024, ...; groups of 32 lanes merge
+// by a shuffle-down tree; thread 0 folds the 32 group results in order.
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const void* __restrict__ logits, uint32_t dtype,
+                                                           uint32_t width, uint32_t* __restrict__ out) {
+    __shared__ float best_value[32];
+    __shared__ uint32_t best_index[32], bad_any[32];
+    const uint32_t tid = threadIdx.x, row = blockIdx.x;
+    const size_t base = (size_t)row * width;
+    float best = -INFINITY;
+    uint32_t index = 0xffffffffu, bad = 0;
+    for (uint32_t j = tid; j < width; j += 1024) {
+        const float x = load_as_f32(logits, base + j, dtype);
+        bad |= (uint32_t)!isfinite(x);
+        if (x > best || index == 0xffffffffu) {
+            best = x;
+            index = j;
+        }
+    }
+    for (uint32_t offset = 16; offset > 0; offset /= 2) {
+        const float other = __shfl_down(best, offset, 32);
+        const uint32_t other_index = __shfl_down(index, offset, 32);
+        if (other > best || (other == best && other_index < index)) {
+            best = other;
+            index = other_index;
+        }
+    }
+    for (uint32_t offset = 16; offset > 0; offset /= 2) bad |= __shfl_xor(bad, offset, 32);
+    if ((tid & 31u) == 0) {
+        best_value[tid >> 5] = best;
+        best_index[tid >> 5] = index;
+        bad_any[tid >> 5] = bad;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (uint32_t s = 1; s < 32; ++s) {
+            if (best_value[s] > best || (best_value[s] == best && best_index[s] < index)) {
+                best = best_value[s];
+                index = best_index[s];
+            }
+            bad |= bad_any[s];
+        }
+        out[2 * (size_t)row] = index;
+        out[2 * (size_t)row + 1] = bad;
+    }
+}
+
+}  // namespace
+
+const char* launch_argmax_rows(hipStream_t s, const void* logits, uint32_t dtype, uint32_t rows, uint32_t width,
+                               uint32_t* out) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(1024), 0, s, logits, dtype, width, out);
+    return "argmax_rows";
+}
+
 void launch_round_to_f16(hipStream_t s, const float* in, uint16_t* out, size_t count) {
     const size_t groups = count / 8;
     size_t blocks = (groups + 255) / 256;

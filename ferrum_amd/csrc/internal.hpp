@@ -74,6 +74,8 @@ inline size_t dtype_bytes(uint32_t dtype) { return dtype == FH_F32 ? 4 : 2; }
 
 // dequant.hip
 // f32 -> f16 (round to nearest even), `count` a multiple of 8: activations on their way to the tile kernels
+const char* launch_argmax_rows(hipStream_t s, const void* logits, uint32_t dtype, uint32_t rows, uint32_t width,
+                               uint32_t* out);
 void launch_round_to_f16(hipStream_t s, const float* in, uint16_t* out, size_t count);
 const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, size_t rows,
                               size_t cols, void* out, uint32_t out_dtype);

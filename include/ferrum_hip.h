@@ -164,6 +164,14 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
 fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
                                uint32_t m, const fh_view* y);
 
+/* MetalDevice::argmax_rows (src/ops/transformer.rs:768-792, kernel
+ * src/metal/shaders/ops.metal:2438-2464): greedy selection over the rows of a
+ * logits matrix, the step after the lm_head projection.  out is an f32 carrier
+ * [rows, 2] holding u32 bits: the first maximal index of the row and a flag
+ * that is 1 when the row holds a non-finite value. */
+fh_status fh_argmax_rows(fh_device* device, const fh_view* logits, uint32_t rows, uint32_t width,
+                         const fh_view* out);
+
 /* ---- mixture of experts -----------------------------------------------------
  * MetalDevice::moe_route (src/ops/mod.rs:23-73; kernel ops.metal:1894-1957).
  * logits [tokens, experts]; bias (may be NULL) [experts] f32; metadata

@@ -336,6 +336,17 @@ public:
         check(fh_project_quantized(handle_->raw, w.raw(), &xv, (uint32_t)dims[0], &yv));
         return {y, {last_operation(), a.byte_size() + w.byte_size(), y.byte_size()}};
     }
+    // [rows, 2] F32 carrier of u32 bits: first maximal index and a non-finite flag.
+    Tensor argmax_rows(const Tensor& logits) const {
+        const auto& dims = logits.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] == 0 || dims[1] > 0xffffffffull)
+            throw Error(ErrorKind::Shape, "argmax requires nonempty [rows,width]");
+        if (!owns(logits)) throw Error(ErrorKind::DeviceMismatch, "tensor belongs to another device");
+        Tensor out = zeros({dims[0], 2}, DType::F32);
+        fh_view lv = logits.c_view(), ov = out.c_view();
+        check(fh_argmax_rows(handle_->raw, &lv, (uint32_t)dims[0], (uint32_t)dims[1], &ov));
+        return out;
+    }
     Tensor moe_route(const Tensor& logits, const Tensor* selection_bias, const MoeRoutingPolicy& policy,
                      const Tensor* out = nullptr) const {
         const auto& dims = logits.shape();

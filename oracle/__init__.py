@@ -67,6 +67,8 @@ def _load() -> ctypes.CDLL:
     lib.fo_expert_project.argtypes = [u32, u8p, sz, sz, sz, f32p, f32p, sz, f32p, i32, i32, i32]
     lib.fo_expert_silu_mul.restype = None
     lib.fo_expert_silu_mul.argtypes = [f32p, sz, sz, u32, f32p]
+    lib.fo_argmax_rows.restype = None
+    lib.fo_argmax_rows.argtypes = [f32p, sz, sz, ctypes.POINTER(ctypes.c_uint32)]
     lib.fo_expert_combine.restype = None
     lib.fo_expert_combine.argtypes = [f32p, f32p, sz, sz, sz, u32, f32p]
     return lib
@@ -205,6 +207,15 @@ def expert_silu_mul(packed_rows, intermediate: int, dtype: int = F32) -> np.ndar
     a = np.ascontiguousarray(packed_rows, dtype=np.float32).reshape(-1, 2 * intermediate)
     out = np.empty((a.shape[0], intermediate), dtype=np.float32)
     _lib.fo_expert_silu_mul(_f32(a), a.shape[0], intermediate, dtype, _f32(out))
+    return out
+
+
+def argmax_rows(logits) -> np.ndarray:
+    """[rows, 2] uint32: first maximal index and a non-finite flag (argmax_rows,
+    src/metal/shaders/ops.metal:2438-2464)."""
+    a = np.ascontiguousarray(logits, dtype=np.float32)
+    out = np.empty((a.shape[0], 2), dtype=np.uint32)
+    _lib.fo_argmax_rows(_f32(a), a.shape[0], a.shape[1], out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
     return out
 
 

@@ -566,3 +566,58 @@ void fo_expert_combine(const float* in, const float* metadata, size_t tokens, si
         }
     }
 }
+
+/* argmax_rows (src/metal/shaders/ops.metal:2438-2464), restated with its own
+ * schedule so that rows holding NaN give the same (flagged) index: 1024
+ * threads scan columns tid, tid + 1024, ...; groups of 32 threads merge by a
+ * shuffle-down tree; thread 0 folds the 32 group results in order.  A later
+ * candidate wins when it is greater, or equal with a lower index.  out[2*row]
+ * = index, out[2*row + 1] = 1 when the row holds a non-finite value.  For
+ * finite rows this is the first maximal index. */
+void fo_argmax_rows(const float* logits, size_t rows, size_t width, uint32_t* out) {
+    enum { THREADS = 1024, GROUP = 32 };
+    static float best[THREADS];
+    static uint32_t index[THREADS];
+    for (size_t row = 0; row < rows; row++) {
+        const float* x = logits + row * width;
+        uint32_t bad = 0;
+        for (uint32_t tid = 0; tid < THREADS; tid++) {
+            best[tid] = -INFINITY;
+            index[tid] = 0xffffffffu;
+            for (size_t j = tid; j < width; j += THREADS) {
+                float v = x[j];
+                if (!isfinite(v)) bad = 1;
+                if (v > best[tid] || index[tid] == 0xffffffffu) {
+                    best[tid] = v;
+                    index[tid] = (uint32_t)j;
+                }
+            }
+        }
+        for (uint32_t offset = GROUP / 2; offset > 0; offset /= 2) {
+            /* shuffle_down reads the pre-step value of lane + offset; ascending tid
+             * only ever reads lanes not yet rewritten in this step */
+            for (uint32_t tid = 0; tid < THREADS; tid++) {
+                uint32_t lane = tid % GROUP;
+                uint32_t from = lane + offset < GROUP ? tid + offset : tid;
+                float other = best[from];
+                uint32_t other_index = index[from];
+                if (other > best[tid] || (other == best[tid] && other_index < index[tid])) {
+                    best[tid] = other;
+                    index[tid] = other_index;
+                }
+            }
+        }
+        float b = best[0];
+        uint32_t bi = index[0];
+        for (uint32_t g = 1; g < THREADS / GROUP; g++) {
+            float v = best[g * GROUP];
+            uint32_t vi = index[g * GROUP];
+            if (v > b || (v == b && vi < bi)) {
+                b = v;
+                bi = vi;
+            }
+        }
+        out[2 * row] = bi;
+        out[2 * row + 1] = bad;
+    }
+}

@@ -397,3 +397,41 @@ def test_releases_asked_for_while_recording_wait_for_its_end(api, d):
     ex.graph.launch()
     assert np.array_equal(y.raw(), want)
     assert np.array_equal(d.project_quantized(x, w).tensor.raw(), want)
+
+
+# ------------------------------------------------------------- greedy selection
+
+@pytest.mark.parametrize("dtype_name", ["F32", "F16", "BF16"])
+def test_argmax_rows_matches_the_oracle(api, d, dtype_name):
+    dtype = api.DType[dtype_name]
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype_name]
+    rng = synth.rng(131)
+    for rows, width in ((1, 1), (3, 33), (4, 1024), (5, 4099), (2, 151936)):
+        x = oracle.round_storage(rng.standard_normal((rows, width)).astype(np.float32), code).reshape(rows, width)
+        if width > 40:
+            x[0, 5] = x[0, width - 3] = 9.0
+            if rows > 2:
+                x[1, 9] = np.inf
+                x[2, 0] = np.nan
+            if rows > 3:
+                x[3, 2047 % width] = np.nan
+        got = d.argmax_rows(api.Tensor.from_f32(d, x.shape, dtype, x))
+        assert d.last_operation() == "argmax_rows"
+        want = oracle.argmax_rows(x)
+        assert np.array_equal(got.raw().view(np.uint32).reshape(rows, 2), want), (rows, width)
+    with pytest.raises(api.ShapeError):
+        d.argmax_rows(api.Tensor.zeros(d, (4,), dtype))
+
+
+def test_lm_head_projection_then_argmax_picks_the_oracle_token(api, d):
+    n, k = 4096, 1024
+    packed = synth.matrix(Q6_K, n, k, seed=141)
+    w = qm(api, d, Q6_K, n, k, packed)
+    x = synth.activations(1, k, seed=142)
+    logits = d.project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x), w).tensor
+    picked = d.argmax_rows(logits).raw().view(np.uint32)
+    want = oracle.project(Q6_K, packed, n, k, x, accumulate="f64")
+    assert picked[1] == 0 and picked[0] == int(np.argmax(logits.to_f32()))
+    top2 = np.sort(want[0])[-2:]
+    if top2[1] - top2[0] > 1e-3 * abs(top2[1]):      # unambiguous in the oracle too
+        assert picked[0] == int(np.argmax(want))

@@ -501,3 +501,27 @@ def test_storage_rounding_points_of_silu_mul_and_combine():
     r = lambda v: oracle.round_storage([v], oracle.BF16)[0]
     want = r(F(r(F(r(meta[0, 2]) * vals[0, 0])) + r(F(r(meta[1, 2]) * vals[1, 0]))))
     assert got == want
+
+
+def test_argmax_rows_is_the_first_maximal_index_and_flags_non_finite_rows():
+    # numpy's argmax (first occurrence of the maximum) pins the finite case; the
+    # flagged cases follow the reference kernel's own scan and merge order
+    rng = np.random.default_rng(17)
+    for width in (1, 31, 1024, 1025, 5000):
+        x = rng.standard_normal((6, width)).astype(np.float32)
+        if width > 40:
+            x[1, 5] = x[1, width - 3] = 9.0       # a tie: the lower index wins
+            x[2, 7] = -np.inf                     # non-finite but not maximal
+            x[3, 11] = np.inf
+        got = oracle.argmax_rows(x)
+        assert np.array_equal(got[:, 0], x.argmax(axis=1).astype(np.uint32)), width
+        assert np.array_equal(got[:, 1], (~np.isfinite(x)).any(axis=1).astype(np.uint32))
+    x = rng.standard_normal((3, 3000)).astype(np.float32)
+    x[0, 0] = np.nan        # thread 0 starts on NaN and never leaves it
+    x[1, 2047] = np.nan     # a NaN later in a thread's scan is skipped
+    x[2, :] = np.nan
+    got = oracle.argmax_rows(x)
+    assert got[:, 1].tolist() == [1, 1, 1]
+    assert got[0, 0] == 0 and got[2, 0] == 0
+    y = x[1].copy(); y[2047] = -np.inf
+    assert got[1, 0] == y.argmax()

@@ -114,6 +114,8 @@ SYMBOLS = {
     "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
+    "fh_moe_route_ranked": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP]),
+    "fh_expert_combine_shared": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
     "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
     "fh_expert_project_fused": (_I32, [_P, _P, _VP, _U32, _U32, _U32, _VP, _VP]),
@@ -604,6 +606,48 @@ class Device:
         _check(_lib.fh_moe_route(self._handle, ctypes.byref(lv), dims[0],
                                  ctypes.byref(bv) if bv is not None else None, ctypes.byref(pc),
                                  ctypes.byref(ov)))
+        return out
+
+    def moe_route_ranked(self, logits: Tensor, policy: MoeRoutingPolicy, x: Tensor | None = None,
+                         gate_vector: Tensor | None = None, want_gate: bool = False):
+        """The hybrid engine's router (h_moe_route, src/metal/shaders/hybrid.metal:2259-2319):
+        metadata rows in selection order, and the shared-expert gate
+        sigmoid(dot(x[t], gate_vector)) per token (ones without a vector).
+        Returns (metadata, shared_gate or None)."""
+        dims = logits.shape()
+        if len(dims) != 2 or dims[0] == 0 or dims[1] != policy.experts:
+            raise ShapeError("invalid sparse routing geometry")
+        if gate_vector is not None and (x is None or x.shape() != (dims[0], gate_vector.shape()[0])
+                                        or gate_vector.dtype != DType.F32):
+            raise ShapeError("the shared-expert gate needs x [tokens, hidden] and an f32 vector [hidden]")
+        meta = Tensor.zeros(self, (dims[0] * policy.top_k, 3), DType.F32)
+        gate = Tensor.zeros(self, (dims[0],), DType.F32) if (want_gate or gate_vector is not None) else None
+        lv, mv, pc = logits._view(), meta._view(), policy._c()
+        xv = x._view() if gate_vector is not None else None
+        wv = gate_vector._view() if gate_vector is not None else None
+        gv = gate._view() if gate is not None else None
+        ref = lambda v: ctypes.byref(v) if v is not None else None
+        _check(_lib.fh_moe_route_ranked(self._handle, ctypes.byref(lv), dims[0], ctypes.byref(pc), ref(xv), ref(wv),
+                                        gate_vector.shape()[0] if gate_vector is not None else 0,
+                                        ctypes.byref(mv), ref(gv)))
+        return meta, gate
+
+    def expert_combine_shared(self, input: Tensor, metadata: Tensor, tokens: int, hidden: int, top_k: int,
+                              shared: Tensor, shared_gate: Tensor | None = None,
+                              out: Tensor | None = None) -> Tensor:
+        """h_moe_combine (hybrid.metal:2374-2388): the weighted sum of the routed rows plus
+        shared_gate[t] * shared[t] (gate 1 when absent)."""
+        if (input.shape() != (tokens * top_k, hidden) or metadata.shape() != (tokens * top_k, 3)
+                or shared.shape() != (tokens, hidden) or shared.dtype != input.dtype
+                or (shared_gate is not None and shared_gate.shape() != (tokens,))):
+            raise ShapeError("expert combine geometry mismatch")
+        if out is None:
+            out = Tensor.zeros(self, (tokens, hidden), input.dtype)
+        iv, mv, sv, ov = input._view(), metadata._view(), shared._view(), out._view()
+        gv = shared_gate._view() if shared_gate is not None else None
+        _check(_lib.fh_expert_combine_shared(self._handle, ctypes.byref(iv), ctypes.byref(mv), tokens, hidden,
+                                             top_k, ctypes.byref(sv),
+                                             ctypes.byref(gv) if gv is not None else None, ctypes.byref(ov)))
         return out
 
     def expert_assign(self, hidden: Tensor, metadata: Tensor, top_k: int,

@@ -579,9 +579,11 @@ fh_status fh_argmax_rows(fh_device* device, const fh_view* logits, uint32_t rows
     return FH_OK;
 }
 
-fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
-                       const fh_view* selection_bias, const fh_routing_policy* policy,
-                       const fh_view* metadata) {
+namespace {
+
+fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const fh_view* selection_bias,
+                const fh_routing_policy* policy, const fh_view* metadata, bool ranked, const fh_view* gate_x,
+                const fh_view* gate_w, uint32_t hidden, const fh_view* shared_gate) {
     if (device == nullptr || policy == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     const fh_routing_policy& p = *policy;
     if (tokens == 0 || p.experts == 0 || p.top_k == 0 || p.top_k > 16 || p.top_k > p.experts ||
@@ -604,11 +606,47 @@ fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens
     st = resolve(device, metadata, (uint64_t)tokens * p.top_k * 3, "routing metadata", &mr, 4);
     if (st != FH_OK) return st;
     if (overlaps(lr, mr)) return fail(FH_ERR_RANGE, "routing metadata aliases the logits");
+    RouteExtras extras;
+    extras.rank_order = ranked ? 1u : 0u;
+    if (shared_gate != nullptr) {
+        if (shared_gate->dtype != FH_F32) return fail(FH_ERR_DTYPE, "the shared-expert gate is f32");
+        Range gr;
+        st = resolve(device, shared_gate, tokens, "shared-expert gate", &gr, 4);
+        if (st != FH_OK) return st;
+        extras.shared_gate = reinterpret_cast<float*>(const_cast<uint8_t*>(gr.begin));
+        if (gate_w != nullptr) {
+            if (gate_w->dtype != FH_F32 || gate_x == nullptr || hidden == 0 || !fits_u32((uint64_t)tokens * hidden))
+                return fail(FH_ERR_SHAPE, "the shared-expert gate needs x [tokens, hidden] and an f32 vector [hidden]");
+            Range xr, wr;
+            st = resolve(device, gate_x, (uint64_t)tokens * hidden, "gate activations", &xr);
+            if (st != FH_OK) return st;
+            st = resolve(device, gate_w, hidden, "gate vector", &wr, 4);
+            if (st != FH_OK) return st;
+            extras.gate_x = xr.begin;
+            extras.gate_x_dtype = gate_x->dtype;
+            extras.gate_w = reinterpret_cast<const float*>(wr.begin);
+            extras.hidden = hidden;
+        }
+    }
     device->last_operation = launch_moe_route(
         device->stream, lr.begin, logits->dtype, reinterpret_cast<const float*>(br.begin),
-        reinterpret_cast<float*>(const_cast<uint8_t*>(mr.begin)), tokens, p);
+        reinterpret_cast<float*>(const_cast<uint8_t*>(mr.begin)), tokens, p, extras);
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
+                       const fh_view* selection_bias, const fh_routing_policy* policy,
+                       const fh_view* metadata) {
+    return route(device, logits, tokens, selection_bias, policy, metadata, false, nullptr, nullptr, 0, nullptr);
+}
+
+fh_status fh_moe_route_ranked(fh_device* device, const fh_view* logits, uint32_t tokens,
+                              const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
+                              uint32_t hidden, const fh_view* metadata, const fh_view* shared_gate) {
+    return route(device, logits, tokens, nullptr, policy, metadata, true, x, gate_vector, hidden, shared_gate);
 }
 
 fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t tokens,
@@ -745,13 +783,15 @@ fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assi
     return FH_OK;
 }
 
-fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
-                            uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out) {
+namespace {
+
+fh_status combine(fh_device* device, const fh_view* in, const fh_view* metadata, uint32_t tokens, uint32_t hidden,
+                  uint32_t top_k, const fh_view* shared, const fh_view* shared_gate, const fh_view* out) {
     if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (top_k == 0 || hidden == 0 || tokens == 0 || metadata == nullptr || metadata->dtype != FH_F32 ||
         !fits_u32((uint64_t)tokens * top_k * hidden))
         return fail(FH_ERR_SHAPE, "expert combine geometry mismatch");
-    Range ir, mr, orr;
+    Range ir, mr, orr, sr{nullptr, 0}, gr{nullptr, 0};
     fh_status st = resolve(device, in, (uint64_t)tokens * top_k * hidden, "combine input", &ir, 4);
     if (st != FH_OK) return st;
     st = resolve(device, metadata, (uint64_t)tokens * top_k * 3, "combine metadata", &mr, 4);
@@ -759,11 +799,37 @@ fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view*
     st = resolve(device, out, (uint64_t)tokens * hidden, "combine output", &orr, 4);
     if (st != FH_OK) return st;
     if (overlaps(ir, orr) || overlaps(mr, orr)) return fail(FH_ERR_RANGE, "combine output aliases an input");
+    if (shared != nullptr) {
+        if (shared->dtype != in->dtype) return fail(FH_ERR_DTYPE, "the shared expert's output has the dtype of the routed rows");
+        st = resolve(device, shared, (uint64_t)tokens * hidden, "shared expert output", &sr, 4);
+        if (st != FH_OK) return st;
+        if (overlaps(sr, orr)) return fail(FH_ERR_RANGE, "combine output aliases an input");
+        if (shared_gate != nullptr) {
+            if (shared_gate->dtype != FH_F32) return fail(FH_ERR_DTYPE, "the shared-expert gate is f32");
+            st = resolve(device, shared_gate, tokens, "shared-expert gate", &gr, 4);
+            if (st != FH_OK) return st;
+        }
+    }
     device->last_operation = launch_expert_combine(
         device->stream, ir.begin, reinterpret_cast<const float*>(mr.begin),
-        const_cast<uint8_t*>(orr.begin), tokens, hidden, top_k, in->dtype, out->dtype);
+        const_cast<uint8_t*>(orr.begin), tokens, hidden, top_k, in->dtype, out->dtype, sr.begin,
+        reinterpret_cast<const float*>(gr.begin));
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
+                            uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out) {
+    return combine(device, in, metadata, tokens, hidden, top_k, nullptr, nullptr, out);
+}
+
+fh_status fh_expert_combine_shared(fh_device* device, const fh_view* in, const fh_view* metadata,
+                                   uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* shared,
+                                   const fh_view* shared_gate, const fh_view* out) {
+    if (shared == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    return combine(device, in, metadata, tokens, hidden, top_k, shared, shared_gate, out);
 }
 
 // ---- batched execution ---------------------------------------------------------------

@@ -139,9 +139,18 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a);
 
 // moe.hip
+// what the hybrid engine's router adds: selection order kept, shared-expert gate
+struct RouteExtras {
+    uint32_t rank_order = 0;
+    const void* gate_x = nullptr;      // [tokens, hidden] activations the gate vector is dotted with
+    uint32_t gate_x_dtype = 0;
+    const float* gate_w = nullptr;     // [hidden], or null: the gate is 1
+    uint32_t hidden = 0;
+    float* shared_gate = nullptr;      // [tokens], or null: no gate output
+};
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
                              const float* bias, float* metadata, uint32_t tokens,
-                             const fh_routing_policy& policy);
+                             const fh_routing_policy& policy, const RouteExtras& extras);
 const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t assignments,
                                 uint32_t experts, uint32_t* offsets, uint32_t* order, void* y,
                                 uint32_t row_bytes);
@@ -151,6 +160,7 @@ const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uin
                                    uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype);
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
                                   uint32_t tokens, uint32_t hidden, uint32_t top_k,
-                                  uint32_t in_dtype, uint32_t out_dtype);
+                                  uint32_t in_dtype, uint32_t out_dtype, const void* shared,
+                                  const float* shared_gate);
 
 }  // namespace fh

@@ -54,7 +54,10 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
                                                        uint32_t tokens, uint32_t experts,
                                                        uint32_t top_k, uint32_t sigmoid,
                                                        uint32_t normalize, float eps,
-                                                       float scaling) {
+                                                       float scaling, uint32_t rank_order,
+                                                       const void* __restrict__ gate_x, uint32_t gate_x_dtype,
+                                                       const float* __restrict__ gate_w, uint32_t hidden,
+                                                       float* __restrict__ shared_gate) {
     extern __shared__ float scores_lds[];  // experts floats
     const uint32_t token = blockIdx.x, lane = threadIdx.x;
     if (token >= tokens) return;
@@ -166,6 +169,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
 #pragma unroll
             for (int other = 0; other < kMaxTopK; ++other)
                 if ((uint32_t)other < top_k && sel_id[other] < sel_id[rank]) ++position;
+            if (rank_order) position = (uint32_t)rank;  // the hybrid engine keeps selection order
             float weight = sel_score[rank];
             if (normalize) weight = weight / denominator;
             weight = weight * scaling;
@@ -174,6 +178,18 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
             out[1] = __uint_as_float(token);
             out[2] = weight;
         }
+    }
+
+    // Shared-expert gate of h_moe_route (src/metal/shaders/hybrid.metal:2259-2319):
+    // sigmoid(dot(x[token], gate_w)), or 1 without a gate vector.
+    if (shared_gate != nullptr) {
+        float dot = 0.f;
+        if (gate_w != nullptr) {
+            for (uint32_t i = lane; i < hidden; i += 64)
+                dot += load_as_f32(gate_x, (size_t)token * hidden + i, gate_x_dtype) * gate_w[i];
+            dot = wave_sum(dot);
+        }
+        if (lane == 0) shared_gate[token] = gate_w != nullptr ? 1.f / (1.f + expf(-dot)) : 1.f;
     }
 }
 
@@ -220,7 +236,9 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(const void* __restr
                                                              void* __restrict__ out,
                                                              uint32_t tokens, uint32_t hidden,
                                                              uint32_t top_k, uint32_t in_dtype,
-                                                             uint32_t out_dtype) {
+                                                             uint32_t out_dtype,
+                                                             const void* __restrict__ shared,
+                                                             const float* __restrict__ shared_gate) {
     size_t total = (size_t)tokens * hidden;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
@@ -231,6 +249,10 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(const void* __restr
             float gate = round_storage(metadata[a * 3 + 2], out_dtype);
             float value = load_as_f32(in, a * hidden + column, in_dtype);
             sum += round_storage(gate * value, out_dtype);
+        }
+        if (shared != nullptr) {
+            const float gate = round_storage(shared_gate != nullptr ? shared_gate[token] : 1.f, out_dtype);
+            sum += round_storage(gate * load_as_f32(shared, i, in_dtype), out_dtype);
         }
         store_from_f32(out, i, out_dtype, sum);
     }
@@ -288,7 +310,9 @@ __global__ __launch_bounds__(256) void expert_combine8_kernel(const void* __rest
                                                               const float* __restrict__ metadata,
                                                               void* __restrict__ out, uint32_t tokens,
                                                               uint32_t hidden, uint32_t top_k,
-                                                              uint32_t in_dtype, uint32_t out_dtype) {
+                                                              uint32_t in_dtype, uint32_t out_dtype,
+                                                              const void* __restrict__ shared,
+                                                              const float* __restrict__ shared_gate) {
     const size_t total = (size_t)tokens * hidden / 8;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
@@ -313,6 +337,13 @@ __global__ __launch_bounds__(256) void expert_combine8_kernel(const void* __rest
                     for (int j = 0; j < 8; ++j) sum[j] += round_storage(weight * value[r][j], out_dtype);
                 }
             }
+        }
+        if (shared != nullptr) {
+            const float weight = round_storage(shared_gate != nullptr ? shared_gate[token] : 1.f, out_dtype);
+            float value[8];
+            load8(shared, i * 8, in_dtype, value);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum[j] += round_storage(weight * value[j], out_dtype);
         }
         store8(out, i * 8, out_dtype, sum);
     }
@@ -379,19 +410,20 @@ __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float
 
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
                              const float* bias, float* metadata, uint32_t tokens,
-                             const fh_routing_policy& p) {
+                             const fh_routing_policy& p, const RouteExtras& x) {
     const size_t lds = ((p.experts + 3u) & ~3u) * sizeof(float);
 #define FH_ROUTE(PL)                                                                                   \
     hipLaunchKernelGGL(moe_route_kernel<PL>, dim3(tokens), dim3(64), lds, s, logits, logits_dtype, bias, \
                        metadata, tokens, p.experts, p.top_k, p.sigmoid, p.normalize_top_k_prob,         \
-                       p.normalization_epsilon, p.routed_scaling_factor)
+                       p.normalization_epsilon, p.routed_scaling_factor, x.rank_order, x.gate_x,        \
+                       x.gate_x_dtype, x.gate_w, x.hidden, x.shared_gate)
     if (p.experts <= 64) FH_ROUTE(1);
     else if (p.experts <= 128) FH_ROUTE(2);
     else if (p.experts <= 256) FH_ROUTE(4);
     else if (p.experts <= 512) FH_ROUTE(8);
     else FH_ROUTE(kMaxPerLane);
 #undef FH_ROUTE
-    return "moe_route";
+    return x.rank_order ? "h_moe_route" : "moe_route";
 }
 
 const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t assignments,
@@ -435,16 +467,18 @@ const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uin
 
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
                                   uint32_t tokens, uint32_t hidden, uint32_t top_k,
-                                  uint32_t in_dtype, uint32_t out_dtype) {
-    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+                                  uint32_t in_dtype, uint32_t out_dtype, const void* shared,
+                                  const float* shared_gate) {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
+                           reinterpret_cast<uintptr_t>(shared)) & 15u) == 0;
     if (hidden % 8 == 0 && aligned) {
         hipLaunchKernelGGL(expert_combine8_kernel, dim3(grid_for((size_t)tokens * hidden / 8)), dim3(256), 0,
-                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype, shared, shared_gate);
     } else {
         hipLaunchKernelGGL(expert_combine_kernel, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0,
-                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype);
+                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype, shared, shared_gate);
     }
-    return "expert_combine";
+    return shared != nullptr ? "h_moe_combine" : "expert_combine";
 }
 
 }  // namespace fh

@@ -194,6 +194,31 @@ fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weigh
                                       const fh_view* x, uint32_t assignments,
                                       const fh_view* metadata, const fh_view* y);
 
+/* The hybrid engine's router and combine (f32 models; HybridModel::moe_ffn,
+ * src/hybrid/engine.rs:2881-3092).
+ *
+ * fh_moe_route_ranked is h_moe_route (src/metal/shaders/hybrid.metal:2259-2319):
+ * softmax over all experts or sigmoid, top-k with ties to the lower index,
+ * weights divided by their sum when policy->normalize_top_k_prob is set, rows
+ * kept in SELECTION order (rank 0 first) instead of expert-id order, and the
+ * shared-expert gate sigmoid(dot(x[t], gate_vector)) written to shared_gate
+ * [tokens] f32 (1 when gate_vector is NULL; nothing when shared_gate is NULL).
+ * The hybrid engine's ids[] and weights[] are columns 0 and 2 of the metadata
+ * rows; expert projections and combine take the rows as they are.  The
+ * policy's epsilon and scaling apply as in fh_moe_route (the hybrid engine
+ * uses 0 and 1); there is no selection bias.
+ *
+ * fh_expert_combine_shared is h_moe_combine (hybrid.metal:2374-2388):
+ * out[t] = sum over ranks of w * down[row] + shared_gate[t] * shared[t]
+ * (gate 1 when shared_gate is NULL), with fh_expert_combine's storage rounding
+ * for 16-bit types. */
+fh_status fh_moe_route_ranked(fh_device* device, const fh_view* logits, uint32_t tokens,
+                              const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
+                              uint32_t hidden, const fh_view* metadata, const fh_view* shared_gate);
+fh_status fh_expert_combine_shared(fh_device* device, const fh_view* in, const fh_view* metadata,
+                                   uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* shared,
+                                   const fh_view* shared_gate, const fh_view* out);
+
 /* Decode-sized fusions.  SparseMoe::forward (src/nn/moe.rs:222-390) encodes
  * expert_assign, the gate|up projection, expert_silu_mul and the down
  * projection back to back; with a handful of assignments each of them is a

@@ -359,6 +359,36 @@ public:
         check(fh_moe_route(handle_->raw, &lv, (uint32_t)dims[0], selection_bias ? &bv : nullptr, &pc, &mv));
         return meta;
     }
+    // The hybrid engine's router (h_moe_route): metadata rows in selection order; when
+    // `shared_gate` is given it receives sigmoid(dot(x[t], gate_vector)) per token, or ones
+    // without a vector.
+    Tensor moe_route_ranked(const Tensor& logits, const MoeRoutingPolicy& policy, const Tensor* x = nullptr,
+                            const Tensor* gate_vector = nullptr, const Tensor* shared_gate = nullptr) const {
+        const auto& dims = logits.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != policy.experts)
+            throw Error(ErrorKind::Shape, "invalid sparse routing geometry");
+        Tensor meta = zeros({dims[0] * policy.top_k, 3}, DType::F32);
+        fh_view lv = logits.c_view(), mv = meta.c_view(), xv{}, wv{}, gv{};
+        if (x) xv = x->c_view();
+        if (gate_vector) wv = gate_vector->c_view();
+        if (shared_gate) gv = shared_gate->c_view();
+        fh_routing_policy pc = policy.c();
+        check(fh_moe_route_ranked(handle_->raw, &lv, (uint32_t)dims[0], &pc, x ? &xv : nullptr,
+                                  gate_vector ? &wv : nullptr, gate_vector ? (uint32_t)gate_vector->numel() : 0, &mv,
+                                  shared_gate ? &gv : nullptr));
+        return meta;
+    }
+    // h_moe_combine: the weighted sum of the routed rows plus shared_gate[t] * shared[t].
+    Tensor expert_combine_shared(const Tensor& input, const Tensor& metadata, size_t tokens, size_t hidden,
+                                 size_t top_k, const Tensor& shared, const Tensor* shared_gate = nullptr,
+                                 const Tensor* out = nullptr) const {
+        Tensor y = out ? *out : zeros({tokens, hidden}, input.dtype());
+        fh_view iv = input.c_view(), mv = metadata.c_view(), sv = shared.c_view(), yv = y.c_view(), gv{};
+        if (shared_gate) gv = shared_gate->c_view();
+        check(fh_expert_combine_shared(handle_->raw, &iv, &mv, (uint32_t)tokens, (uint32_t)hidden, (uint32_t)top_k,
+                                       &sv, shared_gate ? &gv : nullptr, &yv));
+        return y;
+    }
     Tensor expert_assign(const Tensor& hidden, const Tensor& metadata, size_t top_k, const Tensor* out = nullptr) const {
         const auto& x = hidden.shape();
         const auto& m = metadata.shape();

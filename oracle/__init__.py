@@ -67,6 +67,12 @@ def _load() -> ctypes.CDLL:
     lib.fo_expert_project.argtypes = [u32, u8p, sz, sz, sz, f32p, f32p, sz, f32p, i32, i32, i32]
     lib.fo_expert_silu_mul.restype = None
     lib.fo_expert_silu_mul.argtypes = [f32p, sz, sz, u32, f32p]
+    lib.fo_select_routes_ranked.restype = i32
+    lib.fo_select_routes_ranked.argtypes = [f32p, sz, sz, sz, i32, i32, f32p]
+    lib.fo_shared_gate.restype = None
+    lib.fo_shared_gate.argtypes = [f32p, f32p, sz, sz, f32p]
+    lib.fo_expert_combine_shared.restype = None
+    lib.fo_expert_combine_shared.argtypes = [f32p, f32p, sz, sz, sz, u32, f32p, f32p, f32p]
     lib.fo_argmax_rows.restype = None
     lib.fo_argmax_rows.argtypes = [f32p, sz, sz, ctypes.POINTER(ctypes.c_uint32)]
     lib.fo_expert_combine.restype = None
@@ -207,6 +213,37 @@ def expert_silu_mul(packed_rows, intermediate: int, dtype: int = F32) -> np.ndar
     a = np.ascontiguousarray(packed_rows, dtype=np.float32).reshape(-1, 2 * intermediate)
     out = np.empty((a.shape[0], intermediate), dtype=np.float32)
     _lib.fo_expert_silu_mul(_f32(a), a.shape[0], intermediate, dtype, _f32(out))
+    return out
+
+
+def select_routes_ranked(logits, experts: int, top_k: int, sigmoid: bool = False,
+                         normalize: bool = True) -> np.ndarray:
+    """h_moe_route (hybrid.metal:2259-2319): metadata rows in selection order."""
+    a = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1, experts)
+    out = np.empty((a.shape[0] * top_k, 3), dtype=np.float32)
+    status = _lib.fo_select_routes_ranked(_f32(a), a.shape[0], experts, top_k, int(sigmoid), int(normalize), _f32(out))
+    if status:
+        raise ValueError(f"ranked routing failed with status {status}")
+    return out
+
+
+def shared_gate(x, w) -> np.ndarray:
+    a = np.ascontiguousarray(x, dtype=np.float32)
+    v = np.ascontiguousarray(w, dtype=np.float32)
+    out = np.empty(a.shape[0], dtype=np.float32)
+    _lib.fo_shared_gate(_f32(a), _f32(v), a.shape[0], a.shape[1], _f32(out))
+    return out
+
+
+def expert_combine_shared(values, metadata, tokens: int, hidden: int, top_k: int, shared, gate=None,
+                          dtype: int = F32) -> np.ndarray:
+    v = np.ascontiguousarray(values, dtype=np.float32).reshape(tokens * top_k, hidden)
+    meta = np.ascontiguousarray(metadata, dtype=np.float32)
+    sh = np.ascontiguousarray(shared, dtype=np.float32).reshape(tokens, hidden)
+    g = None if gate is None else np.ascontiguousarray(gate, dtype=np.float32)
+    out = np.empty((tokens, hidden), dtype=np.float32)
+    _lib.fo_expert_combine_shared(_f32(v), _f32(meta), tokens, hidden, top_k, dtype, _f32(sh),
+                                  _f32(g) if g is not None else None, _f32(out))
     return out
 
 

@@ -30,6 +30,17 @@
  *       the last ulp (reference tolerance 2e-6).
  *   fo_expert_*            pinned: hand-computed 3-wide MoE of
  *       src/nn/moe.rs:530-664 restated in numpy float64.
+ *   fo_select_routes_ranked, fo_shared_gate
+ *                          ids pinned: the CPU procedure of the reference's
+ *       own routing test (src/hybrid/engine.rs:5004-5024) in numpy float64,
+ *       and equal-logit ties.  Weights and gate: PARITY UNPINNED in the last
+ *       ulps (the reference's threadgroup summation order is its own); held
+ *       to that test's tolerances, 1e-5 and 1e-4.
+ *   fo_expert_combine_shared   pinned: numpy float64 evaluation; equals
+ *       fo_expert_combine when the shared rows are zero.
+ *   fo_argmax_rows         pinned for finite rows: numpy argmax (first
+ *       maximal index) and ties; rows holding NaN follow the reference
+ *       kernel's scan and merge order as read (flagged rows: parity unpinned).
  */
 #include <math.h>
 #include <pthread.h>
@@ -394,8 +405,9 @@ static uint32_t float_to_bits(float f) {
  * the scaling factor; rows sorted by expert id.  metadata is [tokens*k, 3]
  * f32 {expert id bits, token id bits, weight}.  Returns 0, or 1 on invalid
  * logits / geometry, 2 on an invalid normaliser. */
-int fo_select_routes(const float* logits, size_t tokens, size_t experts, size_t top_k, int sigmoid,
-                     int normalize, float eps, float scaling, const float* bias, float* metadata) {
+static int select_routes(const float* logits, size_t tokens, size_t experts, size_t top_k, int sigmoid,
+                         int normalize, float eps, float scaling, const float* bias, float* metadata,
+                         int ranked) {
     if (experts == 0 || top_k == 0 || top_k > experts) return 1;
     for (size_t i = 0; i < tokens * experts; i++)
         if (!isfinite(logits[i])) return 1;
@@ -446,8 +458,8 @@ int fo_select_routes(const float* logits, size_t tokens, size_t experts, size_t 
             for (size_t r = 0; r < top_k; r++) selw[r] = selw[r] / denominator;
         }
         for (size_t r = 0; r < top_k; r++) selw[r] = selw[r] * scaling;
-        /* stable insertion sort by expert id */
-        for (size_t i = 1; i < top_k; i++) {
+        /* stable insertion sort by expert id (the hybrid engine keeps selection order) */
+        for (size_t i = 1; i < top_k && !ranked; i++) {
             size_t id = sel[i];
             float w = selw[i];
             size_t j = i;
@@ -471,6 +483,54 @@ int fo_select_routes(const float* logits, size_t tokens, size_t experts, size_t 
     free(sel);
     free(selw);
     return status;
+}
+
+int fo_select_routes(const float* logits, size_t tokens, size_t experts, size_t top_k, int sigmoid,
+                     int normalize, float eps, float scaling, const float* bias, float* metadata) {
+    return select_routes(logits, tokens, experts, top_k, sigmoid, normalize, eps, scaling, bias, metadata, 0);
+}
+
+/* h_moe_route (src/metal/shaders/hybrid.metal:2259-2319): the same scores and
+ * top-k (greater probability wins, ties to the lower index), weights divided
+ * by the sum of the picked ones taken in rank order, rows left in rank order.
+ * The reference sums the softmax denominator with a threadgroup tree whose
+ * order is its own; this restatement sums in expert order, so weights agree
+ * to the last few ulp, not bitwise (ids are exact away from exact ties). */
+int fo_select_routes_ranked(const float* logits, size_t tokens, size_t experts, size_t top_k, int sigmoid,
+                            int normalize, float* metadata) {
+    return select_routes(logits, tokens, experts, top_k, sigmoid, normalize, 0.0f, 1.0f, NULL, metadata, 1);
+}
+
+/* Shared-expert gate of h_moe_route: sigmoid(dot(x[t], w)); the dot product is
+ * accumulated in f64 here (the reference's threadgroup tree is unpinned). */
+void fo_shared_gate(const float* x, const float* w, size_t tokens, size_t hidden, float* out) {
+    for (size_t t = 0; t < tokens; t++) {
+        double dot = 0.0;
+        for (size_t i = 0; i < hidden; i++) dot += (double)x[t * hidden + i] * (double)w[i];
+        out[t] = (float)(1.0 / (1.0 + exp(-dot)));
+    }
+}
+
+/* h_moe_combine (hybrid.metal:2374-2388) in f32: out[t,c] = sum over ranks of
+ * w * down, then + gate[t] * shared[t,c] (gate may be NULL: 1).  With a 16-bit
+ * dtype the products and the gate are rounded like fo_expert_combine's. */
+void fo_expert_combine_shared(const float* in, const float* metadata, size_t tokens, size_t hidden,
+                              size_t top_k, uint32_t dtype, const float* shared, const float* gate, float* out) {
+    for (size_t t = 0; t < tokens; t++) {
+        for (size_t c = 0; c < hidden; c++) {
+            float total = 0.0f;
+            for (size_t rank = 0; rank < top_k; rank++) {
+                size_t a = t * top_k + rank;
+                float w = fo_round_storage(metadata[a * 3 + 2], dtype);
+                float product = w * in[a * hidden + c];
+                total = total + fo_round_storage(product, dtype);
+            }
+            float g = fo_round_storage(gate ? gate[t] : 1.0f, dtype);
+            float product = g * shared[t * hidden + c];
+            total = total + fo_round_storage(product, dtype);
+            out[t * hidden + c] = fo_round_storage(total, dtype);
+        }
+    }
 }
 
 /* expert_assign (ops.metal:1959-1967): out[a,:] = hidden[token(a),:]. */

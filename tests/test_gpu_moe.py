@@ -406,3 +406,75 @@ def test_sparse_moe_decode_path_matches_the_separate_steps(api, d, tokens):
     separate = moe.forward(xt, lt)
     assert np.array_equal(fused.raw(), separate.raw())
     assert np.abs(fused.to_f32()).max() > 1e-3
+
+
+# ------------------------------------------------- the hybrid engine's router and combine
+
+@pytest.mark.parametrize("sigmoid,norm,shared_gate", [(True, True, False), (False, True, True), (True, False, True)])
+def test_ranked_router_replays_the_hybrid_engines_test(api, d, sigmoid, norm, shared_gate):
+    # src/hybrid/engine.rs:4949-5041: 256 experts, top-6, hidden 2048, three tokens; ids exact,
+    # weights within 1e-5, gate within 1e-4 (the reference's tolerances)
+    experts, top_k, hidden, tokens = 256, 6, 2048, 3
+    rng = synth.rng(151)
+    logits = (rng.standard_normal((tokens, experts)) * 3).astype(np.float32)
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    w = rng.standard_normal(hidden).astype(np.float32)
+    policy = api.MoeRoutingPolicy(experts, top_k, scoring_function=api.MoeScoringFunction.Sigmoid if sigmoid
+                                  else api.MoeScoringFunction.Softmax, normalize_top_k_prob=norm)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F32, x)
+    wt = api.Tensor.from_f32(d, w.shape, api.DType.F32, w)
+    meta, gate = d.moe_route_ranked(lt, policy, xt if shared_gate else None, wt if shared_gate else None,
+                                    want_gate=True)
+    assert d.last_operation() == "h_moe_route"
+    got = meta.to_f32()
+    want = oracle.select_routes_ranked(logits, experts, top_k, sigmoid=sigmoid, normalize=norm)
+    assert np.array_equal(bits(got[:, :2]), bits(want[:, :2]))
+    assert np.abs(got[:, 2] - want[:, 2]).max() < 1e-5
+    want_gate = oracle.shared_gate(x, w) if shared_gate else np.ones(tokens, np.float32)
+    assert np.abs(gate.to_f32() - want_gate).max() < 1e-4
+
+
+def test_hybrid_decode_chain_route_project_combine_with_shared_expert(api, d):
+    # f32 model, one token: ranked route -> gate|up by gathered rows -> down with SiLU*up ->
+    # combine + gate * shared expert, against the oracle's same chain
+    experts, top_k, hidden, inter, tokens = 32, 4, 512, 256, 2
+    fmt = api.QuantizationFormat(Q4_K)
+    w_in = synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=161)
+    w_out = synth.matrix(Q4_K, experts * hidden, inter, seed=162)
+    s_in = synth.matrix(Q4_K, 2 * inter, hidden, seed=163)
+    s_out = synth.matrix(Q4_K, hidden, inter, seed=164)
+    win = api.QuantizedExpertMatrix.new(d, w_in, fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, w_out, fmt, experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, s_in)
+    sout = api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, s_out)
+    rng = synth.rng(165)
+    x = (rng.standard_normal((tokens, hidden)) * 2.0 ** -6).astype(np.float32)
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    gate_w = rng.standard_normal(hidden).astype(np.float32)
+    f32 = api.DType.F32
+    xt = api.Tensor.from_f32(d, x.shape, f32, x)
+    policy = api.MoeRoutingPolicy(experts, top_k)
+    meta, gate = d.moe_route_ranked(api.Tensor.from_f32(d, logits.shape, f32, logits), policy, xt,
+                                    api.Tensor.from_f32(d, gate_w.shape, f32, gate_w))
+    up = d.expert_project_quantized(xt, meta, win, hidden, experts, form="gather")
+    down = d.expert_project_quantized(up, meta, wout, inter, experts, form="silu_mul")
+    shared = d.project_quantized(d.project_quantized(xt, sin).tensor, sout, silu_mul=True).tensor
+    out = d.expert_combine_shared(down, meta, tokens, hidden, top_k, shared, gate)
+    assert d.last_operation() == "h_moe_combine"
+
+    m = oracle.select_routes_ranked(logits, experts, top_k)
+    assert np.array_equal(bits(meta.to_f32()[:, :2]), bits(m[:, :2]))
+    o_up = oracle.expert_project(Q4_K, w_in, experts, 2 * inter, hidden, oracle.expert_assign(x, m), m, accumulate="f64")
+    o_down = oracle.expert_project(Q4_K, w_out, experts, hidden, inter, oracle.expert_silu_mul(o_up, inter), m,
+                                   accumulate="f64")
+    o_sh = oracle.project(Q4_K, s_out, hidden, inter,
+                          oracle.expert_silu_mul(oracle.project(Q4_K, s_in, 2 * inter, hidden, x, accumulate="f64"), inter),
+                          accumulate="f64")
+    want = oracle.expert_combine_shared(o_down, m, tokens, hidden, top_k, o_sh, oracle.shared_gate(x, gate_w))
+    assert np.abs(want).max() > 1e-3
+    assert rel_l2(out.to_f32(), want) <= 2e-5
+    # without a gate tensor the shared expert is added whole
+    whole = d.expert_combine_shared(down, meta, tokens, hidden, top_k, shared).to_f32()
+    plain = d.expert_combine(down, meta, tokens, hidden, top_k).to_f32()
+    assert np.allclose(whole, plain + shared.to_f32(), rtol=1e-6, atol=1e-7)

@@ -525,3 +525,58 @@ def test_argmax_rows_is_the_first_maximal_index_and_flags_non_finite_rows():
     assert got[0, 0] == 0 and got[2, 0] == 0
     y = x[1].copy(); y[2047] = -np.inf
     assert got[1, 0] == y.argmax()
+
+
+def _ranked_by_numpy(logits, top_k, sigmoid, norm):
+    """The CPU procedure of the reference's own routing test
+    (src/hybrid/engine.rs:5004-5024) in float64 numpy."""
+    ids, weights = [], []
+    for row in logits.astype(np.float64):
+        scores = 1 / (1 + np.exp(-row)) if sigmoid else np.exp(row - row.max()) / np.exp(row - row.max()).sum()
+        order = np.lexsort((np.arange(row.size), -scores))[:top_k]
+        w = scores[order]
+        ids.append(order)
+        weights.append(w / w.sum() if norm else w)
+    return np.array(ids), np.array(weights)
+
+
+def test_ranked_routing_follows_the_hybrid_engines_cpu_procedure():
+    rng = np.random.default_rng(21)
+    experts, top_k, tokens = 256, 6, 3
+    logits = (rng.standard_normal((tokens, experts)) * 3).astype(np.float32)
+    for sigmoid, norm in ((True, True), (False, True), (True, False)):
+        meta = oracle.select_routes_ranked(logits, experts, top_k, sigmoid=sigmoid, normalize=norm)
+        want_ids, want_w = _ranked_by_numpy(logits, top_k, sigmoid, norm)
+        assert np.array_equal(meta[:, 0].view(np.uint32).reshape(tokens, top_k), want_ids)
+        assert np.array_equal(meta[:, 1].view(np.uint32).reshape(tokens, top_k),
+                              np.repeat(np.arange(tokens), top_k).reshape(tokens, top_k))
+        assert np.abs(meta[:, 2].reshape(tokens, top_k) - want_w).max() < 1e-6
+    # equal logits: ties go to the lower index, in rank order
+    meta = oracle.select_routes_ranked(np.zeros((1, 8), np.float32), 8, 3)
+    assert meta[:, 0].view(np.uint32).tolist() == [0, 1, 2]
+    # the same selection as the id-ordered form, in a different row order
+    plain = oracle.select_routes(logits, experts, top_k)
+    ranked = oracle.select_routes_ranked(logits, experts, top_k)
+    for t in range(tokens):
+        a = plain[t * top_k:(t + 1) * top_k]
+        b = ranked[t * top_k:(t + 1) * top_k]
+        assert sorted(a[:, 0].view(np.uint32)) == sorted(b[:, 0].view(np.uint32))
+        assert np.all(np.diff(b[:, 2]) <= 0)
+
+
+def test_shared_gate_and_combine_with_a_shared_expert():
+    rng = np.random.default_rng(22)
+    tokens, hidden, top_k = 3, 64, 2
+    x = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    w = rng.standard_normal(hidden).astype(np.float32)
+    gate = oracle.shared_gate(x, w)
+    assert np.allclose(gate, 1 / (1 + np.exp(-(x.astype(np.float64) @ w.astype(np.float64)))), rtol=1e-6)
+    down = rng.standard_normal((tokens * top_k, hidden)).astype(np.float32)
+    shared = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    meta = np.zeros((tokens * top_k, 3), np.float32)
+    meta[:, 2] = rng.random(tokens * top_k).astype(np.float32)
+    got = oracle.expert_combine_shared(down, meta, tokens, hidden, top_k, shared, gate)
+    want = (meta[:, 2:3].astype(np.float64) * down).reshape(tokens, top_k, hidden).sum(1) + gate[:, None] * shared
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    plain = oracle.expert_combine(down, meta, tokens, hidden, top_k)
+    assert np.array_equal(oracle.expert_combine_shared(down, meta, tokens, hidden, top_k, np.zeros_like(shared)), plain)

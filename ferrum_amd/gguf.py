@@ -279,6 +279,16 @@ class GgufReader:
                 return False
         return True
 
+    def read_stacked_experts(self, gate_name: str, up_name: str):
+        return _read_stacked_experts(self, gate_name, up_name)
+
+    def quantized_input_experts(self, device, gate_name: str, up_name: str):
+        """gate|up expert tensors as one api.QuantizedExpertMatrix of [experts, 2I, H]
+        (load_quantized_input_experts, src/model/lfm2_moe/gguf.rs:466-534)."""
+        from . import api
+        payload, fmt, experts, rows_per_expert, columns = self.read_stacked_experts(gate_name, up_name)
+        return api.QuantizedExpertMatrix.new(device, payload, fmt, experts, rows_per_expert, columns)
+
     # ---- device upload ----------------------------------------------------
     def quantized_matrix(self, device, name: str):
         """A rank-2 Q4_K / Q6_K tensor as api.QuantizedMatrix, blocks uploaded verbatim."""
@@ -299,6 +309,48 @@ class GgufReader:
         payload = np.empty(info.byte_len, dtype=np.uint8)
         self.read_tensor_into(name, payload)
         return api.QuantizedExpertMatrix.new(device, payload, fmt, experts, rows, columns)
+
+
+def _read_stacked_experts(reader: "GgufReader", gate_name: str, up_name: str):
+    """Host side of load_quantized_input_experts (src/model/lfm2_moe/gguf.rs:466-534): the
+    gate and up expert tensors ([experts, I, H] each) interleaved per expert into
+    [experts, 2I, H] rows, gate first, streamed 64 rows at a time.  Returns
+    (payload uint8 array, format, experts, rows_per_expert, columns)."""
+    import numpy as np
+    from . import api
+    gate, up = reader.tensor(gate_name), reader.tensor(up_name)
+    experts, intermediate, hidden = gate.logical_expert_shape()
+    if up.logical_expert_shape() != [experts, intermediate, hidden] or up.type_id != gate.type_id:
+        raise api.WeightError(f"{up_name}: gate and up expert tensors differ in shape or type")
+    fmt = api.QuantizationFormat.from_ggml_type(gate.type_id)
+    row_bytes = hidden // fmt.block_elements() * fmt.block_bytes()
+    component_bytes = experts * intermediate * row_bytes
+    rows_per_expert = 2 * intermediate
+    payload = np.empty(experts * rows_per_expert * row_bytes, dtype=np.uint8)
+    view = payload.reshape(experts, 2, intermediate, row_bytes)
+    for component, name in enumerate((gate_name, up_name)):
+        info = reader.tensor(name)
+        if info.byte_len != component_bytes:
+            raise api.WeightError(f"{name}: expected {component_bytes} packed expert bytes")
+        written = 0
+
+        def place(offset, chunk, component=component, name=name):
+            nonlocal written
+            if len(chunk) % row_bytes:
+                raise _error(f"tensor {name} stream ended inside an expert row")
+            rows = np.frombuffer(chunk, dtype=np.uint8).reshape(-1, row_bytes)
+            first = offset // row_bytes
+            for i, row in enumerate(rows):
+                expert, within = divmod(first + i, intermediate)
+                if expert >= experts:
+                    raise _error(f"tensor {name} contains too many expert rows")
+                view[expert, component, within] = row
+            written += len(chunk)
+
+        reader.stream_tensor(name, row_bytes * 64, place)
+        if written != component_bytes:
+            raise _error(f"tensor {name} streamed {written} bytes, expected {component_bytes}")
+    return payload, fmt, experts, rows_per_expert, hidden
 
 
 def builtins_open(path: str):

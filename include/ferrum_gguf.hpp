@@ -363,6 +363,51 @@ inline QuantizedExpertMatrix load_quantized_expert_matrix(const Device& device, 
                                           [&](uint8_t* dst, size_t n) { reader.read_tensor_into(name, dst, n); });
 }
 
+// The gate and up expert tensors ([experts, I, H] each) interleaved per expert into
+// [experts, 2I, H] rows, gate first, streamed 64 rows at a time
+// (load_quantized_input_experts, src/model/lfm2_moe/gguf.rs:466-534).
+inline void read_stacked_experts(Reader& reader, const std::string& gate_name, const std::string& up_name,
+                                 uint8_t* destination, size_t length) {
+    const TensorInfo gate = reader.tensor(gate_name), up = reader.tensor(up_name);
+    const auto shape = gate.logical_expert_shape();
+    if (up.logical_expert_shape() != shape || up.type_id != gate.type_id)
+        throw Error(ErrorKind::Weight, up_name + ": gate and up expert tensors differ in shape or type");
+    const QuantizationFormat format = format_from_ggml_type(gate.type_id);
+    const size_t experts = shape[0], intermediate = shape[1], hidden = shape[2];
+    const size_t row_bytes = hidden / block_elements(format) * block_bytes(format);
+    const size_t component_bytes = experts * intermediate * row_bytes;
+    if (length != 2 * component_bytes) fail("stacked expert destination has " + std::to_string(length) + " bytes");
+    const std::string* names[2] = {&gate_name, &up_name};
+    for (size_t component = 0; component < 2; ++component) {
+        const std::string& name = *names[component];
+        if (reader.tensor(name).byte_len != component_bytes)
+            throw Error(ErrorKind::Weight, name + ": expected " + std::to_string(component_bytes) + " packed expert bytes");
+        size_t written = 0;
+        reader.stream_tensor(name, row_bytes * 64, [&](const uint8_t* chunk, size_t n) {
+            if (n % row_bytes) fail("tensor " + name + " stream ended inside an expert row");
+            for (size_t i = 0; i < n / row_bytes; ++i) {
+                const size_t source_row = written / row_bytes + i;
+                const size_t expert = source_row / intermediate, within = source_row % intermediate;
+                if (expert >= experts) fail("tensor " + name + " contains too many expert rows");
+                std::memcpy(destination + ((expert * 2 + component) * intermediate + within) * row_bytes,
+                            chunk + i * row_bytes, row_bytes);
+            }
+            written += n;
+        });
+        if (written != component_bytes)
+            fail("tensor " + name + " streamed " + std::to_string(written) + " bytes, expected " +
+                 std::to_string(component_bytes));
+    }
+}
+
+inline QuantizedExpertMatrix load_quantized_input_experts(const Device& device, Reader& reader,
+                                                          const std::string& gate_name, const std::string& up_name) {
+    const TensorInfo& gate = reader.tensor(gate_name);
+    const auto shape = gate.logical_expert_shape();
+    return device.quantized_expert_matrix(shape[0], 2 * shape[1], shape[2], format_from_ggml_type(gate.type_id),
+                                          [&](uint8_t* dst, size_t n) { read_stacked_experts(reader, gate_name, up_name, dst, n); });
+}
+
 }  // namespace gguf
 }  // namespace ferrum
 

@@ -31,6 +31,16 @@ static void print(const gguf::MetadataValue& v) {
 int main(int argc, char** argv) {
     if (argc < 2) return 64;
     try {
+        if (argc == 5 && !std::strcmp(argv[2], "stack")) {   // <file> stack <gate> <up>: FNV-1a of the interleaved rows
+            gguf::Reader file = gguf::Reader::open(argv[1]);
+            const auto shape = file.tensor(argv[3]).logical_expert_shape();
+            std::vector<uint8_t> payload(2 * file.tensor(argv[3]).byte_len);
+            gguf::read_stacked_experts(file, argv[3], argv[4], payload.data(), payload.size());
+            uint64_t h = 1469598103934665603ull;
+            for (uint8_t b : payload) h = (h ^ b) * 1099511628211ull;
+            std::printf("stacked %zu %zu %zu fnv %016" PRIx64 "\n", shape[0], 2 * shape[1], shape[2], h);
+            return 0;
+        }
         const uint64_t limit = argc > 2 ? std::strtoull(argv[2], nullptr, 10) : UINT64_MAX;
         gguf::Reader file = gguf::Reader::open(argv[1], limit, !(argc > 3 && !std::strcmp(argv[3], "untagged")));
         std::printf("version %u alignment %" PRIu64 " data %" PRIu64 "\n", file.version(), file.alignment(),

@@ -251,3 +251,31 @@ def test_cpp_reader_agrees_with_the_python_reader(probe, tmp_path):
         if args:
             kw = {"max_array_items": int(args[0])} if len(args) == 1 else {"require_architecture": False}
         assert proc.stdout.splitlines() == _describe(read(data, **kw)), label
+
+
+def test_gate_and_up_expert_tensors_interleave_per_expert(probe, tmp_path):
+    # load_quantized_input_experts (src/model/lfm2_moe/gguf.rs:466-534): [E, I, H] + [E, I, H] -> [E, 2I, H]
+    import subprocess
+    experts, inter, hidden = 3, 70, 512          # 70 rows per expert: chunks of 64 rows cross expert boundaries
+    gate = synth.matrix(12, experts * inter, hidden, seed=31)
+    up = synth.matrix(12, experts * inter, hidden, seed=32)
+    path = tmp_path / "experts.gguf"
+    path.write_bytes(gf.build([("blk.0.ffn_gate_exps.weight", [hidden, inter, experts], 12, gate),
+                               ("blk.0.ffn_up_exps.weight", [hidden, inter, experts], 12, up),
+                               ("blk.0.ffn_down_exps.weight", [inter * 0 + 256, hidden, experts], 12,
+                                synth.matrix(12, experts * hidden, 256, seed=33))]))
+    f = gguf.GgufReader.open(str(path))
+    payload, fmt, e, rows, cols = f.read_stacked_experts("blk.0.ffn_gate_exps.weight", "blk.0.ffn_up_exps.weight")
+    assert (fmt, e, rows, cols) == (api.QuantizationFormat.Q4_K, experts, 2 * inter, hidden)
+    row_bytes = hidden // 256 * 144
+    want = np.concatenate([gate.reshape(experts, inter, row_bytes), up.reshape(experts, inter, row_bytes)], axis=1)
+    assert np.array_equal(payload.reshape(experts, 2 * inter, row_bytes), want)
+    with pytest.raises(api.WeightError):
+        f.read_stacked_experts("blk.0.ffn_gate_exps.weight", "blk.0.ffn_down_exps.weight")
+    h = 1469598103934665603
+    for b in payload.tolist():
+        h = ((h ^ b) * 1099511628211) & (2**64 - 1)
+    proc = subprocess.run([probe, str(path), "stack", "blk.0.ffn_gate_exps.weight", "blk.0.ffn_up_exps.weight"],
+                          capture_output=True, text=True, timeout=30)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert proc.stdout.strip() == f"stacked {experts} {2 * inter} {hidden} fnv {h:016x}"

@@ -56,3 +56,38 @@ def test_tensors_from_a_gguf_file_project_like_the_oracle(tmp_path):
         f.quantized_matrix(d, "blk.0.ffn_gate_exps.weight")    # rank 3
     with pytest.raises(api.GgufError):
         f.quantized_expert_matrix(d, "output.weight")
+
+
+def test_stacked_gate_up_experts_from_a_gguf_file_run_the_fused_decode_chain(tmp_path):
+    from ferrum_amd import api
+    d = api.Device.new()
+    experts, inter, hidden, top_k, tokens = 4, 256, 512, 2, 2
+    gate = synth.matrix(Q4_K, experts * inter, hidden, seed=41)
+    up = synth.matrix(Q4_K, experts * inter, hidden, seed=42)
+    down = synth.matrix(Q4_K, experts * hidden, inter, seed=43)
+    path = tmp_path / "moe.gguf"
+    path.write_bytes(gf.build([("blk.0.ffn_gate_exps.weight", [hidden, inter, experts], Q4_K, gate),
+                               ("blk.0.ffn_up_exps.weight", [hidden, inter, experts], Q4_K, up),
+                               ("blk.0.ffn_down_exps.weight", [inter, hidden, experts], Q4_K, down)]))
+    f = gguf.GgufReader.open(str(path))
+    win = f.quantized_input_experts(d, "blk.0.ffn_gate_exps.weight", "blk.0.ffn_up_exps.weight")
+    wout = f.quantized_expert_matrix(d, "blk.0.ffn_down_exps.weight")
+    assert (win.experts(), win.rows_per_expert(), win.columns()) == (experts, 2 * inter, hidden)
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    rng = synth.rng(44)
+    x = (rng.standard_normal((tokens, hidden)) * 2.0 ** -6).astype(np.float32)
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    got = moe.forward(api.Tensor.from_f32(d, x.shape, api.DType.F32, x),
+                      api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)).to_f32()
+    row_bytes = hidden // 256 * 144
+    stacked = np.concatenate([gate.reshape(experts, inter, row_bytes), up.reshape(experts, inter, row_bytes)],
+                             axis=1).reshape(-1)
+    m = oracle.select_routes(logits, experts, top_k)
+    o_up = oracle.expert_project(Q4_K, stacked, experts, 2 * inter, hidden, oracle.expert_assign(x, m), m,
+                                 accumulate="f64")
+    o_down = oracle.expert_project(Q4_K, down, experts, hidden, inter, oracle.expert_silu_mul(o_up, inter), m,
+                                   accumulate="f64")
+    want = oracle.expert_combine(o_down, m, tokens, hidden, top_k)
+    assert np.abs(want).max() > 1e-4
+    l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    assert l2 <= 2e-5, l2

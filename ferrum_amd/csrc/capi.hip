@@ -700,26 +700,39 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     if (st != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(mr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
     const int64_t grouped_min = tuning(device, "expert_grouped_min_assignments");
-    if (form == FH_INPUT_ROWS && x->dtype != FH_F32 && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
-        weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
+    // f32 rows join the grouped form when the caller has opted f32 activations into the f16
+    // tiles (gemm_f32_min_rows, the hybrid engine's prompt path project_mm_id_in,
+    // src/hybrid/engine.rs:3164): they are rounded to f16 into the scratch first
+    const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
+    const bool f32_grouped = x->dtype == FH_F32 && f32_rows > 0 && assignments >= (uint64_t)f32_rows &&
+                             ((uintptr_t)xr.begin & 15u) == 0;
+    if (form == FH_INPUT_ROWS && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
+        assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
         // grouped form: every expert's weights are streamed once for all of its assignments
-        const size_t words = (size_t)weight->experts + 1 + assignments;
-        st = ensure_scratch(device, words * sizeof(uint32_t));
+        const size_t words = ((size_t)weight->experts + 1 + assignments + 3) & ~(size_t)3;
+        const size_t x16_bytes = f32_grouped ? (size_t)assignments * k * sizeof(uint16_t) : 0;
+        st = ensure_scratch(device, words * sizeof(uint32_t) + x16_bytes);
         if (st != FH_OK) return st;
         uint32_t* offsets = reinterpret_cast<uint32_t*>(scratch_data(device));
         uint32_t* order = offsets + weight->experts + 1;
+        const void* tile_x = xr.begin;
+        if (f32_grouped) {
+            uint16_t* x16 = reinterpret_cast<uint16_t*>(scratch_data(device) + words * sizeof(uint32_t));
+            launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin), x16, (size_t)assignments * k);
+            tile_x = x16;
+        }
         launch_expert_group(device->stream, reinterpret_cast<const float*>(mr.begin), assignments,
                             (uint32_t)weight->experts, offsets, order, const_cast<uint8_t*>(yr.begin),
                             (uint32_t)(rows * dtype_bytes(y->dtype)));
         GemmArgs g{};
         g.ggml_type = weight->ggml_type;
         g.w = weight->ptr;
-        g.x = xr.begin;
+        g.x = tile_x;
         g.y = const_cast<uint8_t*>(yr.begin);
         g.n = (uint32_t)rows;
         g.k = (uint32_t)k;
         g.m = assignments;
-        g.x_dtype = x->dtype;
+        g.x_dtype = f32_grouped ? FH_F16 : x->dtype;
         g.y_dtype = y->dtype;
         g.cu_count = device->props.multiProcessorCount;
         g.experts = (uint32_t)weight->experts;

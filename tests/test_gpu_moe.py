@@ -478,3 +478,29 @@ def test_hybrid_decode_chain_route_project_combine_with_shared_expert(api, d):
     whole = d.expert_combine_shared(down, meta, tokens, hidden, top_k, shared).to_f32()
     plain = d.expert_combine(down, meta, tokens, hidden, top_k).to_f32()
     assert np.allclose(whole, plain + shared.to_f32(), rtol=1e-6, atol=1e-7)
+
+
+def test_f32_assignments_join_the_grouped_projection_on_request(api, d):
+    # gemm_f32_min_rows opts f32 activations into the f16 tiles (the hybrid engine's prompt
+    # path); without it every f32 assignment keeps exact f32 weights
+    experts, rows, cols, a = 6, 64, 512, 48
+    packed = synth.matrix(Q4_K, experts * rows, cols, seed=171)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(Q4_K), experts, rows, cols)
+    ids = synth.rng(172).integers(0, experts, a)
+    meta = _routing_rows(ids)
+    x = synth.activations(a, cols, seed=173)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F32, x)
+    mt = api.Tensor.from_bits(d, meta.shape, meta)
+    exact = d.expert_project_quantized(xt, mt, w, cols, experts)
+    assert d.last_operation() == "expert_project_q4_k_factored"
+    full = oracle.expert_project(Q4_K, packed, experts, rows, cols, x, meta.view(np.float32), accumulate="f64")
+    assert_matmul_parity(exact.to_f32(), full, "exact f32 assignments")
+    d.set_tuning("gemm_f32_min_rows", 5)
+    try:
+        tiled = d.expert_project_quantized(xt, mt, w, cols, experts)
+        assert d.last_operation() == "expert_project_q4_k_grouped_mfma" and tiled.dtype == api.DType.F32
+    finally:
+        d.set_tuning("gemm_f32_min_rows", 0)
+    want = oracle.expert_project(Q4_K, packed, experts, rows, cols, oracle.round_storage(x, oracle.F16).reshape(a, cols),
+                                 meta.view(np.float32), weight_round=oracle.F16, accumulate="f64")
+    assert_matmul_parity(tiled.to_f32(), want, "f32 assignments through the f16 tiles")

@@ -165,6 +165,7 @@ class DType(enum.IntEnum):
 
 class QuantizationFormat(enum.Enum):
     Q4_K = 12
+    Q5_K = 13   # dequantize, embedding gather and the per-row (GEMV) kernels; no tile kernels yet
     Q6_K = 14
 
     @staticmethod
@@ -181,7 +182,7 @@ class QuantizationFormat(enum.Enum):
         return 256
 
     def block_bytes(self) -> int:
-        return 144 if self == QuantizationFormat.Q4_K else 210
+        return {12: 144, 13: 176, 14: 210}[self.value]
 
 
 def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:

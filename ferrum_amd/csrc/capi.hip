@@ -360,7 +360,7 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
     *out = nullptr;
     const size_t bb = block_bytes(ggml_type);
     if (bb == 0) return fail(FH_ERR_GGUF, "unsupported quantized weight type %u", ggml_type);
-    const char* name = ggml_type == kQ4K ? "Q4_K" : "Q6_K";
+    const char* name = ggml_type == kQ4K ? "Q4_K" : ggml_type == kQ5K ? "Q5_K" : "Q6_K";
     if (rows == 0 || cols == 0 || cols % 256 != 0)
         return fail(FH_ERR_SHAPE, "%s matrix requires nonempty rows and columns divisible by block size 256",
                     name);
@@ -377,8 +377,8 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
                     (unsigned long long)byte_len);
     const uint8_t* p = static_cast<const uint8_t*>(packed);
     for (size_t off = 0; off < packed_len; off += bb) {
-        bool ok = ggml_type == kQ4K ? (f16_finite(p + off) && f16_finite(p + off + 2))
-                                    : f16_finite(p + off + 208);
+        bool ok = ggml_type == kQ6K ? f16_finite(p + off + 208)
+                                    : (f16_finite(p + off) && f16_finite(p + off + 2));
         if (!ok) return fail(FH_ERR_WEIGHT, "%s scale must be finite", name);
     }
     FH_HIP(hipSetDevice(device->ordinal));
@@ -495,7 +495,8 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
     // engine does from 5 rows (HybridModel::project, src/hybrid/engine.rs:3407-3500): the
     // activations are then rounded to f16 into the device scratch first.
     const int64_t f32_tile_rows = tuning(device, "gemm_f32_min_rows");
-    const bool f32_tile = !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
+    const bool tiles_exist = weight->ggml_type != kQ5K;   // Q5_K runs on the per-row kernel at every M
+    const bool f32_tile = tiles_exist && !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
                           ((uintptr_t)xr.begin & 15u) == 0;
     const void* tile_x = xr.begin;
     if (f32_tile) {
@@ -505,7 +506,8 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
                             reinterpret_cast<uint16_t*>(scratch_data(device)), (size_t)m * k);
         tile_x = scratch_data(device);
     }
-    const bool tile = f32_tile || (!silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32);
+    const bool tile = f32_tile || (tiles_exist && !silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") &&
+                                   x->dtype != FH_F32);
     if (tile) {
         GemmArgs a{};
         a.ggml_type = weight->ggml_type;
@@ -540,7 +542,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         st = prepare_gemv(device, a);
         if (st != FH_OK) return st;
         const char* name = launch_gemv(device->stream, a);
-        if (m > 1) name = weight->ggml_type == kQ4K ? "q4_k_gemm" : "q6_k_gemm";
+        if (m > 1) name = weight->ggml_type == kQ4K ? "q4_k_gemm" : weight->ggml_type == kQ5K ? "q5_k_gemm" : "q6_k_gemm";
         device->last_operation = name;
     }
     FH_HIP(hipGetLastError());
@@ -706,7 +708,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
     const bool f32_grouped = x->dtype == FH_F32 && f32_rows > 0 && assignments >= (uint64_t)f32_rows &&
                              ((uintptr_t)xr.begin & 15u) == 0;
-    if (form == FH_INPUT_ROWS && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
+    if (form == FH_INPUT_ROWS && weight->ggml_type != kQ5K && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
         assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
         // grouped form: every expert's weights are streamed once for all of its assignments
         const size_t words = ((size_t)weight->experts + 1 + assignments + 3) & ~(size_t)3;

@@ -17,6 +17,8 @@ __device__ __forceinline__ float weight_at(const uint8_t* w, size_t row, uint32_
                                            uint32_t blocks) {
     if constexpr (TYPE == kQ4K) {
         return q4k_weight(w, row, column, blocks);
+    } else if constexpr (TYPE == kQ5K) {
+        return q5k_weight(w, row, column, blocks);
     } else {
         return q6k_weight(w, row, column, blocks);
     }
@@ -94,6 +96,11 @@ const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, 
                            static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
         return "dequantize_q4_k";
     }
+    if (ggml_type == kQ5K) {
+        hipLaunchKernelGGL(dequantize_kernel<kQ5K>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
+        return "dequantize_q5_k";
+    }
     hipLaunchKernelGGL(dequantize_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
                        static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
     return "dequantize_q6_k";
@@ -108,6 +115,12 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                            static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
                            out_dtype);
         return "embedding_gather_q4_k";
+    }
+    if (ggml_type == kQ5K) {
+        hipLaunchKernelGGL(embedding_gather_kernel<kQ5K>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
+                           out_dtype);
+        return "embedding_gather_q5_k";
     }
     hipLaunchKernelGGL(embedding_gather_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
                        static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,

@@ -134,6 +134,27 @@ __device__ __forceinline__ float q4k_weight(const uint8_t* w, size_t row, uint32
     return b - c;
 }
 
+// ---- Q5_K (176 B: f16 d, f16 dmin, scales[12], qh[32], qs[128]) -----------------
+
+// q5_k_weight (src/metal/shaders/ops.metal:846-857): the Q4_K value with bit
+// `group` of qh[lane] as the quant's fifth bit.
+__device__ __forceinline__ float q5k_weight(const uint8_t* w, size_t row, uint32_t column,
+                                            uint32_t blocks) {
+    const uint8_t* block = w + (row * blocks + (column >> 8)) * 176;
+    uint32_t within = column & 255u, group = within >> 5, lane = within & 31u, chunk = within >> 6;
+    uint32_t byte = block[48 + chunk * 32 + lane];
+    uint32_t q = (group & 1u) ? (byte >> 4) : (byte & 15u);
+    q |= (((uint32_t)block[16 + lane] >> group) & 1u) << 4;
+    float d = f16_bits_to_f32(block[0] | (block[1] << 8));
+    float dmin = f16_bits_to_f32(block[2] | (block[3] << 8));
+    uint32_t sc, mn;
+    q4k_scale_min(block + 4, group, sc, mn);
+    float a = d * (float)sc;
+    float b = a * (float)q;
+    float c = dmin * (float)mn;
+    return b - c;
+}
+
 // ---- Q6_K (210 B: ql[128], qh[64], int8 scales[16], f16 d) ---------------------
 
 __device__ __forceinline__ float q6k_weight(const uint8_t* w, size_t row, uint32_t column,

@@ -51,7 +51,7 @@ __device__ __forceinline__ float hi_half(uint32_t v) { return (float)__builtin_b
 // float4 index q (0..63) inside a super-block -> LDS slot u*4 + c (lane c, position u)
 template <uint32_t TYPE>
 __device__ __forceinline__ uint32_t x_slot(uint32_t q) {
-    if constexpr (TYPE == kQ4K) {
+    if constexpr (TYPE != kQ6K) {
         // element 64c + 32hi + 4u' : lane c, float4 u = 8hi + u'
         return (q & 15u) * 4u + (q >> 4);
     } else {
@@ -99,6 +99,54 @@ struct Frag<kQ4K> {
         a_lo += b_lo;
         a_hi += b_hi;
         // low nibbles were q * 2^-24, high nibbles 16q * 2^-24
+        float scaled = fmaf(sc_lo * 16777216.f, a_lo, (sc_hi * 1048576.f) * a_hi);
+        float offset = fmaf(mn_lo, s.x + s.y, mn_hi * (s.z + s.w));
+        return fmaf(d, scaled, -(dmin * offset));
+    }
+};
+
+// Q5_K: the Q4_K lane layout plus the block's 32 qh bytes; bits 2c and 2c + 1 of
+// qh[l] are the fifth bits of chunk c's low- and high-nibble weights at position l.
+// All four lanes of a block fetch the same 32 qh bytes.
+template <>
+struct Frag<kQ5K> {
+    uint4 hdr, ha, hb, qa, qb;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+        ha = *reinterpret_cast<const uint4*>(block + 16);
+        hb = *reinterpret_cast<const uint4*>(block + 32);
+        qa = *reinterpret_cast<const uint4*>(block + 48 + 32 * c);
+        qb = *reinterpret_cast<const uint4*>(block + 64 + 32 * c);
+    }
+    __device__ __forceinline__ float dot(const float4* xc, float4 s, uint32_t c) const {
+        float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc_lo, sc_hi, mn_lo, mn_hi;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, c, sc_lo, sc_hi, mn_lo, mn_hi);
+        float a_lo = 0.f, a_hi = 0.f, b_lo = 0.f, b_hi = 0.f;
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        const uint32_t h[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        const uint32_t shift = 2u * c;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            float4 xl = xc[t * 4], xh = xc[(8 + t) * 4];
+            uint32_t w0 = q[t], w1 = q[t] >> 8;
+            uint32_t p0 = h[t] >> shift, p1 = p0 >> 8;   // fifth bits: bit 0 low group, bit 1 high group
+            // low nibble | fifth bit << 4 reads as q * 2^-24; high nibble in place | fifth bit << 8 as 16q * 2^-24
+            uint32_t l02 = (w0 & 0x000f000fu) | ((p0 & 0x00010001u) << 4);
+            uint32_t l13 = (w1 & 0x000f000fu) | ((p1 & 0x00010001u) << 4);
+            uint32_t h02 = (w0 & 0x00f000f0u) | ((p0 & 0x00020002u) << 7);
+            uint32_t h13 = (w1 & 0x00f000f0u) | ((p1 & 0x00020002u) << 7);
+            a_lo = fmaf(lo_half(l02), xl.x, a_lo);
+            b_lo = fmaf(lo_half(l13), xl.y, b_lo);
+            a_lo = fmaf(hi_half(l02), xl.z, a_lo);
+            b_lo = fmaf(hi_half(l13), xl.w, b_lo);
+            a_hi = fmaf(lo_half(h02), xh.x, a_hi);
+            b_hi = fmaf(lo_half(h13), xh.y, b_hi);
+            a_hi = fmaf(hi_half(h02), xh.z, a_hi);
+            b_hi = fmaf(hi_half(h13), xh.w, b_hi);
+        }
+        a_lo += b_lo;
+        a_hi += b_hi;
         float scaled = fmaf(sc_lo * 16777216.f, a_lo, (sc_hi * 1048576.f) * a_hi);
         float offset = fmaf(mn_lo, s.x + s.y, mn_hi * (s.z + s.w));
         return fmaf(d, scaled, -(dmin * offset));
@@ -204,7 +252,7 @@ struct Params {
 template <uint32_t TYPE, int BS, int IT>
 __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     constexpr int RS = 16 / BS;
-    constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
+    constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
     extern __shared__ float4 xs[];  // seg_len * kXStride float4, then seg_len * 16 run sums
     __shared__ uint32_t last_flag;
     float* rsum = reinterpret_cast<float*>(xs + (size_t)p.seg_len * kXStride);
@@ -419,12 +467,18 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     p.x_rows = a.x_rows;
     const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
     dim3 grid(plan.tiles, plan.segments, a.m);
-    LaunchFn fn = a.ggml_type == kQ4K ? pick<kQ4K>(plan.bs, plan.it) : pick<kQ6K>(plan.bs, plan.it);
+    LaunchFn fn = a.ggml_type == kQ4K   ? pick<kQ4K>(plan.bs, plan.it)
+                  : a.ggml_type == kQ5K ? pick<kQ5K>(plan.bs, plan.it)
+                                        : pick<kQ6K>(plan.bs, plan.it);
     fn(grid, lds, s, p);
-    if (a.metadata != nullptr)
-        return a.ggml_type == kQ4K ? "expert_project_q4_k_factored" : "expert_project_q6_k_factored";
-    if (plan.segments > 1) return a.ggml_type == kQ4K ? "q4_k_gemv_ksplit" : "q6_k_gemv_ksplit";
-    return a.ggml_type == kQ4K ? "q4_k_gemv_factored" : "q6_k_gemv_factored";
+    const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : 2;
+    static const char* const expert_names[3] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
+                                                "expert_project_q6_k_factored"};
+    static const char* const ksplit_names[3] = {"q4_k_gemv_ksplit", "q5_k_gemv_ksplit", "q6_k_gemv_ksplit"};
+    static const char* const factored_names[3] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored"};
+    if (a.metadata != nullptr) return expert_names[f];
+    if (plan.segments > 1) return ksplit_names[f];
+    return factored_names[f];
 }
 
 }  // namespace fh

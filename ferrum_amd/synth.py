@@ -17,8 +17,8 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q6_K = 12, 14
-BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+Q4_K, Q5_K, Q6_K = 12, 13, 14
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210}
 
 
 def rng(seed: int, stream: int = 0) -> np.random.Generator:
@@ -50,6 +50,28 @@ def q4_k_blocks(count: int, g: np.random.Generator) -> np.ndarray:
     blocks[:, 4:16] = pack_q4_k_scales(sc, mn)
     nib = g.integers(0, 16, (count, 4, 2, 32), dtype=np.uint8)      # [chunk][low/high][lane]
     blocks[:, 16:] = (nib[:, :, 0, :] | (nib[:, :, 1, :] << 4)).reshape(count, 128)
+    return blocks
+
+
+def q5_k_blocks(count: int, g: np.random.Generator) -> np.ndarray:
+    """Q4_K's header and scales, then qh[32] (bit 2*chunk + half of byte l is the fifth bit
+    of that group's weight l) and qs[128]."""
+    blocks = np.empty((count, 176), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(count)) * 0.005).astype(np.float32).astype(np.float16)
+    dmin = (np.abs(g.standard_normal(count)) * 0.005).astype(np.float32).astype(np.float16)
+    blocks[:, 0:2] = d.view(np.uint8).reshape(count, 2)
+    blocks[:, 2:4] = dmin.view(np.uint8).reshape(count, 2)
+    sc = g.integers(0, 64, (count, 8), dtype=np.uint8)
+    mn = g.integers(0, 64, (count, 8), dtype=np.uint8)
+    blocks[:, 4:16] = pack_q4_k_scales(sc, mn)
+    q = g.integers(0, 32, (count, 4, 2, 32), dtype=np.uint8)        # [chunk][low/high][lane]
+    low, top = q & 15, q >> 4
+    blocks[:, 48:] = (low[:, :, 0, :] | (low[:, :, 1, :] << 4)).reshape(count, 128)
+    qh = np.zeros((count, 32), dtype=np.uint8)
+    for chunk in range(4):
+        for half in range(2):
+            qh |= top[:, chunk, half, :] << (2 * chunk + half)
+    blocks[:, 16:48] = qh
     return blocks
 
 
@@ -86,6 +108,8 @@ def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> 
     g = rng(seed, stream)
     if ggml_type == Q4_K:
         return q4_k_blocks(count, g).reshape(-1)
+    if ggml_type == Q5_K:
+        return q5_k_blocks(count, g).reshape(-1)
     if ggml_type == Q6_K:
         return q6_k_blocks(count, g).reshape(-1)
     raise ValueError(f"unsupported ggml type {ggml_type}")

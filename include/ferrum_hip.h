@@ -55,7 +55,7 @@ enum {
 enum { FH_F32 = 0, FH_F16 = 1, FH_BF16 = 2 };
 
 /* GGML type ids of the supported formats (src/quantization.rs:24-49). */
-enum { FH_GGML_Q4_K = 12, FH_GGML_Q6_K = 14 };
+enum { FH_GGML_Q4_K = 12, FH_GGML_Q5_K = 13, FH_GGML_Q6_K = 14 };
 
 typedef struct fh_device fh_device;
 typedef struct fh_buffer fh_buffer;

@@ -17,7 +17,7 @@
  *       cases, bf16 ties/NaN cases of tests/correctness.rs:300-318.
  *   fo_q4_k_scale_min      pinned: three restatements agree (direct form,
  *       llama.cpp kmask word form, brute force over all byte pairs).
- *   fo_dequantize (block form) and fo_weight (per-element form)
+ *   fo_dequantize (block form) and fo_weight (per-element form), Q4_K, Q5_K, Q6_K
  *                          pinned: both forms agree bitwise on the
  *       reference's closed-form fixtures; exact-rational step-by-step
  *       rounding on a (d, sc, m, q) grid; Q3_K -> Q6_K value identity.
@@ -49,6 +49,7 @@
 #include <string.h>
 
 #define FO_Q4_K 12u
+#define FO_Q5_K 13u
 #define FO_Q6_K 14u
 
 /* ---------------------------------------------------------------- scalars */
@@ -144,6 +145,7 @@ void fo_round_storage_array(const float* in, size_t n, uint32_t dtype, float* ou
 /* src/quantization.rs:50-74: 256 weights per super-block, 144 / 210 bytes. */
 size_t fo_block_bytes(uint32_t ggml_type) {
     if (ggml_type == FO_Q4_K) return 144;
+    if (ggml_type == FO_Q5_K) return 176;
     if (ggml_type == FO_Q6_K) return 210;
     return 0;
 }
@@ -189,6 +191,34 @@ static void dequant_q4_k_block(const uint8_t* b, float* out) {
     }
 }
 
+/* Block form, Q5_K (176 B: d, dmin, scales[12], qh[32], qs[128]): the Q4_K
+ * walk with bit (2*chunk + half) of qh[l] as the quant's fifth bit
+ * (src/diffusion/tests.rs:811-836, `high` branch). */
+static void dequant_q5_k_block(const uint8_t* b, float* out) {
+    float d = fo_f16_to_f32(le16(b));
+    float dmin = fo_f16_to_f32(le16(b + 2));
+    const uint8_t* scales = b + 4;
+    const uint8_t* qh = b + 16;
+    const uint8_t* qs = b + 48;
+    for (int chunk = 0; chunk < 4; chunk++) {
+        const uint8_t* q = qs + 32 * chunk;
+        for (int half = 0; half < 2; half++) {
+            uint32_t sc, mn;
+            fo_q4_k_scale_min(scales, (uint32_t)(2 * chunk + half), &sc, &mn);
+            float fsc = (float)sc, fmn = (float)mn;
+            uint8_t bit = (uint8_t)(1u << (2 * chunk + half));
+            for (int l = 0; l < 32; l++) {
+                uint32_t low = half == 0 ? (q[l] & 15u) : (uint32_t)(q[l] >> 4);
+                uint32_t top = (qh[l] & bit) ? 16u : 0u;
+                float scaled = d * fsc;
+                float value = scaled * (float)(low + top);
+                float offset = dmin * fmn;
+                *out++ = value - offset;
+            }
+        }
+    }
+}
+
 /* Block form, Q6_K: ggml dequantize_row_q6_K restated at
  * src/diffusion/tests.rs:843-864 and src/hybrid/iq_tests.rs:1481-1500.
  * Expression order (d*scale)*q. */
@@ -217,16 +247,22 @@ static void dequant_q6_k_block(const uint8_t* b, float* out) {
     }
 }
 
+static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) {
+    if (ggml_type == FO_Q4_K)
+        dequant_q4_k_block(block, out);
+    else if (ggml_type == FO_Q5_K)
+        dequant_q5_k_block(block, out);
+    else
+        dequant_q6_k_block(block, out);
+}
+
 /* Dequantize a packed row-major [rows, cols] matrix to f32 (block form). */
 int fo_dequantize(uint32_t ggml_type, const uint8_t* packed, size_t rows, size_t cols, float* out) {
     size_t bb = fo_block_bytes(ggml_type);
     if (bb == 0 || cols % 256 != 0) return 1;
     size_t blocks = rows * (cols / 256);
     for (size_t i = 0; i < blocks; i++) {
-        if (ggml_type == FO_Q4_K)
-            dequant_q4_k_block(packed + i * bb, out + i * 256);
-        else
-            dequant_q6_k_block(packed + i * bb, out + i * 256);
+        dequant_block(ggml_type, packed + i * bb, out + i * 256);
     }
     return 0;
 }
@@ -244,6 +280,23 @@ float fo_weight(uint32_t ggml_type, const uint8_t* packed, size_t row, size_t co
         uint32_t chunk = within >> 6;
         uint8_t byte = block[16 + chunk * 32 + lane];
         uint32_t q = (group & 1) == 0 ? (uint32_t)(byte & 15) : (uint32_t)(byte >> 4);
+        float d = fo_f16_to_f32(le16(block));
+        float dmin = fo_f16_to_f32(le16(block + 2));
+        uint32_t sc, mn;
+        fo_q4_k_scale_min(block + 4, group, &sc, &mn);
+        float a = d * (float)sc;
+        float b = a * (float)q;
+        float c = dmin * (float)mn;
+        return b - c;
+    }
+    if (ggml_type == FO_Q5_K) {
+        /* q5_k_weight (ops.metal:846-857; CPU twin src/ops/transformer.rs:2946-2952) */
+        const uint8_t* block = packed + (row * blocks + block_index) * 176;
+        uint32_t chunk = within >> 6;
+        uint8_t byte = block[48 + chunk * 32 + lane];
+        uint32_t nibble = (group & 1) == 0 ? (uint32_t)(byte & 15) : (uint32_t)(byte >> 4);
+        uint32_t high = ((uint32_t)block[16 + lane] >> group) & 1u;
+        uint32_t q = nibble | (high << 4);
         float d = fo_f16_to_f32(le16(block));
         float dmin = fo_f16_to_f32(le16(block + 2));
         uint32_t sc, mn;
@@ -272,7 +325,7 @@ int fo_validate_payload(uint32_t ggml_type, const uint8_t* payload, size_t len) 
     if (bb == 0 || len % bb != 0) return 1;
     for (size_t off = 0; off < len; off += bb) {
         const uint8_t* b = payload + off;
-        if (ggml_type == FO_Q4_K) {
+        if (ggml_type == FO_Q4_K || ggml_type == FO_Q5_K) {
             if (!isfinite(fo_f16_to_f32(le16(b))) || !isfinite(fo_f16_to_f32(le16(b + 2)))) return 2;
         } else {
             if (!isfinite(fo_f16_to_f32(le16(b + 208)))) return 2;
@@ -303,10 +356,7 @@ static void* project_worker(void* arg) {
     for (size_t row = j->row_begin; row < j->row_end; row++) {
         const uint8_t* src = j->packed + row * blocks * bb;
         for (size_t b = 0; b < blocks; b++) {
-            if (j->ggml_type == FO_Q4_K)
-                dequant_q4_k_block(src + b * bb, w + b * 256);
-            else
-                dequant_q6_k_block(src + b * bb, w + b * 256);
+            dequant_block(j->ggml_type, src + b * bb, w + b * 256);
         }
         if (j->weight_round)
             for (size_t c = 0; c < j->k; c++) w[c] = fo_round_storage(w[c], (uint32_t)j->weight_round);
@@ -560,10 +610,7 @@ int fo_expert_project(uint32_t ggml_type, const uint8_t* packed, size_t experts,
             if (expert < experts) {
                 const uint8_t* src = packed + ((size_t)expert * rows + r) * blocks * bb;
                 for (size_t b = 0; b < blocks; b++) {
-                    if (ggml_type == FO_Q4_K)
-                        dequant_q4_k_block(src + b * bb, w + b * 256);
-                    else
-                        dequant_q6_k_block(src + b * bb, w + b * 256);
+                    dequant_block(ggml_type, src + b * bb, w + b * 256);
                 }
                 if (weight_round)
                     for (size_t c = 0; c < k; c++) w[c] = fo_round_storage(w[c], (uint32_t)weight_round);

@@ -6,6 +6,7 @@ formulas.  Those formulas are restated here so the same bytes and the same
 per-element expectations exist without running the reference:
 
 * ``q4k_packed`` / ``q4k_value``   src/ops/transformer.rs:2833-2956 (qk_tests)
+* ``q5k_packed`` / ``q5k_value``   the Q5_K branch of the same tests (:2843-2847, 2887-2892, 2946-2952)
 * ``q6k_packed`` / ``q6k_value``   src/ops/transformer.rs:4102-4169 (q6_k_tests)
 * ``qk_q6_packed`` / ``qk_q6_value``  the Q6_K branch inside qk_tests
                                    (src/ops/transformer.rs:2863-2878, 2924-2936)
@@ -21,7 +22,7 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 F = np.float32
 
 
@@ -71,6 +72,37 @@ def q4k_value(row: int, column: int) -> np.float32:
     d, dmin = _qk_q4_parameters(row)
     scale, minimum = _unpack_scale_min(_qk_scales(row, block), group)
     return F(F(F(d * F(scale)) * F(nibble)) - F(dmin * F(minimum)))
+
+
+def _qk_q5_parameters(block: int):
+    return F(0.001953125) + F(block) / F(4096.0), F(0.0078125)
+
+
+def q5k_packed(rows: int, columns: int) -> np.ndarray:
+    out = bytearray()
+    for row in range(rows):
+        for block in range(columns // 256):
+            d, dmin = _qk_q5_parameters(block)
+            out += _f16_bytes(d) + _f16_bytes(dmin)
+            out += _qk_scales(row, block).tobytes()
+            out += _qk_qbyte(row + 7, block, np.arange(32)).astype(np.uint8).tobytes()
+            out += _qk_qbyte(row, block, np.arange(128)).astype(np.uint8).tobytes()
+    return np.frombuffer(bytes(out), dtype=np.uint8).copy()
+
+
+def q5k_value(row: int, column: int) -> np.float32:
+    block, within = divmod(column, 256)
+    group, lane, chunk = within // 32, within % 32, within // 64
+    byte = _qk_qbyte(row, block, chunk * 32 + lane)
+    nibble = byte & 15 if group % 2 == 0 else byte >> 4
+    high = (_qk_qbyte(row + 7, block, lane) >> group) & 1
+    d, dmin = _qk_q5_parameters(block)
+    scale, minimum = _unpack_scale_min(_qk_scales(row, block), group)
+    return F(F(F(d * F(scale)) * F(nibble | (high << 4))) - F(dmin * F(minimum)))
+
+
+def q5k_dense(rows: int, columns: int) -> np.ndarray:
+    return np.array([[q5k_value(r, c) for c in range(columns)] for r in range(rows)], dtype=F)
 
 
 def q4k_dense(rows: int, columns: int) -> np.ndarray:

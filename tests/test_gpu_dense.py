@@ -435,3 +435,79 @@ def test_lm_head_projection_then_argmax_picks_the_oracle_token(api, d):
     top2 = np.sort(want[0])[-2:]
     if top2[1] - top2[0] > 1e-3 * abs(top2[1]):      # unambiguous in the oracle too
         assert picked[0] == int(np.argmax(want))
+
+
+# ----------------------------------------------------------------------- Q5_K
+
+Q5_K = 13
+
+
+def test_q5_k_dequantize_and_gather_are_bit_exact(api, d):
+    for rows, cols, packed in ((5, 512, fx.q5k_packed(5, 512)), (133, 2560, fx.q5k_packed(133, 2560)),
+                               (257, 1024, synth.matrix(Q5_K, 257, 1024, seed=181))):
+        w = qm(api, d, Q5_K, rows, cols, packed)
+        assert w.byte_size() == rows * (cols // 256) * 176
+        want = oracle.dequantize(Q5_K, packed, rows, cols)
+        assert np.array_equal(bits(d.dequantize(w).to_f32()), bits(want))
+        assert np.array_equal(bits(d.dequantize(w, api.DType.BF16).to_f32()),
+                              bits(oracle.round_storage(want, oracle.BF16).reshape(rows, cols)))
+        ids = [rows - 1, 0, 3]
+        got = d.embedding_gather_quantized(w, ids, api.DType.F32)
+        assert got.operation == "embedding_gather_q5_k"
+        assert np.array_equal(bits(got.tensor.to_f32()), bits(want[ids]))
+
+
+def test_q5_k_gemv_and_small_batches_replay_the_reference_cases(api, d):
+    # q4_k_and_q5_k_gemv_gemm_cover_blocks_and_batch_tails (src/ops/transformer.rs:2982-3002):
+    # (N, K) = (5, 512), M in 1..7 except 6, f32, abs <= 2e-4 against the f32-sequential sum
+    n, k = 5, 512
+    packed = fx.q5k_packed(n, k)
+    w = qm(api, d, Q5_K, n, k, packed)
+    for m in (1, 2, 3, 4, 5, 7):
+        x = fx.q4k_input(m, k)
+        out = d.project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x), w)
+        assert out.operation == ("q5_k_gemv_factored" if m == 1 else "q5_k_gemm")
+        want = oracle.project(Q5_K, packed, n, k, x, accumulate="f32")
+        assert np.abs(out.tensor.to_f32() - want).max() <= 2e-4, m
+
+
+@pytest.mark.parametrize("n,k,m,dtype_name", [(4099, 5120, 1, "F32"), (1003, 4864, 1, "F32"), (5120, 17408, 1, "F32"),
+                                              (515, 1280, 3, "F32"), (515, 1280, 1, "F16"), (515, 1280, 4, "BF16")])
+def test_q5_k_projection_matches_the_f64_oracle(api, d, n, k, m, dtype_name):
+    dtype = api.DType[dtype_name]
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype_name]
+    packed = synth.matrix(Q5_K, n, k, seed=n + k)
+    w = qm(api, d, Q5_K, n, k, packed)
+    x = oracle.round_storage(synth.activations(m, k, seed=11), code).reshape(m, k)
+    out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), synth.rng(12).integers(0, n, 64)]))
+    want = oracle_columns(Q5_K, packed, n, k, rows, x, accumulate="f64")
+    assert_matmul_parity(out.tensor.to_f32()[:, rows], want, f"q5_k {n}x{k} m={m} {dtype_name}")
+    if k == 17408:
+        assert out.operation == "q5_k_gemv_ksplit"
+
+
+def test_q5_k_expert_projection_and_validation(api, d):
+    experts, rows, cols, a = 4, 40, 768, 9
+    packed = synth.matrix(Q5_K, experts * rows, cols, seed=191)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(Q5_K), experts, rows, cols)
+    meta = np.zeros((a, 3), dtype=np.uint32)
+    meta[:, 0] = [0, 3, 1, 1, 2, 7, 0, 3, 2]          # 7 does not exist: a zero row
+    meta[:, 1] = np.arange(a)
+    meta[:, 2] = np.float32(1.0).view(np.uint32)
+    x = synth.activations(a, cols, seed=192)
+    got = d.expert_project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x),
+                                     api.Tensor.from_bits(d, meta.shape, meta), w, cols, experts)
+    assert d.last_operation() == "expert_project_q5_k_factored"
+    got = got.to_f32()
+    safe = meta.copy(); safe[5, 0] = 0
+    want = oracle.expert_project(Q5_K, packed, experts, rows, cols, x, safe.view(np.float32), accumulate="f64")
+    valid = np.arange(a) != 5
+    assert np.all(got[5] == 0)
+    assert_matmul_parity(got[valid], want[valid], "q5_k expert projection")
+    bad = packed.copy()
+    bad[1] = 0x7c                                       # d = +inf in the first block
+    with pytest.raises(api.WeightError):
+        api.QuantizedMatrix.from_bytes(d, experts * rows, cols, api.QuantizationFormat(Q5_K), bad)
+    with pytest.raises(api.Error):
+        api.QuantizedMatrix.from_bytes(d, experts * rows, cols, api.QuantizationFormat(Q5_K), packed[:-1])

@@ -580,3 +580,45 @@ def test_shared_gate_and_combine_with_a_shared_expert():
     assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
     plain = oracle.expert_combine(down, meta, tokens, hidden, top_k)
     assert np.array_equal(oracle.expert_combine_shared(down, meta, tokens, hidden, top_k, np.zeros_like(shared)), plain)
+
+
+# ------------------------------------------------------------------ Q5_K
+
+Q5_K = 13
+
+
+@pytest.mark.parametrize("rows,cols", [(5, 512), (7, 256), (3, 1024)])
+def test_q5_k_block_decoder_equals_reference_closed_form(rows, cols):
+    # the Q5_K branch of the reference's qk_tests (src/ops/transformer.rs:2843-2952)
+    packed = fx.q5k_packed(rows, cols)
+    assert packed.size == rows * (cols // 256) * 176 == rows * (cols // 256) * oracle.block_bytes(Q5_K)
+    dense = oracle.dequantize(Q5_K, packed, rows, cols)
+    assert np.array_equal(bits(dense), bits(fx.q5k_dense(rows, cols)))
+
+
+def test_q5_k_block_form_per_element_form_and_the_q4_k_special_case_agree():
+    from ferrum_amd import synth
+    rows, cols = 6, 768
+    packed = synth.matrix(Q5_K, rows, cols, seed=71)
+    dense = oracle.dequantize(Q5_K, packed, rows, cols)
+    rng = np.random.default_rng(6)
+    for _ in range(3000):
+        r, c = int(rng.integers(rows)), int(rng.integers(cols))
+        assert bits(np.float32(oracle.weight(Q5_K, packed, r, c, cols))) == bits(dense[r, c])
+    # with every fifth bit clear a Q5_K block is the Q4_K block with the same header and nibbles
+    blocks = packed.reshape(-1, 176).copy()
+    blocks[:, 16:48] = 0
+    as_q4 = np.concatenate([blocks[:, :16], blocks[:, 48:]], axis=1)
+    assert np.array_equal(bits(oracle.dequantize(Q5_K, blocks.reshape(-1), rows, cols)),
+                          bits(oracle.dequantize(Q4_K, as_q4.reshape(-1), rows, cols)))
+    # and setting them all adds 16 * d * sc to every weight
+    blocks[:, 16:48] = 255
+    up = oracle.dequantize(Q5_K, blocks.reshape(-1), rows, cols).astype(np.float64)
+    base = oracle.dequantize(Q4_K, as_q4.reshape(-1), rows, cols).astype(np.float64)
+    d = blocks[:, 0:2].copy().view(np.float16).astype(np.float64).reshape(rows, cols // 256, 1)
+    sc = np.array([[oracle.q4_k_scale_min(b[4:16], g)[0] for g in range(8)] for b in blocks], dtype=np.float64)
+    step = (16 * d * sc.reshape(rows, cols // 256, 8)).repeat(32, axis=2).reshape(rows, cols)
+    assert np.abs(up - base - step).max() <= 1e-6 * np.abs(step).max()
+    x = fx.xorshift_uniform(3 * cols, 9).reshape(3, cols)
+    want = x.astype(np.float64) @ dense.astype(np.float64).T
+    assert np.abs(oracle.project(Q5_K, packed, rows, cols, x, accumulate="f64") - want).max() <= 1e-6 * np.abs(want).max()

@@ -165,7 +165,7 @@ class DType(enum.IntEnum):
 
 class QuantizationFormat(enum.Enum):
     Q4_K = 12
-    Q5_K = 13   # dequantize, embedding gather and the per-row (GEMV) kernels; no tile kernels yet
+    Q5_K = 13
     Q6_K = 14
 
     @staticmethod

@@ -495,8 +495,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
     // engine does from 5 rows (HybridModel::project, src/hybrid/engine.rs:3407-3500): the
     // activations are then rounded to f16 into the device scratch first.
     const int64_t f32_tile_rows = tuning(device, "gemm_f32_min_rows");
-    const bool tiles_exist = weight->ggml_type != kQ5K;   // Q5_K runs on the per-row kernel at every M
-    const bool f32_tile = tiles_exist && !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
+    const bool f32_tile = !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
                           ((uintptr_t)xr.begin & 15u) == 0;
     const void* tile_x = xr.begin;
     if (f32_tile) {
@@ -506,8 +505,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
                             reinterpret_cast<uint16_t*>(scratch_data(device)), (size_t)m * k);
         tile_x = scratch_data(device);
     }
-    const bool tile = f32_tile || (tiles_exist && !silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") &&
-                                   x->dtype != FH_F32);
+    const bool tile = f32_tile || (!silu_mul && m >= (uint32_t)tuning(device, "gemm_min_rows") && x->dtype != FH_F32);
     if (tile) {
         GemmArgs a{};
         a.ggml_type = weight->ggml_type;
@@ -708,7 +706,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
     const bool f32_grouped = x->dtype == FH_F32 && f32_rows > 0 && assignments >= (uint64_t)f32_rows &&
                              ((uintptr_t)xr.begin & 15u) == 0;
-    if (form == FH_INPUT_ROWS && weight->ggml_type != kQ5K && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
+    if (form == FH_INPUT_ROWS && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
         assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
         // grouped form: every expert's weights are streamed once for all of its assignments
         const size_t words = ((size_t)weight->experts + 1 + assignments + 3) & ~(size_t)3;

@@ -72,6 +72,44 @@ struct RawW<kQ4K> {
     }
 };
 
+// Q5_K: Q4_K's walk with the fifth bits: bit 2c (low nibbles) and 2c + 1 (high
+// nibbles) of qh[l], l the position inside the chunk.
+template <>
+struct RawW<kQ5K> {
+    uint4 hdr, qs, qh;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c, uint32_t h) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+        qh = *reinterpret_cast<const uint4*>(block + 16 + 16 * h);
+        qs = *reinterpret_cast<const uint4*>(block + 48 + 32 * c + 16 * h);
+    }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t c, uint32_t (&out_lo)[8],
+                                           uint32_t (&out_hi)[8]) const {
+        float d = f16_bits_to_f32(hdr.x & 0xffffu);
+        float dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc0, sc1, mn0, mn1;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, c, sc0, sc1, mn0, mn1);
+        float a0 = d * sc0, b0 = dmin * mn0;
+        float a1 = d * sc1, b1 = dmin * mn1;
+        const uint32_t q[4] = {qs.x, qs.y, qs.z, qs.w};
+        const uint32_t p[4] = {qh.x, qh.y, qh.z, qh.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t bits = p[t] >> (2 * c);
+            uint32_t lo = (q[t] & 0x0f0f0f0fu) | ((bits & 0x01010101u) << 4);
+            uint32_t hi = ((q[t] >> 4) & 0x0f0f0f0fu) | ((bits & 0x02020202u) << 3);
+            float l0 = fmaf(a0, (float)(lo & 0xffu), -b0), l1 = fmaf(a0, (float)((lo >> 8) & 0xffu), -b0);
+            float l2 = fmaf(a0, (float)((lo >> 16) & 0xffu), -b0), l3 = fmaf(a0, (float)(lo >> 24), -b0);
+            float h0 = fmaf(a1, (float)(hi & 0xffu), -b1), h1 = fmaf(a1, (float)((hi >> 8) & 0xffu), -b1);
+            float h2 = fmaf(a1, (float)((hi >> 16) & 0xffu), -b1), h3 = fmaf(a1, (float)(hi >> 24), -b1);
+            out_lo[2 * t] = pack2<DT>(l0, l1);
+            out_lo[2 * t + 1] = pack2<DT>(l2, l3);
+            out_hi[2 * t] = pack2<DT>(h0, h1);
+            out_hi[2 * t + 1] = pack2<DT>(h2, h3);
+        }
+    }
+};
+
 // Q6_K: the 64-wide K slab c (0..3) of a block, weights 64c .. 64c+63, is
 // slices 2(c&1) and 2(c&1)+1 of half c>>1: the low nibbles (c even) or the
 // high nibbles (c odd) of all 64 ql bytes of that half.  Thread half h covers
@@ -140,7 +178,7 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
     constexpr int WI = TS / 64;  // 32-row tiles per wave
     __shared__ __attribute__((aligned(16))) uint16_t xs[TS * kLd];
     __shared__ __attribute__((aligned(16))) uint16_t ws[TS * kLd];
-    constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
+    constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n0 = blockIdx.x * TS, m0 = blockIdx.y * TS;
@@ -173,7 +211,7 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
     for (uint32_t step = 0; step < steps; ++step) {
         const uint32_t c = step & 3u;
         uint32_t lo[8], hi[8];
-        if constexpr (TYPE == kQ4K) {
+        if constexpr (TYPE != kQ6K) {
             raw.template decode<DT>(c, lo, hi);
         } else {
             raw.template decode<DT>(c, lo, hi, lh);
@@ -181,8 +219,8 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
         __syncthreads();  // previous step's fragment reads are done
         {
             // Q4_K: lo -> k 16h.., hi -> k 32+16h..;  Q6_K: lo -> k 32h.., hi -> k 32h+16..
-            uint32_t k_lo = TYPE == kQ4K ? 16 * lh : 32 * lh;
-            uint32_t k_hi = TYPE == kQ4K ? 32 + 16 * lh : 32 * lh + 16;
+            uint32_t k_lo = TYPE != kQ6K ? 16 * lh : 32 * lh;
+            uint32_t k_hi = TYPE != kQ6K ? 32 + 16 * lh : 32 * lh + 16;
             uint4* dst_lo = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_lo]);
             uint4* dst_hi = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_hi]);
             dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
@@ -254,14 +292,14 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c, uint32_t h,
                                               uint16_t* wrow_lds) {
     uint32_t lo[8], hi[8];
-    if constexpr (TYPE == kQ4K) {
+    if constexpr (TYPE != kQ6K) {
         raw.template decode<DT>(c, lo, hi);
     } else {
         raw.template decode<DT>(c, lo, hi, h);
     }
     // Q4_K: lo -> k 16h.., hi -> k 32+16h..;  Q6_K: lo -> k 32h.., hi -> k 32h+16..
-    const uint32_t k_lo = TYPE == kQ4K ? 16 * h : 32 * h;
-    const uint32_t k_hi = TYPE == kQ4K ? 32 + 16 * h : 32 * h + 16;
+    const uint32_t k_lo = TYPE != kQ6K ? 16 * h : 32 * h;
+    const uint32_t k_hi = TYPE != kQ6K ? 32 + 16 * h : 32 * h + 16;
     uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + k_lo);
     uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + k_hi);
     dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
@@ -309,6 +347,41 @@ struct BlockW<kQ4K> {
         const uint32_t w0 = dword(c, t), w1 = w0 >> 8;
         const uint32_t l02 = w0 & 0x000f000fu, h02 = w0 & 0x00f000f0u;
         const uint32_t l13 = w1 & 0x000f000fu, h13 = w1 & 0x00f000f0u;
+        out[0] = fma_pair<DT>(lo_half(l02), lo_half(l13), s.a_lo, s.b_lo);
+        out[1] = fma_pair<DT>(hi_half(l02), hi_half(l13), s.a_lo, s.b_lo);
+        out[2] = fma_pair<DT>(lo_half(h02), lo_half(h13), s.a_hi, s.b_hi);
+        out[3] = fma_pair<DT>(hi_half(h02), hi_half(h13), s.a_hi, s.b_hi);
+    }
+};
+
+template <>
+struct BlockW<kQ5K> {
+    static constexpr int kDwords = 4;
+    uint4 hdr, qh, q[4];
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+        qh = *reinterpret_cast<const uint4*>(block + 16 + 16 * h);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q[c] = *reinterpret_cast<const uint4*>(block + 48 + 32 * c + 16 * h);
+    }
+    using Scales = BlockW<kQ4K>::Scales;
+    __device__ __forceinline__ Scales scales(int c, uint32_t) const {
+        float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc0, sc1, mn0, mn1;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, (uint32_t)c, sc0, sc1, mn0, mn1);
+        return {(d * sc0) * 16777216.f, (d * sc1) * 1048576.f, -(dmin * mn0), -(dmin * mn1)};
+    }
+    // low nibble | fifth bit << 4 reads as q * 2^-24; high nibble in place | fifth bit << 8 as 16q * 2^-24
+    template <int DT>
+    __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
+        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
+        const uint32_t p[4] = {qh.x, qh.y, qh.z, qh.w};
+        const uint32_t w0 = v[t], w1 = w0 >> 8;
+        const uint32_t p0 = p[t] >> (2 * c), p1 = p0 >> 8;
+        const uint32_t l02 = (w0 & 0x000f000fu) | ((p0 & 0x00010001u) << 4);
+        const uint32_t l13 = (w1 & 0x000f000fu) | ((p1 & 0x00010001u) << 4);
+        const uint32_t h02 = (w0 & 0x00f000f0u) | ((p0 & 0x00020002u) << 7);
+        const uint32_t h13 = (w1 & 0x00f000f0u) | ((p1 & 0x00020002u) << 7);
         out[0] = fma_pair<DT>(lo_half(l02), lo_half(l13), s.a_lo, s.b_lo);
         out[1] = fma_pair<DT>(hi_half(l02), hi_half(l13), s.a_lo, s.b_lo);
         out[2] = fma_pair<DT>(lo_half(h02), lo_half(h13), s.a_hi, s.b_hi);
@@ -377,7 +450,7 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_block_slab(const BlockW<TYPE>& blk, int c, uint32_t h,
                                                   uint16_t* wrow_lds) {
     const auto s = blk.scales(c, h);
-    if constexpr (TYPE == kQ4K) {
+    if constexpr (TYPE != kQ6K) {
         uint32_t lo[8], hi[8];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -414,7 +487,7 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int c, uint32_t h, int t,
                                                    uint16_t* wrow_lds) {
     const auto s = blk.scales(c, h);
-    if constexpr (TYPE == kQ4K) {
+    if constexpr (TYPE != kQ6K) {
         uint32_t out[4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
@@ -444,7 +517,7 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
                                                                  uint32_t y_dtype, uint32_t cols,
                                                                  uint32_t tiles_m, uint32_t tiles_n) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-    constexpr uint32_t kBlockBytes = TYPE == kQ4K ? 144 : 210;
+    constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
     constexpr uint32_t kRowsW = 16 * NT;
     constexpr uint32_t kStage = kRowsW * kLd;  // halfs per buffer
     constexpr bool kExtra = NT > 8;                    // rows 128.. need a second decode task
@@ -473,7 +546,7 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
         const uint32_t er = 128 + (lane >> 3), eh = (lane >> 2) & 1u, et = lane & 3u;
         const uint8_t* esrc = w + (size_t)(n0 + (er < ncols ? er : ncols - 1)) * nb * kBlockBytes;
         // register sets: the block being decoded and the next one or two in flight
-        constexpr bool kDeep = TYPE == kQ4K;   // Q6_K sets are twice as large: one block ahead
+        constexpr bool kDeep = TYPE != kQ6K;   // Q6_K sets are twice as large: one block ahead
         BlockW<TYPE> cur, n1, n2, ecur, en1, en2;
         auto load_block = [&](BlockW<TYPE>& main, BlockW<TYPE>& extra, uint32_t b) {
             main.load(wsrc + (size_t)b * kBlockBytes, wh);
@@ -666,6 +739,10 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan); else launch_wide_nt<kQ4K, 2>(s, a, plan);
             return "q4_k_gemm_mfma_m256";
         }
+        if (a.ggml_type == kQ5K) {
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ5K, 1>(s, a, plan); else launch_wide_nt<kQ5K, 2>(s, a, plan);
+            return "q5_k_gemm_mfma_m256";
+        }
         if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
         return "q6_k_gemm_mfma_m256";
     }
@@ -691,6 +768,14 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             run(gemm_tile_kernel<kQ4K, 2, 128>, gemm_tile_kernel<kQ4K, 2, 64>);
         }
         return "q4_k_gemm_mfma";
+    }
+    if (a.ggml_type == kQ5K) {
+        if (a.x_dtype == FH_F16) {
+            run(gemm_tile_kernel<kQ5K, 1, 128>, gemm_tile_kernel<kQ5K, 1, 64>);
+        } else {
+            run(gemm_tile_kernel<kQ5K, 2, 128>, gemm_tile_kernel<kQ5K, 2, 64>);
+        }
+        return "q5_k_gemm_mfma";
     }
     if (a.x_dtype == FH_F16) {
         run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>);

@@ -78,6 +78,49 @@ struct Quarter<kQ4K> {
 };
 
 template <>
+struct Quarter<kQ5K> {
+    static constexpr uint32_t kBlockBytes = 176;
+    uint4 hdr, ha, hb, qa, qb;   // ha, hb: the block's 32 qh bytes (fifth bits, bit 2g low / 2g + 1 high nibbles)
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t g) {
+        hdr = *reinterpret_cast<const uint4*>(block);
+        ha = *reinterpret_cast<const uint4*>(block + 16);
+        hb = *reinterpret_cast<const uint4*>(block + 32);
+        qa = *reinterpret_cast<const uint4*>(block + 48 + 32 * g);
+        qb = *reinterpret_cast<const uint4*>(block + 64 + 32 * g);
+    }
+    static __device__ __forceinline__ uint32_t klocal(uint32_t g, int s) { return 64 * g + 8 * s; }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t g, uint4 (&a)[8]) const {
+        const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+        float sc0, sc1, mn0, mn1;
+        q4k_chunk_scales(hdr.y, hdr.z, hdr.w, g, sc0, sc1, mn0, mn1);
+        const float a_lo = (d * sc0) * 16777216.f, a_hi = (d * sc1) * 1048576.f;
+        const float b_lo = -(dmin * mn0), b_hi = -(dmin * mn1);
+        const uint32_t v[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        const uint32_t p[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+        uint32_t lo[16], hi[16];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t w0 = v[t], w1 = w0 >> 8;
+            const uint32_t p0 = p[t] >> (2 * g), p1 = p0 >> 8;
+            const uint32_t l02 = (w0 & 0x000f000fu) | ((p0 & 0x00010001u) << 4);
+            const uint32_t l13 = (w1 & 0x000f000fu) | ((p1 & 0x00010001u) << 4);
+            const uint32_t h02 = (w0 & 0x00f000f0u) | ((p0 & 0x00020002u) << 7);
+            const uint32_t h13 = (w1 & 0x00f000f0u) | ((p1 & 0x00020002u) << 7);
+            lo[2 * t] = fma_pair<DT>(lo_half(l02), lo_half(l13), a_lo, b_lo);
+            lo[2 * t + 1] = fma_pair<DT>(hi_half(l02), hi_half(l13), a_lo, b_lo);
+            hi[2 * t] = fma_pair<DT>(lo_half(h02), lo_half(h13), a_hi, b_hi);
+            hi[2 * t + 1] = fma_pair<DT>(hi_half(h02), hi_half(h13), a_hi, b_hi);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            a[s] = make_uint4(lo[4 * s], lo[4 * s + 1], lo[4 * s + 2], lo[4 * s + 3]);
+            a[4 + s] = make_uint4(hi[4 * s], hi[4 * s + 1], hi[4 * s + 2], hi[4 * s + 3]);
+        }
+    }
+};
+
+template <>
 struct Quarter<kQ6K> {
     static constexpr uint32_t kBlockBytes = 210;
     uint4 la, lb, ph, sc;
@@ -511,6 +554,10 @@ const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) launch_tt<kQ4K, 1>(s, a); else launch_tt<kQ4K, 2>(s, a);
         return grouped ? "expert_project_q4_k_grouped_mfma" : "q4_k_gemm_mfma_skinny";
+    }
+    if (a.ggml_type == kQ5K) {
+        if (a.x_dtype == FH_F16) launch_tt<kQ5K, 1>(s, a); else launch_tt<kQ5K, 2>(s, a);
+        return grouped ? "expert_project_q5_k_grouped_mfma" : "q5_k_gemm_mfma_skinny";
     }
     if (a.x_dtype == FH_F16) launch_tt<kQ6K, 1>(s, a); else launch_tt<kQ6K, 2>(s, a);
     return grouped ? "expert_project_q6_k_grouped_mfma" : "q6_k_gemm_mfma_skinny";

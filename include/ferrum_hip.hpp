@@ -98,7 +98,6 @@ inline float f16_bits_to_f32(uint16_t h) {
     return v;
 }
 
-// Q5_K: dequantize, embedding gather and the per-row (GEMV) kernels; no tile kernels yet
 enum class QuantizationFormat : uint32_t { Q4_K = FH_GGML_Q4_K, Q5_K = FH_GGML_Q5_K, Q6_K = FH_GGML_Q6_K };
 inline size_t block_elements(QuantizationFormat) { return 256; }
 inline size_t block_bytes(QuantizationFormat f) {

@@ -481,10 +481,34 @@ def test_q5_k_projection_matches_the_f64_oracle(api, d, n, k, m, dtype_name):
     x = oracle.round_storage(synth.activations(m, k, seed=11), code).reshape(m, k)
     out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
     rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), synth.rng(12).integers(0, n, 64)]))
-    want = oracle_columns(Q5_K, packed, n, k, rows, x, accumulate="f64")
+    tiles = m > 1 and dtype_name != "F32"            # 16-bit batches take the tile kernels: weights rounded once
+    want = oracle_columns(Q5_K, packed, n, k, rows, x, accumulate="f64", **({"weight_round": code} if tiles else {}))
     assert_matmul_parity(out.tensor.to_f32()[:, rows], want, f"q5_k {n}x{k} m={m} {dtype_name}")
     if k == 17408:
         assert out.operation == "q5_k_gemv_ksplit"
+
+
+@pytest.mark.parametrize("m,n,dtype_name", [(8, 1100, "F16"), (20, 1100, "BF16"), (130, 1000, "F16"),
+                                            (130, 16000, "BF16"), (300, 33000, "F16")])
+def test_q5_k_tile_kernels_match_the_rounded_weight_oracle(api, d, m, n, dtype_name):
+    # skinny (M <= 32), 64- and 128-wide tiles, and the 256-row tile (33000 columns x 2 row tiles)
+    k = 512
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    packed = synth.matrix(Q5_K, n, k, seed=201 + n)
+    w = qm(api, d, Q5_K, n, k, packed)
+    x = oracle.round_storage(synth.activations(m, k, seed=202), code).reshape(m, k)
+    out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    want_name = {8: "q5_k_gemm_mfma_skinny", 20: "q5_k_gemm_mfma_skinny", 130: "q5_k_gemm_mfma",
+                 300: "q5_k_gemm_mfma_m256"}[m]
+    assert out.operation == want_name
+    rows = np.unique(np.concatenate([np.arange(0, 140), np.arange(n - 80, n), synth.rng(203).integers(0, n, 64)]))
+    want = oracle_columns(Q5_K, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+    assert_matmul_parity(out.tensor.to_f32()[:, rows], want, f"q5_k tile m={m} n={n}")
+    # the bf16 reference case: result stored in the activation dtype
+    if m == 20:
+        stored = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w).tensor.to_f32()
+        assert np.array_equal(bits(stored), bits(oracle.round_storage(out.tensor.to_f32(), code).reshape(m, n)))
 
 
 def test_q5_k_expert_projection_and_validation(api, d):

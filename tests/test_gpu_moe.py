@@ -204,7 +204,7 @@ def _routing_rows(expert_ids):
     return meta
 
 
-@pytest.mark.parametrize("ggml,dtype", [(Q4_K, "F16"), (Q4_K, "BF16"), (Q6_K, "F16")])
+@pytest.mark.parametrize("ggml,dtype", [(Q4_K, "F16"), (Q4_K, "BF16"), (Q6_K, "F16"), (13, "F16")])
 def test_grouped_expert_projection_matches_the_oracle_and_the_direct_form(api, d, ggml, dtype):
     # 6 experts x 72 rows (a ragged last row tile), K = 768.  Expert 3 gets no
     # assignment, expert 1 gets 37 (more than one pass of 32 tokens), expert 5
@@ -222,8 +222,8 @@ def test_grouped_expert_projection_matches_the_oracle_and_the_direct_form(api, d
     valid = ids < experts
 
     got = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32)
-    assert d.last_operation() == ("expert_project_q4_k_grouped_mfma" if ggml == Q4_K
-                                  else "expert_project_q6_k_grouped_mfma")
+    assert d.last_operation() == {Q4_K: "expert_project_q4_k_grouped_mfma", 13: "expert_project_q5_k_grouped_mfma",
+                                  Q6_K: "expert_project_q6_k_grouped_mfma"}[ggml]
     got = got.to_f32()
     safe = _routing_rows(np.where(valid, ids, 0)).view(np.float32)
     tile = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), safe,

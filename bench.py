@@ -30,8 +30,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
-Q4_K, Q6_K = 12, 14
-BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+Q4_K, Q5_K, Q6_K = 12, 13, 14
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210}
 ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
 
 # HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
@@ -326,6 +326,7 @@ def main():
         timed(Q4_K, 5120, 17408, 1, f32, "Q4_K GEMV M=1 K=17408 N=5120", 1200)
         if not args.only or args.only in "decode layer":
             cases.append(layer_case(api, synth, dev, 400))
+        timed(Q5_K, 17408, 5120, 1, f32, "Q5_K GEMV M=1 K=5120 N=17408", 600)
         timed(Q6_K, 5120, 17408, 1, f32, "Q6_K GEMV M=1 K=17408 N=5120", 600)
         timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
         for m in (8, 16, 128):

@@ -181,7 +181,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
-    d->tuning["gemm_skinny_max_rows"] = 32; // largest M that takes the register-dequant MFMA kernel (0 = never)
+    d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
@@ -250,7 +250,7 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {
-        ok = value >= 0 && value <= 32;
+        ok = value >= 0 && value <= 64;
     } else if (k == "expert_grouped_min_assignments") {
         ok = value >= 0;
     } else if (k == "gemm_f32_min_rows") {

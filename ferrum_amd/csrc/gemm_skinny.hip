@@ -1,5 +1,5 @@
-// Skinny-M projection (2 <= M <= 32 tokens, f16 / bf16 activations) on the
-// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q6_K weights.
+// Skinny-M projection (2 <= M <= 64 tokens, f16 / bf16 activations) on the
+// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q5_K / Q6_K weights.
 //
 // With this few tokens the job is a weight stream (HBM bound), so nothing of
 // the weights goes through LDS.  A wave owns 16 weight rows.  Its 64 lanes are
@@ -544,6 +544,10 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     if (a.m <= 16) {
         hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 1, false>), grid, dim3(kSkThreads), 0, s, w, x, a.y,
                            a.m, a.n, nb, a.y_dtype, nullptr, nullptr);
+    } else if (a.m > 32) {
+        auto kernel = gemm_skinny_kernel<TYPE, DT, 4, false>;
+        hipLaunchKernelGGL(kernel, grid, dim3(kSkThreads), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype, nullptr,
+                           nullptr);
     } else {
         hipLaunchKernelGGL((gemm_skinny_kernel<TYPE, DT, 2, false>), grid, dim3(kSkThreads), 0, s, w, x, a.y,
                            a.m, a.n, nb, a.y_dtype, nullptr, nullptr);

@@ -215,6 +215,25 @@ def test_tile_gemm_both_tile_sizes_match_the_f16_tile_oracle(api, d, ggml, dtype
         assert_matmul_parity(got[:, rows], want, f"tile gemm n={n}")
 
 
+@pytest.mark.parametrize("ggml,dtype_name", [(Q4_K, "F16"), (Q4_K, "BF16"), (synth.Q5_K, "F16"),
+                                             (synth.Q5_K, "BF16"), (Q6_K, "F16"), (Q6_K, "BF16")])
+def test_register_dequant_gemm_up_to_64_rows(api, d, ggml, dtype_name):
+    # 33..64 rows stay on the kernel that dequantises in registers (four 16-row MFMA
+    # operands per wave); 65 is the first row count on the 256-row tile.  N = 1100 leaves
+    # a ragged last row group.
+    n, k = 1100, 1280
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    packed = synth.matrix(ggml, n, k, seed=131)
+    w = qm(api, d, ggml, n, k, packed)
+    for m in (32, 33, 49, 64, 65):
+        x = oracle.round_storage(synth.activations(m, k, seed=132 + m), code).reshape(m, k)
+        out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+        assert out.operation.endswith("_skinny") == (m <= 64), (m, out.operation)
+        want = oracle.project(ggml, packed, n, k, x, weight_round=code, accumulate="f64")
+        assert_matmul_parity(out.tensor.to_f32(), want, f"{dtype_name} m={m}")
+
+
 @pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
 def test_f32_activations_take_the_tile_kernels_from_a_chosen_row_count(api, d, ggml):
     # HybridModel::project (src/hybrid/engine.rs:3407-3500) sends f32 activations to f16
@@ -284,7 +303,8 @@ def test_config3_q4_k_gemm_5120_17408(api, d, m):
     x = synth.activations(m, k, seed=4, f16=True)
     w = qm(api, d, Q4_K, n, k, packed)
     xt = api.Tensor.from_f32(d, (m, k), api.DType.F16, x)
-    got = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+    full = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    got = full.tensor.to_f32()
     rows = np.sort(synth.rng(4, 77).choice(n, size=192, replace=False))
     rows[:4] = [0, 1, 2, 3]
     rows[-2:] = [n - 2, n - 1]
@@ -298,8 +318,11 @@ def test_config3_q4_k_gemm_5120_17408(api, d, m):
     # linearity in M: row i of the product depends only on row i of X
     if m >= 16:
         xt2 = api.Tensor.from_f32(d, (m // 2, k), api.DType.F16, x[: m // 2])
-        half = d.project_quantized(xt2, w, out_dtype=api.DType.F32).tensor.to_f32()
-        assert np.array_equal(half, got[: m // 2])
+        half = d.project_quantized(xt2, w, out_dtype=api.DType.F32)
+        if half.operation == full.operation:
+            assert np.array_equal(half.tensor.to_f32(), got[: m // 2])
+        else:  # another kernel, another summation order
+            assert_matmul_parity(half.tensor.to_f32(), got[: m // 2], f"gemm M={m // 2} vs M={m}")
 
 
 # ------------------------------------------------------------ error behaviour

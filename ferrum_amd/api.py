@@ -20,6 +20,7 @@ from __future__ import annotations
 
 import ctypes
 import enum
+import math
 import os
 import sys
 from dataclasses import dataclass
@@ -113,6 +114,7 @@ SYMBOLS = {
     "fh_embedding_gather_quantized": (_I32, [_P, _P, ctypes.POINTER(_U32), _SZ, _VP]),
     "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
+    "fh_add_rmsnorm": (_I32, [_P, _VP, _VP, _VP, _U32, _U32, ctypes.c_float, _VP, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
     "fh_moe_route_ranked": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP]),
     "fh_expert_combine_shared": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
@@ -591,6 +593,31 @@ class Device:
         lv, ov = logits._view(), out._view()
         _check(_lib.fh_argmax_rows(self._handle, ctypes.byref(lv), dims[0], dims[1], ctypes.byref(ov)))
         return out
+
+    def add_rmsnorm(self, a: Tensor, b: Tensor, weight: Tensor, epsilon: float,
+                    residual: Tensor | None = None, normed: Tensor | None = None) -> tuple[Tensor, Tensor]:
+        """(residual, normed): residual = a + b in the operands' dtype, normed =
+        rmsnorm(residual) * weight (MetalDevice::add_rmsnorm, src/ops/mod.rs:762-820).
+        `residual` / `normed` may be passed in to reuse buffers."""
+        dims = a.shape()
+        if len(dims) == 0 or dims[-1] == 0 or a.numel() == 0:
+            raise ShapeError("last dimension must be nonzero")
+        width = dims[-1]
+        if a.shape() != b.shape() or a.dtype != b.dtype or weight.dtype != a.dtype:
+            raise ShapeError("fused add+RMSNorm operands must match")
+        if weight.shape() != (width,) or width > 0xFFFFFFFF - 256:
+            raise ShapeError("RMSNorm weight must match the last dimension")
+        if not math.isfinite(epsilon) or epsilon <= 0:
+            raise ParameterError("epsilon must be finite and positive")
+        if any(t.buffer.device is not self for t in (a, b, weight)):
+            raise DeviceMismatch("tensor belongs to another device")
+        residual = residual if residual is not None else Tensor.zeros(self, dims, a.dtype)
+        normed = normed if normed is not None else Tensor.zeros(self, dims, a.dtype)
+        views = [t._view() for t in (a, b, weight, residual, normed)]
+        _check(_lib.fh_add_rmsnorm(self._handle, ctypes.byref(views[0]), ctypes.byref(views[1]),
+                                   ctypes.byref(views[2]), a.numel() // width, width, epsilon,
+                                   ctypes.byref(views[3]), ctypes.byref(views[4])))
+        return residual, normed
 
     def moe_route(self, logits: Tensor, selection_bias: Tensor | None, policy: MoeRoutingPolicy,
                   out: Tensor | None = None) -> Tensor:

@@ -579,6 +579,38 @@ fh_status fh_argmax_rows(fh_device* device, const fh_view* logits, uint32_t rows
     return FH_OK;
 }
 
+fh_status fh_add_rmsnorm(fh_device* device, const fh_view* a, const fh_view* b, const fh_view* weight,
+                         uint32_t rows, uint32_t width, float epsilon, const fh_view* residual,
+                         const fh_view* normed) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (rows == 0 || width == 0 || width > 0xffffffffu - 256u || !fits_u32((uint64_t)rows * width))
+        return fail(FH_ERR_SHAPE, "fused add+RMSNorm requires nonempty [rows,width]");
+    if (a == nullptr || b == nullptr || weight == nullptr || residual == nullptr || normed == nullptr)
+        return fail(FH_ERR_RANGE, "fused add+RMSNorm: null view");
+    if (a->dtype != b->dtype || weight->dtype != a->dtype || residual->dtype != a->dtype || normed->dtype != a->dtype)
+        return fail(FH_ERR_SHAPE, "fused add+RMSNorm operands must match");
+    if (!std::isfinite(epsilon) || epsilon <= 0.f)
+        return fail(FH_ERR_PARAMETER, "epsilon must be finite and positive");
+    const uint64_t count = (uint64_t)rows * width;
+    Range ar, br, wr, rr, nr;
+    fh_status st = resolve(device, a, count, "add+RMSNorm a", &ar);
+    if (st != FH_OK) return st;
+    if ((st = resolve(device, b, count, "add+RMSNorm b", &br)) != FH_OK) return st;
+    if ((st = resolve(device, weight, width, "add+RMSNorm weight", &wr)) != FH_OK) return st;
+    if ((st = resolve(device, residual, count, "add+RMSNorm residual", &rr)) != FH_OK) return st;
+    if ((st = resolve(device, normed, count, "add+RMSNorm output", &nr)) != FH_OK) return st;
+    for (const Range* out : {&rr, &nr}) {
+        if (overlaps(*out, ar) || overlaps(*out, br) || overlaps(*out, wr))
+            return fail(FH_ERR_RANGE, "add+RMSNorm outputs alias an operand");
+    }
+    if (overlaps(rr, nr)) return fail(FH_ERR_RANGE, "add+RMSNorm outputs alias each other");
+    device->last_operation = launch_add_rmsnorm(device->stream, ar.begin, br.begin, wr.begin,
+                                                const_cast<uint8_t*>(rr.begin), const_cast<uint8_t*>(nr.begin), rows,
+                                                width, a->dtype, epsilon);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
 namespace {
 
 fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const fh_view* selection_bias,

@@ -320,7 +320,6 @@ struct BlockW;
 
 template <>
 struct BlockW<kQ4K> {
-    static constexpr int kDwords = 4;    // input dwords per (slab, half)
     uint4 hdr, q[4];
     __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
         hdr = *reinterpret_cast<const uint4*>(block);
@@ -356,7 +355,6 @@ struct BlockW<kQ4K> {
 
 template <>
 struct BlockW<kQ5K> {
-    static constexpr int kDwords = 4;
     uint4 hdr, qh, q[4];
     __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
         hdr = *reinterpret_cast<const uint4*>(block);
@@ -391,7 +389,6 @@ struct BlockW<kQ5K> {
 
 template <>
 struct BlockW<kQ6K> {
-    static constexpr int kDwords = 8;
     uint4 l[2][2], p[2][2], sc;  // ql / qh of both halves, the 16 scales
     uint32_t d;
     __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {

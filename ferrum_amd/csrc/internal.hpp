@@ -89,6 +89,12 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                                     const uint32_t* ids_dev, size_t count, void* out,
                                     uint32_t out_dtype);
 
+// norm.hip
+// residual = round(a + b), normed = rmsnorm(residual) * weight; all operands of one dtype,
+// no output overlapping an operand or the other output.
+const char* launch_add_rmsnorm(hipStream_t s, const void* a, const void* b, const void* weight, void* residual,
+                               void* normed, uint32_t rows, uint32_t width, uint32_t dtype, float eps);
+
 // gemv.hip
 // how a GEMV launch reads its activations
 enum : uint32_t {

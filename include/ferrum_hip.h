@@ -172,6 +172,20 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
 fh_status fh_argmax_rows(fh_device* device, const fh_view* logits, uint32_t rows, uint32_t width,
                          const fh_view* out);
 
+/* MetalDevice::add_rmsnorm (src/ops/mod.rs:762-820, kernel
+ * src/metal/shaders/ops.metal:99-124) and the hybrid engine's h_add_rmsnorm
+ * (src/hybrid/engine.rs:3322-3342, src/metal/shaders/hybrid.metal:1576-1595):
+ * the residual add fused with the RMSNorm that feeds the next projection.
+ * a, b, residual, normed are [rows, width], weight is [width], all of one
+ * dtype.  residual = a + b rounded to that dtype (what a separate add
+ * stores); normed = residual * rsqrt(mean(residual^2) + epsilon) * weight.
+ * FH_ERR_SHAPE when the geometry is empty or the dtypes differ,
+ * FH_ERR_PARAMETER unless epsilon is finite and positive, FH_ERR_RANGE when
+ * an output overlaps an operand or the other output. */
+fh_status fh_add_rmsnorm(fh_device* device, const fh_view* a, const fh_view* b, const fh_view* weight,
+                         uint32_t rows, uint32_t width, float epsilon, const fh_view* residual,
+                         const fh_view* normed);
+
 /* ---- mixture of experts -----------------------------------------------------
  * MetalDevice::moe_route (src/ops/mod.rs:23-73; kernel ops.metal:1894-1957).
  * logits [tokens, experts]; bias (may be NULL) [experts] f32; metadata

@@ -350,6 +350,29 @@ public:
         check(fh_argmax_rows(handle_->raw, &lv, (uint32_t)dims[0], (uint32_t)dims[1], &ov));
         return out;
     }
+    // (residual, normed): residual = a + b in the operands' dtype, normed = rmsnorm(residual) * weight
+    // (MetalDevice::add_rmsnorm, src/ops/mod.rs:762-820).  Outputs may be passed in to reuse buffers.
+    std::pair<Tensor, Tensor> add_rmsnorm(const Tensor& a, const Tensor& b, const Tensor& weight, float epsilon,
+                                          const Tensor* residual_out = nullptr,
+                                          const Tensor* normed_out = nullptr) const {
+        const auto& dims = a.shape();
+        if (dims.empty() || dims.back() == 0 || a.numel() == 0)
+            throw Error(ErrorKind::Shape, "last dimension must be nonzero");
+        const uint64_t width = dims.back();
+        if (a.shape() != b.shape() || a.dtype() != b.dtype() || weight.dtype() != a.dtype())
+            throw Error(ErrorKind::Shape, "fused add+RMSNorm operands must match");
+        if (weight.shape().size() != 1 || weight.shape()[0] != width || width > 0xffffffffull - 256)
+            throw Error(ErrorKind::Shape, "RMSNorm weight must match the last dimension");
+        if (!std::isfinite(epsilon) || epsilon <= 0.f)
+            throw Error(ErrorKind::Parameter, "epsilon must be finite and positive");
+        if (!owns(a) || !owns(b) || !owns(weight)) throw Error(ErrorKind::DeviceMismatch, "tensor belongs to another device");
+        Tensor residual = residual_out ? *residual_out : zeros(dims, a.dtype());
+        Tensor normed = normed_out ? *normed_out : zeros(dims, a.dtype());
+        fh_view av = a.c_view(), bv = b.c_view(), wv = weight.c_view(), rv = residual.c_view(), nv = normed.c_view();
+        check(fh_add_rmsnorm(handle_->raw, &av, &bv, &wv, (uint32_t)(a.numel() / width), (uint32_t)width, epsilon, &rv,
+                             &nv));
+        return {residual, normed};
+    }
     Tensor moe_route(const Tensor& logits, const Tensor* selection_bias, const MoeRoutingPolicy& policy,
                      const Tensor* out = nullptr) const {
         const auto& dims = logits.shape();

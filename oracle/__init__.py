@@ -73,6 +73,8 @@ def _load() -> ctypes.CDLL:
     lib.fo_shared_gate.argtypes = [f32p, f32p, sz, sz, f32p]
     lib.fo_expert_combine_shared.restype = None
     lib.fo_expert_combine_shared.argtypes = [f32p, f32p, sz, sz, sz, u32, f32p, f32p, f32p]
+    lib.fo_add_rmsnorm.restype = None
+    lib.fo_add_rmsnorm.argtypes = [f32p, f32p, f32p, sz, sz, ctypes.c_float, ctypes.c_uint32, f32p, f32p]
     lib.fo_argmax_rows.restype = None
     lib.fo_argmax_rows.argtypes = [f32p, sz, sz, ctypes.POINTER(ctypes.c_uint32)]
     lib.fo_expert_combine.restype = None
@@ -245,6 +247,20 @@ def expert_combine_shared(values, metadata, tokens: int, hidden: int, top_k: int
     _lib.fo_expert_combine_shared(_f32(v), _f32(meta), tokens, hidden, top_k, dtype, _f32(sh),
                                   _f32(g) if g is not None else None, _f32(out))
     return out
+
+
+def add_rmsnorm(a, b, weight, eps: float, dtype: int = F32):
+    """(residual, normed) of [rows, width] operands: the storage-rounded sum and the
+    reference's float64 CPU rmsnorm of it (add_rmsnorm, src/metal/shaders/ops.metal:99-124;
+    src/reference.rs:23-35)."""
+    x = np.ascontiguousarray(a, dtype=np.float32)
+    y = np.ascontiguousarray(b, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    assert x.ndim == 2 and x.shape == y.shape and w.shape == (x.shape[1],)
+    residual, normed = np.empty_like(x), np.empty_like(x)
+    _lib.fo_add_rmsnorm(_f32(x), _f32(y), _f32(w), x.shape[0], x.shape[1], eps, dtype, _f32(residual),
+                        _f32(normed))
+    return residual, normed
 
 
 def argmax_rows(logits) -> np.ndarray:

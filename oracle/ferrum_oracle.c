@@ -41,6 +41,10 @@
  *   fo_argmax_rows         pinned for finite rows: numpy argmax (first
  *       maximal index) and ties; rows holding NaN follow the reference
  *       kernel's scan and merge order as read (flagged rows: parity unpinned).
+ *   fo_add_rmsnorm         pinned: the residual is the storage-rounded f32 sum
+ *       (exact); the normalised rows follow the reference's own CPU rmsnorm
+ *       (src/reference.rs:23-35, float64) and are checked against closed
+ *       forms (constant rows, one-hot rows, scale invariance).
  */
 #include <math.h>
 #include <pthread.h>
@@ -726,5 +730,25 @@ void fo_argmax_rows(const float* logits, size_t rows, size_t width, uint32_t* ou
         }
         out[2 * row] = bi;
         out[2 * row + 1] = bad;
+    }
+}
+
+/* add_rmsnorm (src/metal/shaders/ops.metal:99-124): residual = the sum rounded
+ * to the storage type, as a separate `add` stores it; normed = the reference's
+ * CPU rmsnorm (src/reference.rs:23-35) of the residual: float64 mean of
+ * squares, inv = 1 / sqrt(mean + eps), x * inv * w rounded once to f32.  The
+ * caller compares the device's storage-rounded rows against it. */
+void fo_add_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t width,
+                    float eps, uint32_t dtype, float* residual, float* normed) {
+    for (size_t r = 0; r < rows; r++) {
+        double squares = 0.0;
+        for (size_t j = 0; j < width; j++) {
+            float x = fo_round_storage(a[r * width + j] + b[r * width + j], dtype);
+            residual[r * width + j] = x;
+            squares += (double)x * (double)x;
+        }
+        double inv = 1.0 / sqrt(squares / (double)width + (double)eps);
+        for (size_t j = 0; j < width; j++)
+            normed[r * width + j] = (float)((double)residual[r * width + j] * inv * (double)weight[j]);
     }
 }

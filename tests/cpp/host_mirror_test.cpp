@@ -27,6 +27,8 @@ void fo_expert_silu_mul(const float* in, size_t assignments, size_t intermediate
 void fo_expert_combine(const float* in, const float* metadata, size_t tokens, size_t hidden, size_t top_k,
                        uint32_t dtype, float* out);
 void fo_round_storage_array(const float* in, size_t n, uint32_t dtype, float* out);
+void fo_add_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t width, float eps,
+                    uint32_t dtype, float* residual, float* normed);
 }
 
 using namespace ferrum;
@@ -283,6 +285,34 @@ int main() {
             threw = err.kind() == ErrorKind::Gguf;
         }
         report("a rank-3 tensor is not a matrix: Error::Gguf", threw);
+    }
+    {
+        // residual add + RMSNorm (add_rmsnorm, src/ops/mod.rs:762-820): bit-exact residual, normalised
+        // rows against the float64 CPU reference
+        const size_t rows = 3, width = 1000;
+        std::vector<float> a(rows * width), b(rows * width), w(width);
+        for (size_t i = 0; i < a.size(); ++i) {
+            a[i] = (float)((double)((i * 73 + 19) % 257) - 128.0) / 73.f;
+            b[i] = (float)((double)(((i + 11) * 73 + 19) % 257) - 128.0) / 73.f;
+        }
+        for (size_t j = 0; j < width; ++j) w[j] = 1.f + (float)((double)(((j + 3) * 73 + 19) % 257) - 128.0) / 73.f;
+        std::vector<float> want_residual(a.size()), want_normed(a.size());
+        fo_add_rmsnorm(a.data(), b.data(), w.data(), rows, width, 1e-6f, 0, want_residual.data(), want_normed.data());
+        auto [residual, normed] = d.add_rmsnorm(d.from_f32({rows, width}, DType::F32, a),
+                                                d.from_f32({rows, width}, DType::F32, b),
+                                                d.from_f32({width}, DType::F32, w), 1e-6f);
+        const auto got_residual = residual.to_f32();
+        report("add_rmsnorm residual is the f32 sum, bit for bit",
+               std::memcmp(got_residual.data(), want_residual.data(), a.size() * 4) == 0);
+        const double err = rel_l2(normed.to_f32(), want_normed);
+        report("add_rmsnorm rows match the float64 CPU reference", err <= 1e-6, err);
+        bool threw = false;
+        try {
+            d.add_rmsnorm(residual, normed, d.from_f32({width}, DType::F32, w), 0.f);
+        } catch (const Error& err) {
+            threw = err.kind() == ErrorKind::Parameter;
+        }
+        report("a zero epsilon is refused: Error::Parameter", threw);
     }
     std::printf("%d failure(s)\n", failures);
     return failures ? 1 : 0;

@@ -230,6 +230,13 @@ def xorshift_blocks(ggml_type: int, count: int) -> np.ndarray:
     return data.reshape(-1).copy()
 
 
+def deterministic(n: int) -> np.ndarray:
+    """`reference::deterministic(n)`: ((73 i + 19) mod 257 - 128) / 73 in f32
+    (src/reference.rs:67-71), the input of the reference's elementwise and norm tests."""
+    i = np.arange(n, dtype=np.int64)
+    return ((i * 73 + 19) % 257 - 128).astype(F) / F(73.0)
+
+
 def xorshift_uniform(n: int, seed: int, multiplier: int = 0x9E3779B97F4A7C15) -> np.ndarray:
     """`random(n, seed)`: uniform in [-1, 1) (src/diffusion/tests.rs:9-19; the
     hybrid twin at src/hybrid/iq_tests.rs:1251-1262 uses 0x2545F4914F6CDD1D)."""

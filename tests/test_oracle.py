@@ -527,6 +527,43 @@ def test_argmax_rows_is_the_first_maximal_index_and_flags_non_finite_rows():
     assert got[1, 0] == y.argmax()
 
 
+def test_add_rmsnorm_closed_forms():
+    eps = 1e-6
+    # constant rows: every element is c / sqrt(c^2 + eps) times its weight
+    width = 96
+    w = (1.0 + fx.deterministic(width)).astype(np.float32)
+    a = np.full((2, width), 0.75, np.float32)
+    b = np.full((2, width), -0.25, np.float32)
+    residual, normed = oracle.add_rmsnorm(a, b, w, eps)
+    assert np.array_equal(residual, np.full((2, width), 0.5, np.float32))
+    assert np.allclose(normed, (0.5 / np.sqrt(0.25 + eps)) * w.astype(np.float64), rtol=1e-7, atol=0)
+    # a one-hot row: mean of squares is v^2 / width
+    a = np.zeros((1, width), np.float32); b = np.zeros((1, width), np.float32)
+    a[0, 17] = 3.0; b[0, 17] = 1.0
+    residual, normed = oracle.add_rmsnorm(a, b, w, eps)
+    want = np.zeros(width); want[17] = 4.0 / np.sqrt(16.0 / width + eps) * float(w[17])
+    assert np.allclose(normed[0], want, rtol=1e-7, atol=0)
+    # scale invariance up to eps, and unit mean square of normed / weight
+    x = fx.deterministic(4 * 1000).reshape(4, 1000)
+    y = fx.deterministic(4 * 1000 + 11)[11:].reshape(4, 1000)
+    w = (2.0 + fx.deterministic(1003)[3:]).astype(np.float32)      # 0.25 .. 3.8, never zero
+    r1, n1 = oracle.add_rmsnorm(x, y, w, eps)
+    r4, n4 = oracle.add_rmsnorm(4 * x, 4 * y, w, eps)
+    assert np.array_equal(r4, 4 * r1)
+    assert np.allclose(n4, n1, rtol=2e-6, atol=0)
+    ms = ((n1.astype(np.float64) / w) ** 2).mean(axis=1)
+    assert np.allclose(ms, 1.0, atol=1e-5)
+    # the residual of 16-bit rows is the rounded sum, and the norm is taken of the rounded values
+    for code in (oracle.F16, oracle.BF16):
+        xs = oracle.round_storage(x, code).reshape(x.shape); ys = oracle.round_storage(y, code).reshape(y.shape)
+        ws = oracle.round_storage(w, code)
+        residual, normed = oracle.add_rmsnorm(xs, ys, ws, eps, code)
+        assert np.array_equal(residual, oracle.round_storage(xs + ys, code).reshape(x.shape))
+        r64 = residual.astype(np.float64)
+        want = r64 / np.sqrt((r64 ** 2).mean(axis=1, keepdims=True) + eps) * ws.astype(np.float64)
+        assert np.allclose(normed, want, rtol=1e-6, atol=0)
+
+
 def _ranked_by_numpy(logits, top_k, sigmoid, norm):
     """The CPU procedure of the reference's own routing test
     (src/hybrid/engine.rs:5004-5024) in float64 numpy."""

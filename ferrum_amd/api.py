@@ -169,6 +169,7 @@ class QuantizationFormat(enum.Enum):
     Q4_K = 12
     Q5_K = 13
     Q6_K = 14
+    IQ4_XS = 23    # the hybrid engine's Format::Iq4Xs (src/hybrid/weights.rs:38-60)
 
     @staticmethod
     def from_ggml_type(type_id: int) -> "QuantizationFormat":
@@ -184,7 +185,7 @@ class QuantizationFormat(enum.Enum):
         return 256
 
     def block_bytes(self) -> int:
-        return {12: 144, 13: 176, 14: 210}[self.value]
+        return {12: 144, 13: 176, 14: 210, 23: 136}[self.value]
 
 
 def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:

@@ -172,6 +172,56 @@ __device__ __forceinline__ float q6k_weight(const uint8_t* w, size_t row, uint32
     return a * (float)q;
 }
 
+// ---- IQ4_XS (136 B: f16 d, u16 scales_h, scales_l[4], qs[128]) ------------------
+//
+// block_iq4_xs / dequantize_iq4_xs (src/metal/shaders/hybrid.metal:27, 580-596):
+// eight 32-weight sub-blocks.  Sub-block i owns qs[16i .. 16i + 15]: the low
+// nibble of byte j is its weight j, the high nibble its weight 16 + j.  A
+// nibble indexes a 16-entry codebook (kvalues_iq4nl_f, hybrid.metal:34-37);
+// the sub-block scale is d * (ls - 32) with the 6-bit ls = nibble i of
+// scales_l | bits 2i, 2i + 1 of scales_h << 4.  d * (ls - 32) has at most 17
+// significant bits and the codebook 7, so the f32 weight is exact.
+
+// codebook value + 128 (1 .. 241) as unsigned bytes, four per word
+constexpr uint32_t kIq4Table0 = 0x3f2d1801u;  //  -127 -104  -83  -65
+constexpr uint32_t kIq4Table1 = 0x766a5d4fu;  //   -49  -35  -22  -10
+constexpr uint32_t kIq4Table2 = 0xa6998d81u;  //     1   13   25   38
+constexpr uint32_t kIq4Table3 = 0xf1d9c5b5u;  //    53   69   89  113
+
+// The low nibble of each byte of q, looked up: four bytes of codebook + 128.
+// v_perm_b32 picks from eight table bytes by the nibble's low three bits; a
+// third one picks between the two halves of the table by its top bit.
+__device__ __forceinline__ uint32_t iq4_lookup4(uint32_t q) {
+    const uint32_t low3 = q & 0x07070707u;
+    const uint32_t a = __builtin_amdgcn_perm(kIq4Table1, kIq4Table0, low3);
+    const uint32_t b = __builtin_amdgcn_perm(kIq4Table3, kIq4Table2, low3);
+    const uint32_t pick = ((q >> 1) & 0x04040404u) | 0x03020100u;
+    return __builtin_amdgcn_perm(b, a, pick);
+}
+
+// Bytes 0, 1 (or 2, 3) of v, each widened to a 16-bit field: read as f16 these
+// are the subnormals byte * 2^-24.
+__device__ __forceinline__ uint32_t bytes01_as_halves(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c010c00u); }
+__device__ __forceinline__ uint32_t bytes23_as_halves(uint32_t v) { return __builtin_amdgcn_perm(0u, v, 0x0c030c02u); }
+
+// d * (ls - 32) of sub-block i from the header words {d | scales_h << 16, scales_l}
+__device__ __forceinline__ float iq4xs_scale(uint32_t h0, uint32_t h1, uint32_t i) {
+    const uint32_t ls = ((h1 >> (4u * i)) & 15u) | (((h0 >> (16u + 2u * i)) & 3u) << 4);
+    return f16_bits_to_f32(h0 & 0xffffu) * (float)((int)ls - 32);
+}
+
+__device__ __forceinline__ float iq4xs_weight(const uint8_t* w, size_t row, uint32_t column, uint32_t blocks) {
+    const uint8_t* block = w + (row * blocks + (column >> 8)) * 136;
+    const uint32_t within = column & 255u, sub = within >> 5, j = within & 31u;
+    const uint32_t byte = block[8 + 16 * sub + (j & 15u)];
+    const uint32_t index = j < 16 ? (byte & 15u) : (byte >> 4);
+    const uint32_t h0 = block[0] | (block[1] << 8) | (block[2] << 16) | ((uint32_t)block[3] << 24);
+    const uint32_t h1 = block[4] | (block[5] << 8) | (block[6] << 16) | ((uint32_t)block[7] << 24);
+    const uint32_t word = index < 8 ? (index < 4 ? kIq4Table0 : kIq4Table1) : (index < 12 ? kIq4Table2 : kIq4Table3);
+    const int value = (int)((word >> (8u * (index & 3u))) & 0xffu) - 128;
+    return iq4xs_scale(h0, h1, sub) * (float)value;
+}
+
 // ---- wave reductions -----------------------------------------------------------
 
 template <int CTRL>

@@ -1,4 +1,4 @@
-// Dequant-fused tile GEMM for GGUF Q4_K / Q6_K on gfx950:
+// Dequant-fused tile GEMM for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS on gfx950:
 // Y[M,N] = X[M,K] * W[N,K]^T, f16 or bf16 activations, f32 accumulation.
 //
 // Stands in for the reference's tile kernels q4_k_gemm_mpp / q6_k_gemm_mpp
@@ -31,6 +31,16 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
         return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
     }
 }
+
+// How a loader thread's half h (0..1) of a 64-weight K slab maps to K offsets:
+// Q4_K / Q5_K decode 16 low-nibble weights at 16h and 16 high-nibble weights at
+// 32 + 16h; Q6_K and IQ4_XS decode 32 consecutive weights at 32h.
+template <uint32_t TYPE>
+constexpr bool kNibblePlanes = TYPE == kQ4K || TYPE == kQ5K;
+template <uint32_t TYPE>
+__device__ __forceinline__ constexpr uint32_t k_lo_of(uint32_t h) { return kNibblePlanes<TYPE> ? 16 * h : 32 * h; }
+template <uint32_t TYPE>
+__device__ __forceinline__ constexpr uint32_t k_hi_of(uint32_t h) { return kNibblePlanes<TYPE> ? 32 + 16 * h : 32 * h + 16; }
 
 // Raw bytes one thread needs to decode 32 weights (two runs of 16) of one row.
 template <uint32_t TYPE>
@@ -106,6 +116,36 @@ struct RawW<kQ5K> {
             out_lo[2 * t + 1] = pack2<DT>(l2, l3);
             out_hi[2 * t] = pack2<DT>(h0, h1);
             out_hi[2 * t + 1] = pack2<DT>(h2, h3);
+        }
+    }
+};
+
+// IQ4_XS: K slab c is sub-blocks 2c and 2c + 1; thread half h decodes sub-block
+// 2c + h from its 16 qs bytes: low nibbles are weights 0..15, high nibbles 16..31.
+template <>
+struct RawW<kIQ4XS> {
+    uint2 hdr;
+    uint4 qs;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c, uint32_t h) {
+        hdr = *reinterpret_cast<const uint2*>(block);
+        qs = load_u4_unaligned(block + 8 + 32 * c + 16 * h);
+    }
+    // out_lo: 16 weights at k = 32h + i; out_hi: 16 weights at k = 32h + 16 + i
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t c, uint32_t (&out_lo)[8], uint32_t (&out_hi)[8],
+                                           uint32_t h) const {
+        const float dl = iq4xs_scale(hdr.x, hdr.y, 2 * c + h);
+        const float scale = dl * 16777216.f, offset = -128.f * dl;
+        const uint32_t q[4] = {qs.x, qs.y, qs.z, qs.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t l = iq4_lookup4(q[t]), u = iq4_lookup4(q[t] >> 4);
+            const uint32_t l01 = bytes01_as_halves(l), l23 = bytes23_as_halves(l);
+            const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
+            out_lo[2 * t] = fma_pair<DT>(lo_half(l01), hi_half(l01), scale, offset);
+            out_lo[2 * t + 1] = fma_pair<DT>(lo_half(l23), hi_half(l23), scale, offset);
+            out_hi[2 * t] = fma_pair<DT>(lo_half(u01), hi_half(u01), scale, offset);
+            out_hi[2 * t + 1] = fma_pair<DT>(lo_half(u23), hi_half(u23), scale, offset);
         }
     }
 };
@@ -211,16 +251,14 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
     for (uint32_t step = 0; step < steps; ++step) {
         const uint32_t c = step & 3u;
         uint32_t lo[8], hi[8];
-        if constexpr (TYPE != kQ6K) {
+        if constexpr (kNibblePlanes<TYPE>) {
             raw.template decode<DT>(c, lo, hi);
         } else {
             raw.template decode<DT>(c, lo, hi, lh);
         }
         __syncthreads();  // previous step's fragment reads are done
         {
-            // Q4_K: lo -> k 16h.., hi -> k 32+16h..;  Q6_K: lo -> k 32h.., hi -> k 32h+16..
-            uint32_t k_lo = TYPE != kQ6K ? 16 * lh : 32 * lh;
-            uint32_t k_hi = TYPE != kQ6K ? 32 + 16 * lh : 32 * lh + 16;
+            const uint32_t k_lo = k_lo_of<TYPE>(lh), k_hi = k_hi_of<TYPE>(lh);
             uint4* dst_lo = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_lo]);
             uint4* dst_hi = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_hi]);
             dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
@@ -292,14 +330,12 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c, uint32_t h,
                                               uint16_t* wrow_lds) {
     uint32_t lo[8], hi[8];
-    if constexpr (TYPE != kQ6K) {
+    if constexpr (kNibblePlanes<TYPE>) {
         raw.template decode<DT>(c, lo, hi);
     } else {
         raw.template decode<DT>(c, lo, hi, h);
     }
-    // Q4_K: lo -> k 16h.., hi -> k 32+16h..;  Q6_K: lo -> k 32h.., hi -> k 32h+16..
-    const uint32_t k_lo = TYPE != kQ6K ? 16 * h : 32 * h;
-    const uint32_t k_hi = TYPE != kQ6K ? 32 + 16 * h : 32 * h + 16;
+    const uint32_t k_lo = k_lo_of<TYPE>(h), k_hi = k_hi_of<TYPE>(h);
     uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + k_lo);
     uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + k_hi);
     dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
@@ -387,6 +423,35 @@ struct BlockW<kQ5K> {
     }
 };
 
+// IQ4_XS: half h of slab c is sub-block 2c + h; input dword t gives the pair dwords of its
+// weights 4t .. 4t + 3 (low nibbles, out[0..1]) and 16 + 4t .. (high nibbles, out[2..3]).
+template <>
+struct BlockW<kIQ4XS> {
+    uint2 hdr;
+    uint4 q[4];
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
+        hdr = *reinterpret_cast<const uint2*>(block);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q[c] = load_u4_unaligned(block + 8 + 32 * c + 16 * h);
+    }
+    using Scales = BlockW<kQ4K>::Scales;
+    __device__ __forceinline__ Scales scales(int c, uint32_t h) const {
+        const float dl = iq4xs_scale(hdr.x, hdr.y, 2u * (uint32_t)c + h);
+        return {dl * 16777216.f, dl * 16777216.f, -128.f * dl, -128.f * dl};
+    }
+    template <int DT>
+    __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
+        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
+        const uint32_t l = iq4_lookup4(v[t]), u = iq4_lookup4(v[t] >> 4);
+        const uint32_t l01 = bytes01_as_halves(l), l23 = bytes23_as_halves(l);
+        const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
+        out[0] = fma_pair<DT>(lo_half(l01), hi_half(l01), s.a_lo, s.b_lo);
+        out[1] = fma_pair<DT>(lo_half(l23), hi_half(l23), s.a_lo, s.b_lo);
+        out[2] = fma_pair<DT>(lo_half(u01), hi_half(u01), s.a_hi, s.b_hi);
+        out[3] = fma_pair<DT>(lo_half(u23), hi_half(u23), s.a_hi, s.b_hi);
+    }
+};
+
 template <>
 struct BlockW<kQ6K> {
     uint4 l[2][2], p[2][2], sc;  // ql / qh of both halves, the 16 scales
@@ -458,8 +523,8 @@ __device__ __forceinline__ void decode_block_slab(const BlockW<TYPE>& blk, int c
             hi[2 * t] = out[2];
             hi[2 * t + 1] = out[3];
         }
-        uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + 16 * h);        // k = 16h ..
-        uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + 32 + 16 * h);   // k = 32 + 16h ..
+        uint4* dst_lo = reinterpret_cast<uint4*>(wrow_lds + k_lo_of<TYPE>(h));
+        uint4* dst_hi = reinterpret_cast<uint4*>(wrow_lds + k_hi_of<TYPE>(h));
         dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
         dst_lo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
         dst_hi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
@@ -489,8 +554,8 @@ __device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int 
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
             if (tt == t) blk.template decode<DT>(c, h, tt, s, out);
-        *reinterpret_cast<uint2*>(wrow_lds + 16 * h + 4 * t) = make_uint2(out[0], out[1]);
-        *reinterpret_cast<uint2*>(wrow_lds + 32 + 16 * h + 4 * t) = make_uint2(out[2], out[3]);
+        *reinterpret_cast<uint2*>(wrow_lds + k_lo_of<TYPE>(h) + 4 * t) = make_uint2(out[0], out[1]);
+        *reinterpret_cast<uint2*>(wrow_lds + k_hi_of<TYPE>(h) + 4 * t) = make_uint2(out[2], out[3]);
     } else {
         uint32_t a[4] = {0, 0, 0, 0}, b[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -740,6 +805,10 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             if (a.x_dtype == FH_F16) launch_wide_nt<kQ5K, 1>(s, a, plan); else launch_wide_nt<kQ5K, 2>(s, a, plan);
             return "q5_k_gemm_mfma_m256";
         }
+        if (a.ggml_type == kIQ4XS) {
+            if (a.x_dtype == FH_F16) launch_wide_nt<kIQ4XS, 1>(s, a, plan); else launch_wide_nt<kIQ4XS, 2>(s, a, plan);
+            return "iq4_xs_gemm_mfma_m256";
+        }
         if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
         return "q6_k_gemm_mfma_m256";
     }
@@ -773,6 +842,14 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             run(gemm_tile_kernel<kQ5K, 2, 128>, gemm_tile_kernel<kQ5K, 2, 64>);
         }
         return "q5_k_gemm_mfma";
+    }
+    if (a.ggml_type == kIQ4XS) {
+        if (a.x_dtype == FH_F16) {
+            run(gemm_tile_kernel<kIQ4XS, 1, 128>, gemm_tile_kernel<kIQ4XS, 1, 64>);
+        } else {
+            run(gemm_tile_kernel<kIQ4XS, 2, 128>, gemm_tile_kernel<kIQ4XS, 2, 64>);
+        }
+        return "iq4_xs_gemm_mfma";
     }
     if (a.x_dtype == FH_F16) {
         run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>);

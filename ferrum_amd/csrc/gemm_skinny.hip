@@ -1,5 +1,5 @@
 // Skinny-M projection (2 <= M <= 64 tokens, f16 / bf16 activations) on the
-// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q5_K / Q6_K weights.
+// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q5_K / Q6_K / IQ4_XS weights.
 //
 // With this few tokens the job is a weight stream (HBM bound), so nothing of
 // the weights goes through LDS.  A wave owns 16 weight rows.  Its 64 lanes are
@@ -116,6 +116,47 @@ struct Quarter<kQ5K> {
         for (int s = 0; s < 4; ++s) {
             a[s] = make_uint4(lo[4 * s], lo[4 * s + 1], lo[4 * s + 2], lo[4 * s + 3]);
             a[4 + s] = make_uint4(hi[4 * s], hi[4 * s + 1], hi[4 * s + 2], hi[4 * s + 3]);
+        }
+    }
+};
+
+// IQ4_XS: lane group g owns sub-blocks 2g and 2g + 1 (qs bytes [32g, +32)).  Low
+// nibbles are a sub-block's weights 0..15, high nibbles 16..31, so operand s
+// covers weights 64g + 8s .. as for Q4_K.  Codebook bytes (value + 128) become
+// f16 subnormals; fma(byte, scale, -128 scale) is the exact weight.
+template <>
+struct Quarter<kIQ4XS> {
+    static constexpr uint32_t kBlockBytes = 136;
+    uint2 hdr;
+    uint4 qa, qb;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t g) {
+        hdr = *reinterpret_cast<const uint2*>(block);
+        qa = load_u4_unaligned(block + 8 + 32 * g);
+        qb = load_u4_unaligned(block + 24 + 32 * g);
+    }
+    static __device__ __forceinline__ uint32_t klocal(uint32_t g, int s) { return 64 * g + 8 * s; }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t g, uint4 (&a)[8]) const {
+        const uint32_t v[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            const float dl = iq4xs_scale(hdr.x, hdr.y, 2 * g + sub);
+            const float scale = dl * 16777216.f, offset = -128.f * dl;
+            uint32_t lo[8], hi[8];   // pair dwords of weights 0..15 and 16..31 of the sub-block
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const uint32_t l = iq4_lookup4(v[4 * sub + t]), h = iq4_lookup4(v[4 * sub + t] >> 4);
+                const uint32_t l01 = bytes01_as_halves(l), l23 = bytes23_as_halves(l);
+                const uint32_t h01 = bytes01_as_halves(h), h23 = bytes23_as_halves(h);
+                lo[2 * t] = fma_pair<DT>(lo_half(l01), hi_half(l01), scale, offset);
+                lo[2 * t + 1] = fma_pair<DT>(lo_half(l23), hi_half(l23), scale, offset);
+                hi[2 * t] = fma_pair<DT>(lo_half(h01), hi_half(h01), scale, offset);
+                hi[2 * t + 1] = fma_pair<DT>(lo_half(h23), hi_half(h23), scale, offset);
+            }
+            a[4 * sub] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            a[4 * sub + 1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+            a[4 * sub + 2] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            a[4 * sub + 3] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
         }
     }
 };
@@ -565,6 +606,10 @@ const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
     if (a.ggml_type == kQ5K) {
         if (a.x_dtype == FH_F16) launch_tt<kQ5K, 1>(s, a); else launch_tt<kQ5K, 2>(s, a);
         return grouped ? "expert_project_q5_k_grouped_mfma" : "q5_k_gemm_mfma_skinny";
+    }
+    if (a.ggml_type == kIQ4XS) {
+        if (a.x_dtype == FH_F16) launch_tt<kIQ4XS, 1>(s, a); else launch_tt<kIQ4XS, 2>(s, a);
+        return grouped ? "expert_project_iq4_xs_grouped_mfma" : "iq4_xs_gemm_mfma_skinny";
     }
     if (a.x_dtype == FH_F16) launch_tt<kQ6K, 1>(s, a); else launch_tt<kQ6K, 2>(s, a);
     return grouped ? "expert_project_q6_k_grouped_mfma" : "q6_k_gemm_mfma_skinny";

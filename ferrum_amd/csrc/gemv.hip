@@ -1,4 +1,4 @@
-// Dequant-fused GEMV for GGUF Q4_K / Q6_K on gfx950: y[n] = sum_k W[n,k] x[k].
+// Dequant-fused GEMV for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS on gfx950: y[n] = sum_k W[n,k] x[k].
 //
 // Stands in for the reference's M = 1 kernels q4_k_gemv_ksplit / _factored
 // (src/metal/shaders/ops.metal:983-1070) and q6_k_gemv_ksplit / _factored
@@ -150,6 +150,49 @@ struct Frag<kQ5K> {
         float scaled = fmaf(sc_lo * 16777216.f, a_lo, (sc_hi * 1048576.f) * a_hi);
         float offset = fmaf(mn_lo, s.x + s.y, mn_hi * (s.z + s.w));
         return fmaf(d, scaled, -(dmin * offset));
+    }
+};
+
+// IQ4_XS: lane c owns sub-blocks 2c and 2c + 1 (qs bytes [32c, +32)), 32 weights each:
+// low nibbles are a sub-block's first 16 weights, high nibbles its last 16.  The
+// codebook is looked up four nibbles at a time as bytes of value + 128, which
+// reach the FMA as f16 subnormals like the K-quants' nibbles; the 128 comes
+// off through the activation sums of the sub-block.
+template <>
+struct Frag<kIQ4XS> {
+    uint2 hdr;
+    uint4 qa, qb;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c) {
+        hdr = *reinterpret_cast<const uint2*>(block);
+        qa = load_u4_unaligned(block + 8 + 32 * c);
+        qb = load_u4_unaligned(block + 24 + 32 * c);
+    }
+    __device__ __forceinline__ float dot(const float4* xc, float4 s, uint32_t c) const {
+        const float dl0 = iq4xs_scale(hdr.x, hdr.y, 2 * c), dl1 = iq4xs_scale(hdr.x, hdr.y, 2 * c + 1);
+        float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // [sub-block][two chains]
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int sub = t >> 2, u = 8 * sub + (t & 3);      // float4 of the low nibbles; the high ones sit 4 on
+            const float4 xl = xc[u * 4], xh = xc[(u + 4) * 4];
+            const uint32_t lo = iq4_lookup4(q[t]), hi = iq4_lookup4(q[t] >> 4);
+            const uint32_t l01 = bytes01_as_halves(lo), l23 = bytes23_as_halves(lo);
+            const uint32_t h01 = bytes01_as_halves(hi), h23 = bytes23_as_halves(hi);
+            float& a = acc[sub][0];
+            float& b = acc[sub][1];
+            a = fmaf(lo_half(l01), xl.x, a);
+            b = fmaf(hi_half(l01), xl.y, b);
+            a = fmaf(lo_half(l23), xl.z, a);
+            b = fmaf(hi_half(l23), xl.w, b);
+            a = fmaf(lo_half(h01), xh.x, a);
+            b = fmaf(hi_half(h01), xh.y, b);
+            a = fmaf(lo_half(h23), xh.z, a);
+            b = fmaf(hi_half(h23), xh.w, b);
+        }
+        // bytes were (value + 128) * 2^-24
+        const float r0 = fmaf(acc[0][0] + acc[0][1], 16777216.f, -128.f * (s.x + s.y));
+        const float r1 = fmaf(acc[1][0] + acc[1][1], 16777216.f, -128.f * (s.z + s.w));
+        return fmaf(dl0, r0, dl1 * r1);
     }
 };
 
@@ -467,15 +510,18 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     p.x_rows = a.x_rows;
     const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
     dim3 grid(plan.tiles, plan.segments, a.m);
-    LaunchFn fn = a.ggml_type == kQ4K   ? pick<kQ4K>(plan.bs, plan.it)
-                  : a.ggml_type == kQ5K ? pick<kQ5K>(plan.bs, plan.it)
-                                        : pick<kQ6K>(plan.bs, plan.it);
+    LaunchFn fn = a.ggml_type == kQ4K     ? pick<kQ4K>(plan.bs, plan.it)
+                  : a.ggml_type == kQ5K   ? pick<kQ5K>(plan.bs, plan.it)
+                  : a.ggml_type == kIQ4XS ? pick<kIQ4XS>(plan.bs, plan.it)
+                                          : pick<kQ6K>(plan.bs, plan.it);
     fn(grid, lds, s, p);
-    const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : 2;
-    static const char* const expert_names[3] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
-                                                "expert_project_q6_k_factored"};
-    static const char* const ksplit_names[3] = {"q4_k_gemv_ksplit", "q5_k_gemv_ksplit", "q6_k_gemv_ksplit"};
-    static const char* const factored_names[3] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored"};
+    const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : a.ggml_type == kQ6K ? 2 : 3;
+    static const char* const expert_names[4] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
+                                                "expert_project_q6_k_factored", "expert_project_iq4_xs_factored"};
+    static const char* const ksplit_names[4] = {"q4_k_gemv_ksplit", "q5_k_gemv_ksplit", "q6_k_gemv_ksplit",
+                                                "iq4_xs_gemv_ksplit"};
+    static const char* const factored_names[4] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored",
+                                                  "iq4_xs_gemv_factored"};
     if (a.metadata != nullptr) return expert_names[f];
     if (plan.segments > 1) return ksplit_names[f];
     return factored_names[f];

@@ -17,8 +17,8 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q5_K, Q6_K = 12, 13, 14
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210}
+Q4_K, Q5_K, Q6_K, IQ4_XS = 12, 13, 14, 23
+BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}
 
 
 def rng(seed: int, stream: int = 0) -> np.random.Generator:
@@ -100,6 +100,23 @@ def q6_k_blocks(count: int, g: np.random.Generator) -> np.ndarray:
     return blocks
 
 
+def iq4_xs_blocks(count: int, g: np.random.Generator) -> np.ndarray:
+    """f16 d, u16 scales_h, scales_l[4], qs[128]: every 6-bit sub-block scale and every
+    codebook index is drawn uniformly."""
+    blocks = np.empty((count, 136), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(count)) * 0.0005).astype(np.float32).astype(np.float16)
+    blocks[:, 0:2] = d.view(np.uint8).reshape(count, 2)
+    ls = g.integers(0, 64, (count, 8), dtype=np.uint16)
+    high = np.zeros(count, dtype=np.uint16)
+    for i in range(8):
+        high |= (ls[:, i] >> 4) << (2 * i)
+    blocks[:, 2:4] = high.view(np.uint8).reshape(count, 2)
+    low = (ls & 15).astype(np.uint8)
+    blocks[:, 4:8] = low[:, 0::2] | (low[:, 1::2] << 4)
+    blocks[:, 8:] = g.integers(0, 256, (count, 128), dtype=np.uint8)
+    return blocks
+
+
 def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> np.ndarray:
     """Packed row-major ``[rows, cols]`` matrix as a flat uint8 array."""
     if cols % 256:
@@ -112,6 +129,8 @@ def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> 
         return q5_k_blocks(count, g).reshape(-1)
     if ggml_type == Q6_K:
         return q6_k_blocks(count, g).reshape(-1)
+    if ggml_type == IQ4_XS:
+        return iq4_xs_blocks(count, g).reshape(-1)
     raise ValueError(f"unsupported ggml type {ggml_type}")
 
 

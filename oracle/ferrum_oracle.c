@@ -21,6 +21,17 @@
  *                          pinned: both forms agree bitwise on the
  *       reference's closed-form fixtures; exact-rational step-by-step
  *       rounding on a (d, sc, m, q) grid; Q3_K -> Q6_K value identity.
+ *   fo_dequantize / fo_weight, IQ4_XS
+ *                          pinned without a fixture (the reference holds no
+ *       CPU twin or test vector for this format): the block form follows
+ *       dequantize_iq4_xs and the per-element form the indexing of the GEMV
+ *       kernel mv_iq4_xs, two separate statements in the reference, and they
+ *       agree bitwise; with every sub-block scale at ls = 33 a sub-block
+ *       equals the reference's CPU IQ4_NL decoder (src/hybrid/iq_tests.rs:
+ *       1606-1620, src/hybrid/ple.rs:150-158) on the same bytes; the 6-bit
+ *       scale assembly is checked for all 64 values at all 8 positions
+ *       against blocks packed by a separately written packer; the value is
+ *       exact in f32 (17-bit scale x 7-bit codebook), checked in rationals.
  *   fo_project_f32seq / fo_project_f64
  *                          pinned: integer special case (d=1, sc=1, dmin=0)
  *       equals an exact integer dot; all-zero quants equal -dmin*m*sum(x);
@@ -55,6 +66,7 @@
 #define FO_Q4_K 12u
 #define FO_Q5_K 13u
 #define FO_Q6_K 14u
+#define FO_IQ4_XS 23u
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -151,6 +163,7 @@ size_t fo_block_bytes(uint32_t ggml_type) {
     if (ggml_type == FO_Q4_K) return 144;
     if (ggml_type == FO_Q5_K) return 176;
     if (ggml_type == FO_Q6_K) return 210;
+    if (ggml_type == FO_IQ4_XS) return 136; /* src/loader/gguf.rs:111 */
     return 0;
 }
 
@@ -251,11 +264,42 @@ static void dequant_q6_k_block(const uint8_t* b, float* out) {
     }
 }
 
+/* The 16-entry codebook shared by IQ4_NL and IQ4_XS (kvalues_iq4nl_f,
+ * src/metal/shaders/hybrid.metal:34-37; CPU copies src/hybrid/ple.rs:25-27,
+ * src/hybrid/iq_tests.rs:1608-1610). */
+static const float iq4_values[16] = {-127.f, -104.f, -83.f, -65.f, -49.f, -35.f, -22.f, -10.f,
+                                     1.f,    13.f,   25.f,  38.f,  53.f,  69.f,  89.f,  113.f};
+
+/* Block form, IQ4_XS (136 B: f16 d, u16 scales_h, scales_l[4], qs[128]):
+ * dequantize_iq4_xs (src/metal/shaders/hybrid.metal:580-596), which takes the
+ * block 16 values at a time: chunk il is half il % 2 (low or high nibbles) of
+ * the four qs words of sub-block il / 2, scaled by d * (ls - 32). */
+static void dequant_iq4_xs_block(const uint8_t* b, float* out) {
+    float d = fo_f16_to_f32(le16(b));
+    uint32_t scales_h = le16(b + 2);
+    const uint8_t* scales_l = b + 4;
+    const uint8_t* qs = b + 8;
+    for (int il = 0; il < 16; il++) {
+        int ib32 = il / 2, half = il % 2;
+        int ls = (int)(((uint32_t)(scales_l[ib32 / 2] >> (4 * (ib32 % 2))) & 0xfu) | (((scales_h >> (2 * ib32)) & 3u) << 4));
+        float dl = d * (float)(ls - 32);
+        for (int i = 0; i < 4; i++) {
+            const uint8_t* word = qs + 16 * ib32 + 4 * i;
+            for (int j = 0; j < 4; j++) {
+                uint32_t index = ((uint32_t)word[j] >> (4 * half)) & 0xfu;
+                out[16 * il + 4 * i + j] = dl * iq4_values[index];
+            }
+        }
+    }
+}
+
 static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) {
     if (ggml_type == FO_Q4_K)
         dequant_q4_k_block(block, out);
     else if (ggml_type == FO_Q5_K)
         dequant_q5_k_block(block, out);
+    else if (ggml_type == FO_IQ4_XS)
+        dequant_iq4_xs_block(block, out);
     else
         dequant_q6_k_block(block, out);
 }
@@ -310,6 +354,19 @@ float fo_weight(uint32_t ggml_type, const uint8_t* packed, size_t row, size_t co
         float c = dmin * (float)mn;
         return b - c;
     }
+    if (ggml_type == FO_IQ4_XS) {
+        /* the indexing of the GEMV kernel mv_iq4_xs (src/metal/shaders/hybrid.metal:899-951):
+         * sub-block ib = group, byte 16 ib + (lane & 15), low nibble for lanes 0..15 and high
+         * nibble for 16..31, and (d * ls) applied to the codebook value */
+        const uint8_t* block = packed + (row * blocks + block_index) * 136;
+        uint32_t ib = group;
+        uint8_t byte = block[8 + 16 * ib + (lane & 15)];
+        uint32_t index = lane < 16 ? (uint32_t)(byte & 0x0f) : (uint32_t)(byte >> 4);
+        uint32_t scales_h = le16(block + 2);
+        int ls = (int)(((uint32_t)(block[4 + ib / 2] >> (4 * (ib % 2))) & 0xfu) | (((scales_h >> (2 * ib)) & 3u) << 4)) - 32;
+        float dl = fo_f16_to_f32(le16(block)) * (float)ls;
+        return dl * iq4_values[index];
+    }
     const uint8_t* block = packed + (row * blocks + block_index) * 210;
     uint32_t half_block = group >> 2, slice = group & 3;
     uint8_t byte = block[half_block * 64 + (slice & 1) * 32 + lane];
@@ -331,6 +388,8 @@ int fo_validate_payload(uint32_t ggml_type, const uint8_t* payload, size_t len) 
         const uint8_t* b = payload + off;
         if (ggml_type == FO_Q4_K || ggml_type == FO_Q5_K) {
             if (!isfinite(fo_f16_to_f32(le16(b))) || !isfinite(fo_f16_to_f32(le16(b + 2)))) return 2;
+        } else if (ggml_type == FO_IQ4_XS) {
+            if (!isfinite(fo_f16_to_f32(le16(b)))) return 2;
         } else {
             if (!isfinite(fo_f16_to_f32(le16(b + 208)))) return 2;
         }

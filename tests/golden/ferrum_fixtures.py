@@ -230,6 +230,48 @@ def xorshift_blocks(ggml_type: int, count: int) -> np.ndarray:
     return data.reshape(-1).copy()
 
 
+def hybrid_random_blocks(blocks: int, block: int, seed: int) -> np.ndarray:
+    """`random_blocks(blocks, block, seed)` of the hybrid engine's format tests
+    (src/hybrid/iq_tests.rs:1231-1249): xorshift bytes, with the f16 at the start of
+    every block forced to 0.02 + 0.01 * byte0 / 255."""
+    data = _xorshift_bytes(((seed * 0x9E3779B97F4A7C15) & _M64) | 1, blocks * block).reshape(blocks, block)
+    for b in data:
+        scale = F(0.02) + F(0.01) * F(b[0]) / F(255.0)
+        b[0:2] = np.frombuffer(_f16_bytes(scale), dtype=np.uint8)
+    return data.reshape(-1).copy()
+
+
+IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=F)
+
+
+def iq4_nl_dense(blocks: np.ndarray) -> np.ndarray:
+    """`dequant_iq4_nl` (src/hybrid/iq_tests.rs:1606-1620; the same walk at
+    src/hybrid/ple.rs:150-158): 18-byte blocks of 32 values, byte j holds values j (low
+    nibble) and j + 16 (high), each d * VALUES[nibble]."""
+    b = np.asarray(blocks, dtype=np.uint8).reshape(-1, 18)
+    d = b[:, 0:2].copy().view(np.float16).astype(F)            # [blocks, 1]
+    out = np.empty((b.shape[0], 32), dtype=F)
+    out[:, :16] = d * IQ4_VALUES[b[:, 2:] & 15]
+    out[:, 16:] = d * IQ4_VALUES[b[:, 2:] >> 4]
+    return out
+
+
+def iq4_xs_pack(d, ls, index) -> np.ndarray:
+    """IQ4_XS blocks (block_iq4_xs, src/metal/shaders/hybrid.metal:27) from their fields:
+    `d` [blocks] f16-representable, `ls` [blocks, 8] in 0..63, `index` [blocks, 256] in 0..15."""
+    d = np.asarray(d, dtype=np.float16).reshape(-1)
+    ls = np.asarray(ls, dtype=np.uint32).reshape(d.size, 8)
+    index = np.asarray(index, dtype=np.uint8).reshape(d.size, 8, 32)
+    out = np.zeros((d.size, 136), dtype=np.uint8)
+    out[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    high = sum(((ls[:, i] >> 4) & 3) << (2 * i) for i in range(8)).astype(np.uint16)
+    out[:, 2:4] = high.view(np.uint8).reshape(-1, 2)
+    for pair in range(4):
+        out[:, 4 + pair] = (ls[:, 2 * pair] & 15) | ((ls[:, 2 * pair + 1] & 15) << 4)
+    out[:, 8:] = (index[:, :, :16] | (index[:, :, 16:] << 4)).reshape(d.size, 128)
+    return out
+
+
 def deterministic(n: int) -> np.ndarray:
     """`reference::deterministic(n)`: ((73 i + 19) mod 257 - 128) / 73 in f32
     (src/reference.rs:67-71), the input of the reference's elementwise and norm tests."""

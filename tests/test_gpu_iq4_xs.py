@@ -1,0 +1,180 @@
+"""GPU parity of IQ4_XS (GGML type 23, the hybrid engine's Format::Iq4Xs,
+src/hybrid/weights.rs:38-60) through every kernel family, against the CPU oracle and
+through the C ABI.
+
+The reference tests its IQ formats with random blocks, shapes (rows, cols) = (13, 1024),
+M in {1, 3, 16, 64}, f32 activations and |err| <= 5e-3 * max|ref| against the float64
+product of the CPU dequant (src/hybrid/iq_tests.rs:1300-1337); those cases are replayed
+here with its block generator, then held to this build's bars (dequant bit-exact, matmul
+max-rel 1e-3 and rel-L2 1e-5) at larger shapes on seeded blocks.
+"""
+import numpy as np
+import pytest
+
+import ferrum_fixtures as fx
+import oracle
+from helpers import assert_matmul_parity, bits, oracle_columns
+from ferrum_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+IQ4_XS = 23
+
+
+@pytest.fixture(scope="module")
+def api():
+    from ferrum_amd import api as module
+    return module
+
+
+@pytest.fixture(scope="module")
+def d(api):
+    return api.Device.new()
+
+
+def qm(api, d, rows, cols, packed):
+    return api.QuantizedMatrix.from_bytes(d, rows, cols, api.QuantizationFormat(IQ4_XS), packed)
+
+
+def test_dequantize_and_gather_are_bit_exact(api, d):
+    for rows, cols, packed in ((13, 1024, fx.hybrid_random_blocks(13 * 4, 136, 136)),
+                               (257, 2560, synth.matrix(IQ4_XS, 257, 2560, seed=301))):
+        w = qm(api, d, rows, cols, packed)
+        assert w.byte_size() == rows * (cols // 256) * 136
+        want = oracle.dequantize(IQ4_XS, packed, rows, cols)
+        out = d.dequantize(w)
+        assert d.last_operation() == "dequantize_iq4_xs"
+        assert np.array_equal(bits(out.to_f32()), bits(want))
+        for dtype, code in ((api.DType.F16, oracle.F16), (api.DType.BF16, oracle.BF16)):
+            assert np.array_equal(bits(d.dequantize(w, dtype).to_f32()),
+                                  bits(oracle.round_storage(want, code).reshape(rows, cols)))
+        ids = [rows - 1, 0, 3, 3]
+        got = d.embedding_gather_quantized(w, ids, api.DType.F32)
+        assert got.operation == "embedding_gather_iq4_xs"
+        assert np.array_equal(bits(got.tensor.to_f32()), bits(want[ids]))
+
+
+def test_projections_replay_the_reference_iq_cases(api, d):
+    # iq_projections_match_the_cpu_dequant (src/hybrid/iq_tests.rs:1300-1337)
+    rows, cols = 13, 1024
+    packed = fx.hybrid_random_blocks(rows * cols // 256, 136, 136)
+    w = qm(api, d, rows, cols, packed)
+    dense = oracle.dequantize(IQ4_XS, packed, rows, cols).astype(np.float64)
+    for m in (1, 3, 16, 64):
+        x = fx.xorshift_uniform(m * cols, m, multiplier=0x2545F4914F6CDD1D).reshape(m, cols)
+        out = d.project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x), w)
+        assert out.operation == ("iq4_xs_gemv_factored" if m == 1 else "iq4_xs_gemm")
+        want = x.astype(np.float64) @ dense.T
+        scale = np.abs(want).max()
+        assert scale > 1e-2
+        assert np.abs(out.tensor.to_f32() - want).max() <= 5e-3 * scale       # the reference's bound
+        assert_matmul_parity(out.tensor.to_f32(), want, f"iq4_xs m={m}")     # this build's
+
+
+@pytest.mark.parametrize("n,k,m,dtype_name", [(4099, 5120, 1, "F32"), (1003, 4864, 1, "F32"), (5120, 17408, 1, "F32"),
+                                              (17408, 5120, 1, "F32"), (515, 1280, 3, "F32"), (515, 1280, 1, "F16"),
+                                              (515, 1280, 1, "BF16")])
+def test_gemv_matches_the_f64_oracle(api, d, n, k, m, dtype_name):
+    dtype = api.DType[dtype_name]
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype_name]
+    packed = synth.matrix(IQ4_XS, n, k, seed=n + k)
+    w = qm(api, d, n, k, packed)
+    x = oracle.round_storage(synth.activations(m, k, seed=11), code).reshape(m, k)
+    out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), synth.rng(12).integers(0, n, 64)]))
+    want = oracle_columns(IQ4_XS, packed, n, k, rows, x, accumulate="f64")
+    assert_matmul_parity(out.tensor.to_f32()[:, rows], want, f"iq4_xs {n}x{k} m={m} {dtype_name}")
+    if k == 17408:
+        assert out.operation == "iq4_xs_gemv_ksplit"
+
+
+@pytest.mark.parametrize("m,n,dtype_name", [(8, 1100, "F16"), (20, 1100, "BF16"), (50, 1100, "F16"), (130, 1000, "F16"),
+                                            (130, 16000, "BF16"), (300, 33000, "F16"), (300, 33000, "BF16")])
+def test_tile_kernels_match_the_rounded_weight_oracle(api, d, m, n, dtype_name):
+    # register-dequant kernel (M <= 64), 64- and 128-wide tiles, and the 256-row tile
+    k = 768
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    packed = synth.matrix(IQ4_XS, n, k, seed=311 + n)
+    w = qm(api, d, n, k, packed)
+    x = oracle.round_storage(synth.activations(m, k, seed=312), code).reshape(m, k)
+    out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    want_name = {8: "iq4_xs_gemm_mfma_skinny", 20: "iq4_xs_gemm_mfma_skinny", 50: "iq4_xs_gemm_mfma_skinny",
+                 130: "iq4_xs_gemm_mfma", 300: "iq4_xs_gemm_mfma_m256"}[m]
+    assert out.operation == want_name
+    rows = np.unique(np.concatenate([np.arange(0, 150), np.arange(n - 150, n), synth.rng(313).integers(0, n, 64)]))
+    want = oracle_columns(IQ4_XS, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+    assert_matmul_parity(out.tensor.to_f32()[:, rows], want, f"iq4_xs tile m={m} n={n}")
+
+
+def test_tile_values_are_the_dequantised_weights_rounded_once(api, d):
+    # X = identity rows: the product reads the tile values themselves
+    n, k = 200, 256
+    packed = synth.matrix(IQ4_XS, n, k, seed=321)
+    w = qm(api, d, n, k, packed)
+    dense = oracle.dequantize(IQ4_XS, packed, n, k)
+    eye = np.eye(k, dtype=np.float32)
+    for dtype, code in ((api.DType.F16, oracle.F16), (api.DType.BF16, oracle.BF16)):
+        for m0, m1 in ((0, 40), (40, 256)):              # register-dequant kernel, then the tiles
+            x = eye[m0:m1]
+            out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+            want = oracle.round_storage(dense[:, m0:m1].T.copy(), code).reshape(m1 - m0, n)
+            # equal as numbers: a sub-block scale of zero gives -0 in the decoder and +0 from a sum
+            got = out.tensor.to_f32()
+            assert np.array_equal(got, want), (dtype, out.operation, np.argwhere(got != want)[:4])
+            nonzero = want != 0
+            assert np.array_equal(bits(got[nonzero]), bits(want[nonzero]))
+
+
+def test_expert_projection_per_assignment_and_grouped(api, d):
+    # iq_expert_projections_match_the_cpu_dequant (src/hybrid/iq_tests.rs:1398-1437) in shape:
+    # each route multiplies its own expert's slice
+    experts, rows, cols = 3, 13, 1024
+    packed = fx.hybrid_random_blocks(experts * rows * cols // 256, 136, 7 + 136)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(IQ4_XS), experts, rows, cols)
+    ids = [2, 0, 1, 1, 2]
+    a = len(ids)
+    meta = np.zeros((a, 3), dtype=np.uint32)
+    meta[:, 0] = ids
+    meta[:, 1] = np.arange(a)
+    meta[:, 2] = np.float32(1.0).view(np.uint32)
+    x = fx.xorshift_uniform(a * cols, 11, multiplier=0x2545F4914F6CDD1D).reshape(a, cols)
+    got = d.expert_project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F32, x),
+                                     api.Tensor.from_bits(d, meta.shape, meta), w, cols, experts).to_f32()
+    assert d.last_operation() == "expert_project_iq4_xs_factored"
+    want = oracle.expert_project(IQ4_XS, packed, experts, rows, cols, x, meta.view(np.float32), accumulate="f64")
+    assert np.abs(got - want).max() <= 5e-3 * np.abs(want).max()
+    assert_matmul_parity(got, want, "iq4_xs routes")
+
+    # the grouped MFMA form: many assignments, f16 rows, ragged expert sizes (one empty)
+    experts, rows, cols, a = 6, 200, 768, 150
+    packed = synth.matrix(IQ4_XS, experts * rows, cols, seed=331)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(IQ4_XS), experts, rows, cols)
+    rng = synth.rng(332)
+    ids = rng.choice([0, 1, 2, 4, 5], size=a, p=[0.4, 0.05, 0.25, 0.2, 0.1])   # expert 3 gets nothing
+    meta = np.zeros((a, 3), dtype=np.uint32)
+    meta[:, 0] = np.sort(ids)
+    meta[:, 1] = rng.integers(0, 64, a)
+    meta[:, 2] = np.float32(1.0).view(np.uint32)
+    x = oracle.round_storage(synth.activations(a, cols, seed=333) * 0.25, oracle.F16).reshape(a, cols)
+    got = d.expert_project_quantized(api.Tensor.from_f32(d, x.shape, api.DType.F16, x),
+                                     api.Tensor.from_bits(d, meta.shape, meta), w, cols, experts,
+                                     out_dtype=api.DType.F32).to_f32()
+    assert d.last_operation() == "expert_project_iq4_xs_grouped_mfma"
+    want = oracle.expert_project(IQ4_XS, packed, experts, rows, cols, x, meta.view(np.float32), accumulate="f64",
+                                 weight_round=oracle.F16)
+    assert_matmul_parity(got, want, "iq4_xs grouped routes")
+
+
+def test_validation(api, d):
+    rows, cols = 4, 512
+    packed = synth.matrix(IQ4_XS, rows, cols, seed=341)
+    bad = packed.copy()
+    bad[1] = 0x7c                                       # d = +inf in the first block
+    with pytest.raises(api.WeightError):
+        qm(api, d, rows, cols, bad)
+    ok = packed.copy()
+    ok[2:4] = 0xff                                      # scales_h is not a float: any bits are fine
+    qm(api, d, rows, cols, ok)
+    with pytest.raises(api.Error):
+        qm(api, d, rows, cols, packed[:-1])

@@ -659,3 +659,84 @@ def test_q5_k_block_form_per_element_form_and_the_q4_k_special_case_agree():
     x = fx.xorshift_uniform(3 * cols, 9).reshape(3, cols)
     want = x.astype(np.float64) @ dense.astype(np.float64).T
     assert np.abs(oracle.project(Q5_K, packed, rows, cols, x, accumulate="f64") - want).max() <= 1e-6 * np.abs(want).max()
+
+
+# ---------------------------------------------------------------- IQ4_XS
+
+IQ4_XS = 23
+
+
+def test_iq4_xs_two_reference_statements_agree_and_values_are_exact():
+    # block form = dequantize_iq4_xs, per-element form = the indexing of mv_iq4_xs
+    rows, cols = 13, 1024          # the geometry of the hybrid engine's own format tests
+    packed = fx.hybrid_random_blocks(rows * cols // 256, 136, 136)
+    assert oracle.block_bytes(IQ4_XS) == 136 and oracle.validate_payload(IQ4_XS, packed) == 0
+    dense = oracle.dequantize(IQ4_XS, packed, rows, cols)
+    rng = np.random.default_rng(23)
+    for _ in range(4000):
+        r, c = int(rng.integers(rows)), int(rng.integers(cols))
+        assert bits(np.float32(oracle.weight(IQ4_XS, packed, r, c, cols))) == bits(dense[r, c])
+    # every value is d * (ls - 32) * codebook exactly: no rounding happens in f32
+    blocks = packed.reshape(-1, 136)
+    for bi in (0, 7, 51):
+        b = blocks[bi]
+        d = Fraction(float(b[0:2].copy().view(np.float16)[0]))
+        scales_h = int(b[2]) | (int(b[3]) << 8)
+        for sub in range(8):
+            ls = ((int(b[4 + sub // 2]) >> (4 * (sub % 2))) & 15) | (((scales_h >> (2 * sub)) & 3) << 4)
+            for j in range(32):
+                byte = int(b[8 + 16 * sub + (j & 15)])
+                value = int(fx.IQ4_VALUES[byte & 15 if j < 16 else byte >> 4])
+                want = d * (ls - 32) * value
+                got = Fraction(float(dense.reshape(-1, 256)[bi, 32 * sub + j]))
+                assert got == want
+
+
+def test_iq4_xs_reduces_to_the_reference_iq4_nl_decoder():
+    # with ls = 33 every sub-block is an IQ4_NL block of the same d and the same 16 bytes
+    count = 40
+    rng = np.random.default_rng(5)
+    d = (0.01 + 0.02 * rng.random(count)).astype(np.float16)
+    index = rng.integers(0, 16, (count, 256), dtype=np.uint8)
+    packed = fx.iq4_xs_pack(d, np.full((count, 8), 33), index)
+    dense = oracle.dequantize(IQ4_XS, packed.reshape(-1), count, 256)
+    nl = np.empty((count, 8, 18), dtype=np.uint8)
+    nl[:, :, 0:2] = d.view(np.uint8).reshape(count, 1, 2)
+    nl[:, :, 2:] = packed[:, 8:].reshape(count, 8, 16)
+    assert np.array_equal(bits(dense), bits(fx.iq4_nl_dense(nl).reshape(count, 256)))
+
+
+def test_iq4_xs_scale_bits_at_every_position():
+    # all 64 scale values at each of the 8 sub-block positions, the others held at 32 (zero)
+    d = np.float16(0.03125)
+    index = np.full((1, 256), 15, dtype=np.uint8)        # codebook value 113
+    for position in range(8):
+        for ls in range(64):
+            scales = np.full((1, 8), 32)
+            scales[0, position] = ls
+            dense = oracle.dequantize(IQ4_XS, fx.iq4_xs_pack([d], scales, index).reshape(-1), 1, 256)[0]
+            want = np.zeros(256, dtype=np.float32)
+            want[32 * position: 32 * position + 32] = np.float32(d) * np.float32(ls - 32) * np.float32(113)
+            assert np.array_equal(bits(dense), bits(want)), (position, ls)
+
+
+def test_iq4_xs_projection_is_the_float64_product_of_the_dequantised_matrix():
+    from ferrum_amd import synth
+    rows, cols = 9, 1280
+    packed = synth.matrix(IQ4_XS, rows, cols, seed=81)
+    dense = oracle.dequantize(IQ4_XS, packed, rows, cols)
+    assert np.isfinite(dense).all() and np.abs(dense).max() > 0
+    # the synthetic packer and the fixture packer are separate code: same fields, same bytes
+    blocks = packed.reshape(-1, 136)
+    scales_h = blocks[:, 2].astype(np.uint32) | (blocks[:, 3].astype(np.uint32) << 8)
+    ls = np.stack([((blocks[:, 4 + i // 2] >> (4 * (i % 2))) & 15) | (((scales_h >> (2 * i)) & 3) << 4)
+                   for i in range(8)], axis=1)
+    q = blocks[:, 8:].reshape(-1, 8, 16)
+    index = np.concatenate([q & 15, q >> 4], axis=2).reshape(-1, 256)
+    assert np.array_equal(fx.iq4_xs_pack(blocks[:, 0:2].copy().view(np.float16).reshape(-1), ls, index), blocks)
+    x = fx.xorshift_uniform(3 * cols, 9).reshape(3, cols)
+    want = x.astype(np.float64) @ dense.astype(np.float64).T
+    assert np.abs(oracle.project(IQ4_XS, packed, rows, cols, x, accumulate="f64") - want).max() <= 1e-6 * np.abs(want).max()
+    assert oracle.validate_payload(IQ4_XS, packed[:-1]) == 1
+    bad = packed.copy(); bad[0:2] = np.frombuffer(np.float16(np.inf).tobytes(), dtype=np.uint8)
+    assert oracle.validate_payload(IQ4_XS, bad) == 2

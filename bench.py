@@ -30,8 +30,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA, published
-Q4_K, Q5_K, Q6_K, IQ4_XS = 12, 13, 14, 23
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
+BLOCK_BYTES = {Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}    # per 256 weights
 ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
 
 # HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
@@ -328,6 +328,7 @@ def main():
             cases.append(layer_case(api, synth, dev, 400))
         timed(Q5_K, 17408, 5120, 1, f32, "Q5_K GEMV M=1 K=5120 N=17408", 600)
         timed(IQ4_XS, 17408, 5120, 1, f32, "IQ4_XS GEMV M=1 K=5120 N=17408", 600)
+        timed(Q8_0, 17408, 5120, 1, f32, "Q8_0 GEMV M=1 K=5120 N=17408", 400)
         timed(Q6_K, 5120, 17408, 1, f32, "Q6_K GEMV M=1 K=17408 N=5120", 600)
         timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
         for m in (8, 16, 128):
@@ -335,6 +336,7 @@ def main():
         gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
         for m in (8, 512):
             timed(IQ4_XS, 17408, 5120, m, f16, f"IQ4_XS GEMM M={m} K=5120 N=17408 f16 x", 240)
+            timed(Q8_0, 17408, 5120, m, f16, f"Q8_0 GEMM M={m} K=5120 N=17408 f16 x", 240)
         if not args.only or args.only in "Q4_K GEMM M=512 K=5120 N=17408 f32 x":
             dev.set_tuning("gemm_f32_min_rows", 5)   # the hybrid engine's tiering: f16 tiles from 5 rows on
             timed(Q4_K, 17408, 5120, 512, f32, "Q4_K GEMM M=512 K=5120 N=17408 f32 x (rounded to f16 for the tiles)", 120)

@@ -166,6 +166,7 @@ class DType(enum.IntEnum):
 
 
 class QuantizationFormat(enum.Enum):
+    Q8_0 = 8       # the hybrid engine's Format::Q8_0; rows in runs of eight 34-byte blocks
     Q4_K = 12
     Q5_K = 13
     Q6_K = 14
@@ -182,10 +183,12 @@ class QuantizationFormat(enum.Enum):
         return self.value
 
     def block_elements(self) -> int:
+        """Weights per unit of a row: a super-block, or for Q8_0 eight 32-weight GGML blocks
+        (rows are a multiple of 256 weights long in every format)."""
         return 256
 
     def block_bytes(self) -> int:
-        return {12: 144, 13: 176, 14: 210, 23: 136}[self.value]
+        return {8: 272, 12: 144, 13: 176, 14: 210, 23: 136}[self.value]
 
 
 def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:

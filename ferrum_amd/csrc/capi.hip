@@ -360,7 +360,11 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
     *out = nullptr;
     const size_t bb = block_bytes(ggml_type);
     if (bb == 0) return fail(FH_ERR_GGUF, "unsupported quantized weight type %u", ggml_type);
-    const char* name = ggml_type == kQ4K ? "Q4_K" : ggml_type == kQ5K ? "Q5_K" : ggml_type == kQ6K ? "Q6_K" : "IQ4_XS";
+    const char* name = ggml_type == kQ4K   ? "Q4_K"
+                       : ggml_type == kQ5K ? "Q5_K"
+                       : ggml_type == kQ6K ? "Q6_K"
+                       : ggml_type == kQ8_0 ? "Q8_0"
+                                            : "IQ4_XS";
     if (rows == 0 || cols == 0 || cols % 256 != 0)
         return fail(FH_ERR_SHAPE, "%s matrix requires nonempty rows and columns divisible by block size 256",
                     name);
@@ -377,6 +381,11 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
                     (unsigned long long)byte_len);
     const uint8_t* p = static_cast<const uint8_t*>(packed);
     for (size_t off = 0; off < packed_len; off += bb) {
+        if (ggml_type == kQ8_0) {
+            for (size_t sub = 0; sub < 272; sub += 34)
+                if (!f16_finite(p + off + sub)) return fail(FH_ERR_WEIGHT, "%s scale must be finite", name);
+            continue;
+        }
         bool ok = ggml_type == kQ6K     ? f16_finite(p + off + 208)
                   : ggml_type == kIQ4XS ? f16_finite(p + off)
                                         : (f16_finite(p + off) && f16_finite(p + off + 2));
@@ -545,7 +554,8 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
             name = weight->ggml_type == kQ4K   ? "q4_k_gemm"
                    : weight->ggml_type == kQ5K ? "q5_k_gemm"
                    : weight->ggml_type == kQ6K ? "q6_k_gemm"
-                                               : "iq4_xs_gemm";
+                   : weight->ggml_type == kQ8_0 ? "q8_0_gemm"
+                                                : "iq4_xs_gemm";
         device->last_operation = name;
     }
     FH_HIP(hipGetLastError());

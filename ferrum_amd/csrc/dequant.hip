@@ -1,4 +1,4 @@
-// Whole-matrix dequantisation and embedding gather for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS.
+// Whole-matrix dequantisation and embedding gather for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS / Q8_0.
 //
 // Values follow the reference's per-element decoders (q4_k_weight,
 // src/metal/shaders/ops.metal:834-845; q6_k_weight, :1316-1329); the gather
@@ -21,6 +21,8 @@ __device__ __forceinline__ float weight_at(const uint8_t* w, size_t row, uint32_
         return q5k_weight(w, row, column, blocks);
     } else if constexpr (TYPE == kIQ4XS) {
         return iq4xs_weight(w, row, column, blocks);
+    } else if constexpr (TYPE == kQ8_0) {
+        return q8_0_weight(w, row, column, blocks);
     } else {
         return q6k_weight(w, row, column, blocks);
     }
@@ -108,6 +110,11 @@ const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, 
                            static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
         return "dequantize_iq4_xs";
     }
+    if (ggml_type == kQ8_0) {
+        hipLaunchKernelGGL(dequantize_kernel<kQ8_0>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
+        return "dequantize_q8_0";
+    }
     hipLaunchKernelGGL(dequantize_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
                        static_cast<const uint8_t*>(w), rows, (uint32_t)cols, out, out_dtype);
     return "dequantize_q6_k";
@@ -134,6 +141,12 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                            static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
                            out_dtype);
         return "embedding_gather_iq4_xs";
+    }
+    if (ggml_type == kQ8_0) {
+        hipLaunchKernelGGL(embedding_gather_kernel<kQ8_0>, dim3(grid), dim3(256), 0, s,
+                           static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,
+                           out_dtype);
+        return "embedding_gather_q8_0";
     }
     hipLaunchKernelGGL(embedding_gather_kernel<kQ6K>, dim3(grid), dim3(256), 0, s,
                        static_cast<const uint8_t*>(w), (uint32_t)cols, ids_dev, count, out,

@@ -222,6 +222,52 @@ __device__ __forceinline__ float iq4xs_weight(const uint8_t* w, size_t row, uint
     return iq4xs_scale(h0, h1, sub) * (float)value;
 }
 
+// ---- Q8_0 (34 B: f16 d, int8 qs[32]; eight blocks per 256 weights) ---------------
+//
+// block_q8_0 / dequantize_q8_0 (src/metal/shaders/hybrid.metal:23, 499-508; CPU
+// twin src/hybrid/draft/gguf.rs:331-338): weight = d * q, exact in f32.
+
+__device__ __forceinline__ float q8_0_weight(const uint8_t* w, size_t row, uint32_t column, uint32_t blocks) {
+    const uint8_t* block = w + (row * blocks + (column >> 8)) * 272 + 34 * ((column & 255u) >> 5);
+    const float d = f16_bits_to_f32(block[0] | (block[1] << 8));
+    return d * (float)(int)(int8_t)block[2 + (column & 31u)];
+}
+
+// 4-byte aligned 16-byte and 4-byte loads
+__device__ __forceinline__ uint32_t load_u32_unaligned(const uint8_t* p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+
+// One lane's 64 weights of a 256-weight run: blocks 2c and 2c + 1, 68 bytes at 68c,
+// [d0][q0 x 32][d1][q1 x 32].  The quants of the first block straddle dwords by two
+// bytes; v_alignbyte_b32 puts them back.  q + 128 (a byte xor) is then widened like
+// the other formats' quants.
+struct Q8Pair {
+    uint32_t w[17];
+    __device__ __forceinline__ void load(const uint8_t* p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 v;
+            __builtin_memcpy(&v, p + 16 * i, 16);
+            w[4 * i] = v.x;
+            w[4 * i + 1] = v.y;
+            w[4 * i + 2] = v.z;
+            w[4 * i + 3] = v.w;
+        }
+        w[16] = load_u32_unaligned(p + 64);
+    }
+    __device__ __forceinline__ float d(int block) const {
+        return f16_bits_to_f32(block == 0 ? (w[0] & 0xffffu) : (w[8] >> 16));
+    }
+    // quant dword j (0..7) of block `block`, four bytes of q + 128
+    __device__ __forceinline__ uint32_t biased(int block, int j) const {
+        const uint32_t q = block == 0 ? __builtin_amdgcn_alignbyte(w[j + 1], w[j], 2) : w[9 + j];
+        return q ^ 0x80808080u;
+    }
+};
+
 // ---- wave reductions -----------------------------------------------------------
 
 template <int CTRL>

@@ -1,4 +1,4 @@
-// Dequant-fused tile GEMM for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS on gfx950:
+// Dequant-fused tile GEMM for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS / Q8_0 on gfx950:
 // Y[M,N] = X[M,K] * W[N,K]^T, f16 or bf16 activations, f32 accumulation.
 //
 // Stands in for the reference's tile kernels q4_k_gemm_mpp / q6_k_gemm_mpp
@@ -37,6 +37,9 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 // 32 + 16h; Q6_K and IQ4_XS decode 32 consecutive weights at 32h.
 template <uint32_t TYPE>
 constexpr bool kNibblePlanes = TYPE == kQ4K || TYPE == kQ5K;
+// a producer's task reads eight input dwords (one value per byte) instead of four (two nibbles per byte)
+template <uint32_t TYPE>
+constexpr bool kEightDwords = TYPE == kQ6K || TYPE == kQ8_0;
 template <uint32_t TYPE>
 __device__ __forceinline__ constexpr uint32_t k_lo_of(uint32_t h) { return kNibblePlanes<TYPE> ? 16 * h : 32 * h; }
 template <uint32_t TYPE>
@@ -146,6 +149,35 @@ struct RawW<kIQ4XS> {
             out_lo[2 * t + 1] = fma_pair<DT>(lo_half(l23), hi_half(l23), scale, offset);
             out_hi[2 * t] = fma_pair<DT>(lo_half(u01), hi_half(u01), scale, offset);
             out_hi[2 * t + 1] = fma_pair<DT>(lo_half(u23), hi_half(u23), scale, offset);
+        }
+    }
+};
+
+// Q8_0: K slab c is blocks 2c and 2c + 1 of the 256-weight run; thread half h decodes
+// block 2c + h: 34 bytes at 34 (2c + h), two-byte aligned.
+template <>
+struct RawW<kQ8_0> {
+    uint4 qa, qb;
+    uint32_t dh;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c, uint32_t h) {
+        const uint8_t* b = block + 34 * (2 * c + h);
+        dh = load_u16_unaligned(b);
+        qa = load_u4_unaligned(b + 2);
+        qb = load_u4_unaligned(b + 18);
+    }
+    // out_lo: 16 weights at k = 32h + i; out_hi: 16 weights at k = 32h + 16 + i
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t, uint32_t (&out_lo)[8], uint32_t (&out_hi)[8], uint32_t) const {
+        const float d = f16_bits_to_f32(dh);
+        const float scale = d * 16777216.f, offset = -128.f * d;
+        const uint32_t q[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t u = q[t] ^ 0x80808080u;
+            const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
+            uint32_t* out = t < 4 ? out_lo : out_hi;
+            out[2 * (t & 3)] = fma_pair<DT>(lo_half(u01), hi_half(u01), scale, offset);
+            out[2 * (t & 3) + 1] = fma_pair<DT>(lo_half(u23), hi_half(u23), scale, offset);
         }
     }
 };
@@ -452,6 +484,40 @@ struct BlockW<kIQ4XS> {
     }
 };
 
+// Q8_0: half h of slab c is block 2c + h; input dword t (0..7) gives the pair dwords of its
+// weights 4t .. 4t + 3.
+template <>
+struct BlockW<kQ8_0> {
+    uint4 q[4][2];
+    uint32_t dh[4];
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t h) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint8_t* b = block + 34 * (2 * c + h);
+            dh[c] = load_u16_unaligned(b);
+            q[c][0] = load_u4_unaligned(b + 2);
+            q[c][1] = load_u4_unaligned(b + 18);
+        }
+    }
+    struct Scales {
+        float scale, offset;
+    };
+    __device__ __forceinline__ Scales scales(int c, uint32_t) const {
+        const float d = f16_bits_to_f32(dh[c]);
+        return {d * 16777216.f, -128.f * d};
+    }
+    template <int DT>
+    __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
+        const uint32_t v[8] = {q[c][0].x, q[c][0].y, q[c][0].z, q[c][0].w, q[c][1].x, q[c][1].y, q[c][1].z, q[c][1].w};
+        const uint32_t u = v[t] ^ 0x80808080u;
+        const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
+        out[0] = fma_pair<DT>(lo_half(u01), hi_half(u01), s.scale, s.offset);
+        out[1] = fma_pair<DT>(lo_half(u23), hi_half(u23), s.scale, s.offset);
+        out[2] = 0;
+        out[3] = 0;
+    }
+};
+
 template <>
 struct BlockW<kQ6K> {
     uint4 l[2][2], p[2][2], sc;  // ql / qh of both halves, the 16 scales
@@ -512,7 +578,7 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_block_slab(const BlockW<TYPE>& blk, int c, uint32_t h,
                                                   uint16_t* wrow_lds) {
     const auto s = blk.scales(c, h);
-    if constexpr (TYPE != kQ6K) {
+    if constexpr (!kEightDwords<TYPE>) {
         uint32_t lo[8], hi[8];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -549,7 +615,7 @@ template <uint32_t TYPE, int DT>
 __device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int c, uint32_t h, int t,
                                                    uint16_t* wrow_lds) {
     const auto s = blk.scales(c, h);
-    if constexpr (TYPE != kQ6K) {
+    if constexpr (!kEightDwords<TYPE>) {
         uint32_t out[4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
@@ -608,7 +674,7 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
         const uint32_t er = 128 + (lane >> 3), eh = (lane >> 2) & 1u, et = lane & 3u;
         const uint8_t* esrc = w + (size_t)(n0 + (er < ncols ? er : ncols - 1)) * nb * kBlockBytes;
         // register sets: the block being decoded and the next one or two in flight
-        constexpr bool kDeep = TYPE != kQ6K;   // Q6_K sets are twice as large: one block ahead
+        constexpr bool kDeep = !kEightDwords<TYPE>;   // Q6_K and Q8_0 sets are twice as large: one block ahead
         BlockW<TYPE> cur, n1, n2, ecur, en1, en2;
         auto load_block = [&](BlockW<TYPE>& main, BlockW<TYPE>& extra, uint32_t b) {
             main.load(wsrc + (size_t)b * kBlockBytes, wh);
@@ -809,6 +875,10 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             if (a.x_dtype == FH_F16) launch_wide_nt<kIQ4XS, 1>(s, a, plan); else launch_wide_nt<kIQ4XS, 2>(s, a, plan);
             return "iq4_xs_gemm_mfma_m256";
         }
+        if (a.ggml_type == kQ8_0) {
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ8_0, 1>(s, a, plan); else launch_wide_nt<kQ8_0, 2>(s, a, plan);
+            return "q8_0_gemm_mfma_m256";
+        }
         if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
         return "q6_k_gemm_mfma_m256";
     }
@@ -850,6 +920,14 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
             run(gemm_tile_kernel<kIQ4XS, 2, 128>, gemm_tile_kernel<kIQ4XS, 2, 64>);
         }
         return "iq4_xs_gemm_mfma";
+    }
+    if (a.ggml_type == kQ8_0) {
+        if (a.x_dtype == FH_F16) {
+            run(gemm_tile_kernel<kQ8_0, 1, 128>, gemm_tile_kernel<kQ8_0, 1, 64>);
+        } else {
+            run(gemm_tile_kernel<kQ8_0, 2, 128>, gemm_tile_kernel<kQ8_0, 2, 64>);
+        }
+        return "q8_0_gemm_mfma";
     }
     if (a.x_dtype == FH_F16) {
         run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>);

@@ -1,5 +1,5 @@
 // Skinny-M projection (2 <= M <= 64 tokens, f16 / bf16 activations) on the
-// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q5_K / Q6_K / IQ4_XS weights.
+// matrix cores: Y[M,N] = X[M,K] . W[N,K]^T for Q4_K / Q5_K / Q6_K / IQ4_XS / Q8_0 weights.
 //
 // With this few tokens the job is a weight stream (HBM bound), so nothing of
 // the weights goes through LDS.  A wave owns 16 weight rows.  Its 64 lanes are
@@ -157,6 +157,34 @@ struct Quarter<kIQ4XS> {
             a[4 * sub + 1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
             a[4 * sub + 2] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
             a[4 * sub + 3] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+        }
+    }
+};
+
+// Q8_0: lane group g owns blocks 2g and 2g + 1 of the 256-weight run; operand s covers
+// weights 64g + 8s .., two quant dwords of one block.
+template <>
+struct Quarter<kQ8_0> {
+    static constexpr uint32_t kBlockBytes = 272;
+    Q8Pair p;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t g) { p.load(block + 68 * g); }
+    static __device__ __forceinline__ uint32_t klocal(uint32_t g, int s) { return 64 * g + 8 * s; }
+    template <int DT>
+    __device__ __forceinline__ void decode(uint32_t, uint4 (&a)[8]) const {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const float d = p.d(blk);
+            const float scale = d * 16777216.f, offset = -128.f * d;   // fma(q + 128, d, -128 d) = d q, exact
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const uint32_t u0 = p.biased(blk, 2 * s), u1 = p.biased(blk, 2 * s + 1);
+                const uint32_t a01 = bytes01_as_halves(u0), a23 = bytes23_as_halves(u0);
+                const uint32_t b01 = bytes01_as_halves(u1), b23 = bytes23_as_halves(u1);
+                a[4 * blk + s] = make_uint4(fma_pair<DT>(lo_half(a01), hi_half(a01), scale, offset),
+                                            fma_pair<DT>(lo_half(a23), hi_half(a23), scale, offset),
+                                            fma_pair<DT>(lo_half(b01), hi_half(b01), scale, offset),
+                                            fma_pair<DT>(lo_half(b23), hi_half(b23), scale, offset));
+            }
         }
     }
 };
@@ -610,6 +638,10 @@ const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
     if (a.ggml_type == kIQ4XS) {
         if (a.x_dtype == FH_F16) launch_tt<kIQ4XS, 1>(s, a); else launch_tt<kIQ4XS, 2>(s, a);
         return grouped ? "expert_project_iq4_xs_grouped_mfma" : "iq4_xs_gemm_mfma_skinny";
+    }
+    if (a.ggml_type == kQ8_0) {
+        if (a.x_dtype == FH_F16) launch_tt<kQ8_0, 1>(s, a); else launch_tt<kQ8_0, 2>(s, a);
+        return grouped ? "expert_project_q8_0_grouped_mfma" : "q8_0_gemm_mfma_skinny";
     }
     if (a.x_dtype == FH_F16) launch_tt<kQ6K, 1>(s, a); else launch_tt<kQ6K, 2>(s, a);
     return grouped ? "expert_project_q6_k_grouped_mfma" : "q6_k_gemm_mfma_skinny";

@@ -1,4 +1,4 @@
-// Dequant-fused GEMV for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS on gfx950: y[n] = sum_k W[n,k] x[k].
+// Dequant-fused GEMV for GGUF Q4_K / Q5_K / Q6_K / IQ4_XS / Q8_0 on gfx950: y[n] = sum_k W[n,k] x[k].
 //
 // Stands in for the reference's M = 1 kernels q4_k_gemv_ksplit / _factored
 // (src/metal/shaders/ops.metal:983-1070) and q6_k_gemv_ksplit / _factored
@@ -193,6 +193,33 @@ struct Frag<kIQ4XS> {
         const float r0 = fmaf(acc[0][0] + acc[0][1], 16777216.f, -128.f * (s.x + s.y));
         const float r1 = fmaf(acc[1][0] + acc[1][1], 16777216.f, -128.f * (s.z + s.w));
         return fmaf(dl0, r0, dl1 * r1);
+    }
+};
+
+// Q8_0: lane c owns blocks 2c and 2c + 1 of the 256-weight run (68 bytes).  q + 128
+// is widened like a nibble; the 128 comes off through the activation sums.
+template <>
+struct Frag<kQ8_0> {
+    Q8Pair p;
+    __device__ __forceinline__ void load(const uint8_t* block, uint32_t c) { p.load(block + 68 * c); }
+    __device__ __forceinline__ float dot(const float4* xc, float4 s, uint32_t) const {
+        float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // [block][two chains]
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float4 x = xc[(8 * blk + j) * 4];
+                const uint32_t u = p.biased(blk, j);
+                const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
+                acc[blk][0] = fmaf(lo_half(u01), x.x, acc[blk][0]);
+                acc[blk][1] = fmaf(hi_half(u01), x.y, acc[blk][1]);
+                acc[blk][0] = fmaf(lo_half(u23), x.z, acc[blk][0]);
+                acc[blk][1] = fmaf(hi_half(u23), x.w, acc[blk][1]);
+            }
+        }
+        const float r0 = fmaf(acc[0][0] + acc[0][1], 16777216.f, -128.f * (s.x + s.y));
+        const float r1 = fmaf(acc[1][0] + acc[1][1], 16777216.f, -128.f * (s.z + s.w));
+        return fmaf(p.d(0), r0, p.d(1) * r1);
     }
 };
 
@@ -513,15 +540,17 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     LaunchFn fn = a.ggml_type == kQ4K     ? pick<kQ4K>(plan.bs, plan.it)
                   : a.ggml_type == kQ5K   ? pick<kQ5K>(plan.bs, plan.it)
                   : a.ggml_type == kIQ4XS ? pick<kIQ4XS>(plan.bs, plan.it)
+                  : a.ggml_type == kQ8_0  ? pick<kQ8_0>(plan.bs, plan.it)
                                           : pick<kQ6K>(plan.bs, plan.it);
     fn(grid, lds, s, p);
-    const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : a.ggml_type == kQ6K ? 2 : 3;
-    static const char* const expert_names[4] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
-                                                "expert_project_q6_k_factored", "expert_project_iq4_xs_factored"};
-    static const char* const ksplit_names[4] = {"q4_k_gemv_ksplit", "q5_k_gemv_ksplit", "q6_k_gemv_ksplit",
-                                                "iq4_xs_gemv_ksplit"};
-    static const char* const factored_names[4] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored",
-                                                  "iq4_xs_gemv_factored"};
+    const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : a.ggml_type == kQ6K ? 2 : a.ggml_type == kIQ4XS ? 3 : 4;
+    static const char* const expert_names[5] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
+                                                "expert_project_q6_k_factored", "expert_project_iq4_xs_factored",
+                                                "expert_project_q8_0_factored"};
+    static const char* const ksplit_names[5] = {"q4_k_gemv_ksplit", "q5_k_gemv_ksplit", "q6_k_gemv_ksplit",
+                                                "iq4_xs_gemv_ksplit", "q8_0_gemv_ksplit"};
+    static const char* const factored_names[5] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored",
+                                                  "iq4_xs_gemv_factored", "q8_0_gemv_factored"};
     if (a.metadata != nullptr) return expert_names[f];
     if (plan.segments > 1) return ksplit_names[f];
     return factored_names[f];

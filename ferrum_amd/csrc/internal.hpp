@@ -66,10 +66,16 @@ constexpr uint32_t kQ4K = FH_GGML_Q4_K;
 constexpr uint32_t kQ5K = FH_GGML_Q5_K;
 constexpr uint32_t kQ6K = FH_GGML_Q6_K;
 constexpr uint32_t kIQ4XS = FH_GGML_IQ4_XS;
+constexpr uint32_t kQ8_0 = FH_GGML_Q8_0;
 
-// bytes of one 256-weight super-block
+// bytes of 256 weights: one super-block, or eight 34-byte blocks of Q8_0
 constexpr uint32_t block_bytes_of(uint32_t ggml_type) {
-    return ggml_type == kQ4K ? 144u : ggml_type == kQ5K ? 176u : ggml_type == kQ6K ? 210u : ggml_type == kIQ4XS ? 136u : 0u;
+    return ggml_type == kQ4K     ? 144u
+           : ggml_type == kQ5K   ? 176u
+           : ggml_type == kQ6K   ? 210u
+           : ggml_type == kIQ4XS ? 136u
+           : ggml_type == kQ8_0  ? 272u
+                                 : 0u;
 }
 
 inline size_t block_bytes(uint32_t ggml_type) {

@@ -17,8 +17,8 @@ from __future__ import annotations
 
 import numpy as np
 
-Q4_K, Q5_K, Q6_K, IQ4_XS = 12, 13, 14, 23
-BLOCK_BYTES = {Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}
+Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
+BLOCK_BYTES = {Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}    # per 256 weights
 
 
 def rng(seed: int, stream: int = 0) -> np.random.Generator:
@@ -117,6 +117,15 @@ def iq4_xs_blocks(count: int, g: np.random.Generator) -> np.ndarray:
     return blocks
 
 
+def q8_0_blocks(count: int, g: np.random.Generator) -> np.ndarray:
+    """`count` runs of 256 weights: eight 34-byte blocks (f16 d, int8 qs[32]) each."""
+    blocks = np.empty((count * 8, 34), dtype=np.uint8)
+    d = (np.abs(g.standard_normal(count * 8)) * 0.0005).astype(np.float32).astype(np.float16)
+    blocks[:, 0:2] = d.view(np.uint8).reshape(-1, 2)
+    blocks[:, 2:] = g.integers(-128, 128, (count * 8, 32), dtype=np.int8).view(np.uint8)
+    return blocks.reshape(count, 272)
+
+
 def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> np.ndarray:
     """Packed row-major ``[rows, cols]`` matrix as a flat uint8 array."""
     if cols % 256:
@@ -131,6 +140,8 @@ def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> 
         return q6_k_blocks(count, g).reshape(-1)
     if ggml_type == IQ4_XS:
         return iq4_xs_blocks(count, g).reshape(-1)
+    if ggml_type == Q8_0:
+        return q8_0_blocks(count, g).reshape(-1)
     raise ValueError(f"unsupported ggml type {ggml_type}")
 
 

@@ -98,19 +98,28 @@ inline float f16_bits_to_f32(uint16_t h) {
     return v;
 }
 
-// IQ4_XS is the hybrid engine's Format::Iq4Xs (src/hybrid/weights.rs:38-60)
+// IQ4_XS and Q8_0 are the hybrid engine's Format::Iq4Xs / Format::Q8_0 (src/hybrid/weights.rs:29-60).
+// Rows are a multiple of 256 weights long in every format; for Q8_0 a unit is eight 34-byte GGML blocks.
 enum class QuantizationFormat : uint32_t {
-    Q4_K = FH_GGML_Q4_K, Q5_K = FH_GGML_Q5_K, Q6_K = FH_GGML_Q6_K, IQ4_XS = FH_GGML_IQ4_XS
+    Q8_0 = FH_GGML_Q8_0, Q4_K = FH_GGML_Q4_K, Q5_K = FH_GGML_Q5_K, Q6_K = FH_GGML_Q6_K, IQ4_XS = FH_GGML_IQ4_XS
 };
 inline size_t block_elements(QuantizationFormat) { return 256; }
 inline size_t block_bytes(QuantizationFormat f) {
-    return f == QuantizationFormat::Q4_K ? 144 : f == QuantizationFormat::Q5_K ? 176 : f == QuantizationFormat::Q6_K ? 210 : 136;
+    switch (f) {
+        case QuantizationFormat::Q8_0: return 272;
+        case QuantizationFormat::Q4_K: return 144;
+        case QuantizationFormat::Q5_K: return 176;
+        case QuantizationFormat::Q6_K: return 210;
+        case QuantizationFormat::IQ4_XS: return 136;
+    }
+    return 0;
 }
 inline QuantizationFormat format_from_ggml_type(uint32_t id) {
     if (id == FH_GGML_Q4_K) return QuantizationFormat::Q4_K;
     if (id == FH_GGML_Q5_K) return QuantizationFormat::Q5_K;
     if (id == FH_GGML_Q6_K) return QuantizationFormat::Q6_K;
     if (id == FH_GGML_IQ4_XS) return QuantizationFormat::IQ4_XS;
+    if (id == FH_GGML_Q8_0) return QuantizationFormat::Q8_0;
     throw Error(ErrorKind::Gguf, "unsupported GGML type " + std::to_string(id));
 }
 

@@ -32,6 +32,9 @@
  *       scale assembly is checked for all 64 values at all 8 positions
  *       against blocks packed by a separately written packer; the value is
  *       exact in f32 (17-bit scale x 7-bit codebook), checked in rationals.
+ *   fo_dequantize / fo_weight, Q8_0
+ *                          pinned: numpy (int8 view times float16 view) on the
+ *       reference's random-block generator; block form = per-element form.
  *   fo_project_f32seq / fo_project_f64
  *                          pinned: integer special case (d=1, sc=1, dmin=0)
  *       equals an exact integer dot; all-zero quants equal -dmin*m*sum(x);
@@ -67,6 +70,7 @@
 #define FO_Q5_K 13u
 #define FO_Q6_K 14u
 #define FO_IQ4_XS 23u
+#define FO_Q8_0 8u
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -164,6 +168,7 @@ size_t fo_block_bytes(uint32_t ggml_type) {
     if (ggml_type == FO_Q5_K) return 176;
     if (ggml_type == FO_Q6_K) return 210;
     if (ggml_type == FO_IQ4_XS) return 136; /* src/loader/gguf.rs:111 */
+    if (ggml_type == FO_Q8_0) return 8 * 34;  /* 256 weights = eight 34-byte blocks, src/loader/gguf.rs:99 */
     return 0;
 }
 
@@ -293,6 +298,17 @@ static void dequant_iq4_xs_block(const uint8_t* b, float* out) {
     }
 }
 
+/* Q8_0, 256 weights = eight blocks of {f16 d, int8 qs[32]}: value = q * d
+ * (src/hybrid/draft/gguf.rs:331-338; dequantize_q8_0,
+ * src/metal/shaders/hybrid.metal:499-508). */
+static void dequant_q8_0_run(const uint8_t* b, float* out) {
+    for (int block = 0; block < 8; block++) {
+        const uint8_t* p = b + 34 * block;
+        float d = fo_f16_to_f32(le16(p));
+        for (int j = 0; j < 32; j++) out[32 * block + j] = (float)(int8_t)p[2 + j] * d;
+    }
+}
+
 static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) {
     if (ggml_type == FO_Q4_K)
         dequant_q4_k_block(block, out);
@@ -300,6 +316,8 @@ static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) 
         dequant_q5_k_block(block, out);
     else if (ggml_type == FO_IQ4_XS)
         dequant_iq4_xs_block(block, out);
+    else if (ggml_type == FO_Q8_0)
+        dequant_q8_0_run(block, out);
     else
         dequant_q6_k_block(block, out);
 }
@@ -354,6 +372,11 @@ float fo_weight(uint32_t ggml_type, const uint8_t* packed, size_t row, size_t co
         float c = dmin * (float)mn;
         return b - c;
     }
+    if (ggml_type == FO_Q8_0) {
+        /* one value of the row's flat run of 34-byte blocks: block column / 32, quant column % 32 */
+        const uint8_t* block = packed + row * (blocks * 272) + (column >> 5) * 34;
+        return fo_f16_to_f32(le16(block)) * (float)(int8_t)block[2 + (column & 31)];
+    }
     if (ggml_type == FO_IQ4_XS) {
         /* the indexing of the GEMV kernel mv_iq4_xs (src/metal/shaders/hybrid.metal:899-951):
          * sub-block ib = group, byte 16 ib + (lane & 15), low nibble for lanes 0..15 and high
@@ -390,6 +413,9 @@ int fo_validate_payload(uint32_t ggml_type, const uint8_t* payload, size_t len) 
             if (!isfinite(fo_f16_to_f32(le16(b))) || !isfinite(fo_f16_to_f32(le16(b + 2)))) return 2;
         } else if (ggml_type == FO_IQ4_XS) {
             if (!isfinite(fo_f16_to_f32(le16(b)))) return 2;
+        } else if (ggml_type == FO_Q8_0) {
+            for (int block = 0; block < 8; block++)
+                if (!isfinite(fo_f16_to_f32(le16(b + 34 * block)))) return 2;
         } else {
             if (!isfinite(fo_f16_to_f32(le16(b + 208)))) return 2;
         }

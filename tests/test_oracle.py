@@ -740,3 +740,30 @@ def test_iq4_xs_projection_is_the_float64_product_of_the_dequantised_matrix():
     assert oracle.validate_payload(IQ4_XS, packed[:-1]) == 1
     bad = packed.copy(); bad[0:2] = np.frombuffer(np.float16(np.inf).tobytes(), dtype=np.uint8)
     assert oracle.validate_payload(IQ4_XS, bad) == 2
+
+
+# ------------------------------------------------------------------ Q8_0
+
+Q8_0 = 8
+
+
+def test_q8_0_decoder_equals_numpy_on_the_reference_generator():
+    # value = q * d (src/hybrid/draft/gguf.rs:331-338); 256 weights are eight 34-byte blocks
+    rows, cols = 13, 1024
+    packed = fx.hybrid_random_blocks(rows * cols // 32, 34, 34)
+    assert oracle.block_bytes(Q8_0) == 272 and oracle.validate_payload(Q8_0, packed) == 0
+    b = packed.reshape(-1, 34)
+    want = (b[:, 2:].view(np.int8).astype(np.float32)
+            * b[:, 0:2].copy().view(np.float16).astype(np.float32)).reshape(rows, cols)
+    dense = oracle.dequantize(Q8_0, packed, rows, cols)
+    assert np.array_equal(bits(dense), bits(want))
+    rng = np.random.default_rng(8)
+    for _ in range(3000):
+        r, c = int(rng.integers(rows)), int(rng.integers(cols))
+        assert bits(np.float32(oracle.weight(Q8_0, packed, r, c, cols))) == bits(dense[r, c])
+    x = fx.xorshift_uniform(3 * cols, 9).reshape(3, cols)
+    ref = x.astype(np.float64) @ dense.astype(np.float64).T
+    assert np.abs(oracle.project(Q8_0, packed, rows, cols, x, accumulate="f64") - ref).max() <= 1e-6 * np.abs(ref).max()
+    assert oracle.validate_payload(Q8_0, packed[:-1]) == 1
+    bad = packed.copy(); bad[34 * 5: 34 * 5 + 2] = np.frombuffer(np.float16(np.nan).tobytes(), dtype=np.uint8)
+    assert oracle.validate_payload(Q8_0, bad) == 2

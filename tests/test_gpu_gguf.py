@@ -91,3 +91,24 @@ def test_stacked_gate_up_experts_from_a_gguf_file_run_the_fused_decode_chain(tmp
     assert np.abs(want).max() > 1e-4
     l2 = float(np.linalg.norm(got - want) / np.linalg.norm(want))
     assert l2 <= 2e-5, l2
+
+
+@pytest.mark.parametrize("ggml", [23, 8, 13], ids=["iq4_xs", "q8_0", "q5_k"])
+def test_other_formats_load_from_a_gguf_file(tmp_path, ggml):
+    # the file's bytes are the device payload unchanged, also for Q8_0 whose GGUF block is 32 weights
+    from ferrum_amd import api
+    d = api.Device.new()
+    n, k, experts, rows = 70, 768, 3, 20
+    dense = synth.matrix(ggml, n, k, seed=51)
+    ex = synth.matrix(ggml, experts * rows, k, seed=52)
+    path = tmp_path / "formats.gguf"
+    path.write_bytes(gf.build([("blk.0.attn_q.weight", [k, n], ggml, dense),
+                               ("blk.0.ffn_down_exps.weight", [k, rows, experts], ggml, ex)]))
+    f = gguf.GgufReader.open(str(path))
+    w = f.quantized_matrix(d, "blk.0.attn_q.weight")
+    assert (w.rows(), w.columns(), w.format().value) == (n, k, ggml)
+    assert np.array_equal(bits(d.dequantize(w).to_f32()), bits(oracle.dequantize(ggml, dense, n, k)))
+    e = f.quantized_expert_matrix(d, "blk.0.ffn_down_exps.weight")
+    assert (e.experts(), e.rows_per_expert(), e.columns()) == (experts, rows, k)
+    assert np.array_equal(bits(d.dequantize(e.matrix_view()).to_f32()),
+                          bits(oracle.dequantize(ggml, ex, experts * rows, k)))

@@ -18,34 +18,29 @@ __device__ __forceinline__ uint32_t total_order_key(float x) {
 }
 
 template <int CTRL>
-__device__ __forceinline__ unsigned long long dpp_max_u64(unsigned long long v) {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, 0xf, 0xf, false);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, 0xf, 0xf, false);
-    const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+__device__ __forceinline__ uint32_t dpp_max_u32(uint32_t v) {
+    const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
     return other > v ? other : v;
 }
 
-// Maximum over the 64 lanes, returned in all lanes; every lane must be active.
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-    v = dpp_max_u64<0xB1>(v);   // quad_perm [1,0,3,2]
-    v = dpp_max_u64<0x4E>(v);   // quad_perm [2,3,0,1]
-    v = dpp_max_u64<0x141>(v);  // row_half_mirror
-    v = dpp_max_u64<0x140>(v);  // row_mirror: every lane now holds its row's maximum
-    unsigned long long best = 0ull;
-#pragma unroll
-    for (int row = 0; row < 4; ++row) {
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 16 * row);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 16 * row);
-        const unsigned long long other = ((unsigned long long)hi << 32) | lo;
-        best = other > best ? other : best;
-    }
-    return best;
+// Maximum over the 64 lanes as a wave-uniform value; every lane must be active.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = dpp_max_u32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_u32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_u32<0x141>(v);  // row_half_mirror
+    v = dpp_max_u32<0x140>(v);  // row_mirror: every lane now holds its row's maximum
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
 }
 
 // One wave per token.  Scores are computed by all lanes in parallel; the
 // softmax normaliser is then summed by one lane in expert order so it carries
 // the same f32 rounding as a sequential host loop.  Selection runs top_k
-// rounds of a wave-wide arg-max over (total-order key, lower id wins).
+// rounds of a wave-wide arg-max over (total-order key, lower id wins).  With one
+// token the kernel is one wave's dependent instruction stream, so its length is
+// its duration: reductions are DPP, owners are found by ballot.
 template <int kPerLane>   // experts <= 64 * kPerLane
 __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ logits,
                                                        uint32_t logits_dtype,
@@ -116,68 +111,79 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
         for (int i = 0; i < kPerLane; ++i) score[i] = score[i] / normalizer;
     }
 
-    unsigned long long packed[kPerLane];
+    // Selection: top_k rounds of a wave-wide arg-max over the total-order key of the
+    // biased score, the lower expert id winning ties.  The maximum is a 32-bit DPP
+    // reduction; its owner is then found by ballot: expert ids grow with the slot i first
+    // and the lane second, so the lowest id is the first lane of the first slot that holds it.
+    uint32_t key[kPerLane];
+    uint32_t alive = 0;
 #pragma unroll
     for (int i = 0; i < kPerLane; ++i) {
-        uint32_t e = lane + 64u * i;
-        float selection = score[i] + (bias != nullptr && e < experts ? bias[e] : 0.f);
-        // 0 marks "not a candidate"; valid entries have low word >= 1
-        packed[i] = e < experts ? ((unsigned long long)total_order_key(selection) << 32) |
-                                      (0xffffffffu - e)
-                                : 0ull;
+        const uint32_t e = lane + 64u * i;
+        const float selection = score[i] + (bias != nullptr && e < experts ? bias[e] : 0.f);
+        key[i] = e < experts ? total_order_key(selection) : 0u;
+        alive |= e < experts ? 1u << i : 0u;
     }
 
-    uint32_t sel_id[kMaxTopK];
-    float sel_score[kMaxTopK];
+    uint32_t my_id = 0xffffffffu;   // lane r < top_k: the expert of rank r and its raw score
+    float my_score = 0.f;
+    float selected_sum = 0.f;
 #pragma unroll
     for (int rank = 0; rank < kMaxTopK; ++rank) {
         if ((uint32_t)rank < top_k) {
-            unsigned long long best = 0ull;
+            uint32_t best = 0;
 #pragma unroll
-            for (int i = 0; i < kPerLane; ++i) best = packed[i] > best ? packed[i] : best;
-            best = wave_max_u64(best);
-            uint32_t id = 0xffffffffu - (uint32_t)best;
+            for (int i = 0; i < kPerLane; ++i) best = key[i] > best ? key[i] : best;
+            best = wave_max_u32(best);
+            uint32_t slot = kPerLane;
+            unsigned long long owners = 0ull;
+#pragma unroll
+            for (int i = kPerLane - 1; i >= 0; --i) {
+                const unsigned long long mask = __ballot(((alive >> i) & 1u) != 0 && key[i] == best);
+                if (mask != 0ull) {
+                    slot = (uint32_t)i;
+                    owners = mask;
+                }
+            }
+            const uint32_t owner = (uint32_t)__ffsll((long long)owners) - 1u;
             float mine = 0.f;
 #pragma unroll
             for (int i = 0; i < kPerLane; ++i) {
-                if (lane + 64u * i == id) {
-                    mine = score[i];
-                    packed[i] = 0ull;
+                if ((uint32_t)i == slot && lane == owner) {
+                    mine = score[i];   // the raw score (bias excluded)
+                    key[i] = 0u;
+                    alive &= ~(1u << i);
                 }
             }
-            // the owner lane publishes the raw score (bias excluded)
-            sel_score[rank] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), id & 63u));
-            sel_id[rank] = id;
-        } else {
-            sel_id[rank] = 0xffffffffu;
-            sel_score[rank] = 0.f;
+            const float chosen = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), owner));
+            selected_sum += chosen;
+            if (lane == (uint32_t)rank) {
+                my_id = owner + 64u * slot;
+                my_score = chosen;
+            }
         }
     }
-
-    float selected_sum = 0.f;
-#pragma unroll
-    for (int rank = 0; rank < kMaxTopK; ++rank)
-        if ((uint32_t)rank < top_k) selected_sum += sel_score[rank];
     const float denominator = selected_sum + eps;
 
-    // Rows are written in expert-id order: lane r places entry r at the
-    // number of selected ids below its own.
+    // Rows are written in expert-id order (lane r places entry r at the number of selected
+    // ids below its own), or in selection order for the hybrid engine's router.
+    uint32_t position = 0;
 #pragma unroll
-    for (int rank = 0; rank < kMaxTopK; ++rank) {
-        if ((uint32_t)rank < top_k && lane == (uint32_t)rank) {
-            uint32_t position = 0;
-#pragma unroll
-            for (int other = 0; other < kMaxTopK; ++other)
-                if ((uint32_t)other < top_k && sel_id[other] < sel_id[rank]) ++position;
-            if (rank_order) position = (uint32_t)rank;  // the hybrid engine keeps selection order
-            float weight = sel_score[rank];
-            if (normalize) weight = weight / denominator;
-            weight = weight * scaling;
-            float* out = metadata + ((size_t)token * top_k + position) * 3;
-            out[0] = __uint_as_float(sel_id[rank]);
-            out[1] = __uint_as_float(token);
-            out[2] = weight;
+    for (int other = 0; other < kMaxTopK; ++other) {
+        if ((uint32_t)other < top_k) {
+            const uint32_t id = (uint32_t)__builtin_amdgcn_readlane((int)my_id, other);
+            position += id < my_id ? 1u : 0u;
         }
+    }
+    if (rank_order) position = lane;
+    if (lane < top_k) {
+        float weight = my_score;
+        if (normalize) weight = weight / denominator;
+        weight = weight * scaling;
+        float* out = metadata + ((size_t)token * top_k + position) * 3;
+        out[0] = __uint_as_float(my_id);
+        out[1] = __uint_as_float(token);
+        out[2] = weight;
     }
 
     // Shared-expert gate of h_moe_route (src/metal/shaders/hybrid.metal:2259-2319):
@@ -306,13 +312,18 @@ __global__ __launch_bounds__(256) void expert_silu_mul8_kernel(const void* __res
     }
 }
 
+// The dtypes are template parameters: with one token the kernel is a single short
+// dependent instruction stream, and every runtime dtype switch lengthens it.
+template <uint32_t in_dtype, uint32_t out_dtype>
 __global__ __launch_bounds__(256) void expert_combine8_kernel(const void* __restrict__ in,
                                                               const float* __restrict__ metadata,
                                                               void* __restrict__ out, uint32_t tokens,
                                                               uint32_t hidden, uint32_t top_k,
-                                                              uint32_t in_dtype, uint32_t out_dtype,
                                                               const void* __restrict__ shared,
                                                               const float* __restrict__ shared_gate) {
+    // each product is rounded before it is added: with f32 storage round_storage is the
+    // identity and would not keep the compiler from fusing the two into an fma
+#pragma clang fp contract(off)
     const size_t total = (size_t)tokens * hidden / 8;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
@@ -472,8 +483,15 @@ const char* launch_expert_combine(hipStream_t s, const void* in, const float* me
     const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
                            reinterpret_cast<uintptr_t>(shared)) & 15u) == 0;
     if (hidden % 8 == 0 && aligned) {
-        hipLaunchKernelGGL(expert_combine8_kernel, dim3(grid_for((size_t)tokens * hidden / 8)), dim3(256), 0,
-                           s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype, shared, shared_gate);
+        const dim3 grid(grid_for((size_t)tokens * hidden / 8));
+#define FH_COMBINE(I, O)                                                                                       \
+    if (in_dtype == I && out_dtype == O)                                                                       \
+        hipLaunchKernelGGL((expert_combine8_kernel<I, O>), grid, dim3(256), 0, s, in, metadata, out, tokens,   \
+                           hidden, top_k, shared, shared_gate);
+        FH_COMBINE(0, 0) FH_COMBINE(0, 1) FH_COMBINE(0, 2)
+        FH_COMBINE(1, 0) FH_COMBINE(1, 1) FH_COMBINE(1, 2)
+        FH_COMBINE(2, 0) FH_COMBINE(2, 1) FH_COMBINE(2, 2)
+#undef FH_COMBINE
     } else {
         hipLaunchKernelGGL(expert_combine_kernel, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0,
                            s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype, shared, shared_gate);

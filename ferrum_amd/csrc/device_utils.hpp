@@ -290,9 +290,24 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    // lanes the pattern leaves unwritten keep the old value (the first operand): their own v
+    int moved = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, false);
+    return fmaxf(v, __int_as_float(moved));
+}
+
+// Maximum over the 64 lanes, returned in all lanes; every lane of the wave must be active.
 __device__ __forceinline__ float wave_max(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    v = dpp_max<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max<0x141>(v);  // row_half_mirror
+    v = dpp_max<0x140>(v);  // row_mirror
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
 }  // namespace fh

@@ -272,57 +272,58 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    const uint32_t steps = nb * 4;
-    RawW<TYPE> raw;
-    uint4 xr[4];
-    raw.load(wsrc, 0, lh);
+    // One register stage per K slab of a super-block: the loads of a slab are issued a whole
+    // block (four slabs) before it is decoded, so a memory round trip is spread over four steps.
+    RawW<TYPE> raw[4];
+    uint4 xr[4][4];
+    auto fetch = [&](int c, uint32_t block) {
+        raw[c].load(wsrc + (size_t)block * kBlockBytes, (uint32_t)c, lh);
+        const uint4* xp = reinterpret_cast<const uint4*>(xsrc + ((size_t)block * 4 + c) * kBK);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        xr[i] = xlive ? reinterpret_cast<const uint4*>(xsrc)[i] : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) xr[c][i] = xlive ? xp[i] : make_uint4(0, 0, 0, 0);
+    };
+#pragma unroll
+    for (int c = 0; c < 4; ++c) fetch(c, 0);
 
-    for (uint32_t step = 0; step < steps; ++step) {
-        const uint32_t c = step & 3u;
-        uint32_t lo[8], hi[8];
-        if constexpr (kNibblePlanes<TYPE>) {
-            raw.template decode<DT>(c, lo, hi);
-        } else {
-            raw.template decode<DT>(c, lo, hi, lh);
-        }
-        __syncthreads();  // previous step's fragment reads are done
-        {
-            const uint32_t k_lo = k_lo_of<TYPE>(lh), k_hi = k_hi_of<TYPE>(lh);
-            uint4* dst_lo = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_lo]);
-            uint4* dst_hi = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_hi]);
-            dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-            dst_lo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
-            dst_hi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-            dst_hi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-            uint4* xdst = reinterpret_cast<uint4*>(&xs[lrow * kLd + 32 * lh]);
+    for (uint32_t block = 0; block < nb; ++block) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) xdst[i] = xr[i];
-        }
-        if (step + 1 < steps) {
-            uint32_t nstep = step + 1;
-            raw.load(wsrc + (size_t)(nstep >> 2) * kBlockBytes, nstep & 3u, lh);
-            const uint4* xp = reinterpret_cast<const uint4*>(xsrc + (size_t)nstep * kBK);
+        for (int c = 0; c < 4; ++c) {
+            uint32_t lo[8], hi[8];
+            if constexpr (kNibblePlanes<TYPE>) {
+                raw[c].template decode<DT>((uint32_t)c, lo, hi);
+            } else {
+                raw[c].template decode<DT>((uint32_t)c, lo, hi, lh);
+            }
+            __syncthreads();  // previous step's fragment reads are done
+            {
+                const uint32_t k_lo = k_lo_of<TYPE>(lh), k_hi = k_hi_of<TYPE>(lh);
+                uint4* dst_lo = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_lo]);
+                uint4* dst_hi = reinterpret_cast<uint4*>(&ws[lrow * kLd + k_hi]);
+                dst_lo[0] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                dst_lo[1] = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+                dst_hi[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                dst_hi[1] = make_uint4(hi[4], hi[5], hi[6], hi[7]);
+                uint4* xdst = reinterpret_cast<uint4*>(&xs[lrow * kLd + 32 * lh]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) xr[i] = xlive ? xp[i] : make_uint4(0, 0, 0, 0);
-        }
-        __syncthreads();
+                for (int i = 0; i < 4; ++i) xdst[i] = xr[c][i];
+            }
+            if (block + 1 < nb) fetch(c, block + 1);
+            __syncthreads();
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            uint32_t koff = kk * 16 + 8 * (lane >> 5);
-            uint4 a[WI], b[2];
+            for (int kk = 0; kk < 4; ++kk) {
+                uint32_t koff = kk * 16 + 8 * (lane >> 5);
+                uint4 a[WI], b[2];
 #pragma unroll
-            for (int i = 0; i < WI; ++i)
-                a[i] = *reinterpret_cast<const uint4*>(&xs[(wm + 32 * i + (lane & 31u)) * kLd + koff]);
+                for (int i = 0; i < WI; ++i)
+                    a[i] = *reinterpret_cast<const uint4*>(&xs[(wm + 32 * i + (lane & 31u)) * kLd + koff]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                b[j] = *reinterpret_cast<const uint4*>(&ws[(wn + 32 * j + (lane & 31u)) * kLd + koff]);
+                for (int j = 0; j < 2; ++j)
+                    b[j] = *reinterpret_cast<const uint4*>(&ws[(wn + 32 * j + (lane & 31u)) * kLd + koff]);
 #pragma unroll
-            for (int i = 0; i < WI; ++i)
+                for (int i = 0; i < WI; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = mfma<DT>(a[i], b[j], acc[i][j]);
+                    for (int j = 0; j < 2; ++j) acc[i][j] = mfma<DT>(a[i], b[j], acc[i][j]);
+            }
         }
     }
 

@@ -118,6 +118,12 @@ SYMBOLS = {
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
     "fh_moe_route_ranked": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP]),
     "fh_expert_combine_shared": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
+    "fh_hybrid_moe_route": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP, _VP]),
+    "fh_hybrid_project_id": (_I32, [_P, _P, _VP, _VP, _U32, _U32, _VP]),
+    "fh_hybrid_moe_map": (_I32, [_P, _VP, _U32, _U32, _VP, _VP, _VP]),
+    "fh_hybrid_moe_gather": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
+    "fh_hybrid_project_mm_id": (_I32, [_P, _P, _VP, _VP, _U32, _VP]),
+    "fh_hybrid_moe_combine": (_I32, [_P, _VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
     "fh_expert_project_fused": (_I32, [_P, _P, _VP, _U32, _U32, _U32, _VP, _VP]),
@@ -663,6 +669,96 @@ class Device:
                                         gate_vector.shape()[0] if gate_vector is not None else 0,
                                         ctypes.byref(mv), ref(gv)))
         return meta, gate
+
+    # ---- the hybrid engine's routed FFN in its own layout (ids / weights as plain arrays) ----
+
+    def hybrid_moe_route(self, logits: Tensor, policy: MoeRoutingPolicy, x: Tensor | None = None,
+                         gate_vector: Tensor | None = None):
+        """h_moe_route (src/metal/shaders/hybrid.metal:2259-2319): (ids, weights, shared_gate),
+        ids and weights [tokens * top_k] in selection order, ids as u32 bits in an F32 carrier."""
+        dims = logits.shape()
+        if len(dims) != 2 or dims[0] == 0 or dims[1] != policy.experts:
+            raise ShapeError("invalid sparse routing geometry")
+        if gate_vector is not None and (x is None or x.shape() != (dims[0], gate_vector.shape()[0])
+                                        or gate_vector.dtype != DType.F32):
+            raise ShapeError("the shared-expert gate needs x [tokens, hidden] and an f32 vector [hidden]")
+        ids = Tensor.zeros(self, (dims[0] * policy.top_k,), DType.F32)
+        weights = Tensor.zeros(self, (dims[0] * policy.top_k,), DType.F32)
+        gate = Tensor.zeros(self, (dims[0],), DType.F32)
+        lv, iv, wtv, gv, pc = logits._view(), ids._view(), weights._view(), gate._view(), policy._c()
+        xv = x._view() if gate_vector is not None else None
+        wv = gate_vector._view() if gate_vector is not None else None
+        ref = lambda v: ctypes.byref(v) if v is not None else None
+        _check(_lib.fh_hybrid_moe_route(self._handle, ctypes.byref(lv), dims[0], ctypes.byref(pc), ref(xv), ref(wv),
+                                        gate_vector.shape()[0] if gate_vector is not None else 0,
+                                        ctypes.byref(iv), ctypes.byref(wtv), ctypes.byref(gv)))
+        return ids, weights, gate
+
+    def hybrid_project_id(self, weight: "QuantizedExpertMatrix", x: Tensor, ids: Tensor, routes: int, x_div: int,
+                          out_dtype: DType | None = None) -> Tensor:
+        """HybridModel::project_id (src/hybrid/engine.rs:3113-3148): route r multiplies activation
+        row r / x_div by expert ids[r]."""
+        if (routes == 0 or x_div == 0 or routes % x_div or ids.shape() != (routes,) or ids.dtype != DType.F32
+                or x.shape() != (routes // x_div, weight.columns())):
+            raise ShapeError("expert projection geometry")
+        y = Tensor.zeros(self, (routes, weight.rows_per_expert()), out_dtype or x.dtype)
+        xv, iv, yv = x._view(), ids._view(), y._view()
+        _check(_lib.fh_hybrid_project_id(self._handle, _handle_of(weight), ctypes.byref(xv), ctypes.byref(iv), routes,
+                                         x_div, ctypes.byref(yv)))
+        return y
+
+    def hybrid_moe_map(self, ids: Tensor, experts: int):
+        """h_moe_map (hybrid.metal:2321-2358): (offsets [experts + 1], sorted [routes], position
+        [routes]) as u32 bits in F32 carriers."""
+        routes = ids.numel()
+        if routes == 0 or ids.dtype != DType.F32:
+            raise ShapeError("route map needs routes")
+        offsets = Tensor.zeros(self, (experts + 1,), DType.F32)
+        order = Tensor.zeros(self, (routes,), DType.F32)
+        position = Tensor.zeros(self, (routes,), DType.F32)
+        iv, ov, sv, pv = ids._view(), offsets._view(), order._view(), position._view()
+        _check(_lib.fh_hybrid_moe_map(self._handle, ctypes.byref(iv), experts, routes, ctypes.byref(ov),
+                                      ctypes.byref(sv), ctypes.byref(pv)))
+        return offsets, order, position
+
+    def hybrid_moe_gather(self, x: Tensor, order: Tensor, used: int) -> Tensor:
+        """h_moe_gather (hybrid.metal:2360-2370): out[p] = x[sorted[p] / used]."""
+        dims, routes = x.shape(), order.numel()
+        if len(dims) != 2 or used == 0 or routes != dims[0] * used:
+            raise ShapeError("route gather needs [tokens, hidden] and tokens * used routes")
+        out = Tensor.zeros(self, (routes, dims[1]), x.dtype)
+        xv, sv, ov = x._view(), order._view(), out._view()
+        _check(_lib.fh_hybrid_moe_gather(self._handle, ctypes.byref(xv), ctypes.byref(sv), dims[1], used, routes,
+                                         ctypes.byref(ov)))
+        return out
+
+    def hybrid_project_mm_id(self, weight: "QuantizedExpertMatrix", x: Tensor, offsets: Tensor,
+                             out_dtype: DType | None = None) -> Tensor:
+        """HybridModel::project_mm_id (src/hybrid/engine.rs:3150-3220): rows offsets[e] ..
+        offsets[e + 1] of the expert-sorted x are multiplied by expert e."""
+        dims = x.shape()
+        if len(dims) != 2 or dims[0] == 0 or dims[1] != weight.columns() or offsets.shape() != (weight.experts() + 1,):
+            raise ShapeError("expert projection geometry")
+        y = Tensor.zeros(self, (dims[0], weight.rows_per_expert()), out_dtype or x.dtype)
+        xv, fv, yv = x._view(), offsets._view(), y._view()
+        _check(_lib.fh_hybrid_project_mm_id(self._handle, _handle_of(weight), ctypes.byref(xv), ctypes.byref(fv),
+                                            dims[0], ctypes.byref(yv)))
+        return y
+
+    def hybrid_moe_combine(self, down: Tensor, weights: Tensor, position: Tensor | None, shared: Tensor,
+                           shared_gate: Tensor, used: int) -> Tensor:
+        """h_moe_combine (hybrid.metal:2372-2388), f32: the weighted sum of each token's routed rows
+        (row = position[route], or the route itself when position is None) plus gate * shared."""
+        tokens, hidden = shared.shape()
+        if (down.shape() != (tokens * used, hidden) or weights.numel() != tokens * used
+                or shared_gate.shape() != (tokens,) or (position is not None and position.numel() != tokens * used)):
+            raise ShapeError("expert combine geometry mismatch")
+        out = Tensor.zeros(self, (tokens, hidden), DType.F32)
+        views = [t._view() if t is not None else None for t in (down, weights, position, shared, shared_gate, out)]
+        ref = lambda v: ctypes.byref(v) if v is not None else None
+        _check(_lib.fh_hybrid_moe_combine(self._handle, ref(views[0]), ref(views[1]), ref(views[2]), ref(views[3]),
+                                          ref(views[4]), hidden, used, tokens, ref(views[5])))
+        return out
 
     def expert_combine_shared(self, input: Tensor, metadata: Tensor, tokens: int, hidden: int, top_k: int,
                               shared: Tensor, shared_gate: Tensor | None = None,

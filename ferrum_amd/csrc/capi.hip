@@ -144,6 +144,7 @@ int64_t tuning(const fh_device* d, const char* key) {
 
 using namespace fh;
 
+static_assert(kXDivide > FH_INPUT_SILU_MUL, "the row-divide mode is internal: it has no public input form");
 static_assert(kXPlain == FH_INPUT_ROWS && kXGather == FH_INPUT_GATHER && kXSiluMul == FH_INPUT_SILU_MUL,
               "the kernel's input modes are the ABI's input forms");
 
@@ -630,7 +631,8 @@ namespace {
 
 fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const fh_view* selection_bias,
                 const fh_routing_policy* policy, const fh_view* metadata, bool ranked, const fh_view* gate_x,
-                const fh_view* gate_w, uint32_t hidden, const fh_view* shared_gate) {
+                const fh_view* gate_w, uint32_t hidden, const fh_view* shared_gate, const fh_view* ids = nullptr,
+                const fh_view* weights = nullptr) {
     if (device == nullptr || policy == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     const fh_routing_policy& p = *policy;
     if (tokens == 0 || p.experts == 0 || p.top_k == 0 || p.top_k > 16 || p.top_k > p.experts ||
@@ -648,13 +650,29 @@ fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const
         st = resolve(device, selection_bias, p.experts, "selection bias", &br, 4);
         if (st != FH_OK) return st == FH_ERR_DEVICE_MISMATCH ? fail(FH_ERR_SHAPE, "invalid sparse routing geometry") : st;
     }
-    if (metadata == nullptr || metadata->dtype != FH_F32)
-        return fail(FH_ERR_DTYPE, "routing metadata must be f32");
-    st = resolve(device, metadata, (uint64_t)tokens * p.top_k * 3, "routing metadata", &mr, 4);
-    if (st != FH_OK) return st;
-    if (overlaps(lr, mr)) return fail(FH_ERR_RANGE, "routing metadata aliases the logits");
     RouteExtras extras;
     extras.rank_order = ranked ? 1u : 0u;
+    mr = Range{nullptr, 0};
+    if (ids == nullptr) {
+        if (metadata == nullptr || metadata->dtype != FH_F32)
+            return fail(FH_ERR_DTYPE, "routing metadata must be f32");
+        st = resolve(device, metadata, (uint64_t)tokens * p.top_k * 3, "routing metadata", &mr, 4);
+        if (st != FH_OK) return st;
+        if (overlaps(lr, mr)) return fail(FH_ERR_RANGE, "routing metadata aliases the logits");
+    } else {
+        // the hybrid engine's layout: ids and weights as two [tokens, top_k] f32 carriers
+        if (weights == nullptr || ids->dtype != FH_F32 || weights->dtype != FH_F32)
+            return fail(FH_ERR_DTYPE, "route ids and weights are f32 carriers");
+        Range ir, wr;
+        st = resolve(device, ids, (uint64_t)tokens * p.top_k, "route ids", &ir, 4);
+        if (st != FH_OK) return st;
+        st = resolve(device, weights, (uint64_t)tokens * p.top_k, "route weights", &wr, 4);
+        if (st != FH_OK) return st;
+        if (overlaps(lr, ir) || overlaps(lr, wr) || overlaps(ir, wr))
+            return fail(FH_ERR_RANGE, "route outputs alias the logits or each other");
+        extras.ids_out = reinterpret_cast<float*>(const_cast<uint8_t*>(ir.begin));
+        extras.weights_out = reinterpret_cast<float*>(const_cast<uint8_t*>(wr.begin));
+    }
     if (shared_gate != nullptr) {
         if (shared_gate->dtype != FH_F32) return fail(FH_ERR_DTYPE, "the shared-expert gate is f32");
         Range gr;
@@ -694,6 +712,182 @@ fh_status fh_moe_route_ranked(fh_device* device, const fh_view* logits, uint32_t
                               const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
                               uint32_t hidden, const fh_view* metadata, const fh_view* shared_gate) {
     return route(device, logits, tokens, nullptr, policy, metadata, true, x, gate_vector, hidden, shared_gate);
+}
+
+// ---- the hybrid engine's MoE stages over plain id / weight arrays ----------------------
+
+fh_status fh_hybrid_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
+                              const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
+                              uint32_t hidden, const fh_view* ids, const fh_view* weights,
+                              const fh_view* shared_gate) {
+    if (ids == nullptr) return fail(FH_ERR_RANGE, "route ids: null view");
+    return route(device, logits, tokens, nullptr, policy, nullptr, true, x, gate_vector, hidden, shared_gate, ids,
+                 weights);
+}
+
+fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
+                               uint32_t routes, uint32_t x_div, const fh_view* y) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device || routes == 0 || x_div == 0 || routes % x_div != 0 || ids == nullptr ||
+        ids->dtype != FH_F32)
+        return fail(FH_ERR_SHAPE, "expert projection geometry");
+    const uint64_t rows = weight->rows, k = weight->cols;
+    if (!fits_u32((uint64_t)routes * rows) || !fits_u32((uint64_t)routes / x_div * k))
+        return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+    Range xr, ir, yr;
+    fh_status st = resolve(device, x, (uint64_t)routes / x_div * k, "expert input", &xr);
+    if (st != FH_OK) return st;
+    st = resolve(device, ids, routes, "route ids", &ir, 4);
+    if (st != FH_OK) return st;
+    st = resolve(device, y, (uint64_t)routes * rows, "expert output", &yr);
+    if (st != FH_OK) return st;
+    if (overlaps(xr, yr) || overlaps(ir, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    GemvArgs a{};
+    a.ggml_type = weight->ggml_type;
+    a.w = weight->ptr;
+    a.x = xr.begin;
+    a.y = const_cast<uint8_t*>(yr.begin);
+    a.n = (uint32_t)rows;
+    a.k = (uint32_t)k;
+    a.m = routes;
+    a.x_dtype = x->dtype;
+    a.y_dtype = y->dtype;
+    a.metadata = reinterpret_cast<const float*>(ir.begin);
+    a.meta_stride = 1;
+    a.experts = (uint32_t)weight->experts;
+    a.x_mode = kXDivide;
+    a.x_div = x_div;
+    a.x_rows = routes / x_div;
+    st = prepare_gemv(device, a);
+    if (st != FH_OK) return st;
+    launch_gemv(device->stream, a);
+    device->last_operation = weight->ggml_type == kQ4K     ? "h_mv_id_q4_k"
+                             : weight->ggml_type == kQ5K   ? "h_mv_id_q5_k"
+                             : weight->ggml_type == kQ6K   ? "h_mv_id_q6_k"
+                             : weight->ggml_type == kQ8_0  ? "h_mv_id_q8_0"
+                                                           : "h_mv_id_iq4_xs";
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_hybrid_moe_map(fh_device* device, const fh_view* ids, uint32_t experts, uint32_t routes,
+                            const fh_view* offsets, const fh_view* sorted, const fh_view* position) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (experts == 0 || experts > 1024 || routes == 0) return fail(FH_ERR_SHAPE, "route map needs 1..1024 experts and routes");
+    for (const fh_view* v : {ids, offsets, sorted, position})
+        if (v == nullptr || v->dtype != FH_F32) return fail(FH_ERR_DTYPE, "route map operands are f32 carriers of u32");
+    Range ir, fr, sr, pr;
+    fh_status st = resolve(device, ids, routes, "route ids", &ir, 4);
+    if (st != FH_OK) return st;
+    if ((st = resolve(device, offsets, (uint64_t)experts + 1, "expert offsets", &fr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, sorted, routes, "sorted routes", &sr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, position, routes, "route positions", &pr, 4)) != FH_OK) return st;
+    if (overlaps(ir, fr) || overlaps(ir, sr) || overlaps(ir, pr) || overlaps(fr, sr) || overlaps(fr, pr) ||
+        overlaps(sr, pr))
+        return fail(FH_ERR_RANGE, "route map operands alias");
+    auto words = [](const Range& r) { return reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(r.begin)); };
+    device->last_operation = launch_moe_map(device->stream, words(ir), experts, routes, words(fr), words(sr), words(pr));
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_hybrid_moe_gather(fh_device* device, const fh_view* x, const fh_view* sorted, uint32_t hidden,
+                               uint32_t used, uint32_t routes, const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (hidden == 0 || used == 0 || routes == 0 || routes % used != 0 || !fits_u32((uint64_t)routes * hidden))
+        return fail(FH_ERR_SHAPE, "route gather needs [tokens, hidden] and tokens * used routes");
+    if (sorted == nullptr || sorted->dtype != FH_F32 || x == nullptr || out == nullptr || out->dtype != x->dtype)
+        return fail(FH_ERR_DTYPE, "route gather: sorted is an f32 carrier, output dtype is the input's");
+    Range xr, sr, orr;
+    fh_status st = resolve(device, x, (uint64_t)routes / used * hidden, "gather input", &xr);
+    if (st != FH_OK) return st;
+    if ((st = resolve(device, sorted, routes, "sorted routes", &sr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, out, (uint64_t)routes * hidden, "gather output", &orr)) != FH_OK) return st;
+    if (overlaps(xr, orr) || overlaps(sr, orr)) return fail(FH_ERR_RANGE, "gather output aliases an input");
+    device->last_operation = launch_moe_gather_sorted(
+        device->stream, xr.begin, reinterpret_cast<const uint32_t*>(sr.begin), const_cast<uint8_t*>(orr.begin), routes,
+        used, routes / used, hidden * (uint32_t)dtype_bytes(x->dtype));
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                  const fh_view* offsets, uint32_t routes, const fh_view* y) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device || routes == 0 || weight->experts > 1024 || offsets == nullptr ||
+        offsets->dtype != FH_F32 || x == nullptr || y == nullptr)
+        return fail(FH_ERR_SHAPE, "expert projection geometry");
+    const uint64_t rows = weight->rows, k = weight->cols;
+    if (!fits_u32((uint64_t)routes * rows) || !fits_u32((uint64_t)routes * k))
+        return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+    if ((rows * dtype_bytes(y->dtype)) % 4 != 0) return fail(FH_ERR_SHAPE, "expert output rows must be whole words");
+    Range xr, fr, yr;
+    fh_status st = resolve(device, x, (uint64_t)routes * k, "expert input", &xr);
+    if (st != FH_OK) return st;
+    if ((st = resolve(device, offsets, weight->experts + 1, "expert offsets", &fr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, y, (uint64_t)routes * rows, "expert output", &yr)) != FH_OK) return st;
+    if (overlaps(xr, yr) || overlaps(fr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    // the tiles are f16 / bf16, as the reference's h_mm_id kernels make theirs; f32 rows are rounded to f16 first
+    const void* tile_x = xr.begin;
+    if (x->dtype == FH_F32) {
+        st = ensure_scratch(device, (size_t)routes * k * sizeof(uint16_t));
+        if (st != FH_OK) return st;
+        uint16_t* x16 = reinterpret_cast<uint16_t*>(scratch_data(device));
+        launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin), x16, (size_t)routes * k);
+        tile_x = x16;
+    }
+    GemmArgs g{};
+    g.ggml_type = weight->ggml_type;
+    g.w = weight->ptr;
+    g.x = tile_x;
+    g.y = const_cast<uint8_t*>(yr.begin);
+    g.n = (uint32_t)rows;
+    g.k = (uint32_t)k;
+    g.m = routes;
+    g.x_dtype = x->dtype == FH_F32 ? FH_F16 : x->dtype;
+    g.y_dtype = y->dtype;
+    g.cu_count = device->props.multiProcessorCount;
+    g.experts = (uint32_t)weight->experts;
+    g.expert_offsets = reinterpret_cast<const uint32_t*>(fr.begin);
+    g.expert_order = nullptr;   // rows are already expert-sorted
+    launch_gemm_skinny(device->stream, g);
+    device->last_operation = weight->ggml_type == kQ4K     ? "h_mm_id_q4_k"
+                             : weight->ggml_type == kQ5K   ? "h_mm_id_q5_k"
+                             : weight->ggml_type == kQ6K   ? "h_mm_id_q6_k"
+                             : weight->ggml_type == kQ8_0  ? "h_mm_id_q8_0"
+                                                           : "h_mm_id_iq4_xs";
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_hybrid_moe_combine(fh_device* device, const fh_view* down, const fh_view* weights,
+                                const fh_view* position, const fh_view* shared, const fh_view* shared_gate,
+                                uint32_t hidden, uint32_t used, uint32_t tokens, const fh_view* out) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (hidden == 0 || used == 0 || tokens == 0 || !fits_u32((uint64_t)tokens * used * hidden))
+        return fail(FH_ERR_SHAPE, "route combine needs [tokens * used, hidden]");
+    for (const fh_view* v : {down, weights, shared, shared_gate, out})
+        if (v == nullptr || v->dtype != FH_F32) return fail(FH_ERR_DTYPE, "the hybrid combine works on f32 rows");
+    if (position != nullptr && position->dtype != FH_F32) return fail(FH_ERR_DTYPE, "positions are an f32 carrier of u32");
+    const uint64_t routes = (uint64_t)tokens * used;
+    Range dr, wr, pr{nullptr, 0}, sr, gr, orr;
+    fh_status st = resolve(device, down, routes * hidden, "expert rows", &dr);
+    if (st != FH_OK) return st;
+    if ((st = resolve(device, weights, routes, "route weights", &wr, 4)) != FH_OK) return st;
+    if (position != nullptr && (st = resolve(device, position, routes, "route positions", &pr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, shared, (uint64_t)tokens * hidden, "shared rows", &sr)) != FH_OK) return st;
+    if ((st = resolve(device, shared_gate, tokens, "shared gate", &gr, 4)) != FH_OK) return st;
+    if ((st = resolve(device, out, (uint64_t)tokens * hidden, "combine output", &orr)) != FH_OK) return st;
+    if (overlaps(dr, orr) || overlaps(wr, orr) || overlaps(sr, orr) || overlaps(gr, orr) ||
+        (position != nullptr && overlaps(pr, orr)))
+        return fail(FH_ERR_RANGE, "combine output aliases an input");
+    device->last_operation = launch_hybrid_combine(
+        device->stream, reinterpret_cast<const float*>(dr.begin), reinterpret_cast<const float*>(wr.begin),
+        reinterpret_cast<const uint32_t*>(pr.begin), reinterpret_cast<const float*>(sr.begin),
+        reinterpret_cast<const float*>(gr.begin), reinterpret_cast<float*>(const_cast<uint8_t*>(orr.begin)), hidden, used,
+        tokens, (uint32_t)routes);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
 }
 
 fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t tokens,

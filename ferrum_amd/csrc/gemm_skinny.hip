@@ -269,7 +269,8 @@ struct SlabRegs {
 
 // GROUPED = false: the dense projection, tokens 0 .. m-1 of x, one weight matrix.
 // GROUPED = true: the routed-expert projection.  blockIdx.y is an expert; its
-// tokens are the assignments order[offsets[e]] .. order[offsets[e+1] - 1] (rows
+// tokens are the assignments order[offsets[e]] .. order[offsets[e+1] - 1], or rows
+// offsets[e] .. offsets[e+1] - 1 themselves when order is null (rows
 // of x and of y), its weights rows [e*n, e*n + n), and the workgroup makes as
 // many passes of 16*TT tokens as the expert's count needs (the weights of the
 // later passes come from L2).
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
 #pragma unroll
         for (int p = 0; p < kXP; ++p) {
             uint32_t token = first_token + t0 + min(xtok + 8 * p, mt - 1);
-            if constexpr (GROUPED) token = order[token];
+            if constexpr (GROUPED) token = order != nullptr ? order[token] : token;
             rows.row[p] = x + (size_t)token * k + xcol;
         }
 
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
             const uint32_t tok = 16 * t + r;
             if (tok >= mt) continue;
             uint32_t token = first_token + t0 + tok;
-            if constexpr (GROUPED) token = order[token];
+            if constexpr (GROUPED) token = order != nullptr ? order[token] : token;
             const size_t base = (size_t)token * n + out_row;
             if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
                 *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
@@ -459,7 +460,8 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                 const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
                 const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
                 dst[j] = tok * ld + 8 * pc;
-                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)order[first_token + t0 + tok] * k + 8 * pc);
+                const uint32_t slot = first_token + t0 + tok;
+                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)(order != nullptr ? order[slot] : slot) * k + 8 * pc);
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
@@ -474,7 +476,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
         for (int t = 0; t < TT; ++t) {
             const uint32_t tok = min(16u * t + r, mt - 1);
             boff[t] = tok * ld;
-            out_token[t] = order[first_token + t0 + tok];
+            out_token[t] = order != nullptr ? order[first_token + t0 + tok] : first_token + t0 + tok;
         }
         uint32_t kl[8];
 #pragma unroll

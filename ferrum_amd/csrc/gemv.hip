@@ -315,7 +315,10 @@ struct Params {
     uint32_t segments;
     uint32_t x_dtype, y_dtype, experts;
     uint32_t x_rows;     // rows of x, for kXGather
-    uint32_t x_mode;     // kXPlain, kXGather (row = token of the assignment) or kXSiluMul (x = silu(gate) * up)
+    uint32_t x_mode;     // kXPlain, kXGather (row = token of the assignment), kXSiluMul (x = silu(gate) * up)
+                         // or kXDivide (row = m / x_div: the routes of a token share its row)
+    uint32_t meta_stride;  // floats per batch entry in `metadata`: 3 (id, token, weight) or 1 (ids only)
+    uint32_t x_div;
 };
 
 // grid: (row tiles, K segments, m)
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     size_t row_base = 0;
     bool live = true;
     if (p.metadata != nullptr) {
-        uint32_t expert = __float_as_uint(p.metadata[3 * (size_t)m]);
+        uint32_t expert = __float_as_uint(p.metadata[p.meta_stride * (size_t)m]);
         live = expert < p.experts;
         row_base = live ? (size_t)expert * p.n : 0;
     }
@@ -349,6 +352,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     if (p.x_mode == kXGather) {
         const uint32_t token = __float_as_uint(p.metadata[3 * (size_t)m + 1]);
         xrow = token < p.x_rows ? token : p.x_rows - 1;
+    } else if (p.x_mode == kXDivide) {
+        xrow = m / p.x_div;
     }
     const size_t xbase = (xrow * (p.x_mode == kXSiluMul ? 2 : 1) * p.nb + b0) * 64;
     // the SiLU form computes on what it loads, so it fetches after the weight
@@ -535,6 +540,8 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     p.experts = a.experts;
     p.x_mode = a.x_mode;
     p.x_rows = a.x_rows;
+    p.meta_stride = a.meta_stride == 0 ? 3u : a.meta_stride;
+    p.x_div = a.x_div == 0 ? 1u : a.x_div;
     const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
     dim3 grid(plan.tiles, plan.segments, a.m);
     LaunchFn fn = a.ggml_type == kQ4K     ? pick<kQ4K>(plan.bs, plan.it)

@@ -108,6 +108,7 @@ enum : uint32_t {
     kXPlain = 0,    // row m of x
     kXGather = 1,   // row token(m) of x, the token id from the routing metadata (expert_assign fused)
     kXSiluMul = 2,  // x is [m, 2K]: silu(x[:, :K]) * x[:, K:] with expert_silu_mul's rounding
+    kXDivide = 3,   // row m / x_div of x: the hybrid engine's project_id, whose routes share a token's row
 };
 
 struct GemvArgs {
@@ -124,6 +125,8 @@ struct GemvArgs {
     int ksplit;           // 0 = automatic, else at least this many K segments
     uint32_t x_mode;      // kXPlain, kXGather or kXSiluMul
     uint32_t x_rows;      // rows of x (kXGather clamps the token id to it)
+    uint32_t meta_stride; // floats per entry of `metadata`: 0 or 3 = {id, token, weight}, 1 = ids only
+    uint32_t x_div;       // kXDivide: batch entries per row of x (0 = 1)
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
 };
@@ -166,10 +169,20 @@ struct RouteExtras {
     const float* gate_w = nullptr;     // [hidden], or null: the gate is 1
     uint32_t hidden = 0;
     float* shared_gate = nullptr;      // [tokens], or null: no gate output
+    float* ids_out = nullptr;          // [tokens, top_k] expert ids as u32 bits, or null
+    float* weights_out = nullptr;      // [tokens, top_k] route weights, or null
 };
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
                              const float* bias, float* metadata, uint32_t tokens,
                              const fh_routing_policy& policy, const RouteExtras& extras);
+// the hybrid engine's stages over plain id / weight arrays (h_moe_map, h_moe_gather, h_moe_combine)
+const char* launch_moe_map(hipStream_t s, const uint32_t* ids, uint32_t experts, uint32_t routes, uint32_t* offsets,
+                           uint32_t* sorted, uint32_t* position);
+const char* launch_moe_gather_sorted(hipStream_t s, const void* x, const uint32_t* sorted, void* out, uint32_t routes,
+                                     uint32_t used, uint32_t tokens, uint32_t row_bytes);
+const char* launch_hybrid_combine(hipStream_t s, const float* down, const float* weights, const uint32_t* position,
+                                  const float* shared, const float* shared_gate, float* out, uint32_t hidden,
+                                  uint32_t used, uint32_t tokens, uint32_t rows);
 const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t assignments,
                                 uint32_t experts, uint32_t* offsets, uint32_t* order, void* y,
                                 uint32_t row_bytes);

@@ -52,7 +52,9 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
                                                        float scaling, uint32_t rank_order,
                                                        const void* __restrict__ gate_x, uint32_t gate_x_dtype,
                                                        const float* __restrict__ gate_w, uint32_t hidden,
-                                                       float* __restrict__ shared_gate) {
+                                                       float* __restrict__ shared_gate,
+                                                       float* __restrict__ ids_out,
+                                                       float* __restrict__ weights_out) {
     extern __shared__ float scores_lds[];  // experts floats
     const uint32_t token = blockIdx.x, lane = threadIdx.x;
     if (token >= tokens) return;
@@ -180,10 +182,16 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const void* __restrict__ 
         float weight = my_score;
         if (normalize) weight = weight / denominator;
         weight = weight * scaling;
-        float* out = metadata + ((size_t)token * top_k + position) * 3;
-        out[0] = __uint_as_float(my_id);
-        out[1] = __uint_as_float(token);
-        out[2] = weight;
+        const size_t slot = (size_t)token * top_k + position;
+        if (metadata != nullptr) {
+            float* out = metadata + slot * 3;
+            out[0] = __uint_as_float(my_id);
+            out[1] = __uint_as_float(token);
+            out[2] = weight;
+        }
+        // the hybrid engine's layout: ids and weights as two [tokens, top_k] arrays
+        if (ids_out != nullptr) ids_out[slot] = __uint_as_float(my_id);
+        if (weights_out != nullptr) weights_out[slot] = weight;
     }
 
     // Shared-expert gate of h_moe_route (src/metal/shaders/hybrid.metal:2259-2319):
@@ -417,6 +425,136 @@ __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float
     }
 }
 
+// h_moe_map (src/metal/shaders/hybrid.metal:2321-2358): the deterministic expert-major
+// order of routes.  offsets[e] .. offsets[e + 1] are expert e's rows, sorted[p] is the route
+// at row p, position[r] the row of route r; inside an expert routes keep their order.
+// Routes whose id is not an expert are left out, as there.  One workgroup; experts <= 1024.
+// Routes are placed 1024 at a time: a wave ranks its 64 routes among themselves by ballot
+// and leaves one count per expert, and a route's row is its expert's next free row plus the
+// counts of the waves before its own plus its rank.
+constexpr int kMapThreads = 1024;
+constexpr int kMapWaves = kMapThreads / 64;
+
+__global__ __launch_bounds__(kMapThreads) void moe_map_kernel(const uint32_t* __restrict__ ids, uint32_t experts,
+                                                              uint32_t routes, uint32_t* __restrict__ offsets,
+                                                              uint32_t* __restrict__ sorted,
+                                                              uint32_t* __restrict__ position) {
+    __shared__ uint32_t next[kMapThreads];                 // counts, then the next free row of each expert
+    __shared__ uint32_t scan[kMapThreads];
+    __shared__ uint8_t wave_count[kMapWaves][kMapThreads];  // routes of expert e in wave w of this round
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    next[tid] = 0;
+    __syncthreads();
+    for (uint32_t r = tid; r < routes; r += kMapThreads) {
+        const uint32_t e = ids[r];
+        if (e < experts) atomicAdd(&next[e], 1u);
+    }
+    __syncthreads();
+    const uint32_t mine = next[tid];
+    scan[tid] = mine;
+    __syncthreads();
+    for (uint32_t step = 1; step < kMapThreads; step <<= 1) {
+        const uint32_t add = tid >= step ? scan[tid - step] : 0u;
+        __syncthreads();
+        scan[tid] += add;
+        __syncthreads();
+    }
+    const uint32_t first = scan[tid] - mine;
+    if (tid < experts) offsets[tid] = first;
+    if (tid == experts - 1) offsets[experts] = scan[tid];
+    next[tid] = first;
+
+    uint32_t id_bits = 0;
+    while ((1u << id_bits) < experts) ++id_bits;
+    for (uint32_t r0 = 0; r0 < routes; r0 += kMapThreads) {
+#pragma unroll
+        for (int w = 0; w < kMapWaves; ++w) wave_count[w][tid] = 0;
+        __syncthreads();
+        const uint32_t r = r0 + tid;
+        const uint32_t e = r < routes ? ids[r] : 0xffffffffu;
+        const bool valid = e < experts;
+        // lanes of this wave that hold the same expert
+        unsigned long long peers = __ballot(valid);
+        for (uint32_t b = 0; b < id_bits; ++b) {
+            const bool bit = (e >> b) & 1u;
+            const unsigned long long with_bit = __ballot(bit);
+            peers &= bit ? with_bit : ~with_bit;
+        }
+        const uint32_t rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+        if (valid && rank == 0) wave_count[wave][e] = (uint8_t)__popcll(peers);
+        __syncthreads();
+        if (valid) {
+            uint32_t row = next[e] + rank;
+            for (uint32_t w = 0; w < wave; ++w) row += wave_count[w][e];
+            sorted[row] = r;
+            position[r] = row;
+        }
+        __syncthreads();
+        uint32_t total = 0;
+#pragma unroll
+        for (int w = 0; w < kMapWaves; ++w) total += wave_count[w][tid];
+        next[tid] += total;
+        __syncthreads();
+    }
+}
+
+// h_moe_gather (src/metal/shaders/hybrid.metal:2360-2370): row p of the output is the
+// activation row of the token that route sorted[p] belongs to.  Rows move in pieces of sizeof(V).
+template <typename V>
+__global__ __launch_bounds__(256) void moe_gather_sorted_kernel(const V* __restrict__ x,
+                                                                const uint32_t* __restrict__ sorted,
+                                                                V* __restrict__ out, uint32_t used,
+                                                                uint32_t tokens, uint32_t pieces) {
+    const uint32_t row = blockIdx.x;
+    uint32_t token = sorted[row] / used;
+    token = token < tokens ? token : tokens - 1;
+    for (uint32_t i = threadIdx.x; i < pieces; i += blockDim.x) out[(size_t)row * pieces + i] = x[(size_t)token * pieces + i];
+}
+
+// h_moe_combine (src/metal/shaders/hybrid.metal:2372-2388), f32:
+// out[t] = sum_s weights[t, s] * down[row(t, s)] + shared_gate[t] * shared[t], the sum in
+// rank order; row(t, s) is the route itself or position[route].
+template <int VEC>
+__global__ __launch_bounds__(256) void hybrid_combine_kernel(const float* __restrict__ down,
+                                                             const float* __restrict__ weights,
+                                                             const uint32_t* __restrict__ position,
+                                                             const float* __restrict__ shared,
+                                                             const float* __restrict__ shared_gate,
+                                                             float* __restrict__ out, uint32_t hidden,
+                                                             uint32_t used, uint32_t tokens, uint32_t rows) {
+    const size_t total = (size_t)tokens * hidden / VEC;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = (i * VEC) / hidden, column = (i * VEC) % hidden;
+        float acc[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = 0.f;
+        for (uint32_t s = 0; s < used; ++s) {
+            const size_t r = t * used + s;
+            uint32_t row = position != nullptr ? position[r] : (uint32_t)r;
+            row = row < rows ? row : rows - 1;
+            const float w = weights[r];
+            const float* src = down + (size_t)row * hidden + column;
+            if constexpr (VEC == 4) {
+                const float4 v = *reinterpret_cast<const float4*>(src);
+                acc[0] += w * v.x;
+                acc[1] += w * v.y;
+                acc[2] += w * v.z;
+                acc[3] += w * v.w;
+            } else {
+                acc[0] += w * src[0];
+            }
+        }
+        const float g = shared_gate[t];
+        if constexpr (VEC == 4) {
+            const float4 sv = *reinterpret_cast<const float4*>(shared + i * 4);
+            *reinterpret_cast<float4*>(out + i * 4) =
+                make_float4(acc[0] + g * sv.x, acc[1] + g * sv.y, acc[2] + g * sv.z, acc[3] + g * sv.w);
+        } else {
+            out[i] = acc[0] + g * shared[i];
+        }
+    }
+}
+
 }  // namespace
 
 const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_dtype,
@@ -427,7 +565,7 @@ const char* launch_moe_route(hipStream_t s, const void* logits, uint32_t logits_
     hipLaunchKernelGGL(moe_route_kernel<PL>, dim3(tokens), dim3(64), lds, s, logits, logits_dtype, bias, \
                        metadata, tokens, p.experts, p.top_k, p.sigmoid, p.normalize_top_k_prob,         \
                        p.normalization_epsilon, p.routed_scaling_factor, x.rank_order, x.gate_x,        \
-                       x.gate_x_dtype, x.gate_w, x.hidden, x.shared_gate)
+                       x.gate_x_dtype, x.gate_w, x.hidden, x.shared_gate, x.ids_out, x.weights_out)
     if (p.experts <= 64) FH_ROUTE(1);
     else if (p.experts <= 128) FH_ROUTE(2);
     else if (p.experts <= 256) FH_ROUTE(4);
@@ -497,6 +635,42 @@ const char* launch_expert_combine(hipStream_t s, const void* in, const float* me
                            s, in, metadata, out, tokens, hidden, top_k, in_dtype, out_dtype, shared, shared_gate);
     }
     return shared != nullptr ? "h_moe_combine" : "expert_combine";
+}
+
+const char* launch_moe_map(hipStream_t s, const uint32_t* ids, uint32_t experts, uint32_t routes, uint32_t* offsets,
+                           uint32_t* sorted, uint32_t* position) {
+    hipLaunchKernelGGL(moe_map_kernel, dim3(1), dim3(kMapThreads), 0, s, ids, experts, routes, offsets, sorted,
+                       position);
+    return "h_moe_map";
+}
+
+const char* launch_moe_gather_sorted(hipStream_t s, const void* x, const uint32_t* sorted, void* out, uint32_t routes,
+                                     uint32_t used, uint32_t tokens, uint32_t row_bytes) {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (row_bytes % 16 == 0 && aligned) {
+        hipLaunchKernelGGL(moe_gather_sorted_kernel<uint4>, dim3(routes), dim3(256), 0, s, static_cast<const uint4*>(x),
+                           sorted, static_cast<uint4*>(out), used, tokens, row_bytes / 16);
+    } else {
+        hipLaunchKernelGGL(moe_gather_sorted_kernel<uint16_t>, dim3(routes), dim3(256), 0, s,
+                           static_cast<const uint16_t*>(x), sorted, static_cast<uint16_t*>(out), used, tokens,
+                           row_bytes / 2);
+    }
+    return "h_moe_gather";
+}
+
+const char* launch_hybrid_combine(hipStream_t s, const float* down, const float* weights, const uint32_t* position,
+                                  const float* shared, const float* shared_gate, float* out, uint32_t hidden,
+                                  uint32_t used, uint32_t tokens, uint32_t rows) {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(down) | reinterpret_cast<uintptr_t>(shared) |
+                           reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (hidden % 4 == 0 && aligned) {
+        hipLaunchKernelGGL(hybrid_combine_kernel<4>, dim3(grid_for((size_t)tokens * hidden / 4)), dim3(256), 0, s, down,
+                           weights, position, shared, shared_gate, out, hidden, used, tokens, rows);
+    } else {
+        hipLaunchKernelGGL(hybrid_combine_kernel<1>, dim3(grid_for((size_t)tokens * hidden)), dim3(256), 0, s, down,
+                           weights, position, shared, shared_gate, out, hidden, used, tokens, rows);
+    }
+    return "h_moe_combine";
 }
 
 }  // namespace fh

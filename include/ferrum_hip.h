@@ -237,6 +237,47 @@ fh_status fh_expert_combine_shared(fh_device* device, const fh_view* in, const f
                                    uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* shared,
                                    const fh_view* shared_gate, const fh_view* out);
 
+/* The hybrid engine's routed FFN in its own data layout: expert ids and route
+ * weights are two [tokens, used] arrays (ids as u32 bits in an f32 carrier, as
+ * the engine's Tensor::from_le_bytes(.., DType::F32, ..) holds them), not
+ * metadata triples.  HybridModel::moe_ffn, src/hybrid/engine.rs:2881-3080.
+ *
+ * fh_hybrid_moe_route  = h_moe_route (src/metal/shaders/hybrid.metal:2259-2319):
+ *   fh_moe_route_ranked writing ids, weights [tokens * top_k] and shared_gate.
+ * fh_hybrid_project_id = HybridModel::project_id (engine.rs:3113-3148, kernels
+ *   h_mv_id_*, hybrid.metal:2391-2425): route r multiplies activation row
+ *   r / x_div of x [routes / x_div, K] by expert ids[r]; y is [routes, rows].
+ *   An id that is not an expert gives a zero row.  FH_ERR_SHAPE when x_div
+ *   does not divide routes.
+ * fh_hybrid_moe_map    = h_moe_map (hybrid.metal:2321-2358): the expert-major
+ *   order of routes, stable inside an expert: offsets [experts + 1], sorted
+ *   [routes] (route at each row), position [routes] (row of each route).
+ * fh_hybrid_moe_gather = h_moe_gather (hybrid.metal:2360-2370):
+ *   out[p] = x[sorted[p] / used], x [routes / used, hidden].
+ * fh_hybrid_project_mm_id = HybridModel::project_mm_id (engine.rs:3150-3220
+ *   without arena slots, kernels h_mm_id_*): rows offsets[e] .. offsets[e+1]
+ *   of x [routes, K] are multiplied by expert e; y [routes, rows] in the same
+ *   row order.  The tiles are f16 (f32 rows are rounded first), as there.
+ * fh_hybrid_moe_combine = h_moe_combine (hybrid.metal:2372-2388), f32:
+ *   out[t] = sum_s weights[t, s] * down[row(t, s)] + shared_gate[t] * shared[t],
+ *   row(t, s) = position[t * used + s], or the route itself when position is
+ *   NULL (the engine's `identity`). */
+fh_status fh_hybrid_moe_route(fh_device* device, const fh_view* logits, uint32_t tokens,
+                              const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
+                              uint32_t hidden, const fh_view* ids, const fh_view* weights,
+                              const fh_view* shared_gate);
+fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
+                               uint32_t routes, uint32_t x_div, const fh_view* y);
+fh_status fh_hybrid_moe_map(fh_device* device, const fh_view* ids, uint32_t experts, uint32_t routes,
+                            const fh_view* offsets, const fh_view* sorted, const fh_view* position);
+fh_status fh_hybrid_moe_gather(fh_device* device, const fh_view* x, const fh_view* sorted, uint32_t hidden,
+                               uint32_t used, uint32_t routes, const fh_view* out);
+fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                  const fh_view* offsets, uint32_t routes, const fh_view* y);
+fh_status fh_hybrid_moe_combine(fh_device* device, const fh_view* down, const fh_view* weights,
+                                const fh_view* position, const fh_view* shared, const fh_view* shared_gate,
+                                uint32_t hidden, uint32_t used, uint32_t tokens, const fh_view* out);
+
 /* Decode-sized fusions.  SparseMoe::forward (src/nn/moe.rs:222-390) encodes
  * expert_assign, the gate|up projection, expert_silu_mul and the down
  * projection back to back; with a handful of assignments each of them is a

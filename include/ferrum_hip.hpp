@@ -428,6 +428,82 @@ public:
                                        &sv, shared_gate ? &gv : nullptr, &yv));
         return y;
     }
+    // ---- the hybrid engine's routed FFN in its own layout: ids / weights as plain arrays
+    // (HybridModel::moe_ffn, src/hybrid/engine.rs:2881-3080); u32 values ride in F32 carriers ----
+    struct HybridRoutes {
+        Tensor ids, weights, shared_gate;
+    };
+    // h_moe_route: ids and weights [tokens * top_k] in selection order, and the shared-expert gate
+    HybridRoutes hybrid_moe_route(const Tensor& logits, const MoeRoutingPolicy& policy, const Tensor* x = nullptr,
+                                  const Tensor* gate_vector = nullptr) const {
+        const auto& dims = logits.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != policy.experts)
+            throw Error(ErrorKind::Shape, "invalid sparse routing geometry");
+        HybridRoutes r{zeros({dims[0] * policy.top_k}, DType::F32), zeros({dims[0] * policy.top_k}, DType::F32),
+                       zeros({dims[0]}, DType::F32)};
+        fh_view lv = logits.c_view(), iv = r.ids.c_view(), wtv = r.weights.c_view(), gv = r.shared_gate.c_view(), xv{}, wv{};
+        if (x) xv = x->c_view();
+        if (gate_vector) wv = gate_vector->c_view();
+        fh_routing_policy pc = policy.c();
+        check(fh_hybrid_moe_route(handle_->raw, &lv, (uint32_t)dims[0], &pc, x ? &xv : nullptr,
+                                  gate_vector ? &wv : nullptr, gate_vector ? (uint32_t)gate_vector->numel() : 0, &iv,
+                                  &wtv, &gv));
+        return r;
+    }
+    // HybridModel::project_id: route r multiplies activation row r / x_div by expert ids[r]
+    Tensor hybrid_project_id(const QuantizedExpertMatrix& w, const Tensor& x, const Tensor& ids, size_t routes,
+                             size_t x_div) const {
+        if (routes == 0 || x_div == 0 || routes % x_div != 0 || ids.numel() != routes)
+            throw Error(ErrorKind::Shape, "expert projection geometry");
+        Tensor y = zeros({routes, w.rows_per_expert()}, x.dtype());
+        fh_view xv = x.c_view(), iv = ids.c_view(), yv = y.c_view();
+        check(fh_hybrid_project_id(handle_->raw, w.matrix().raw(), &xv, &iv, (uint32_t)routes, (uint32_t)x_div, &yv));
+        return y;
+    }
+    struct HybridMap {
+        Tensor offsets, sorted, position;
+    };
+    // h_moe_map: expert-major order of the routes, stable inside an expert
+    HybridMap hybrid_moe_map(const Tensor& ids, size_t experts) const {
+        const size_t routes = ids.numel();
+        HybridMap m{zeros({experts + 1}, DType::F32), zeros({routes}, DType::F32), zeros({routes}, DType::F32)};
+        fh_view iv = ids.c_view(), ov = m.offsets.c_view(), sv = m.sorted.c_view(), pv = m.position.c_view();
+        check(fh_hybrid_moe_map(handle_->raw, &iv, (uint32_t)experts, (uint32_t)routes, &ov, &sv, &pv));
+        return m;
+    }
+    // h_moe_gather: out[p] = x[sorted[p] / used]
+    Tensor hybrid_moe_gather(const Tensor& x, const Tensor& sorted, size_t used) const {
+        const auto& dims = x.shape();
+        if (dims.size() != 2 || used == 0 || sorted.numel() != dims[0] * used)
+            throw Error(ErrorKind::Shape, "route gather needs [tokens, hidden] and tokens * used routes");
+        Tensor out = zeros({sorted.numel(), dims[1]}, x.dtype());
+        fh_view xv = x.c_view(), sv = sorted.c_view(), ov = out.c_view();
+        check(fh_hybrid_moe_gather(handle_->raw, &xv, &sv, (uint32_t)dims[1], (uint32_t)used, (uint32_t)sorted.numel(), &ov));
+        return out;
+    }
+    // HybridModel::project_mm_id: rows offsets[e] .. offsets[e + 1] of the expert-sorted x times expert e
+    Tensor hybrid_project_mm_id(const QuantizedExpertMatrix& w, const Tensor& x, const Tensor& offsets) const {
+        const auto& dims = x.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != w.columns() || offsets.numel() != w.experts() + 1)
+            throw Error(ErrorKind::Shape, "expert projection geometry");
+        Tensor y = zeros({dims[0], w.rows_per_expert()}, x.dtype());
+        fh_view xv = x.c_view(), fv = offsets.c_view(), yv = y.c_view();
+        check(fh_hybrid_project_mm_id(handle_->raw, w.matrix().raw(), &xv, &fv, (uint32_t)dims[0], &yv));
+        return y;
+    }
+    // h_moe_combine (f32): weighted sum of each token's routed rows through `position` (or the routes
+    // themselves when null) plus shared_gate[t] * shared[t]
+    Tensor hybrid_moe_combine(const Tensor& down, const Tensor& weights, const Tensor* position, const Tensor& shared,
+                              const Tensor& shared_gate, size_t used) const {
+        const auto& dims = shared.shape();
+        if (dims.size() != 2 || used == 0) throw Error(ErrorKind::Shape, "expert combine geometry mismatch");
+        Tensor out = zeros({dims[0], dims[1]}, DType::F32);
+        fh_view dv = down.c_view(), wv = weights.c_view(), sv = shared.c_view(), gv = shared_gate.c_view(), ov = out.c_view(), pv{};
+        if (position) pv = position->c_view();
+        check(fh_hybrid_moe_combine(handle_->raw, &dv, &wv, position ? &pv : nullptr, &sv, &gv, (uint32_t)dims[1],
+                                    (uint32_t)used, (uint32_t)dims[0], &ov));
+        return out;
+    }
     Tensor expert_assign(const Tensor& hidden, const Tensor& metadata, size_t top_k, const Tensor* out = nullptr) const {
         const auto& x = hidden.shape();
         const auto& m = metadata.shape();

@@ -73,6 +73,11 @@ def _load() -> ctypes.CDLL:
     lib.fo_shared_gate.argtypes = [f32p, f32p, sz, sz, f32p]
     lib.fo_expert_combine_shared.restype = None
     lib.fo_expert_combine_shared.argtypes = [f32p, f32p, sz, sz, sz, u32, f32p, f32p, f32p]
+    u32p = c.POINTER(c.c_uint32)
+    lib.fo_moe_map.restype = None
+    lib.fo_moe_map.argtypes = [u32p, sz, sz, u32p, u32p, u32p]
+    lib.fo_hybrid_combine.restype = None
+    lib.fo_hybrid_combine.argtypes = [f32p, f32p, u32p, f32p, f32p, sz, sz, sz, f32p]
     lib.fo_add_rmsnorm.restype = None
     lib.fo_add_rmsnorm.argtypes = [f32p, f32p, f32p, sz, sz, ctypes.c_float, ctypes.c_uint32, f32p, f32p]
     lib.fo_argmax_rows.restype = None
@@ -246,6 +251,35 @@ def expert_combine_shared(values, metadata, tokens: int, hidden: int, top_k: int
     out = np.empty((tokens, hidden), dtype=np.float32)
     _lib.fo_expert_combine_shared(_f32(v), _f32(meta), tokens, hidden, top_k, dtype, _f32(sh),
                                   _f32(g) if g is not None else None, _f32(out))
+    return out
+
+
+def _u32(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+
+
+def moe_map(ids, experts: int):
+    """(offsets, sorted, position) of h_moe_map (src/metal/shaders/hybrid.metal:2321-2358);
+    entries of routes whose id is not an expert are 0xffffffff."""
+    i = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+    offsets = np.zeros(experts + 1, dtype=np.uint32)
+    order = np.full(i.size, 0xFFFFFFFF, dtype=np.uint32)
+    position = np.full(i.size, 0xFFFFFFFF, dtype=np.uint32)
+    _lib.fo_moe_map(_u32(i), experts, i.size, _u32(offsets), _u32(order), _u32(position))
+    return offsets, order, position
+
+
+def hybrid_combine(down, weights, position, shared, shared_gate, used: int) -> np.ndarray:
+    """h_moe_combine (src/metal/shaders/hybrid.metal:2372-2388) in f32, rank order."""
+    sh = np.ascontiguousarray(shared, dtype=np.float32)
+    tokens, hidden = sh.shape
+    d = np.ascontiguousarray(down, dtype=np.float32).reshape(tokens * used, hidden)
+    w = np.ascontiguousarray(weights, dtype=np.float32).reshape(-1)
+    g = np.ascontiguousarray(shared_gate, dtype=np.float32).reshape(-1)
+    p = None if position is None else np.ascontiguousarray(position, dtype=np.uint32).reshape(-1)
+    out = np.empty((tokens, hidden), dtype=np.float32)
+    _lib.fo_hybrid_combine(_f32(d), _f32(w), _u32(p) if p is not None else None, _f32(sh), _f32(g), hidden, used,
+                           tokens, _f32(out))
     return out
 
 

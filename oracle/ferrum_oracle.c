@@ -55,6 +55,11 @@
  *   fo_argmax_rows         pinned for finite rows: numpy argmax (first
  *       maximal index) and ties; rows holding NaN follow the reference
  *       kernel's scan and merge order as read (flagged rows: parity unpinned).
+ *   fo_moe_map             pinned: numpy's stable argsort and bincount (integer
+ *       work, exact).
+ *   fo_hybrid_combine      pinned: numpy float64 evaluation (f32 sums in rank
+ *       order; the reference kernel's own fma contraction is its compiler's
+ *       choice, so the last ulp is held to the reference test's 1e-4).
  *   fo_add_rmsnorm         pinned: the residual is the storage-rounded f32 sum
  *       (exact); the normalised rows follow the reference's own CPU rmsnorm
  *       (src/reference.rs:23-35, float64) and are checked against closed
@@ -835,5 +840,49 @@ void fo_add_rmsnorm(const float* a, const float* b, const float* weight, size_t 
         double inv = 1.0 / sqrt(squares / (double)width + (double)eps);
         for (size_t j = 0; j < width; j++)
             normed[r * width + j] = (float)((double)residual[r * width + j] * inv * (double)weight[j]);
+    }
+}
+
+/* h_moe_map (src/metal/shaders/hybrid.metal:2321-2358): expert-major order of
+ * routes, stable inside an expert.  offsets[experts + 1], sorted[routes],
+ * position[routes]; routes whose id is not an expert are left untouched. */
+void fo_moe_map(const uint32_t* ids, size_t experts, size_t routes, uint32_t* offsets, uint32_t* sorted,
+                uint32_t* position) {
+    uint32_t acc = 0;
+    for (size_t e = 0; e < experts; e++) {
+        offsets[e] = acc;
+        for (size_t r = 0; r < routes; r++) acc += ids[r] == e ? 1u : 0u;
+    }
+    offsets[experts] = acc;
+    for (size_t e = 0; e < experts; e++) {
+        uint32_t at = offsets[e];
+        for (size_t r = 0; r < routes; r++) {
+            if (ids[r] == e) {
+                sorted[at] = (uint32_t)r;
+                position[r] = at;
+                at++;
+            }
+        }
+    }
+}
+
+/* h_moe_combine (src/metal/shaders/hybrid.metal:2372-2388), f32, each product
+ * and sum rounded to f32 in rank order: out[t] = sum_s weights[t*used + s] *
+ * down[row] + shared_gate[t] * shared[t], row = position[r] or r itself when
+ * position is NULL. */
+void fo_hybrid_combine(const float* down, const float* weights, const uint32_t* position, const float* shared,
+                       const float* shared_gate, size_t hidden, size_t used, size_t tokens, float* out) {
+    for (size_t t = 0; t < tokens; t++) {
+        for (size_t i = 0; i < hidden; i++) {
+            float acc = 0.0f;
+            for (size_t s = 0; s < used; s++) {
+                size_t r = t * used + s;
+                size_t row = position ? position[r] : r;
+                float product = weights[r] * down[row * hidden + i];
+                acc = acc + product;
+            }
+            float tail = shared_gate[t] * shared[t * hidden + i];
+            out[t * hidden + i] = acc + tail;
+        }
     }
 }

@@ -27,6 +27,8 @@ void fo_expert_silu_mul(const float* in, size_t assignments, size_t intermediate
 void fo_expert_combine(const float* in, const float* metadata, size_t tokens, size_t hidden, size_t top_k,
                        uint32_t dtype, float* out);
 void fo_round_storage_array(const float* in, size_t n, uint32_t dtype, float* out);
+void fo_moe_map(const uint32_t* ids, size_t experts, size_t routes, uint32_t* offsets, uint32_t* sorted,
+                uint32_t* position);
 void fo_add_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t width, float eps,
                     uint32_t dtype, float* residual, float* normed);
 }
@@ -313,6 +315,40 @@ int main() {
             threw = err.kind() == ErrorKind::Parameter;
         }
         report("a zero epsilon is refused: Error::Parameter", threw);
+    }
+    {
+        // the hybrid engine's layout: route map (h_moe_map) and per-route expert GEMV (project_id)
+        const size_t experts = 6, routes = 300, rows = 24, k = 512;
+        std::vector<uint32_t> ids(routes);
+        for (size_t r = 0; r < routes; ++r) ids[r] = (uint32_t)((r * 7 + r / 5) % experts);
+        std::vector<uint32_t> want_offsets(experts + 1), want_sorted(routes), want_position(routes);
+        fo_moe_map(ids.data(), experts, routes, want_offsets.data(), want_sorted.data(), want_position.data());
+        Tensor id_tensor = d.from_bits({routes}, ids);
+        auto map = d.hybrid_moe_map(id_tensor, experts);
+        auto words = [](const Tensor& t) {
+            const std::vector<float> f = t.to_f32();
+            std::vector<uint32_t> u(f.size());
+            std::memcpy(u.data(), f.data(), f.size() * 4);
+            return u;
+        };
+        report("hybrid route map equals the h_moe_map restatement",
+               words(map.offsets) == want_offsets && words(map.sorted) == want_sorted &&
+                   words(map.position) == want_position);
+        const auto packed = blocks(QuantizationFormat::Q4_K, experts * rows, k, 77);
+        QuantizedExpertMatrix w = d.quantized_expert_matrix(
+            experts, rows, k, QuantizationFormat::Q4_K,
+            [&packed](uint8_t* dst, size_t bytes) { std::memcpy(dst, packed.data(), bytes); });
+        std::vector<float> x(routes / 3 * k);
+        for (size_t i = 0; i < x.size(); ++i) x[i] = (float)((double)((i * 41 + 11) % 127) / 113.0 - 0.55);
+        Tensor y = d.hybrid_project_id(w, d.from_f32({routes / 3, k}, DType::F32, x), id_tensor, routes, 3);
+        std::vector<float> xr(routes * k), meta(routes * 3, 0.f), want(routes * rows);
+        for (size_t r = 0; r < routes; ++r) {
+            std::memcpy(&xr[r * k], &x[(r / 3) * k], k * 4);
+            std::memcpy(&meta[r * 3], &ids[r], 4);
+        }
+        fo_expert_project(FH_GGML_Q4_K, packed.data(), experts, rows, k, xr.data(), meta.data(), routes, want.data(), 0, 0, 1);
+        const double err = rel_l2(y.to_f32(), want);
+        report("hybrid project_id: each route times its expert", err <= 1e-5, err);
     }
     std::printf("%d failure(s)\n", failures);
     return failures ? 1 : 0;

@@ -767,3 +767,40 @@ def test_q8_0_decoder_equals_numpy_on_the_reference_generator():
     assert oracle.validate_payload(Q8_0, packed[:-1]) == 1
     bad = packed.copy(); bad[34 * 5: 34 * 5 + 2] = np.frombuffer(np.float16(np.nan).tobytes(), dtype=np.uint8)
     assert oracle.validate_payload(Q8_0, bad) == 2
+
+
+# ----------------------------------------------- the hybrid engine's route map and combine
+
+def test_moe_map_is_numpy_stable_argsort():
+    rng = np.random.default_rng(31)
+    for experts, routes in ((4, 1), (8, 40), (256, 4096), (60, 1000)):
+        ids = rng.integers(0, experts, routes).astype(np.uint32)
+        if routes > 10:
+            ids[ids == 3] = 5                      # an empty expert
+        offsets, order, position = oracle.moe_map(ids, experts)
+        counts = np.bincount(ids, minlength=experts)
+        assert np.array_equal(offsets, np.concatenate([[0], np.cumsum(counts)]).astype(np.uint32))
+        want = np.argsort(ids, kind="stable").astype(np.uint32)
+        assert np.array_equal(order, want)
+        assert np.array_equal(position[want], np.arange(routes, dtype=np.uint32))
+    ids = np.array([1, 9, 0, 1], dtype=np.uint32)     # 9 is not an expert: left out
+    offsets, order, position = oracle.moe_map(ids, 2)
+    assert offsets.tolist() == [0, 1, 3] and order[:3].tolist() == [2, 0, 3] and position.tolist() == [1, 0xFFFFFFFF, 0, 2]
+
+
+def test_hybrid_combine_is_the_weighted_sum_plus_gated_shared_rows():
+    rng = np.random.default_rng(32)
+    tokens, used, hidden = 5, 4, 24
+    down = rng.standard_normal((tokens * used, hidden)).astype(np.float32)
+    weights = rng.random(tokens * used).astype(np.float32)
+    shared = rng.standard_normal((tokens, hidden)).astype(np.float32)
+    gate = rng.random(tokens).astype(np.float32)
+    position = rng.permutation(tokens * used).astype(np.uint32)
+    for pos in (None, position):
+        rows = down if pos is None else down[pos]
+        want = (weights[:, None].astype(np.float64) * rows).reshape(tokens, used, hidden).sum(1) + gate[:, None] * shared.astype(np.float64)
+        got = oracle.hybrid_combine(down, weights, pos, shared, gate, used)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    # one route of weight 1, no shared contribution: the row itself
+    one = oracle.hybrid_combine(down[:tokens], np.ones(tokens, np.float32), None, shared, np.zeros(tokens, np.float32), 1)
+    assert np.array_equal(one, down[:tokens])

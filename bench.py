@@ -37,7 +37,7 @@ ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer rep
 # HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
 # FETCH_SIZE 24723.1 KiB x 1.94485 + WRITE_SIZE 68.0 KiB x 1.0, the factors being
 # known bytes / counter reading for the row-copy kernel of `--cases copy`.
-MEASURED_TRAFFIC_BYTES = 49306489
+MEASURED_TRAFFIC_BYTES = 49319405
 
 
 def algorithmic_bytes(ggml, n, k, m, x_size, y_size):

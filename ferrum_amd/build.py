@@ -82,12 +82,14 @@ def build_host_test() -> str:
     return out
 
 
-def build_gguf_probe() -> str:
+def build_gguf_probe(sanitize: bool = False) -> str:
     """Compiles tests/cpp/gguf_probe.cpp (the C++ GGUF reader's CPU test
-    program; host code only, nothing to link)."""
+    program; host code only, nothing to link).  `sanitize` builds a second
+    binary under AddressSanitizer and UBSan, any report of which is fatal."""
     root = os.path.dirname(HERE)
-    out = os.path.join(root, "tests", "cpp", "gguf_probe")
-    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Werror", "-I" + os.path.join(root, "include"),
+    out = os.path.join(root, "tests", "cpp", "gguf_probe_san" if sanitize else "gguf_probe")
+    flags = ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all"] if sanitize else ["-O2"]
+    cmd = ["g++", "-std=c++17", *flags, "-Wall", "-Werror", "-I" + os.path.join(root, "include"),
            os.path.join(root, "tests", "cpp", "gguf_probe.cpp"), "-o", out]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:

@@ -253,6 +253,49 @@ def test_cpp_reader_agrees_with_the_python_reader(probe, tmp_path):
         assert proc.stdout.splitlines() == _describe(read(data, **kw)), label
 
 
+def test_both_readers_survive_truncated_and_corrupted_files(tmp_path):
+    # an untrusted file may be cut anywhere or carry any byte: the C++ reader, built under
+    # AddressSanitizer and UBSan, must either read it or refuse it (exit 0 or 2, never a report
+    # or a crash), and the Python reader must do the same with GgufError
+    import subprocess
+    from ferrum_amd import build
+    probe = build.build_gguf_probe(sanitize=True)
+    metadata = gf.STANDARD + [("tokenizer.ggml.tokens", gf.ARRAY, ["a", "bc"], gf.STRING),
+                              ("general.alignment", gf.U32, 32), ("x.f64", gf.F64, 2.5)]
+    tensors = [("blk.0.ffn_up.weight", [256, 3], 12, synth.matrix(12, 3, 256, seed=21)),
+               ("blk.0.ffn_up_exps.weight", [256, 2, 2], 23, synth.matrix(23, 4, 256, seed=22)),
+               ("norm.weight", [4], 0, np.arange(4, dtype=np.float32).view(np.uint8))]
+    good = gf.build(tensors, metadata)
+    header = len(good) - 32 * -(-(3 * 144 + 4 * 136 + 16 + 64) // 32)      # at most: where the tensor data starts
+    header = max(header, 200)
+    rng = np.random.default_rng(7)
+    variants = [good[:n] for n in range(0, min(len(good), header + 40), 5)]
+    for _ in range(250):
+        data = bytearray(good)
+        at = int(rng.integers(0, header))
+        data[at] = int(rng.integers(0, 256))
+        variants.append(bytes(data))
+    for _ in range(60):                                       # a huge count or length field
+        data = bytearray(good)
+        at = int(rng.integers(8, header - 8))
+        data[at:at + 8] = int(rng.integers(1 << 40, 1 << 63)).to_bytes(8, "little")
+        variants.append(bytes(data))
+    path = tmp_path / "case.gguf"
+    outcomes = {0: 0, 2: 0}
+    for i, data in enumerate(variants):
+        path.write_bytes(data)
+        proc = subprocess.run([probe, str(path)], capture_output=True, text=True, timeout=30)
+        assert proc.returncode in (0, 2), (i, len(data), proc.returncode, proc.stderr[-600:])
+        outcomes[proc.returncode] += 1
+        try:
+            read(data)
+            ok = True
+        except api.GgufError:
+            ok = False
+        assert ok == (proc.returncode == 0), (i, len(data), proc.returncode)
+    assert outcomes[0] > 0 and outcomes[2] > 100
+
+
 def test_gate_and_up_expert_tensors_interleave_per_expert(probe, tmp_path):
     # load_quantized_input_experts (src/model/lfm2_moe/gguf.rs:466-534): [E, I, H] + [E, I, H] -> [E, 2I, H]
     import subprocess

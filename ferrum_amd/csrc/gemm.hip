@@ -240,14 +240,16 @@ __device__ __forceinline__ float16v mfma(uint4 a, uint4 b, float16v c) {
 }
 
 // TS = 128: four waves, 64 x 64 each; TS = 64: two waves, 32 x 64 each (four times the
-// workgroups, for matrices too small to fill the chip with 128 x 128 tiles).
+// workgroups, for matrices too small to fill the chip with 128 x 128 tiles); TS = 32: one
+// wave and one 32 x 32 tile, when even 64 x 64 tiles number fewer than the compute units.
 template <uint32_t TYPE, int DT, int TS>
 __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __restrict__ w,
                                                              const uint16_t* __restrict__ x,
                                                              void* __restrict__ y, uint32_t m,
                                                              uint32_t n, uint32_t nb,
                                                              uint32_t y_dtype) {
-    constexpr int WI = TS / 64;  // 32-row tiles per wave
+    constexpr int WI = TS == 128 ? 2 : 1;  // 32-row tiles per wave
+    constexpr int WJ = TS == 32 ? 1 : 2;   // 32-column tiles per wave
     __shared__ __attribute__((aligned(16))) uint16_t xs[TS * kLd];
     __shared__ __attribute__((aligned(16))) uint16_t ws[TS * kLd];
     constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
@@ -263,12 +265,12 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
     const bool xlive = m0 + lrow < m;
     const uint16_t* xsrc = x + (size_t)(xlive ? m0 + lrow : 0) * k + 32 * lh;
 
-    const uint32_t wm = TS == 128 ? (wave >> 1) * 64 : wave * 32, wn = TS == 128 ? (wave & 1u) * 64 : 0;
-    float16v acc[WI][2];
+    const uint32_t wm = TS == 128 ? (wave >> 1) * 64 : TS == 64 ? wave * 32 : 0, wn = TS == 128 ? (wave & 1u) * 64 : 0;
+    float16v acc[WI][WJ];
 #pragma unroll
     for (int i = 0; i < WI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < WJ; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
@@ -312,17 +314,17 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 uint32_t koff = kk * 16 + 8 * (lane >> 5);
-                uint4 a[WI], b[2];
+                uint4 a[WI], b[WJ];
 #pragma unroll
                 for (int i = 0; i < WI; ++i)
                     a[i] = *reinterpret_cast<const uint4*>(&xs[(wm + 32 * i + (lane & 31u)) * kLd + koff]);
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < WJ; ++j)
                     b[j] = *reinterpret_cast<const uint4*>(&ws[(wn + 32 * j + (lane & 31u)) * kLd + koff]);
 #pragma unroll
                 for (int i = 0; i < WI; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) acc[i][j] = mfma<DT>(a[i], b[j], acc[i][j]);
+                    for (int j = 0; j < WJ; ++j) acc[i][j] = mfma<DT>(a[i], b[j], acc[i][j]);
             }
         }
     }
@@ -330,7 +332,7 @@ __global__ __launch_bounds__(2 * TS) void gemm_tile_kernel(const uint8_t* __rest
 #pragma unroll
     for (int i = 0; i < WI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < WJ; ++j) {
             uint32_t col = n0 + wn + 32 * j + (lane & 31u);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -886,13 +888,17 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     // 128 x 128 tiles, or 64 x 64 when those would leave most of the chip idle
     const uint64_t big_wgs = (uint64_t)((a.n + kBN - 1) / kBN) * ((a.m + kBM - 1) / kBM);
     const bool small = big_wgs * 2 < (uint64_t)a.cu_count;
-    const uint32_t ts = small ? 64 : 128;
+    const uint64_t mid_wgs = (uint64_t)((a.n + 63) / 64) * ((a.m + 63) / 64);
+    const bool tiny = small && mid_wgs < (uint64_t)a.cu_count;
+    const uint32_t ts = tiny ? 32 : small ? 64 : 128;
     dim3 grid((a.n + ts - 1) / ts, (a.m + ts - 1) / ts);
     const uint32_t nb = a.k / 256;
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
-    auto run = [&](auto big, auto little) {
-        if (small) {
+    auto run = [&](auto big, auto little, auto least) {
+        if (tiny) {
+            hipLaunchKernelGGL(least, grid, dim3(64), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype);
+        } else if (small) {
             hipLaunchKernelGGL(little, grid, dim3(128), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype);
         } else {
             hipLaunchKernelGGL(big, grid, dim3(256), 0, s, w, x, a.y, a.m, a.n, nb, a.y_dtype);
@@ -900,40 +906,40 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     };
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) {
-            run(gemm_tile_kernel<kQ4K, 1, 128>, gemm_tile_kernel<kQ4K, 1, 64>);
+            run(gemm_tile_kernel<kQ4K, 1, 128>, gemm_tile_kernel<kQ4K, 1, 64>, gemm_tile_kernel<kQ4K, 1, 32>);
         } else {
-            run(gemm_tile_kernel<kQ4K, 2, 128>, gemm_tile_kernel<kQ4K, 2, 64>);
+            run(gemm_tile_kernel<kQ4K, 2, 128>, gemm_tile_kernel<kQ4K, 2, 64>, gemm_tile_kernel<kQ4K, 2, 32>);
         }
         return "q4_k_gemm_mfma";
     }
     if (a.ggml_type == kQ5K) {
         if (a.x_dtype == FH_F16) {
-            run(gemm_tile_kernel<kQ5K, 1, 128>, gemm_tile_kernel<kQ5K, 1, 64>);
+            run(gemm_tile_kernel<kQ5K, 1, 128>, gemm_tile_kernel<kQ5K, 1, 64>, gemm_tile_kernel<kQ5K, 1, 32>);
         } else {
-            run(gemm_tile_kernel<kQ5K, 2, 128>, gemm_tile_kernel<kQ5K, 2, 64>);
+            run(gemm_tile_kernel<kQ5K, 2, 128>, gemm_tile_kernel<kQ5K, 2, 64>, gemm_tile_kernel<kQ5K, 2, 32>);
         }
         return "q5_k_gemm_mfma";
     }
     if (a.ggml_type == kIQ4XS) {
         if (a.x_dtype == FH_F16) {
-            run(gemm_tile_kernel<kIQ4XS, 1, 128>, gemm_tile_kernel<kIQ4XS, 1, 64>);
+            run(gemm_tile_kernel<kIQ4XS, 1, 128>, gemm_tile_kernel<kIQ4XS, 1, 64>, gemm_tile_kernel<kIQ4XS, 1, 32>);
         } else {
-            run(gemm_tile_kernel<kIQ4XS, 2, 128>, gemm_tile_kernel<kIQ4XS, 2, 64>);
+            run(gemm_tile_kernel<kIQ4XS, 2, 128>, gemm_tile_kernel<kIQ4XS, 2, 64>, gemm_tile_kernel<kIQ4XS, 2, 32>);
         }
         return "iq4_xs_gemm_mfma";
     }
     if (a.ggml_type == kQ8_0) {
         if (a.x_dtype == FH_F16) {
-            run(gemm_tile_kernel<kQ8_0, 1, 128>, gemm_tile_kernel<kQ8_0, 1, 64>);
+            run(gemm_tile_kernel<kQ8_0, 1, 128>, gemm_tile_kernel<kQ8_0, 1, 64>, gemm_tile_kernel<kQ8_0, 1, 32>);
         } else {
-            run(gemm_tile_kernel<kQ8_0, 2, 128>, gemm_tile_kernel<kQ8_0, 2, 64>);
+            run(gemm_tile_kernel<kQ8_0, 2, 128>, gemm_tile_kernel<kQ8_0, 2, 64>, gemm_tile_kernel<kQ8_0, 2, 32>);
         }
         return "q8_0_gemm_mfma";
     }
     if (a.x_dtype == FH_F16) {
-        run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>);
+        run(gemm_tile_kernel<kQ6K, 1, 128>, gemm_tile_kernel<kQ6K, 1, 64>, gemm_tile_kernel<kQ6K, 1, 32>);
     } else {
-        run(gemm_tile_kernel<kQ6K, 2, 128>, gemm_tile_kernel<kQ6K, 2, 64>);
+        run(gemm_tile_kernel<kQ6K, 2, 128>, gemm_tile_kernel<kQ6K, 2, 64>, gemm_tile_kernel<kQ6K, 2, 32>);
     }
     return "q6_k_gemm_mfma";
 }

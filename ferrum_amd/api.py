@@ -119,6 +119,7 @@ SYMBOLS = {
     "fh_moe_route_ranked": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP]),
     "fh_expert_combine_shared": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_route": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP, _VP]),
+    "fh_hybrid_project": (_I32, [_P, _P, _VP, _U32, _VP, _U32]),
     "fh_hybrid_project_id": (_I32, [_P, _P, _VP, _VP, _U32, _U32, _VP]),
     "fh_hybrid_moe_map": (_I32, [_P, _VP, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_gather": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
@@ -693,6 +694,19 @@ class Device:
                                         gate_vector.shape()[0] if gate_vector is not None else 0,
                                         ctypes.byref(iv), ctypes.byref(wtv), ctypes.byref(gv)))
         return ids, weights, gate
+
+    def hybrid_project(self, weight: QuantizedMatrix, x: Tensor, exact: bool = False,
+                       out_dtype: DType | None = None) -> Output:
+        """HybridModel::project (src/hybrid/engine.rs:3407-3500): exact f32 weights for 1..4 rows
+        (or always with `exact`), f16 tiles from 5 rows on."""
+        dims = x.shape()
+        if len(dims) != 2 or dims[0] == 0 or dims[1] != weight.columns():
+            raise ShapeError("quantized projection requires [M,K] matching [N,K]")
+        y = Tensor.zeros(self, (dims[0], weight.rows()), out_dtype or x.dtype)
+        xv, yv = x._view(), y._view()
+        _check(_lib.fh_hybrid_project(self._handle, _handle_of(weight), ctypes.byref(xv), dims[0], ctypes.byref(yv),
+                                      1 if exact else 0))
+        return Output(y, self.last_operation(), x.byte_size() + weight.byte_size(), y.byte_size())
 
     def hybrid_project_id(self, weight: "QuantizedExpertMatrix", x: Tensor, ids: Tensor, routes: int, x_div: int,
                           out_dtype: DType | None = None) -> Tensor:

@@ -481,8 +481,10 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
 
 namespace {
 
+// `f32_tile_from`: row count from which f32 activations take the f16 tiles; negative = the
+// device's gemm_f32_min_rows setting
 fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t m,
-                  const fh_view* y, bool silu_mul) {
+                  const fh_view* y, bool silu_mul, int64_t f32_tile_from = -1) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device) {
         g_last_error = "weight belongs to another device";
@@ -505,7 +507,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
     // caller asks for the tile kernels from some row count on, as the reference's hybrid
     // engine does from 5 rows (HybridModel::project, src/hybrid/engine.rs:3407-3500): the
     // activations are then rounded to f16 into the device scratch first.
-    const int64_t f32_tile_rows = tuning(device, "gemm_f32_min_rows");
+    const int64_t f32_tile_rows = f32_tile_from >= 0 ? f32_tile_from : tuning(device, "gemm_f32_min_rows");
     const bool f32_tile = !silu_mul && x->dtype == FH_F32 && f32_tile_rows > 0 && m >= (uint64_t)f32_tile_rows &&
                           ((uintptr_t)xr.begin & 15u) == 0;
     const void* tile_x = xr.begin;
@@ -723,6 +725,25 @@ fh_status fh_hybrid_moe_route(fh_device* device, const fh_view* logits, uint32_t
     if (ids == nullptr) return fail(FH_ERR_RANGE, "route ids: null view");
     return route(device, logits, tokens, nullptr, policy, nullptr, true, x, gate_vector, hidden, shared_gate, ids,
                  weights);
+}
+
+fh_status fh_hybrid_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t m,
+                            const fh_view* y, uint32_t exact) {
+    // HybridModel::project (src/hybrid/engine.rs:3407-3500): one row and `exact` keep f32
+    // weights; 2..4 rows are a batched GEMV, also exact; from 5 rows (MVB_MAX_ROWS + 1,
+    // :3584) the rows go through f16 tiles
+    const fh_status st = project(device, weight, x, m, y, false, exact ? 0 : 5);
+    if (st != FH_OK) return st;
+    static const char* const names[4][5] = {
+        {"h_mv_q4_k", "h_mv_q5_k", "h_mv_q6_k", "h_mv_q8_0", "h_mv_iq4_xs"},
+        {"h_mvb_q4_k", "h_mvb_q5_k", "h_mvb_q6_k", "h_mvb_q8_0", "h_mvb_iq4_xs"},
+        {"h_mms_q4_k", "h_mms_q5_k", "h_mms_q6_k", "h_mms_q8_0", "h_mms_iq4_xs"},
+        {"h_mm_q4_k", "h_mm_q5_k", "h_mm_q6_k", "h_mm_q8_0", "h_mm_iq4_xs"}};
+    const int tier = m == 1 || exact ? 0 : m <= 4 ? 1 : m <= 32 ? 2 : 3;
+    const int f = weight->ggml_type == kQ4K ? 0 : weight->ggml_type == kQ5K ? 1 : weight->ggml_type == kQ6K ? 2
+                  : weight->ggml_type == kQ8_0 ? 3 : 4;
+    device->last_operation = names[tier][f];
+    return FH_OK;
 }
 
 fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,

@@ -266,6 +266,15 @@ fh_status fh_hybrid_moe_route(fh_device* device, const fh_view* logits, uint32_t
                               const fh_routing_policy* policy, const fh_view* x, const fh_view* gate_vector,
                               uint32_t hidden, const fh_view* ids, const fh_view* weights,
                               const fh_view* shared_gate);
+/* HybridModel::project (src/hybrid/engine.rs:3407-3500) with its tiers
+ * (MVB_MAX_ROWS = 4, MMS_MAX_ROWS = 32, :3584-3585): one row, or any row count
+ * when `exact` is set (the engine's exact_math flag), multiplies exact f32
+ * weights; 2..4 rows do the same row by row (the batched GEMV h_mvb_*); from 5
+ * rows on f32 activations are rounded to f16 and take the tile kernels
+ * (h_mms_* up to 32 rows, h_mm_* beyond), whatever gemm_f32_min_rows says.
+ * fh_last_operation names the tier, e.g. "h_mms_q4_k". */
+fh_status fh_hybrid_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t m,
+                            const fh_view* y, uint32_t exact);
 fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
                                uint32_t routes, uint32_t x_div, const fh_view* y);
 fh_status fh_hybrid_moe_map(fh_device* device, const fh_view* ids, uint32_t experts, uint32_t routes,

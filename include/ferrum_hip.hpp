@@ -450,6 +450,16 @@ public:
                                   &wtv, &gv));
         return r;
     }
+    // HybridModel::project: exact f32 weights for 1..4 rows (or always with `exact`), f16 tiles from 5 rows on
+    Output hybrid_project(const QuantizedMatrix& w, const Tensor& a, bool exact = false) const {
+        const auto& dims = a.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != w.columns())
+            throw Error(ErrorKind::Shape, "quantized projection requires [M,K] matching [N,K]");
+        Tensor y = zeros({dims[0], w.rows()}, a.dtype());
+        fh_view xv = a.c_view(), yv = y.c_view();
+        check(fh_hybrid_project(handle_->raw, w.raw(), &xv, (uint32_t)dims[0], &yv, exact ? 1u : 0u));
+        return {y, {last_operation(), a.byte_size() + w.byte_size(), y.byte_size()}};
+    }
     // HybridModel::project_id: route r multiplies activation row r / x_div by expert ids[r]
     Tensor hybrid_project_id(const QuantizedExpertMatrix& w, const Tensor& x, const Tensor& ids, size_t routes,
                              size_t x_div) const {

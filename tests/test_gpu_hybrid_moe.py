@@ -181,6 +181,32 @@ def test_prompt_chain_map_gather_mm_id_combine_matches_the_decode_chain_and_the_
     assert np.abs(out1).max() > 1e-4
 
 
+@pytest.mark.parametrize("ggml", [Q4_K, IQ4_XS])
+def test_project_tiers_follow_the_engine(api, d, ggml):
+    # HybridModel::project (src/hybrid/engine.rs:3407-3500) and the cases of its format tests
+    # (M = 1, 3, 16, 64: GEMV, batched GEMV, narrow tiles, tensor-op tiles; iq_tests.rs:1300-1337)
+    n, k = 300, 1024
+    packed = synth.matrix(ggml, n, k, seed=431)
+    w = api.QuantizedMatrix.from_bytes(d, n, k, api.QuantizationFormat(ggml), packed)
+    name = {Q4_K: "q4_k", IQ4_XS: "iq4_xs"}[ggml]
+    for m, tier in ((1, "h_mv_"), (3, "h_mvb_"), (4, "h_mvb_"), (5, "h_mms_"), (16, "h_mms_"), (64, "h_mm_"), (200, "h_mm_")):
+        x = synth.activations(m, k, seed=432 + m)
+        out = d.hybrid_project(w, api.Tensor.from_f32(d, x.shape, api.DType.F32, x))
+        assert out.operation == tier + name and out.tensor.dtype == api.DType.F32
+        if m < 5:
+            want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
+        else:
+            want = oracle.project(ggml, packed, n, k, oracle.round_storage(x, oracle.F16).reshape(m, k),
+                                  weight_round=oracle.F16, accumulate="f64")
+        assert_matmul_parity(out.tensor.to_f32(), want, f"{tier}{name} m={m}")
+        plain = oracle.project(ggml, packed, n, k, x, accumulate="f64")
+        assert np.abs(out.tensor.to_f32() - plain).max() <= 5e-3 * np.abs(plain).max()      # the reference's bound
+    x = synth.activations(16, k, seed=433)
+    exact = d.hybrid_project(w, api.Tensor.from_f32(d, x.shape, api.DType.F32, x), exact=True)
+    assert exact.operation == "h_mv_" + name
+    assert_matmul_parity(exact.tensor.to_f32(), oracle.project(ggml, packed, n, k, x, accumulate="f64"), "exact")
+
+
 def test_hybrid_entry_points_reject_bad_geometry(api, d):
     f32 = api.DType.F32
     ids = carrier(api, d, np.zeros(8, np.uint32))

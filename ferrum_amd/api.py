@@ -892,6 +892,8 @@ class SparseMoe:
         # most assignments that take the fused per-assignment kernels; above it the
         # separate steps run (and group by expert from 32 assignments on)
         self.fused_max_assignments = 31
+        # False: expert_assign and expert_silu_mul always run as launches of their own
+        self.fuse_inputs = True
 
     def workspace(self, tokens: int, dtype: DType):
         a, h, i = tokens * self.routing.top_k, self.hidden_size, self.intermediate_size
@@ -914,8 +916,9 @@ class SparseMoe:
         d, k = self.device, self.routing.top_k
         ws = self._ws if self._ws and self._ws["tokens"] == dims[0] and self._ws["dtype"] == hidden.dtype else {}
         metadata = d.moe_route(router_logits, self.selection_bias, self.routing, out=ws.get("metadata"))
-        if dims[0] * k <= self.fused_max_assignments:
-            # decode: the copy and the activation ride inside the projections
+        if self.fuse_inputs and (dims[0] * k <= self.fused_max_assignments or hidden.dtype != DType.F32):
+            # the copy and the activation ride inside the projections: per assignment in
+            # decode, and in the grouped kernel's gather of an expert's rows beyond it
             projected = d.expert_project_quantized(hidden, metadata, self.input_experts, self.hidden_size,
                                                    self.expert_count, out=ws.get("projected"), form="gather")
             expert_output = d.expert_project_quantized(projected, metadata, self.output_experts,

@@ -930,7 +930,7 @@ fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t to
     if (overlaps(hr, orr) || overlaps(mr, orr)) return fail(FH_ERR_RANGE, "assign output aliases an input");
     device->last_operation = launch_expert_assign(
         device->stream, hr.begin, reinterpret_cast<const float*>(mr.begin),
-        const_cast<uint8_t*>(orr.begin), assignments, width * (uint32_t)dtype_bytes(hidden->dtype));
+        const_cast<uint8_t*>(orr.begin), assignments, width * (uint32_t)dtype_bytes(hidden->dtype), tokens);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -966,22 +966,37 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     // tiles (gemm_f32_min_rows, the hybrid engine's prompt path project_mm_id_in,
     // src/hybrid/engine.rs:3164): they are rounded to f16 into the scratch first
     const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
-    const bool f32_grouped = x->dtype == FH_F32 && f32_rows > 0 && assignments >= (uint64_t)f32_rows &&
-                             ((uintptr_t)xr.begin & 15u) == 0;
-    if (form == FH_INPUT_ROWS && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
-        assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
-        // grouped form: every expert's weights are streamed once for all of its assignments
+    const bool f32_grouped = form == FH_INPUT_ROWS && x->dtype == FH_F32 && f32_rows > 0 &&
+                             assignments >= (uint64_t)f32_rows && ((uintptr_t)xr.begin & 15u) == 0;
+    if ((x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
+        weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
+        // grouped form: every expert's weights are streamed once for all of its assignments.
+        // The kernel that keeps an expert's rows in LDS gathers them from the token rows
+        // itself; where they do not fit, and for the SiLU form, the rows are written out
+        // first, as the separate expert_assign / expert_silu_mul launches would.
+        const bool gathers = form == FH_INPUT_GATHER &&
+                             expert_rows_fit_lds((uint32_t)k, assignments, (uint32_t)weight->experts);
+        const bool staged = f32_grouped || (form != FH_INPUT_ROWS && !gathers);
         const size_t words = ((size_t)weight->experts + 1 + assignments + 3) & ~(size_t)3;
-        const size_t x16_bytes = f32_grouped ? (size_t)assignments * k * sizeof(uint16_t) : 0;
-        st = ensure_scratch(device, words * sizeof(uint32_t) + x16_bytes);
+        const size_t staged_bytes = staged ? (size_t)assignments * k * sizeof(uint16_t) : 0;
+        st = ensure_scratch(device, words * sizeof(uint32_t) + staged_bytes);
         if (st != FH_OK) return st;
         uint32_t* offsets = reinterpret_cast<uint32_t*>(scratch_data(device));
         uint32_t* order = offsets + weight->experts + 1;
         const void* tile_x = xr.begin;
-        if (f32_grouped) {
-            uint16_t* x16 = reinterpret_cast<uint16_t*>(scratch_data(device) + words * sizeof(uint32_t));
-            launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin), x16, (size_t)assignments * k);
-            tile_x = x16;
+        if (staged) {
+            uint8_t* rows_x = scratch_data(device) + words * sizeof(uint32_t);
+            if (f32_grouped) {
+                launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin),
+                                    reinterpret_cast<uint16_t*>(rows_x), (size_t)assignments * k);
+            } else if (form == FH_INPUT_GATHER) {
+                launch_expert_assign(device->stream, xr.begin, reinterpret_cast<const float*>(mr.begin), rows_x,
+                                     assignments, (uint32_t)(k * sizeof(uint16_t)), x_rows);
+            } else {
+                launch_expert_silu_mul(device->stream, xr.begin, rows_x, assignments, (uint32_t)k, x->dtype,
+                                       x->dtype);
+            }
+            tile_x = rows_x;
         }
         launch_expert_group(device->stream, reinterpret_cast<const float*>(mr.begin), assignments,
                             (uint32_t)weight->experts, offsets, order, const_cast<uint8_t*>(yr.begin),
@@ -1000,6 +1015,8 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.experts = (uint32_t)weight->experts;
         g.expert_offsets = offsets;
         g.expert_order = order;
+        g.gather_metadata = gathers ? reinterpret_cast<const float*>(mr.begin) : nullptr;
+        g.x_rows = x_rows;
         device->last_operation = launch_gemm_skinny(device->stream, g);
         FH_HIP(hipGetLastError());
         return FH_OK;

@@ -66,6 +66,15 @@ __device__ __forceinline__ float round_storage(float v, uint32_t dtype) {
     return v;
 }
 
+// SiLU in the branch-stable form of expert_silu_mul (src/metal/shaders/ops.metal:2223-2232):
+// 1 / (1 + exp(-g)) for g >= 0 and exp(g) / (1 + exp(g)) below.  Both sides are one
+// exponential of -|g| and one division, so they are written as that: the same values with
+// half the work of evaluating the two sides.
+__device__ __forceinline__ float silu_stable(float gate) {
+    const float e = expf(-fabsf(gate));
+    return gate * ((gate >= 0.f ? 1.f : e) / (1.f + e));
+}
+
 // 16-byte and 2-byte loads from addresses that are only 2-byte aligned (Q6_K
 // blocks are 210 bytes); gfx950 global loads accept unaligned addresses.
 __device__ __forceinline__ uint4 load_u4_unaligned(const uint8_t* p) {

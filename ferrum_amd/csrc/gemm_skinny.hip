@@ -420,6 +420,12 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
 // and walks (tile, super-block) units through a register ring, so the prefetch
 // runs across tile boundaries.  blockIdx.y = expert, blockIdx.x = which share
 // of the expert's rows.  Dynamic LDS: 16*TT rows of (K + 8) halfs.
+//
+// The rows are [A, K] rows or, with metadata given, the row of the assignment's
+// token in [tokens, K]: expert_assign folded into the gather.  (SiLU * up is not
+// folded in: it is bound by its exponentials and divisions, and one workgroup
+// per compute unit doing them ahead of its first MFMA costs more than the
+// launch that spreads them over the whole chip: +11 us against -5 us.)
 constexpr int kResRing = 6;
 constexpr int kResWaves = 8;                    // two waves per SIMD hide each other's decode and MFMA waits
 constexpr int kResThreads = 64 * kResWaves;
@@ -431,7 +437,9 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                                                                      uint32_t nb, uint32_t y_dtype,
                                                                      const uint32_t* __restrict__ offsets,
                                                                      const uint32_t* __restrict__ order,
-                                                                     uint32_t tiles_per_wg) {
+                                                                     uint32_t tiles_per_wg,
+                                                                     const float* __restrict__ metadata,
+                                                                     uint32_t x_rows) {
     constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
     constexpr int kTokens = 16 * TT;
     extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
@@ -461,7 +469,12 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                 const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
                 dst[j] = tok * ld + 8 * pc;
                 const uint32_t slot = first_token + t0 + tok;
-                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)(order != nullptr ? order[slot] : slot) * k + 8 * pc);
+                uint32_t row = order != nullptr ? order[slot] : slot;
+                if (metadata != nullptr) {
+                    const uint32_t token = __float_as_uint(metadata[3 * (size_t)row + 1]);
+                    row = token < x_rows ? token : x_rows - 1;
+                }
+                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)row * k + 8 * pc);
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
@@ -575,7 +588,7 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     if (a.expert_offsets != nullptr) {
         const bool wide = a.m > 8 * a.experts;   // mean tokens per expert > 8: 32 tokens a pass
         const size_t lds = (size_t)(wide ? 32 : 16) * (a.k + 8) * 2;
-        if (lds <= 150u * 1024) {
+        if (expert_rows_fit_lds(a.k, a.m, a.experts)) {
             // the expert's rows are cut into shares so that about one workgroup per compute unit
             // exists: every share gathers the expert's tokens again, and at 256 experts one share
             // each (236 us for the 512-token routed FFN) beats four (264 us)
@@ -591,13 +604,13 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows);
             } else {
                 auto kernel = expert_resident_kernel<TYPE, DT, 1>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows);
             }
             return;
         }
@@ -626,6 +639,11 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
 }
 
 }  // namespace
+
+bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts) {
+    // more than 8 tokens per expert on average: 32 tokens a pass, else 16
+    return (size_t)(m > 8 * experts ? 32 : 16) * (k + 8) * 2 <= 150u * 1024;
+}
 
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
     const bool grouped = a.expert_offsets != nullptr;

@@ -288,19 +288,13 @@ __device__ __forceinline__ float4 load_x4(const void* x, uint32_t dtype, size_t 
                        bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
 }
 
-// SiLU in the branch-stable form of expert_silu_mul (src/metal/shaders/ops.metal:2223-2232)
-__device__ __forceinline__ float gemv_silu(float gate) {
-    float s = gate >= 0.f ? 1.f / (1.f + expf(-gate)) : expf(gate) / (1.f + expf(gate));
-    return gate * s;
-}
-
 // What expert_silu_mul would have stored for four columns, rounded to the
 // activation dtype at the same two points.
 __device__ __forceinline__ float4 silu_mul4(float4 g, float4 u, uint32_t dtype) {
-    return make_float4(round_storage(round_storage(gemv_silu(g.x), dtype) * u.x, dtype),
-                       round_storage(round_storage(gemv_silu(g.y), dtype) * u.y, dtype),
-                       round_storage(round_storage(gemv_silu(g.z), dtype) * u.z, dtype),
-                       round_storage(round_storage(gemv_silu(g.w), dtype) * u.w, dtype));
+    return make_float4(round_storage(round_storage(silu_stable(g.x), dtype) * u.x, dtype),
+                       round_storage(round_storage(silu_stable(g.y), dtype) * u.y, dtype),
+                       round_storage(round_storage(silu_stable(g.z), dtype) * u.z, dtype),
+                       round_storage(round_storage(silu_stable(g.w), dtype) * u.w, dtype));
 }
 
 struct Params {

@@ -154,11 +154,19 @@ struct GemmArgs {
     uint32_t experts;
     const uint32_t* expert_offsets;
     const uint32_t* expert_order;
+    // routed form with the expert's rows resident in LDS (expert_rows_fit_lds): when set,
+    // x is [x_rows, k] token rows and assignment a reads the row of its token,
+    // gather_metadata[3a + 1], as expert_assign would have copied it
+    const float* gather_metadata;
+    uint32_t x_rows;
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 
 // gemm_skinny.hip
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a);
+// whether the routed form keeps an expert's activation rows of width k in LDS,
+// which is the kernel that takes the gathered input form
+bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts);
 
 // moe.hip
 // what the hybrid engine's router adds: selection order kept, shared-expert gate
@@ -187,7 +195,7 @@ const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t a
                                 uint32_t experts, uint32_t* offsets, uint32_t* order, void* y,
                                 uint32_t row_bytes);
 const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,
-                                 void* out, uint32_t assignments, uint32_t row_bytes);
+                                 void* out, uint32_t assignments, uint32_t row_bytes, uint32_t tokens);
 const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,
                                    uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype);
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,

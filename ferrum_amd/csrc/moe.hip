@@ -213,18 +213,14 @@ __global__ __launch_bounds__(256) void expert_assign_kernel(const V* __restrict_
                                                             const float* __restrict__ metadata,
                                                             V* __restrict__ out,
                                                             uint32_t assignments,
-                                                            uint32_t row_pieces) {
+                                                            uint32_t row_pieces, uint32_t tokens) {
     const uint32_t a = blockIdx.x;
     if (a >= assignments) return;
-    const uint32_t token = __float_as_uint(metadata[3 * (size_t)a + 1]);
+    uint32_t token = __float_as_uint(metadata[3 * (size_t)a + 1]);
+    token = token < tokens ? token : tokens - 1;  // a damaged triple reads a wrong row, never outside
     const V* src = hidden + (size_t)token * row_pieces;
     V* dst = out + (size_t)a * row_pieces;
     for (uint32_t i = threadIdx.x; i < row_pieces; i += blockDim.x) dst[i] = src[i];
-}
-
-__device__ __forceinline__ float silu(float gate) {
-    float s = gate >= 0.f ? 1.f / (1.f + expf(-gate)) : expf(gate) / (1.f + expf(gate));
-    return gate * s;
 }
 
 __global__ __launch_bounds__(256) void expert_silu_mul_kernel(const void* __restrict__ in,
@@ -240,7 +236,7 @@ __global__ __launch_bounds__(256) void expert_silu_mul_kernel(const void* __rest
         size_t base = a * 2 * intermediate;
         float gate = load_as_f32(in, base + column, in_dtype);
         float up = load_as_f32(in, base + intermediate + column, in_dtype);
-        float activated = round_storage(silu(gate), out_dtype);
+        float activated = round_storage(silu_stable(gate), out_dtype);
         store_from_f32(out, i, out_dtype, activated * up);
     }
 }
@@ -315,7 +311,7 @@ __global__ __launch_bounds__(256) void expert_silu_mul8_kernel(const void* __res
         load8(in, a * 2 * intermediate + column, in_dtype, gate);
         load8(in, a * 2 * intermediate + intermediate + column, in_dtype, up);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) result[j] = round_storage(silu(gate[j]), out_dtype) * up[j];
+        for (int j = 0; j < 8; ++j) result[j] = round_storage(silu_stable(gate[j]), out_dtype) * up[j];
         store8(out, i * 8, out_dtype, result);
     }
 }
@@ -584,19 +580,19 @@ const char* launch_expert_group(hipStream_t s, const float* metadata, uint32_t a
 }
 
 const char* launch_expert_assign(hipStream_t s, const void* hidden, const float* metadata,
-                                 void* out, uint32_t assignments, uint32_t row_bytes) {
+                                 void* out, uint32_t assignments, uint32_t row_bytes, uint32_t tokens) {
     if (row_bytes % 16 == 0) {
         hipLaunchKernelGGL(expert_assign_kernel<uint4>, dim3(assignments), dim3(256), 0, s,
                            static_cast<const uint4*>(hidden), metadata, static_cast<uint4*>(out),
-                           assignments, row_bytes / 16);
+                           assignments, row_bytes / 16, tokens);
     } else if (row_bytes % 4 == 0) {
         hipLaunchKernelGGL(expert_assign_kernel<uint32_t>, dim3(assignments), dim3(256), 0, s,
                            static_cast<const uint32_t*>(hidden), metadata,
-                           static_cast<uint32_t*>(out), assignments, row_bytes / 4);
+                           static_cast<uint32_t*>(out), assignments, row_bytes / 4, tokens);
     } else {
         hipLaunchKernelGGL(expert_assign_kernel<uint16_t>, dim3(assignments), dim3(256), 0, s,
                            static_cast<const uint16_t*>(hidden), metadata,
-                           static_cast<uint16_t*>(out), assignments, row_bytes / 2);
+                           static_cast<uint16_t*>(out), assignments, row_bytes / 2, tokens);
     }
     return "expert_assign";
 }

@@ -626,8 +626,9 @@ public:
         if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
             throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
         Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
-        if (dims[0] * routing_.top_k <= fused_max_assignments) {
-            // decode: the copy and the activation ride inside the projections
+        if (fuse_inputs && (dims[0] * routing_.top_k <= fused_max_assignments || hidden.dtype() != DType::F32)) {
+            // the copy and the activation ride inside the projections: per assignment in
+            // decode, and in the grouped kernel's gather of an expert's rows beyond it
             Tensor projected = device_.expert_project_gathered(hidden, meta, input_);
             Tensor expert_output = device_.expert_project_silu_mul(projected, meta, output_);
             return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
@@ -639,8 +640,11 @@ public:
         return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
     }
 
-    // most assignments that take the fused per-assignment kernels
+    // most f32 assignments that take the fused per-assignment kernels (f32 rows have no
+    // grouped form by default, and the per-assignment SiLU is recomputed by every workgroup)
     size_t fused_max_assignments = 31;
+    // false: expert_assign and expert_silu_mul always run as launches of their own
+    bool fuse_inputs = true;
 
 private:
     const Device& device_;

@@ -223,7 +223,7 @@ int main() {
         Tensor xs = d.from_f32({few, hidden}, DType::F16, std::vector<float>(x.begin(), x.begin() + few * hidden));
         Tensor ls = d.from_f32({few, experts}, DType::F32, std::vector<float>(logits.begin(), logits.begin() + few * experts));
         const auto fused = moe.forward(xs, ls).to_f32();
-        moe.fused_max_assignments = 0;
+        moe.fuse_inputs = false;
         const auto separate = moe.forward(xs, ls).to_f32();
         report("SparseMoe::forward decode path equals the separate steps bitwise",
                std::memcmp(fused.data(), separate.data(), fused.size() * 4) == 0);

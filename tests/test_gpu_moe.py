@@ -388,8 +388,11 @@ def test_dense_projection_with_silu_mul_input_matches_the_two_calls(api, d, dtyp
         d.project_quantized(api.Tensor.zeros(d, (m, k), dt), w, silu_mul=True)
 
 
-@pytest.mark.parametrize("tokens", [1, 3])
-def test_sparse_moe_decode_path_matches_the_separate_steps(api, d, tokens):
+# one and three tokens take the per-assignment kernels; 20 and 300 the grouped kernel, whose
+# gather of an expert's rows reads the token rows and applies SiLU * up itself (16 and then
+# 32 tokens a pass)
+@pytest.mark.parametrize("tokens", [1, 3, 20, 300])
+def test_sparse_moe_fused_inputs_match_the_separate_steps(api, d, tokens):
     experts, hidden, inter, top_k = 16, 512, 256, 4
     fmt = api.QuantizationFormat(Q4_K)
     win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=81), fmt,
@@ -402,7 +405,34 @@ def test_sparse_moe_decode_path_matches_the_separate_steps(api, d, tokens):
     xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
     lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
     fused = moe.forward(xt, lt)
-    moe.fused_max_assignments = 0
+    fused_op = d.last_operation()
+    moe.fuse_inputs = False
+    separate = moe.forward(xt, lt)
+    assert np.array_equal(fused.raw(), separate.raw())
+    assert np.abs(fused.to_f32()).max() > 1e-3
+    meta = d.moe_route(lt, None, moe.routing)
+    d.expert_project_quantized(xt, meta, win, hidden, experts, form="gather")
+    assert d.last_operation() == ("expert_project_q4_k_grouped_mfma" if tokens * top_k >= 32 else "expert_project_q4_k_factored")
+
+
+@pytest.mark.parametrize("dtype", ["F16", "BF16"])
+def test_grouped_input_forms_when_an_experts_rows_do_not_fit_lds(api, d, dtype):
+    # 32 rows of 2560 halves are more than the kernel's LDS: the library writes the gathered
+    # and the activated rows out itself and the result is still that of the separate steps
+    experts, hidden, inter, top_k, tokens = 4, 2560, 2560, 2, 40
+    fmt = api.QuantizationFormat(Q4_K)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=85), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * hidden, inter, seed=86), fmt,
+                                         experts, hidden, inter)
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    dt = getattr(api.DType, dtype)
+    x = synth.activations(tokens, hidden, seed=87, f16=True) * np.float32(2.0 ** -5)
+    logits = synth.rng(88).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    fused = moe.forward(xt, lt)
+    moe.fuse_inputs = False
     separate = moe.forward(xt, lt)
     assert np.array_equal(fused.raw(), separate.raw())
     assert np.abs(fused.to_f32()).max() > 1e-3

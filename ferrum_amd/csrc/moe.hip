@@ -380,6 +380,24 @@ unsigned grid_for(size_t threads) {
 // leaves them.  One workgroup; experts <= 1024.
 constexpr int kGroupThreads = 1024;
 
+// Inclusive sum over the 1024 threads of a workgroup, in thread order: each wave scans its
+// own 64 values through lane shuffles and adds the totals of the waves before it, so two
+// barriers replace the twenty of a step-doubling scan through LDS.  wave_total: 16 words.
+__device__ __forceinline__ uint32_t block_inclusive_scan_1024(uint32_t v, uint32_t* wave_total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t sum = v;
+#pragma unroll
+    for (uint32_t step = 1; step < 64; step <<= 1) {
+        const uint32_t below = (uint32_t)__shfl_up((int)sum, step, 64);
+        if (lane >= step) sum += below;
+    }
+    __syncthreads();  // wave_total may still be read from an earlier scan
+    if (lane == 63) wave_total[wave] = sum;
+    __syncthreads();
+    for (uint32_t w = 0; w < wave; ++w) sum += wave_total[w];
+    return sum;
+}
+
 __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float* __restrict__ metadata,
                                                                      uint32_t assignments, uint32_t experts,
                                                                      uint32_t* __restrict__ offsets,
@@ -387,36 +405,47 @@ __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float
                                                                      uint32_t* __restrict__ y_words,
                                                                      uint32_t row_words) {
     __shared__ uint32_t count[kGroupThreads];
-    __shared__ uint32_t scan[kGroupThreads];
+    __shared__ uint32_t wave_total[kGroupThreads / 64];
     const uint32_t tid = threadIdx.x;
     count[tid] = 0;
     __syncthreads();
-    for (uint32_t a = tid; a < assignments; a += kGroupThreads) {
-        const uint32_t e = __float_as_uint(metadata[3 * (size_t)a]);
-        if (e < experts) atomicAdd(&count[e], 1u);
+    // eight ids per thread are requested together: one memory latency per 8192 assignments
+    for (uint32_t base = 0; base < assignments; base += 8 * kGroupThreads) {
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t a = base + i * kGroupThreads + tid;
+            e[i] = a < assignments ? __float_as_uint(metadata[3 * (size_t)a]) : 0xffffffffu;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (e[i] < experts) atomicAdd(&count[e[i]], 1u);
     }
     __syncthreads();
     // inclusive scan over the expert counts
-    uint32_t v = count[tid];
-    scan[tid] = v;
-    __syncthreads();
-    for (uint32_t step = 1; step < kGroupThreads; step <<= 1) {
-        const uint32_t add = tid >= step ? scan[tid - step] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
-    const uint32_t first = scan[tid] - v;
+    const uint32_t v = count[tid];
+    const uint32_t upto = block_inclusive_scan_1024(v, wave_total);
+    const uint32_t first = upto - v;
     if (tid < experts) offsets[tid] = first;
-    if (tid == experts - 1) offsets[experts] = scan[tid];
+    if (tid == experts - 1) offsets[experts] = upto;
     count[tid] = first;  // now the next free slot of each expert
     __syncthreads();
-    for (uint32_t a = tid; a < assignments; a += kGroupThreads) {
-        const uint32_t e = __float_as_uint(metadata[3 * (size_t)a]);
-        if (e < experts) {
-            order[atomicAdd(&count[e], 1u)] = a;
-        } else {
-            for (uint32_t i = 0; i < row_words; ++i) y_words[(size_t)a * row_words + i] = 0u;
+    for (uint32_t base = 0; base < assignments; base += 8 * kGroupThreads) {
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t a = base + i * kGroupThreads + tid;
+            e[i] = a < assignments ? __float_as_uint(metadata[3 * (size_t)a]) : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t a = base + i * kGroupThreads + tid;
+            if (a >= assignments) continue;
+            if (e[i] < experts) {
+                order[atomicAdd(&count[e[i]], 1u)] = a;
+            } else {
+                for (uint32_t j = 0; j < row_words; ++j) y_words[(size_t)a * row_words + j] = 0u;
+            }
         }
     }
 }
@@ -430,34 +459,35 @@ __global__ __launch_bounds__(kGroupThreads) void expert_group_kernel(const float
 // counts of the waves before its own plus its rank.
 constexpr int kMapThreads = 1024;
 constexpr int kMapWaves = kMapThreads / 64;
+static_assert(kMapThreads == 1024 && kGroupThreads == 1024, "block_inclusive_scan_1024 covers 1024 threads");
 
 __global__ __launch_bounds__(kMapThreads) void moe_map_kernel(const uint32_t* __restrict__ ids, uint32_t experts,
                                                               uint32_t routes, uint32_t* __restrict__ offsets,
                                                               uint32_t* __restrict__ sorted,
                                                               uint32_t* __restrict__ position) {
     __shared__ uint32_t next[kMapThreads];                 // counts, then the next free row of each expert
-    __shared__ uint32_t scan[kMapThreads];
+    __shared__ uint32_t wave_total[kMapWaves];
     __shared__ uint8_t wave_count[kMapWaves][kMapThreads];  // routes of expert e in wave w of this round
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     next[tid] = 0;
     __syncthreads();
-    for (uint32_t r = tid; r < routes; r += kMapThreads) {
-        const uint32_t e = ids[r];
-        if (e < experts) atomicAdd(&next[e], 1u);
+    for (uint32_t base = 0; base < routes; base += 8 * kMapThreads) {
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t r = base + i * kMapThreads + tid;
+            e[i] = r < routes ? ids[r] : 0xffffffffu;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (e[i] < experts) atomicAdd(&next[e[i]], 1u);
     }
     __syncthreads();
     const uint32_t mine = next[tid];
-    scan[tid] = mine;
-    __syncthreads();
-    for (uint32_t step = 1; step < kMapThreads; step <<= 1) {
-        const uint32_t add = tid >= step ? scan[tid - step] : 0u;
-        __syncthreads();
-        scan[tid] += add;
-        __syncthreads();
-    }
-    const uint32_t first = scan[tid] - mine;
+    const uint32_t upto = block_inclusive_scan_1024(mine, wave_total);
+    const uint32_t first = upto - mine;
     if (tid < experts) offsets[tid] = first;
-    if (tid == experts - 1) offsets[experts] = scan[tid];
+    if (tid == experts - 1) offsets[experts] = upto;
     next[tid] = first;
 
     uint32_t id_bits = 0;

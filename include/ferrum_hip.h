@@ -287,13 +287,18 @@ fh_status fh_hybrid_moe_combine(fh_device* device, const fh_view* down, const fh
                                 const fh_view* position, const fh_view* shared, const fh_view* shared_gate,
                                 uint32_t hidden, uint32_t used, uint32_t tokens, const fh_view* out);
 
-/* Decode-sized fusions.  SparseMoe::forward (src/nn/moe.rs:222-390) encodes
+/* Input forms.  SparseMoe::forward (src/nn/moe.rs:222-390) encodes
  * expert_assign, the gate|up projection, expert_silu_mul and the down
  * projection back to back; with a handful of assignments each of them is a
  * launch that lasts microseconds.  These two entry points fold the copy or the
  * activation into the projection that follows and give the same bits as the
- * separate calls.  They always take the per-assignment (per-row) kernel, so
- * callers keep the separate calls for prefill-sized batches.
+ * separate calls.  fh_expert_project_fused is good at every batch size for
+ * 16-bit activations: beyond the per-assignment kernel the grouped kernel
+ * gathers the token rows itself, and what it cannot read in place the library
+ * stages in its scratch with the kernels of the separate calls.  With f32
+ * activations (per-assignment kernel only) and in the dense
+ * fh_project_silu_mul_quantized (per-row kernel only) the forms are for
+ * decode-sized batches, and callers keep the separate calls beyond them.
  *
  * fh_expert_project_fused: input_form FH_INPUT_ROWS is
  * fh_expert_project_quantized; FH_INPUT_GATHER reads x as hidden [x_rows, K]

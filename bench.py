@@ -194,10 +194,11 @@ def layer_case(api, synth, dev, steps, layers=4):
 
 def moe_case(api, synth, dev, tokens, steps):
     """A3B-style routed FFN: hidden 2048, 256 experts x intermediate 512 in Q4_K,
-    top-8 softmax routing with renormalised weights, plus one shared expert;
-    f16 activations.  One step = route, gather, gate|up, SiLU*up, down, combine
-    and the shared expert's two projections.  Distinct router logits per step
-    move the set of experts that are hit."""
+    top-8 softmax routing with renormalised weights, plus one shared expert
+    whose output the combine adds; f16 activations.  One step =
+    SparseMoe.forward: route, gate|up, SiLU*up, down and the shared expert's
+    two projections, combine.  Distinct router logits per step move the set of
+    experts that are hit."""
     hidden, inter, experts, top_k = 2048, 512, 256, 8
     fmt = api.QuantizationFormat.Q4_K
     f16, f32 = api.DType.F16, api.DType.F32
@@ -209,7 +210,7 @@ def moe_case(api, synth, dev, tokens, steps):
                                          experts, hidden, inter)
     sin = api.QuantizedMatrix.from_bytes(dev, 2 * inter, hidden, fmt, synth.matrix(Q4_K, 2 * inter, hidden, seed=13))
     sout = api.QuantizedMatrix.from_bytes(dev, hidden, inter, fmt, synth.matrix(Q4_K, hidden, inter, seed=14))
-    moe = api.SparseMoe(dev, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    moe = api.SparseMoe(dev, win, wout, api.MoeRoutingPolicy(experts, top_k), shared_input=sin, shared_output=sout)
     moe.workspace(tokens, f16)
     x = api.Tensor.from_f32(dev, (tokens, hidden), f16,
                             synth.activations(tokens, hidden, seed=15, f16=True) * np.float32(2.0 ** -6))
@@ -219,20 +220,11 @@ def moe_case(api, synth, dev, tokens, steps):
         values = synth.rng(16, i).standard_normal((tokens, experts)).astype(np.float32)
         logit_sets.append(api.Tensor.from_f32(dev, values.shape, f32, values))
         hit.append(len(np.unique(np.argsort(-values, axis=1)[:, :top_k])))
-    s_up = api.Tensor.zeros(dev, (tokens, 2 * inter), f16)
-    s_act = api.Tensor.zeros(dev, (tokens, inter), f16)
-    s_out = api.Tensor.zeros(dev, (tokens, hidden), f16)
     names = []
 
     def enqueue(i):
         moe.forward(x, logit_sets[i % variants])
         names.append(dev.last_operation())
-        dev.project_quantized(x, sin, out=s_up)
-        if tokens * top_k <= moe.fused_max_assignments:
-            dev.project_quantized(s_up, sout, out=s_out, silu_mul=True)   # decode: SiLU*up rides in the projection
-        else:
-            dev.expert_silu_mul(s_up, inter, out=s_act)
-            dev.project_quantized(s_act, sout, out=s_out)
 
     best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(2)) / steps
     per_expert = (2 * inter * hidden + hidden * inter) // 256 * BLOCK_BYTES[Q4_K]
@@ -242,7 +234,8 @@ def moe_case(api, synth, dev, tokens, steps):
     flops = 2 * tokens * (top_k + 1) * (2 * inter * hidden + hidden * inter)
     return {
         "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
-        "operation": "moe_route + expert_assign + 2 x expert_project + silu_mul + combine + shared FFN",
+        "operation": ("moe_route + 2 x (expert_project with the shared expert riding) + combine" if tokens * top_k <= 31
+                      else "moe_route + 2 x expert_project (grouped) + silu_mul + shared FFN + combine"),
         "us": round(best * 1e6, 2),
         "GB/s": round(nbytes / best / 1e9, 1),
         "frac_hbm": round(nbytes / best / 1e9 / HBM_PEAK_GBS, 4),

@@ -129,6 +129,7 @@ SYMBOLS = {
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
     "fh_expert_project_fused": (_I32, [_P, _P, _VP, _U32, _U32, _U32, _VP, _VP]),
     "fh_project_silu_mul_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
+    "fh_expert_project_with_shared": (_I32, [_P, _P, _P, _VP, _U32, _U32, _U32, _VP, _VP, _VP, _VP]),
     "fh_expert_silu_mul": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_expert_combine": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_execution_begin": (_I32, [_P]),
@@ -834,6 +835,41 @@ class Device:
                                                 meta[0], ctypes.byref(mv), ctypes.byref(ov)))
         return out
 
+    def expert_project_with_shared(self, input: Tensor, metadata: Tensor, weight: QuantizedExpertMatrix,
+                                   shared_weight: QuantizedMatrix, tokens: int, form: str,
+                                   shared_input: Tensor | None = None, out: Tensor | None = None,
+                                   shared_out: Tensor | None = None):
+        """The routed projection of ``expert_project_quantized(form=...)`` and, in the same
+        launch, the shared expert's dense projection of every token: ``form="gather"`` reads
+        both from ``input`` [tokens, K]; ``form="silu_mul"`` reads the routed rows from
+        ``input`` [A, 2K] and the shared ones from ``shared_input`` [tokens, 2K].  Returns
+        (routed [A, N], shared [tokens, N]).  For decode-sized batches."""
+        code = {"gather": 1, "silu_mul": 2}[form]
+        x, meta, k = input.shape(), metadata.shape(), weight.columns()
+        if (len(x) != 2 or len(meta) != 2 or meta[1] != 3 or meta[0] == 0 or tokens == 0
+                or metadata.dtype != DType.F32
+                or x != ((tokens, k) if code == 1 else (meta[0], 2 * k))
+                or (code == 2) != (shared_input is not None)
+                or (shared_input is not None and (shared_input.shape() != (tokens, 2 * k)
+                                                  or shared_input.dtype != input.dtype))
+                or shared_weight.rows() != weight.rows_per_expert() or shared_weight.columns() != k
+                or shared_weight.format().ggml_type() != weight.format().ggml_type()
+                or input.buffer.device is not self or metadata.buffer.device is not self
+                or weight.device is not self or shared_weight.device is not self):
+            raise ShapeError("quantized expert projection geometry mismatch")
+        n = weight.rows_per_expert()
+        if out is None:
+            out = Tensor.zeros(self, (meta[0], n), input.dtype)
+        if shared_out is None:
+            shared_out = Tensor.zeros(self, (tokens, n), input.dtype)
+        xv, mv, ov, sov = input._view(), metadata._view(), out._view(), shared_out._view()
+        sxv = shared_input._view() if shared_input is not None else None
+        _check(_lib.fh_expert_project_with_shared(
+            self._handle, weight._handle, _handle_of(shared_weight), ctypes.byref(xv), tokens, code, meta[0],
+            ctypes.byref(mv), ctypes.byref(sxv) if sxv is not None else None, ctypes.byref(ov),
+            ctypes.byref(sov)))
+        return out, shared_out
+
     def expert_silu_mul(self, input: Tensor, intermediate: int, out: Tensor | None = None) -> Tensor:
         x = input.shape()
         if len(x) != 2 or intermediate == 0 or intermediate * 2 != x[1]:
@@ -877,7 +913,12 @@ class SparseMoe:
 
     def __init__(self, device: "Device", input_experts: QuantizedExpertMatrix,
                  output_experts: QuantizedExpertMatrix, routing: MoeRoutingPolicy,
-                 selection_bias: Tensor | None = None):
+                 selection_bias: Tensor | None = None, shared_input: QuantizedMatrix | None = None,
+                 shared_output: QuantizedMatrix | None = None):
+        """``shared_input`` [2*I_s, H] (gate rows first) and ``shared_output`` [H, I_s]: a
+        shared expert that every token runs next to its routed ones, as the hybrid engine's
+        moe_ffn does (src/hybrid/engine.rs:2925); its output is added in the combine,
+        scaled by ``forward``'s ``shared_gate`` when given."""
         e, two_i, h = input_experts.experts(), input_experts.rows_per_expert(), input_experts.columns()
         if (two_i == 0 or two_i % 2 or output_experts.experts() != e
                 or output_experts.rows_per_expert() != h or output_experts.columns() * 2 != two_i
@@ -885,12 +926,23 @@ class SparseMoe:
                 or routing.use_expert_bias != (selection_bias is not None)
                 or input_experts.device is not device or output_experts.device is not device):
             raise ConfigError("invalid sparse expert weight geometry")
+        if (shared_input is None) != (shared_output is None) or (shared_input is not None and (
+                shared_input.columns() != h or shared_output.rows() != h or shared_input.rows() == 0
+                or shared_input.rows() != 2 * shared_output.columns()
+                or shared_input.device is not device or shared_output.device is not device)):
+            raise ConfigError("invalid shared expert weight geometry")
         self.device, self.routing, self.selection_bias = device, routing, selection_bias
         self.input_experts, self.output_experts = input_experts, output_experts
+        self.shared_input, self.shared_output = shared_input, shared_output
         self.expert_count, self.hidden_size, self.intermediate_size = e, h, two_i // 2
+        # the shared expert can ride in the routed launches when it has an expert's shape and format
+        self._shared_rides = (shared_input is not None and shared_input.rows() == two_i
+                              and shared_input.format().ggml_type() == input_experts.format().ggml_type()
+                              and shared_output.format().ggml_type() == output_experts.format().ggml_type())
         self._ws = None
-        # most assignments that take the fused per-assignment kernels; above it the
-        # separate steps run (and group by expert from 32 assignments on)
+        # most f32 assignments that take the fused per-assignment kernels (f32 rows have no
+        # grouped form by default, and the per-assignment SiLU is recomputed by every workgroup);
+        # also the most assignments whose shared expert rides in the routed launches
         self.fused_max_assignments = 31
         # False: expert_assign and expert_silu_mul always run as launches of their own
         self.fuse_inputs = True
@@ -905,9 +957,14 @@ class SparseMoe:
                     "activated": Tensor.zeros(d, (a, i), dtype),
                     "expert_output": Tensor.zeros(d, (a, h), dtype),
                     "combined": Tensor.zeros(d, (tokens, h), dtype)}
+        if self.shared_input is not None:
+            si = self.shared_output.columns()
+            self._ws.update({"shared_projected": Tensor.zeros(d, (tokens, 2 * si), dtype),
+                             "shared_activated": Tensor.zeros(d, (tokens, si), dtype),
+                             "shared_output": Tensor.zeros(d, (tokens, h), dtype)})
         return self._ws
 
-    def forward(self, hidden: Tensor, router_logits: Tensor) -> Tensor:
+    def forward(self, hidden: Tensor, router_logits: Tensor, shared_gate: Tensor | None = None) -> Tensor:
         dims = hidden.shape()
         if len(dims) != 2 or dims[1] != self.hidden_size or dims[0] == 0:
             raise ShapeError("sparse expert input requires [tokens,hidden]")
@@ -916,6 +973,8 @@ class SparseMoe:
         d, k = self.device, self.routing.top_k
         ws = self._ws if self._ws and self._ws["tokens"] == dims[0] and self._ws["dtype"] == hidden.dtype else {}
         metadata = d.moe_route(router_logits, self.selection_bias, self.routing, out=ws.get("metadata"))
+        if self.shared_input is not None:
+            return self._forward_with_shared(hidden, metadata, shared_gate, ws)
         if self.fuse_inputs and (dims[0] * k <= self.fused_max_assignments or hidden.dtype != DType.F32):
             # the copy and the activation ride inside the projections: per assignment in
             # decode, and in the grouped kernel's gather of an expert's rows beyond it
@@ -934,6 +993,45 @@ class SparseMoe:
                                                        out=ws.get("expert_output"))
         return d.expert_combine(expert_output, metadata, dims[0], self.hidden_size, k,
                                 out=ws.get("combined"))
+
+    def _forward_with_shared(self, hidden, metadata, shared_gate, ws):
+        d, k, tokens = self.device, self.routing.top_k, hidden.shape()[0]
+        a = tokens * k
+        if self.fuse_inputs and self._shared_rides and a <= self.fused_max_assignments:
+            # decode: four launches, the shared expert's rows are batch entries of the routed ones
+            projected, shared_projected = d.expert_project_with_shared(
+                hidden, metadata, self.input_experts, self.shared_input, tokens, "gather",
+                out=ws.get("projected"), shared_out=ws.get("shared_projected"))
+            expert_output, shared_output = d.expert_project_with_shared(
+                projected, metadata, self.output_experts, self.shared_output, tokens, "silu_mul",
+                shared_input=shared_projected, out=ws.get("expert_output"), shared_out=ws.get("shared_output"))
+        else:
+            fused = self.fuse_inputs and (a <= self.fused_max_assignments or hidden.dtype != DType.F32)
+            if fused:
+                projected = d.expert_project_quantized(hidden, metadata, self.input_experts, self.hidden_size,
+                                                       self.expert_count, out=ws.get("projected"), form="gather")
+                expert_output = d.expert_project_quantized(projected, metadata, self.output_experts,
+                                                           self.intermediate_size, self.expert_count,
+                                                           out=ws.get("expert_output"), form="silu_mul")
+            else:
+                assigned = d.expert_assign(hidden, metadata, k, out=ws.get("assigned"))
+                projected = d.expert_project_quantized(assigned, metadata, self.input_experts, self.hidden_size,
+                                                       self.expert_count, out=ws.get("projected"))
+                activated = d.expert_silu_mul(projected, self.intermediate_size, out=ws.get("activated"))
+                expert_output = d.expert_project_quantized(activated, metadata, self.output_experts,
+                                                           self.intermediate_size, self.expert_count,
+                                                           out=ws.get("expert_output"))
+            shared_projected = d.project_quantized(hidden, self.shared_input, out=ws.get("shared_projected")).tensor
+            if self.fuse_inputs and tokens <= self.fused_max_assignments:
+                shared_output = d.project_quantized(shared_projected, self.shared_output, out=ws.get("shared_output"),
+                                                    silu_mul=True).tensor
+            else:
+                shared_activated = d.expert_silu_mul(shared_projected, self.shared_output.columns(),
+                                                     out=ws.get("shared_activated"))
+                shared_output = d.project_quantized(shared_activated, self.shared_output,
+                                                    out=ws.get("shared_output")).tensor
+        return d.expert_combine_shared(expert_output, metadata, tokens, self.hidden_size, k, shared_output,
+                                       shared_gate, out=ws.get("combined"))
 
 
 def _handle_of(weight):

@@ -937,10 +937,22 @@ fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t to
 
 namespace {
 
+// A shared expert (dense [rows, k] matrix every token also runs) can ride in the launch:
+// tokens entries more, reading x (gather form) or shared_x (SiLU form), writing shared_y.
+struct SharedExpert {
+    const fh_qmatrix* weight = nullptr;
+    uint32_t tokens = 0;
+    const fh_view* x = nullptr;
+    const fh_view* y = nullptr;
+};
+
 fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t x_rows,
-                         uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y) {
+                         uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y,
+                         const SharedExpert* shared = nullptr) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (form > FH_INPUT_SILU_MUL) return fail(FH_ERR_PARAMETER, "unknown input form %u", form);
+    if (shared != nullptr && form == FH_INPUT_ROWS)
+        return fail(FH_ERR_PARAMETER, "a shared expert needs the gathered or the SiLU input form");
     if (form == FH_INPUT_GATHER && x_rows == 0) return fail(FH_ERR_SHAPE, "gathered expert projection needs tokens");
     if (weight->device != device || assignments == 0 || metadata == nullptr ||
         metadata->dtype != FH_F32 || metadata->buffer == nullptr ||
@@ -961,6 +973,33 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     st = resolve(device, y, (uint64_t)assignments * rows, "expert output", &yr);
     if (st != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(mr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    Range sxr{nullptr, 0}, syr{nullptr, 0};
+    if (shared != nullptr) {
+        const fh_qmatrix* sw = shared->weight;
+        if (sw == nullptr || shared->y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+        if (sw->device != device) {
+            g_last_error = "weight belongs to another device";
+            return FH_ERR_DEVICE_MISMATCH;
+        }
+        if (sw->experts != 1 || sw->rows != rows || sw->cols != k || sw->ggml_type != weight->ggml_type)
+            return fail(FH_ERR_SHAPE, "the shared expert's matrix must have one expert's shape and format");
+        if (shared->tokens == 0 || (form == FH_INPUT_GATHER && shared->tokens != x_rows) ||
+            !fits_u32((uint64_t)assignments + shared->tokens) || !fits_u32((uint64_t)shared->tokens * rows))
+            return fail(FH_ERR_SHAPE, "the shared expert runs once per token");
+        if ((form == FH_INPUT_SILU_MUL) != (shared->x != nullptr))
+            return fail(FH_ERR_PARAMETER, "the shared expert takes its own input in the SiLU form only");
+        if (shared->y->dtype != y->dtype || (shared->x != nullptr && shared->x->dtype != x->dtype))
+            return fail(FH_ERR_DTYPE, "the shared expert's tensors differ in dtype from the routed ones");
+        st = resolve(device, shared->y, (uint64_t)shared->tokens * rows, "shared expert output", &syr);
+        if (st != FH_OK) return st;
+        if (shared->x != nullptr) {
+            st = resolve(device, shared->x, (uint64_t)shared->tokens * k * 2, "shared expert input", &sxr);
+            if (st != FH_OK) return st;
+            if (overlaps(sxr, syr) || overlaps(sxr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+        }
+        if (overlaps(xr, syr) || overlaps(mr, syr) || overlaps(yr, syr))
+            return fail(FH_ERR_RANGE, "shared expert output aliases another tensor");
+    }
     const int64_t grouped_min = tuning(device, "expert_grouped_min_assignments");
     // f32 rows join the grouped form when the caller has opted f32 activations into the f16
     // tiles (gemm_f32_min_rows, the hybrid engine's prompt path project_mm_id_in,
@@ -968,8 +1007,8 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
     const bool f32_grouped = form == FH_INPUT_ROWS && x->dtype == FH_F32 && f32_rows > 0 &&
                              assignments >= (uint64_t)f32_rows && ((uintptr_t)xr.begin & 15u) == 0;
-    if ((x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 && assignments >= (uint64_t)grouped_min &&
-        weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
+    if (shared == nullptr && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
+        assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
         // grouped form: every expert's weights are streamed once for all of its assignments.
         // The kernel that keeps an expert's rows in LDS gathers them from the token rows
         // itself; where they do not fit, and for the SiLU form, the rows are written out
@@ -1036,6 +1075,13 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     a.ksplit = 0;
     a.x_mode = form;
     a.x_rows = form == FH_INPUT_GATHER ? x_rows : assignments;
+    if (shared != nullptr) {
+        a.m = assignments + shared->tokens;
+        a.shared_w = shared->weight->ptr;
+        a.shared_rows = shared->tokens;
+        a.shared_x = sxr.begin;
+        a.shared_y = const_cast<uint8_t*>(syr.begin);
+    }
     st = prepare_gemv(device, a);
     if (st != FH_OK) return st;
     device->last_operation = launch_gemv(device->stream, a);
@@ -1044,6 +1090,19 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
 }
 
 }  // namespace
+
+fh_status fh_expert_project_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                        const fh_qmatrix* shared_weight, const fh_view* x, uint32_t tokens,
+                                        uint32_t input_form, uint32_t assignments, const fh_view* metadata,
+                                        const fh_view* shared_x, const fh_view* y, const fh_view* shared_y) {
+    SharedExpert shared;
+    shared.weight = shared_weight;
+    shared.tokens = tokens;
+    shared.x = shared_x;
+    shared.y = shared_y;
+    if (shared_weight == nullptr || shared_y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    return expert_project(device, weight, x, tokens, input_form, assignments, metadata, y, &shared);
+}
 
 fh_status fh_expert_project_quantized(fh_device* device, const fh_qmatrix* weight,
                                       const fh_view* x, uint32_t assignments,

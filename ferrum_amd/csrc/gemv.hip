@@ -313,6 +313,14 @@ struct Params {
                          // or kXDivide (row = m / x_div: the routes of a token share its row)
     uint32_t meta_stride;  // floats per batch entry in `metadata`: 3 (id, token, weight) or 1 (ids only)
     uint32_t x_div;
+    // Batch entries from `routed` on belong to a shared expert that every token also runs:
+    // entry routed + t multiplies token t's row with the dense matrix w_shared [n, k] into
+    // row t of y_shared.  Its input is row t of x (kXGather: x holds the token rows) or of
+    // x_shared (kXSiluMul: the shared expert's own packed gate|up rows).
+    uint32_t routed;
+    const uint8_t* w_shared;
+    const void* x_shared;
+    void* y_shared;
 };
 
 // grid: (row tiles, K segments, m)
@@ -332,18 +340,25 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
 
     size_t row_base = 0;
     bool live = true;
-    if (p.metadata != nullptr) {
+    const bool shared = m >= p.routed;             // uniform over the workgroup
+    const uint8_t* wmat = shared ? p.w_shared : p.w;
+    const void* xmat = shared && p.x_mode == kXSiluMul ? p.x_shared : p.x;
+    void* ymat = shared ? p.y_shared : p.y;
+    const uint32_t ym = shared ? m - p.routed : m;  // row of y this entry writes
+    if (p.metadata != nullptr && !shared) {
         uint32_t expert = __float_as_uint(p.metadata[p.meta_stride * (size_t)m]);
         live = expert < p.experts;
         row_base = live ? (size_t)expert * p.n : 0;
     }
     const uint32_t row = (blockIdx.x * kWaves + wave) * RS + rs;
-    const uint8_t* rp = p.w + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
+    const uint8_t* rp = wmat + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
 
     // 1. activations of this segment (requested first, consumed first)
     // float4 index of the segment start in the row this batch entry reads
-    size_t xrow = m;
-    if (p.x_mode == kXGather) {
+    size_t xrow = ym;
+    if (shared) {
+        // token ym's own row, in either form
+    } else if (p.x_mode == kXGather) {
         const uint32_t token = __float_as_uint(p.metadata[3 * (size_t)m + 1]);
         xrow = token < p.x_rows ? token : p.x_rows - 1;
     } else if (p.x_mode == kXDivide) {
@@ -354,8 +369,8 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     // loads are queued instead of ahead of them
     const bool early = p.x_mode != kXSiluMul;
     auto fetch = [&](uint32_t q) {
-        float4 v = load_x4(p.x, p.x_dtype, xbase + q);
-        if (p.x_mode == kXSiluMul) v = silu_mul4(v, load_x4(p.x, p.x_dtype, xbase + (size_t)p.nb * 64 + q), p.x_dtype);
+        float4 v = load_x4(xmat, p.x_dtype, xbase + q);
+        if (p.x_mode == kXSiluMul) v = silu_mul4(v, load_x4(xmat, p.x_dtype, xbase + (size_t)p.nb * 64 + q), p.x_dtype);
         return v;
     };
     const uint32_t xq = cb * 64;
@@ -364,7 +379,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
 #pragma unroll
     for (int i = 0; i < kXPer; ++i) {
         uint32_t q = tid + i * kThreads;
-        xr[i] = q < xq && early ? load_x4(p.x, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
+        xr[i] = q < xq && early ? load_x4(xmat, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     asm volatile("" ::: "memory");
 
@@ -417,7 +432,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     if (!live) acc = 0.f;
 
     if (p.segments == 1) {
-        if (writer) store_from_f32(p.y, (size_t)m * p.n + row, p.y_dtype, acc);
+        if (writer) store_from_f32(ymat, (size_t)ym * p.n + row, p.y_dtype, acc);
         return;
     }
     // 5. K segments meet in the scratch buffer; the last workgroup of a tile adds
@@ -444,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
             for (uint32_t s = 0; s < p.segments; ++s)
                 total += __hip_atomic_load(&p.partials[((size_t)s * p.m + m) * p.n + r], __ATOMIC_RELAXED,
                                            __HIP_MEMORY_SCOPE_AGENT);
-            store_from_f32(p.y, (size_t)m * p.n + r, p.y_dtype, total);
+            store_from_f32(ymat, (size_t)ym * p.n + r, p.y_dtype, total);
         }
     }
 }
@@ -536,6 +551,10 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     p.x_rows = a.x_rows;
     p.meta_stride = a.meta_stride == 0 ? 3u : a.meta_stride;
     p.x_div = a.x_div == 0 ? 1u : a.x_div;
+    p.routed = a.shared_w != nullptr ? a.m - a.shared_rows : 0xffffffffu;
+    p.w_shared = static_cast<const uint8_t*>(a.shared_w);
+    p.x_shared = a.shared_x;
+    p.y_shared = a.shared_y;
     const size_t lds = (size_t)plan.seg_len * kXStride * 16 + (size_t)plan.seg_len * 64;
     dim3 grid(plan.tiles, plan.segments, a.m);
     LaunchFn fn = a.ggml_type == kQ4K     ? pick<kQ4K>(plan.bs, plan.it)

@@ -127,6 +127,13 @@ struct GemvArgs {
     uint32_t x_rows;      // rows of x (kXGather clamps the token id to it)
     uint32_t meta_stride; // floats per entry of `metadata`: 0 or 3 = {id, token, weight}, 1 = ids only
     uint32_t x_div;       // kXDivide: batch entries per row of x (0 = 1)
+    // A shared expert riding in the same launch: the last shared_rows of the m batch entries
+    // are tokens 0 .. shared_rows - 1 on the dense matrix shared_w [n, k], writing shared_y
+    // [shared_rows, n]; they read x (kXGather) or shared_x (kXSiluMul).  Null = none.
+    const void* shared_w;
+    uint32_t shared_rows;
+    const void* shared_x;
+    void* shared_y;
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
 };

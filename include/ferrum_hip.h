@@ -315,6 +315,25 @@ fh_status fh_expert_project_fused(fh_device* device, const fh_qmatrix* weight, c
 fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* weight,
                                         const fh_view* packed, uint32_t m, const fh_view* y);
 
+/* The routed projection with a shared expert in the same launch.  Models with
+ * a shared expert run it as a dense FFN on every token next to the routed
+ * experts (the hybrid engine's moe_ffn, src/hybrid/engine.rs:2925, right
+ * after routing); in decode that is two more launches of a few microseconds.
+ * Here the `tokens` rows of the shared expert are further batch entries of
+ * fh_expert_project_fused's per-assignment kernel: y gets what
+ * fh_expert_project_fused(weight, x, tokens, input_form, ..) writes and
+ * shared_y [tokens, N] what fh_project_quantized(shared_weight, x) (gathered
+ * form; shared_x must be NULL) or fh_project_silu_mul_quantized(shared_weight,
+ * shared_x) (SiLU form; shared_x is the shared expert's own packed
+ * [tokens, 2K] rows) writes, bit for bit while both would take that kernel.
+ * shared_weight is dense with one expert's rows, columns and format;
+ * input_form is FH_INPUT_GATHER or FH_INPUT_SILU_MUL.  Always the
+ * per-assignment kernel: for decode-sized batches. */
+fh_status fh_expert_project_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                        const fh_qmatrix* shared_weight, const fh_view* x, uint32_t tokens,
+                                        uint32_t input_form, uint32_t assignments, const fh_view* metadata,
+                                        const fh_view* shared_x, const fh_view* y, const fh_view* shared_y);
+
 /* MetalDevice::expert_silu_mul (src/ops/mod.rs:487-508): in [A, 2*I] (gate
  * first), out [A, I] = round(silu(gate)) * up, stored in out.dtype. */
 fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assignments,

@@ -18,6 +18,7 @@
 #include <cstring>
 #include <functional>
 #include <memory>
+#include <optional>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -546,6 +547,34 @@ public:
                                    const Tensor* out = nullptr) const {
         return expert_project_fused(packed, metadata, w, FH_INPUT_SILU_MUL, out);
     }
+    // The routed projection and, in the same launch, the shared expert's dense projection of
+    // every token (fh_expert_project_with_shared): form FH_INPUT_GATHER reads both from
+    // input [tokens, K]; FH_INPUT_SILU_MUL reads the routed rows from input [A, 2K] and the
+    // shared ones from shared_input [tokens, 2K].  Returns {routed [A, N], shared [tokens, N]}.
+    std::pair<Tensor, Tensor> expert_project_with_shared(const Tensor& input, const Tensor& metadata,
+                                                         const QuantizedExpertMatrix& w, const QuantizedMatrix& shared_w,
+                                                         size_t tokens, uint32_t form,
+                                                         const Tensor* shared_input = nullptr) const {
+        const auto& x = input.shape();
+        const auto& m = metadata.shape();
+        const size_t k = w.columns();
+        const bool silu = form == FH_INPUT_SILU_MUL;
+        if ((form != FH_INPUT_GATHER && !silu) || x.size() != 2 || m.size() != 2 || m[0] == 0 || m[1] != 3 || tokens == 0 ||
+            x[0] != (silu ? m[0] : tokens) || x[1] != (silu ? 2 * k : k) || silu != (shared_input != nullptr) ||
+            (shared_input && (shared_input->shape() != std::vector<size_t>{tokens, 2 * k} ||
+                              shared_input->dtype() != input.dtype())) ||
+            shared_w.rows() != w.rows_per_expert() || shared_w.columns() != k || shared_w.format() != w.format())
+            throw Error(ErrorKind::Shape, "quantized expert projection geometry mismatch");
+        if (!owns(input) || !owns(metadata) || shared_w.owner() != handle_)
+            throw Error(ErrorKind::DeviceMismatch, "tensor or weight belongs to another device");
+        Tensor y = zeros({m[0], w.rows_per_expert()}, input.dtype());
+        Tensor ys = zeros({tokens, w.rows_per_expert()}, input.dtype());
+        fh_view xv = input.c_view(), mv = metadata.c_view(), yv = y.c_view(), ysv = ys.c_view(), sxv{};
+        if (shared_input) sxv = shared_input->c_view();
+        check(fh_expert_project_with_shared(handle_->raw, w.matrix().raw(), shared_w.raw(), &xv, (uint32_t)tokens, form,
+                                            (uint32_t)m[0], &mv, shared_input ? &sxv : nullptr, &yv, &ysv));
+        return {y, ys};
+    }
     Output project_silu_mul_quantized(const Tensor& packed, const QuantizedMatrix& w, const Tensor* out = nullptr) const {
         const auto& dims = packed.shape();
         if (dims.size() != 2 || dims[1] != 2 * w.columns() || dims[0] == 0)
@@ -620,36 +649,74 @@ public:
             routing_.experts != input_.experts() || routing_.top_k == 0 || routing_.top_k > routing_.experts)
             throw Error(ErrorKind::Config, "invalid sparse expert weight geometry");
     }
-    Tensor forward(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias = nullptr) const {
+    // A shared expert that every token runs next to its routed ones, as the hybrid engine's
+    // moe_ffn does (src/hybrid/engine.rs:2925): input [2*I_s, H] with the gate rows first,
+    // output [H, I_s].  Its result is added in the combine, scaled by forward's shared_gate.
+    void set_shared_expert(QuantizedMatrix input, QuantizedMatrix output) {
+        if (input.columns() != input_.columns() || output.rows() != input_.columns() || input.rows() == 0 ||
+            input.rows() != 2 * output.columns())
+            throw Error(ErrorKind::Config, "invalid shared expert weight geometry");
+        shared_rides_ = input.rows() == input_.rows_per_expert() && input.format() == input_.format() &&
+                        output.format() == output_.format();
+        shared_input_ = std::move(input);
+        shared_output_ = std::move(output);
+    }
+    Tensor forward(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias = nullptr,
+                   const Tensor* shared_gate = nullptr) const {
         const auto& dims = hidden.shape();
         const size_t h = input_.columns(), i = input_.rows_per_expert() / 2, e = input_.experts();
         if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
             throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
         Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
-        if (fuse_inputs && (dims[0] * routing_.top_k <= fused_max_assignments || hidden.dtype() != DType::F32)) {
-            // the copy and the activation ride inside the projections: per assignment in
-            // decode, and in the grouped kernel's gather of an expert's rows beyond it
-            Tensor projected = device_.expert_project_gathered(hidden, meta, input_);
-            Tensor expert_output = device_.expert_project_silu_mul(projected, meta, output_);
-            return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
+        if (shared_input_) {
+            const size_t tokens = dims[0], a = tokens * routing_.top_k;
+            if (fuse_inputs && shared_rides_ && a <= fused_max_assignments) {
+                // decode: four launches, the shared expert's rows are batch entries of the routed ones
+                auto up = device_.expert_project_with_shared(hidden, meta, input_, *shared_input_, tokens, FH_INPUT_GATHER);
+                auto down = device_.expert_project_with_shared(up.first, meta, output_, *shared_output_, tokens,
+                                                               FH_INPUT_SILU_MUL, &up.second);
+                return device_.expert_combine_shared(down.first, meta, tokens, h, routing_.top_k, down.second, shared_gate);
+            }
+            Tensor expert_output = routed(hidden, meta, h, i, e);
+            Tensor shared_projected = device_.project_quantized(hidden, *shared_input_).tensor;
+            Tensor shared_output =
+                fuse_inputs && tokens <= fused_max_assignments
+                    ? device_.project_silu_mul_quantized(shared_projected, *shared_output_).tensor
+                    : device_.project_quantized(device_.expert_silu_mul(shared_projected, shared_output_->columns()),
+                                                *shared_output_).tensor;
+            return device_.expert_combine_shared(expert_output, meta, tokens, h, routing_.top_k, shared_output, shared_gate);
         }
-        Tensor assigned = device_.expert_assign(hidden, meta, routing_.top_k);
-        Tensor projected = device_.expert_project_quantized(assigned, meta, input_, h, e);
-        Tensor activated = device_.expert_silu_mul(projected, i);
-        Tensor expert_output = device_.expert_project_quantized(activated, meta, output_, i, e);
-        return device_.expert_combine(expert_output, meta, dims[0], h, routing_.top_k);
+        return device_.expert_combine(routed(hidden, meta, h, i, e), meta, dims[0], h, routing_.top_k);
     }
 
     // most f32 assignments that take the fused per-assignment kernels (f32 rows have no
-    // grouped form by default, and the per-assignment SiLU is recomputed by every workgroup)
+    // grouped form by default, and the per-assignment SiLU is recomputed by every workgroup);
+    // also the most assignments whose shared expert rides in the routed launches
     size_t fused_max_assignments = 31;
     // false: expert_assign and expert_silu_mul always run as launches of their own
     bool fuse_inputs = true;
 
 private:
+    // the routed experts' outputs [A, H], before the combine
+    Tensor routed(const Tensor& hidden, const Tensor& meta, size_t h, size_t i, size_t e) const {
+        const auto& dims = hidden.shape();
+        if (fuse_inputs && (dims[0] * routing_.top_k <= fused_max_assignments || hidden.dtype() != DType::F32)) {
+            // the copy and the activation ride inside the projections: per assignment in
+            // decode, and in the grouped kernel's gather of an expert's rows beyond it
+            Tensor projected = device_.expert_project_gathered(hidden, meta, input_);
+            return device_.expert_project_silu_mul(projected, meta, output_);
+        }
+        Tensor assigned = device_.expert_assign(hidden, meta, routing_.top_k);
+        Tensor projected = device_.expert_project_quantized(assigned, meta, input_, h, e);
+        Tensor activated = device_.expert_silu_mul(projected, i);
+        return device_.expert_project_quantized(activated, meta, output_, i, e);
+    }
+
     const Device& device_;
     QuantizedExpertMatrix input_, output_;
     MoeRoutingPolicy routing_;
+    std::optional<QuantizedMatrix> shared_input_, shared_output_;
+    bool shared_rides_ = false;
 };
 
 }  // namespace ferrum

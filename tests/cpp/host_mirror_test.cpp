@@ -228,6 +228,33 @@ int main() {
         report("SparseMoe::forward decode path equals the separate steps bitwise",
                std::memcmp(fused.data(), separate.data(), fused.size() * 4) == 0);
 
+        // a shared expert: with one token it rides in the routed launches, and every launch is the
+        // per-row kernel either way, so the two orchestrations give the same bits
+        const auto sin = blocks(QuantizationFormat::Q4_K, 2 * inter, hidden, 25);
+        const auto sout = blocks(QuantizationFormat::Q4_K, hidden, inter, 26);
+        moe.set_shared_expert(upload(d, QuantizationFormat::Q4_K, 2 * inter, hidden, sin),
+                              upload(d, QuantizationFormat::Q4_K, hidden, inter, sout));
+        Tensor x1 = d.from_f32({1, hidden}, DType::F16, std::vector<float>(x.begin(), x.begin() + hidden));
+        Tensor l1 = d.from_f32({1, experts}, DType::F32, std::vector<float>(logits.begin(), logits.begin() + experts));
+        Tensor gate1 = d.from_f32({1}, DType::F32, std::vector<float>{0.625f});
+        moe.fuse_inputs = true;
+        const auto riding = moe.forward(x1, l1, nullptr, &gate1).to_f32();
+        const bool rode = d.last_operation() == std::string("h_moe_combine");
+        moe.fuse_inputs = false;
+        const auto apart = moe.forward(x1, l1, nullptr, &gate1).to_f32();
+        float peak = 0.f;
+        for (float v : riding) peak = std::max(peak, std::fabs(v));
+        report("SparseMoe with a shared expert: riding in the routed launches equals the separate calls bitwise",
+               rode && peak > 1e-4f && std::memcmp(riding.data(), apart.data(), riding.size() * 4) == 0, peak);
+        bool refused = false;
+        try {
+            moe.set_shared_expert(upload(d, QuantizationFormat::Q4_K, 2 * inter, hidden, sin),
+                                  upload(d, QuantizationFormat::Q4_K, 2 * inter, hidden, sin));
+        } catch (const Error& e) {
+            refused = e.kind() == ErrorKind::Config;
+        }
+        report("a shared expert whose output matrix does not fit is Error::Config", refused);
+
         Device other(0);
         bool threw = false;
         try {

@@ -389,8 +389,8 @@ def test_dense_projection_with_silu_mul_input_matches_the_two_calls(api, d, dtyp
 
 
 # one and three tokens take the per-assignment kernels; 20 and 300 the grouped kernel, whose
-# gather of an expert's rows reads the token rows and applies SiLU * up itself (16 and then
-# 32 tokens a pass)
+# gather of an expert's rows reads the token rows itself (16 and then 32 tokens a pass) and
+# whose SiLU * up rows the library writes into its scratch
 @pytest.mark.parametrize("tokens", [1, 3, 20, 300])
 def test_sparse_moe_fused_inputs_match_the_separate_steps(api, d, tokens):
     experts, hidden, inter, top_k = 16, 512, 256, 4
@@ -436,6 +436,108 @@ def test_grouped_input_forms_when_an_experts_rows_do_not_fit_lds(api, d, dtype):
     separate = moe.forward(xt, lt)
     assert np.array_equal(fused.raw(), separate.raw())
     assert np.abs(fused.to_f32()).max() > 1e-3
+
+
+def _shared_case(api, d, dtype, tokens, seed):
+    experts, hidden, inter, top_k = 16, 512, 256, 4
+    fmt = api.QuantizationFormat(Q4_K)
+    packed = {"win": synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=seed),
+              "wout": synth.matrix(Q4_K, experts * hidden, inter, seed=seed + 1),
+              "sin": synth.matrix(Q4_K, 2 * inter, hidden, seed=seed + 2),
+              "sout": synth.matrix(Q4_K, hidden, inter, seed=seed + 3)}
+    w = {"win": api.QuantizedExpertMatrix.new(d, packed["win"], fmt, experts, 2 * inter, hidden),
+         "wout": api.QuantizedExpertMatrix.new(d, packed["wout"], fmt, experts, hidden, inter),
+         "sin": api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, packed["sin"]),
+         "sout": api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, packed["sout"])}
+    dt = getattr(api.DType, dtype)
+    x = synth.activations(tokens, hidden, seed=seed + 4, f16=True) * np.float32(2.0 ** -4)
+    logits = synth.rng(seed + 5).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    return (experts, hidden, inter, top_k), packed, w, x, logits, xt, lt
+
+
+@pytest.mark.parametrize("dtype", ["F32", "F16", "BF16"])
+@pytest.mark.parametrize("tokens", [1, 3])
+def test_shared_expert_rides_in_the_routed_launch(api, d, dtype, tokens):
+    (experts, hidden, inter, top_k), _, w, _, _, xt, lt = _shared_case(api, d, dtype, tokens, 171)
+    meta = d.moe_route(lt, None, api.MoeRoutingPolicy(experts, top_k))
+    d.set_tuning("gemm_min_rows", 1000)  # the dense reference calls below take the per-row kernel too
+    try:
+        up, shared_up = d.expert_project_with_shared(xt, meta, w["win"], w["sin"], tokens, "gather")
+        assert d.last_operation() == "expert_project_q4_k_factored"
+        assert np.array_equal(up.raw(), d.expert_project_quantized(xt, meta, w["win"], hidden, experts,
+                                                                   form="gather").raw())
+        assert np.array_equal(shared_up.raw(), d.project_quantized(xt, w["sin"]).tensor.raw())
+        down, shared_down = d.expert_project_with_shared(up, meta, w["wout"], w["sout"], tokens, "silu_mul",
+                                                         shared_input=shared_up)
+        assert np.array_equal(down.raw(), d.expert_project_quantized(up, meta, w["wout"], inter, experts,
+                                                                     form="silu_mul").raw())
+        assert np.array_equal(shared_down.raw(), d.project_quantized(shared_up, w["sout"], silu_mul=True).tensor.raw())
+        assert np.abs(shared_down.to_f32()).max() > 1e-4 and np.abs(down.to_f32()).max() > 1e-4
+    finally:
+        d.set_tuning("gemm_min_rows", 2)
+
+
+def test_shared_expert_projection_rejects_what_it_cannot_run(api, d):
+    (experts, hidden, inter, top_k), packed, w, _, _, xt, lt = _shared_case(api, d, "F16", 2, 181)
+    meta = d.moe_route(lt, None, api.MoeRoutingPolicy(experts, top_k))
+    fmt = api.QuantizationFormat(Q4_K)
+    with pytest.raises(api.ShapeError):   # a shared matrix of another shape
+        d.expert_project_with_shared(xt, meta, w["win"], w["sout"], 2, "gather")
+    with pytest.raises(api.ShapeError):   # the SiLU form needs the shared expert's own rows
+        up, _ = d.expert_project_with_shared(xt, meta, w["win"], w["sin"], 2, "gather")
+        d.expert_project_with_shared(up, meta, w["wout"], w["sout"], 2, "silu_mul")
+    q6 = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, api.QuantizationFormat(Q6_K),
+                                        synth.matrix(Q6_K, 2 * inter, hidden, seed=182))
+    with pytest.raises(api.ShapeError):   # another format
+        d.expert_project_with_shared(xt, meta, w["win"], q6, 2, "gather")
+    # the C entry point itself: the rows form has no shared variant, and outputs must not alias
+    from ferrum_amd.api import _lib
+    import ctypes
+    up = api.Tensor.zeros(d, (2 * top_k, 2 * inter), api.DType.F16)
+    sup = api.Tensor.zeros(d, (2, 2 * inter), api.DType.F16)
+    xv, mv, ov, sv = xt._view(), meta._view(), up._view(), sup._view()
+    call = lambda form, out, shared_out: _lib.fh_expert_project_with_shared(
+        d._handle, w["win"]._handle, w["sin"]._handle, ctypes.byref(xv), 2, form, 2 * top_k, ctypes.byref(mv), None,
+        ctypes.byref(out), ctypes.byref(shared_out))
+    last_error = lambda: _lib.fh_last_error().decode()
+    assert call(0, ov, sv) != 0 and "gathered or the SiLU" in last_error()
+    assert call(1, ov, ov) != 0 and "aliases" in last_error()
+    assert call(1, ov, sv) == 0
+
+
+@pytest.mark.parametrize("tokens,gated", [(1, False), (3, True), (40, True)])
+def test_sparse_moe_with_a_shared_expert(api, d, tokens, gated):
+    # one and three tokens: the shared expert rides in the routed launches; 40: separate dense calls
+    (experts, hidden, inter, top_k), packed, w, x, logits, xt, lt = _shared_case(api, d, "F16", tokens, 191)
+    moe = api.SparseMoe(d, w["win"], w["wout"], api.MoeRoutingPolicy(experts, top_k),
+                        shared_input=w["sin"], shared_output=w["sout"])
+    gate = None
+    gate_values = None
+    if gated:
+        gate_values = (0.25 + 0.5 * synth.rng(192).random(tokens)).astype(np.float32)
+        gate = api.Tensor.from_f32(d, (tokens,), api.DType.F32, gate_values)
+    got = moe.forward(xt, lt, shared_gate=gate)
+    moe.fuse_inputs = False
+    separate = moe.forward(xt, lt, shared_gate=gate)
+    if tokens == 1:
+        assert np.array_equal(got.raw(), separate.raw())   # every launch is the per-row kernel either way
+    # the whole FFN against the host statement, f16 storage at every step
+    code = oracle.F16
+    xr = oracle.round_storage(x, code)
+    meta = oracle.select_routes(logits, experts, top_k)
+    up = oracle.round_storage(oracle.expert_project(Q4_K, packed["win"], experts, 2 * inter, hidden,
+                                                    oracle.expert_assign(xr, meta), meta), code)
+    down = oracle.round_storage(oracle.expert_project(Q4_K, packed["wout"], experts, hidden, inter,
+                                                      oracle.expert_silu_mul(up, inter, code), meta), code)
+    sup = oracle.round_storage(oracle.project(Q4_K, packed["sin"], 2 * inter, hidden, xr), code)
+    sdown = oracle.round_storage(oracle.project(Q4_K, packed["sout"], hidden, inter,
+                                                oracle.expert_silu_mul(sup, inter, code)), code)
+    want = oracle.expert_combine_shared(down, meta, tokens, hidden, top_k, sdown, gate_values, dtype=code)
+    for result in (got, separate):
+        assert rel_l2(result.to_f32(), want) <= 3e-3
+    assert np.abs(want).max() > 1e-3
 
 
 # ------------------------------------------------- the hybrid engine's router and combine

@@ -121,6 +121,7 @@ SYMBOLS = {
     "fh_hybrid_moe_route": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP, _VP]),
     "fh_hybrid_project": (_I32, [_P, _P, _VP, _U32, _VP, _U32]),
     "fh_hybrid_project_id": (_I32, [_P, _P, _VP, _VP, _U32, _U32, _VP]),
+    "fh_hybrid_project_id_with_shared": (_I32, [_P, _P, _P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_map": (_I32, [_P, _VP, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_gather": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_hybrid_project_mm_id": (_I32, [_P, _P, _VP, _VP, _U32, _VP]),
@@ -721,6 +722,30 @@ class Device:
         _check(_lib.fh_hybrid_project_id(self._handle, _handle_of(weight), ctypes.byref(xv), ctypes.byref(iv), routes,
                                          x_div, ctypes.byref(yv)))
         return y
+
+    def hybrid_project_id_with_shared(self, weight: "QuantizedExpertMatrix", shared_weight: "QuantizedMatrix",
+                                      x: Tensor, ids: Tensor, routes: int, x_div: int, tokens: int,
+                                      shared_x: Tensor | None = None):
+        """``hybrid_project_id`` and, in the same launch, the shared expert's projection of every
+        token with the dense ``shared_weight``: from ``shared_x`` [tokens, K] when given (the down
+        projection), else from the token rows ``x`` (gate, up).  Returns (y [routes, N],
+        shared_y [tokens, N])."""
+        if (routes == 0 or x_div == 0 or routes % x_div or ids.shape() != (routes,) or ids.dtype != DType.F32
+                or x.shape() != (routes // x_div, weight.columns()) or tokens == 0
+                or (shared_x is None and tokens != routes // x_div)
+                or (shared_x is not None and (shared_x.shape() != (tokens, weight.columns())
+                                              or shared_x.dtype != x.dtype))
+                or shared_weight.rows() != weight.rows_per_expert() or shared_weight.columns() != weight.columns()
+                or shared_weight.format().ggml_type() != weight.format().ggml_type()):
+            raise ShapeError("expert projection geometry")
+        y = Tensor.zeros(self, (routes, weight.rows_per_expert()), x.dtype)
+        ys = Tensor.zeros(self, (tokens, weight.rows_per_expert()), x.dtype)
+        xv, iv, yv, ysv = x._view(), ids._view(), y._view(), ys._view()
+        sxv = shared_x._view() if shared_x is not None else None
+        _check(_lib.fh_hybrid_project_id_with_shared(
+            self._handle, _handle_of(weight), _handle_of(shared_weight), ctypes.byref(xv), ctypes.byref(iv), routes,
+            x_div, tokens, ctypes.byref(sxv) if sxv is not None else None, ctypes.byref(yv), ctypes.byref(ysv)))
+        return y, ys
 
     def hybrid_moe_map(self, ids: Tensor, experts: int):
         """h_moe_map (hybrid.metal:2321-2358): (offsets [experts + 1], sorted [routes], position

@@ -746,8 +746,19 @@ fh_status fh_hybrid_project(fh_device* device, const fh_qmatrix* weight, const f
     return FH_OK;
 }
 
-fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
-                               uint32_t routes, uint32_t x_div, const fh_view* y) {
+namespace {
+
+// A shared expert (dense [rows, k] matrix every token also runs) can ride in a routed
+// launch: tokens entries more, reading the token rows or rows of its own (x), writing y.
+struct SharedExpert {
+    const fh_qmatrix* weight = nullptr;
+    uint32_t tokens = 0;
+    const fh_view* x = nullptr;
+    const fh_view* y = nullptr;
+};
+
+fh_status hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
+                            uint32_t routes, uint32_t x_div, const fh_view* y, const SharedExpert* shared) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device || routes == 0 || x_div == 0 || routes % x_div != 0 || ids == nullptr ||
         ids->dtype != FH_F32)
@@ -763,6 +774,33 @@ fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, cons
     st = resolve(device, y, (uint64_t)routes * rows, "expert output", &yr);
     if (st != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(ir, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    Range sxr{nullptr, 0}, syr{nullptr, 0};
+    if (shared != nullptr) {
+        const fh_qmatrix* sw = shared->weight;
+        if (sw == nullptr || shared->y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+        if (sw->device != device) {
+            g_last_error = "weight belongs to another device";
+            return FH_ERR_DEVICE_MISMATCH;
+        }
+        if (sw->experts != 1 || sw->rows != rows || sw->cols != k || sw->ggml_type != weight->ggml_type)
+            return fail(FH_ERR_SHAPE, "the shared expert's matrix must have one expert's shape and format");
+        // without rows of its own the shared expert reads the token rows of x, one per x_div routes
+        if (shared->tokens == 0 || (shared->x == nullptr && shared->tokens != routes / x_div) ||
+            !fits_u32((uint64_t)routes + shared->tokens) || !fits_u32((uint64_t)shared->tokens * rows) ||
+            !fits_u32((uint64_t)shared->tokens * k))
+            return fail(FH_ERR_SHAPE, "the shared expert runs once per token");
+        if (shared->y->dtype != y->dtype || (shared->x != nullptr && shared->x->dtype != x->dtype))
+            return fail(FH_ERR_DTYPE, "the shared expert's tensors differ in dtype from the routed ones");
+        st = resolve(device, shared->y, (uint64_t)shared->tokens * rows, "shared expert output", &syr);
+        if (st != FH_OK) return st;
+        if (shared->x != nullptr) {
+            st = resolve(device, shared->x, (uint64_t)shared->tokens * k, "shared expert input", &sxr);
+            if (st != FH_OK) return st;
+            if (overlaps(sxr, syr) || overlaps(sxr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+        }
+        if (overlaps(xr, syr) || overlaps(ir, syr) || overlaps(yr, syr))
+            return fail(FH_ERR_RANGE, "shared expert output aliases another tensor");
+    }
     GemvArgs a{};
     a.ggml_type = weight->ggml_type;
     a.w = weight->ptr;
@@ -779,6 +817,13 @@ fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, cons
     a.x_mode = kXDivide;
     a.x_div = x_div;
     a.x_rows = routes / x_div;
+    if (shared != nullptr) {
+        a.m = routes + shared->tokens;
+        a.shared_w = shared->weight->ptr;
+        a.shared_rows = shared->tokens;
+        a.shared_x = sxr.begin;
+        a.shared_y = const_cast<uint8_t*>(syr.begin);
+    }
     st = prepare_gemv(device, a);
     if (st != FH_OK) return st;
     launch_gemv(device->stream, a);
@@ -789,6 +834,26 @@ fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, cons
                                                            : "h_mv_id_iq4_xs";
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
+                               uint32_t routes, uint32_t x_div, const fh_view* y) {
+    return hybrid_project_id(device, weight, x, ids, routes, x_div, y, nullptr);
+}
+
+fh_status fh_hybrid_project_id_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                           const fh_qmatrix* shared_weight, const fh_view* x, const fh_view* ids,
+                                           uint32_t routes, uint32_t x_div, uint32_t tokens, const fh_view* shared_x,
+                                           const fh_view* y, const fh_view* shared_y) {
+    if (shared_weight == nullptr || shared_y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    SharedExpert shared;
+    shared.weight = shared_weight;
+    shared.tokens = tokens;
+    shared.x = shared_x;
+    shared.y = shared_y;
+    return hybrid_project_id(device, weight, x, ids, routes, x_div, y, &shared);
 }
 
 fh_status fh_hybrid_moe_map(fh_device* device, const fh_view* ids, uint32_t experts, uint32_t routes,
@@ -936,15 +1001,6 @@ fh_status fh_expert_assign(fh_device* device, const fh_view* hidden, uint32_t to
 }
 
 namespace {
-
-// A shared expert (dense [rows, k] matrix every token also runs) can ride in the launch:
-// tokens entries more, reading x (gather form) or shared_x (SiLU form), writing shared_y.
-struct SharedExpert {
-    const fh_qmatrix* weight = nullptr;
-    uint32_t tokens = 0;
-    const fh_view* x = nullptr;
-    const fh_view* y = nullptr;
-};
 
 fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t x_rows,
                          uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y,

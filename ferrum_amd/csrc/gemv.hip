@@ -315,8 +315,9 @@ struct Params {
     uint32_t x_div;
     // Batch entries from `routed` on belong to a shared expert that every token also runs:
     // entry routed + t multiplies token t's row with the dense matrix w_shared [n, k] into
-    // row t of y_shared.  Its input is row t of x (kXGather: x holds the token rows) or of
-    // x_shared (kXSiluMul: the shared expert's own packed gate|up rows).
+    // row t of y_shared.  Its input is row t of x_shared when that is set (the shared
+    // expert's own rows: packed gate|up for kXSiluMul, activated rows otherwise), else row
+    // t of x (x holds the token rows: kXGather, kXDivide).
     uint32_t routed;
     const uint8_t* w_shared;
     const void* x_shared;
@@ -342,7 +343,7 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     bool live = true;
     const bool shared = m >= p.routed;             // uniform over the workgroup
     const uint8_t* wmat = shared ? p.w_shared : p.w;
-    const void* xmat = shared && p.x_mode == kXSiluMul ? p.x_shared : p.x;
+    const void* xmat = shared && p.x_shared != nullptr ? p.x_shared : p.x;
     void* ymat = shared ? p.y_shared : p.y;
     const uint32_t ym = shared ? m - p.routed : m;  // row of y this entry writes
     if (p.metadata != nullptr && !shared) {

@@ -129,7 +129,7 @@ struct GemvArgs {
     uint32_t x_div;       // kXDivide: batch entries per row of x (0 = 1)
     // A shared expert riding in the same launch: the last shared_rows of the m batch entries
     // are tokens 0 .. shared_rows - 1 on the dense matrix shared_w [n, k], writing shared_y
-    // [shared_rows, n]; they read x (kXGather) or shared_x (kXSiluMul).  Null = none.
+    // [shared_rows, n]; they read row t of shared_x when set, else row t of x.  Null = none.
     const void* shared_w;
     uint32_t shared_rows;
     const void* shared_x;

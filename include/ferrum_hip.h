@@ -277,6 +277,21 @@ fh_status fh_hybrid_project(fh_device* device, const fh_qmatrix* weight, const f
                             const fh_view* y, uint32_t exact);
 fh_status fh_hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
                                uint32_t routes, uint32_t x_div, const fh_view* y);
+/* fh_hybrid_project_id with the shared expert's projection in the same launch.
+ * moe_ffn runs the shared expert as a dense FFN of three more per-row
+ * projections right after routing (engine.rs:2925); in its identity branch
+ * (a few routes) each is a launch of a few microseconds.  Here the shared
+ * expert's `tokens` rows are further entries of the per-route kernel on the
+ * dense matrix shared_weight (one expert's rows, columns and format): entry t
+ * reads row t of shared_x [tokens, K] when that is given (the down projection:
+ * the shared expert's own activated rows) and row t of x otherwise (gate and
+ * up: x holds one row per token, tokens == routes / x_div), and writes row t
+ * of shared_y [tokens, rows].  y and shared_y are bit for bit what
+ * fh_hybrid_project_id and a one-row-at-a-time fh_hybrid_project write. */
+fh_status fh_hybrid_project_id_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                           const fh_qmatrix* shared_weight, const fh_view* x, const fh_view* ids,
+                                           uint32_t routes, uint32_t x_div, uint32_t tokens, const fh_view* shared_x,
+                                           const fh_view* y, const fh_view* shared_y);
 fh_status fh_hybrid_moe_map(fh_device* device, const fh_view* ids, uint32_t experts, uint32_t routes,
                             const fh_view* offsets, const fh_view* sorted, const fh_view* position);
 fh_status fh_hybrid_moe_gather(fh_device* device, const fh_view* x, const fh_view* sorted, uint32_t hidden,

@@ -471,6 +471,25 @@ public:
         check(fh_hybrid_project_id(handle_->raw, w.matrix().raw(), &xv, &iv, (uint32_t)routes, (uint32_t)x_div, &yv));
         return y;
     }
+    // project_id with the shared expert's projection in the same launch: its `tokens` rows read
+    // shared_x [tokens, K] when given (down), else the token rows x (gate, up).
+    // Returns {y [routes, N], shared_y [tokens, N]}.
+    std::pair<Tensor, Tensor> hybrid_project_id_with_shared(const QuantizedExpertMatrix& w, const QuantizedMatrix& shared_w,
+                                                            const Tensor& x, const Tensor& ids, size_t routes,
+                                                            size_t x_div, size_t tokens,
+                                                            const Tensor* shared_x = nullptr) const {
+        if (routes == 0 || x_div == 0 || routes % x_div != 0 || ids.numel() != routes || tokens == 0 ||
+            (!shared_x && tokens != routes / x_div) || shared_w.rows() != w.rows_per_expert() ||
+            shared_w.columns() != w.columns() || shared_w.format() != w.format())
+            throw Error(ErrorKind::Shape, "expert projection geometry");
+        Tensor y = zeros({routes, w.rows_per_expert()}, x.dtype());
+        Tensor ys = zeros({tokens, w.rows_per_expert()}, x.dtype());
+        fh_view xv = x.c_view(), iv = ids.c_view(), yv = y.c_view(), ysv = ys.c_view(), sxv{};
+        if (shared_x) sxv = shared_x->c_view();
+        check(fh_hybrid_project_id_with_shared(handle_->raw, w.matrix().raw(), shared_w.raw(), &xv, &iv, (uint32_t)routes,
+                                               (uint32_t)x_div, (uint32_t)tokens, shared_x ? &sxv : nullptr, &yv, &ysv));
+        return {y, ys};
+    }
     struct HybridMap {
         Tensor offsets, sorted, position;
     };

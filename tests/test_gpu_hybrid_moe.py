@@ -101,6 +101,37 @@ def test_project_id_multiplies_each_route_by_its_expert(api, d, ggml):
         d.hybrid_project_id(w, api.Tensor.from_f32(d, (2, cols), api.DType.F32, x[:2]), carrier(api, d, ids[:5]), 5, 2)
 
 
+@pytest.mark.parametrize("ggml", [Q4_K, IQ4_XS])
+def test_project_id_carries_the_shared_expert(api, d, ggml):
+    # moe_ffn's identity branch with its shared expert (src/hybrid/engine.rs:2925): the shared
+    # rows ride in the routed launches and equal the separate one-row projections bit for bit
+    experts, rows, cols, used, tokens = 4, 24, 512, 3, 2
+    fmt = api.QuantizationFormat(ggml)
+    w = api.QuantizedExpertMatrix.new(d, synth.matrix(ggml, experts * rows, cols, seed=421), fmt, experts, rows, cols)
+    sw = api.QuantizedMatrix.from_bytes(d, rows, cols, fmt, synth.matrix(ggml, rows, cols, seed=422))
+    ids = carrier(api, d, np.array([2, 0, 3, 1, 9, 0], dtype=np.uint32))   # 9 is not an expert: a zero row
+    routes = tokens * used
+    f32 = api.DType.F32
+    x = api.Tensor.from_f32(d, (tokens, cols), f32, synth.activations(tokens, cols, seed=423))
+    # gate / up: every route of a token and the shared expert read the token's row
+    y, ys = d.hybrid_project_id_with_shared(w, sw, x, ids, routes, used, tokens)
+    assert d.last_operation().startswith("h_mv_id_")
+    assert np.array_equal(bits(y.to_f32()), bits(d.hybrid_project_id(w, x, ids, routes, used).to_f32()))
+    assert np.array_equal(bits(ys.to_f32()), bits(d.hybrid_project(sw, x, exact=True).tensor.to_f32()))
+    assert np.abs(ys.to_f32()).max() > 1e-3 and not y.to_f32()[4].any()
+    # down: a row per route, and the shared expert's own rows
+    act = api.Tensor.from_f32(d, (routes, cols), f32, synth.activations(routes, cols, seed=424))
+    shared_act = api.Tensor.from_f32(d, (tokens, cols), f32, synth.activations(tokens, cols, seed=425))
+    y, ys = d.hybrid_project_id_with_shared(w, sw, act, ids, routes, 1, tokens, shared_x=shared_act)
+    assert np.array_equal(bits(y.to_f32()), bits(d.hybrid_project_id(w, act, ids, routes, 1).to_f32()))
+    assert np.array_equal(bits(ys.to_f32()), bits(d.hybrid_project(sw, shared_act, exact=True).tensor.to_f32()))
+    with pytest.raises(api.ShapeError):   # without rows of its own the shared expert runs once per token row of x
+        d.hybrid_project_id_with_shared(w, sw, act, ids, routes, 1, tokens)
+    other = api.QuantizedMatrix.from_bytes(d, rows + 8, cols, fmt, synth.matrix(ggml, rows + 8, cols, seed=426))
+    with pytest.raises(api.ShapeError):
+        d.hybrid_project_id_with_shared(w, other, x, ids, routes, used, tokens)
+
+
 def test_prompt_chain_map_gather_mm_id_combine_matches_the_decode_chain_and_the_oracle(api, d):
     # HybridModel::moe_ffn's two branches (src/hybrid/engine.rs:3030-3075): per-route GEMVs with
     # `identity` rows, or map -> gather -> expert GEMM over sorted rows -> combine through position

@@ -868,7 +868,7 @@ class Device:
         launch, the shared expert's dense projection of every token: ``form="gather"`` reads
         both from ``input`` [tokens, K]; ``form="silu_mul"`` reads the routed rows from
         ``input`` [A, 2K] and the shared ones from ``shared_input`` [tokens, 2K].  Returns
-        (routed [A, N], shared [tokens, N]).  For decode-sized batches."""
+        (routed [A, N], shared [tokens, N])."""
         code = {"gather": 1, "silu_mul": 2}[form]
         x, meta, k = input.shape(), metadata.shape(), weight.columns()
         if (len(x) != 2 or len(meta) != 2 or meta[1] != 3 or meta[0] == 0 or tokens == 0
@@ -1022,8 +1022,9 @@ class SparseMoe:
     def _forward_with_shared(self, hidden, metadata, shared_gate, ws):
         d, k, tokens = self.device, self.routing.top_k, hidden.shape()[0]
         a = tokens * k
-        if self.fuse_inputs and self._shared_rides and a <= self.fused_max_assignments:
-            # decode: four launches, the shared expert's rows are batch entries of the routed ones
+        if self.fuse_inputs and self._shared_rides and (a <= self.fused_max_assignments or hidden.dtype != DType.F32):
+            # four launches: the shared expert's rows are batch entries of the routed ones in
+            # decode and further token groups of the grouped kernel beyond it
             projected, shared_projected = d.expert_project_with_shared(
                 hidden, metadata, self.input_experts, self.shared_input, tokens, "gather",
                 out=ws.get("projected"), shared_out=ws.get("shared_projected"))

@@ -1063,8 +1063,40 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     const int64_t f32_rows = tuning(device, "gemm_f32_min_rows");
     const bool f32_grouped = form == FH_INPUT_ROWS && x->dtype == FH_F32 && f32_rows > 0 &&
                              assignments >= (uint64_t)f32_rows && ((uintptr_t)xr.begin & 15u) == 0;
-    if (shared == nullptr && (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
-        assignments >= (uint64_t)grouped_min && weight->experts <= 1024 && (rows * dtype_bytes(y->dtype)) % 4 == 0) {
+    const bool grouped = (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
+                         assignments >= (uint64_t)grouped_min && weight->experts <= 1024 &&
+                         (rows * dtype_bytes(y->dtype)) % 4 == 0;
+    if (grouped && shared != nullptr &&
+        !expert_rows_fit_lds((uint32_t)k, assignments, (uint32_t)weight->experts)) {
+        // a shared expert rides in the grouped form only in the kernel that keeps rows in LDS;
+        // with rows too wide for it the two run apart, as the separate calls would
+        st = expert_project(device, weight, x, x_rows, form, assignments, metadata, y, nullptr);
+        if (st != FH_OK) return st;
+        if (form == FH_INPUT_GATHER) return project(device, shared->weight, x, shared->tokens, shared->y, false);
+        if (shared->tokens < (uint64_t)tuning(device, "gemm_min_rows") || ((uintptr_t)sxr.begin & 15u) != 0)
+            return project(device, shared->weight, shared->x, shared->tokens, shared->y, true);
+        st = ensure_scratch(device, (size_t)shared->tokens * k * sizeof(uint16_t));
+        if (st != FH_OK) return st;
+        launch_expert_silu_mul(device->stream, sxr.begin, scratch_data(device), shared->tokens, (uint32_t)k, x->dtype,
+                               x->dtype);
+        GemmArgs g{};
+        g.ggml_type = weight->ggml_type;
+        g.w = shared->weight->ptr;
+        g.x = scratch_data(device);
+        g.y = const_cast<uint8_t*>(syr.begin);
+        g.n = (uint32_t)rows;
+        g.k = (uint32_t)k;
+        g.m = shared->tokens;
+        g.x_dtype = x->dtype;
+        g.y_dtype = y->dtype;
+        g.cu_count = device->props.multiProcessorCount;
+        g.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
+        g.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
+        device->last_operation = launch_gemm(device->stream, g);
+        FH_HIP(hipGetLastError());
+        return FH_OK;
+    }
+    if (grouped) {
         // grouped form: every expert's weights are streamed once for all of its assignments.
         // The kernel that keeps an expert's rows in LDS gathers them from the token rows
         // itself; where they do not fit, and for the SiLU form, the rows are written out
@@ -1073,12 +1105,15 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
                              expert_rows_fit_lds((uint32_t)k, assignments, (uint32_t)weight->experts);
         const bool staged = f32_grouped || (form != FH_INPUT_ROWS && !gathers);
         const size_t words = ((size_t)weight->experts + 1 + assignments + 3) & ~(size_t)3;
-        const size_t staged_bytes = staged ? (size_t)assignments * k * sizeof(uint16_t) : 0;
+        // the SiLU form stages the shared expert's rows behind the routed ones
+        const size_t staged_rows = (size_t)assignments + (shared != nullptr && form == FH_INPUT_SILU_MUL ? shared->tokens : 0);
+        const size_t staged_bytes = staged ? staged_rows * k * sizeof(uint16_t) : 0;
         st = ensure_scratch(device, words * sizeof(uint32_t) + staged_bytes);
         if (st != FH_OK) return st;
         uint32_t* offsets = reinterpret_cast<uint32_t*>(scratch_data(device));
         uint32_t* order = offsets + weight->experts + 1;
         const void* tile_x = xr.begin;
+        uint8_t* shared_rows_x = nullptr;  // the shared expert's own rows, when it does not read the token rows
         if (staged) {
             uint8_t* rows_x = scratch_data(device) + words * sizeof(uint32_t);
             if (f32_grouped) {
@@ -1090,6 +1125,11 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
             } else {
                 launch_expert_silu_mul(device->stream, xr.begin, rows_x, assignments, (uint32_t)k, x->dtype,
                                        x->dtype);
+                if (shared != nullptr) {
+                    shared_rows_x = rows_x + (size_t)assignments * k * sizeof(uint16_t);
+                    launch_expert_silu_mul(device->stream, sxr.begin, shared_rows_x, shared->tokens, (uint32_t)k,
+                                           x->dtype, x->dtype);
+                }
             }
             tile_x = rows_x;
         }
@@ -1112,6 +1152,13 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.expert_order = order;
         g.gather_metadata = gathers ? reinterpret_cast<const float*>(mr.begin) : nullptr;
         g.x_rows = x_rows;
+        if (shared != nullptr) {
+            g.shared_w = shared->weight->ptr;
+            g.shared_rows = shared->tokens;
+            // gathered form: the token rows themselves, in place or as staged for the routed rows' gather
+            g.shared_x = form == FH_INPUT_GATHER ? xr.begin : shared_rows_x;
+            g.shared_y = const_cast<uint8_t*>(syr.begin);
+        }
         device->last_operation = launch_gemm_skinny(device->stream, g);
         FH_HIP(hipGetLastError());
         return FH_OK;

@@ -430,6 +430,21 @@ constexpr int kResRing = 6;
 constexpr int kResWaves = 8;                    // two waves per SIMD hide each other's decode and MFMA waits
 constexpr int kResThreads = 64 * kResWaves;
 
+// A shared expert in the same launch: every token also runs the dense matrix w [n, k];
+// token t reads row t of x (null: row t of the routed x, which then holds token rows) and
+// writes row t of y.  Its work is cut into pieces of 16*TT consecutive tokens times
+// tiles_per_slice row tiles, `slices` of them per token group, and the workgroups share the
+// pieces out after their own expert, so the grid and its one round of workgroups stay as
+// they are.
+struct ResidentShared {
+    const uint8_t* w;
+    const uint16_t* x;
+    void* y;
+    uint32_t tokens;
+    uint32_t slices;
+    uint32_t tiles_per_slice;
+};
+
 template <uint32_t TYPE, int DT, int TT>
 __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint8_t* __restrict__ w,
                                                                      const uint16_t* __restrict__ x,
@@ -439,7 +454,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                                                                      const uint32_t* __restrict__ order,
                                                                      uint32_t tiles_per_wg,
                                                                      const float* __restrict__ metadata,
-                                                                     uint32_t x_rows) {
+                                                                     uint32_t x_rows, const ResidentShared sh) {
     constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
     constexpr int kTokens = 16 * TT;
     extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
@@ -447,18 +462,38 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t r = lane & 15u, g = lane >> 4;
     const uint32_t k = nb * 256, ld = k + 8;
-    const uint32_t first_token = offsets[blockIdx.y];
-    const uint32_t count = offsets[blockIdx.y + 1] - first_token;
+    const uint32_t expert_first = offsets[blockIdx.y];
+    const uint32_t count = offsets[blockIdx.y + 1] - expert_first;
     const uint32_t tiles = (n + 15) / 16;
-    const uint32_t tile_begin = blockIdx.x * tiles_per_wg + wave;
-    const uint32_t tile_end = min(tiles, (blockIdx.x + 1) * tiles_per_wg);
-    const uint8_t* wexpert = w + (size_t)blockIdx.y * n * nb * kBB;
     const uint32_t pieces = k / 8;  // 16-byte pieces per activation row
 
-    for (uint32_t t0 = 0; t0 < count; t0 += kTokens) {
-        const uint32_t mt = min((uint32_t)kTokens, count - t0);
-        if (t0 != 0) __syncthreads();  // the previous pass is done with the rows
-        // gather the expert's rows, eight 16-byte pieces per thread in flight at a time
+    // work items of this workgroup: its expert's tokens, 16*TT at a time, then its part of
+    // the shared expert's pieces
+    const uint32_t passes = (count + kTokens - 1) / kTokens;
+    const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, wgs = gridDim.x * gridDim.y;
+    const uint32_t shared_pieces = sh.w != nullptr ? (sh.tokens + kTokens - 1) / kTokens * sh.slices : 0;
+    const uint32_t my_pieces = shared_pieces > wg ? (shared_pieces - wg + wgs - 1) / wgs : 0;
+    for (uint32_t item = 0; item < passes + my_pieces; ++item) {
+        const bool shared = item >= passes;  // uniform over the workgroup
+        uint32_t first_token, mt, tile_begin, tile_end;
+        if (!shared) {
+            first_token = expert_first + item * kTokens;
+            mt = min((uint32_t)kTokens, count - item * kTokens);
+            tile_begin = blockIdx.x * tiles_per_wg + wave;
+            tile_end = min(tiles, (blockIdx.x + 1) * tiles_per_wg);
+        } else {
+            const uint32_t piece = wg + (item - passes) * wgs;
+            const uint32_t group = piece / sh.slices, slice = piece - group * sh.slices;
+            first_token = group * kTokens;
+            mt = min((uint32_t)kTokens, sh.tokens - first_token);
+            tile_begin = slice * sh.tiles_per_slice + wave;
+            tile_end = min(tiles, (slice + 1) * sh.tiles_per_slice);
+        }
+        const uint8_t* wexpert = shared ? sh.w : w + (size_t)blockIdx.y * n * nb * kBB;
+        const uint16_t* xsrc = shared && sh.x != nullptr ? sh.x : x;
+        void* ydst = shared ? sh.y : y;
+        if (item != 0) __syncthreads();  // the previous item is done with the rows
+        // gather the rows, eight 16-byte pieces per thread in flight at a time
         const uint32_t total = mt * pieces;
         for (uint32_t base = 0; base < total; base += 8 * kResThreads) {
             u32x4 v[8];
@@ -468,19 +503,22 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                 const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
                 const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
                 dst[j] = tok * ld + 8 * pc;
-                const uint32_t slot = first_token + t0 + tok;
-                uint32_t row = order != nullptr ? order[slot] : slot;
-                if (metadata != nullptr) {
-                    const uint32_t token = __float_as_uint(metadata[3 * (size_t)row + 1]);
-                    row = token < x_rows ? token : x_rows - 1;
+                const uint32_t slot = first_token + tok;
+                uint32_t row = slot;  // a shared group's slots are its tokens
+                if (!shared) {
+                    row = order != nullptr ? order[slot] : slot;
+                    if (metadata != nullptr) {
+                        const uint32_t token = __float_as_uint(metadata[3 * (size_t)row + 1]);
+                        row = token < x_rows ? token : x_rows - 1;
+                    }
                 }
-                v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)row * k + 8 * pc);
+                v[j] = *reinterpret_cast<const u32x4*>(xsrc + (size_t)row * k + 8 * pc);
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
         }
         __syncthreads();
-        if (tile_begin >= tile_end) continue;  // uniform per wave; no barrier follows in this pass
+        if (tile_begin >= tile_end) continue;  // uniform per wave; no barrier follows in this item
 
         // B operand rows: token 16t + r, clamped (columns past mt are never stored)
         uint32_t boff[TT];
@@ -489,7 +527,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
         for (int t = 0; t < TT; ++t) {
             const uint32_t tok = min(16u * t + r, mt - 1);
             boff[t] = tok * ld;
-            out_token[t] = order != nullptr ? order[first_token + t0 + tok] : first_token + t0 + tok;
+            out_token[t] = order != nullptr && !shared ? order[first_token + tok] : first_token + tok;
         }
         uint32_t kl[8];
 #pragma unroll
@@ -542,7 +580,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                     if (16u * t + r < mt) {
                         const size_t base = (size_t)out_token[t] * n + out_row;
                         if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
-                            *reinterpret_cast<float4*>(static_cast<float*>(y) + base) =
+                            *reinterpret_cast<float4*>(static_cast<float*>(ydst) + base) =
                                 make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
                         } else if (y_dtype != FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
                             uint2 packed;
@@ -553,11 +591,11 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                                 packed.x = f32_to_bf16_bits(acc[t][0]) | (f32_to_bf16_bits(acc[t][1]) << 16);
                                 packed.y = f32_to_bf16_bits(acc[t][2]) | (f32_to_bf16_bits(acc[t][3]) << 16);
                             }
-                            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + base) = packed;
+                            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(ydst) + base) = packed;
                         } else {
 #pragma unroll
                             for (int v = 0; v < 4; ++v)
-                                if (out_row + v < n) store_from_f32(y, base + v, y_dtype, acc[t][v]);
+                                if (out_row + v < n) store_from_f32(ydst, base + v, y_dtype, acc[t][v]);
                         }
                     }
                     acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
@@ -599,18 +637,31 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
             uint32_t tiles_per_wg = (tiles + shares - 1) / shares;
             tiles_per_wg = (tiles_per_wg + kResWaves - 1) / kResWaves * kResWaves;
             const dim3 rgrid((tiles + tiles_per_wg - 1) / tiles_per_wg, a.experts);
+            ResidentShared sh{};
+            if (a.shared_w != nullptr) {
+                sh.w = static_cast<const uint8_t*>(a.shared_w);
+                sh.x = static_cast<const uint16_t*>(a.shared_x);
+                sh.y = a.shared_y;
+                sh.tokens = a.shared_rows;
+                // about one piece per workgroup: a token group's rows are cut into as many slices
+                const uint32_t per_group = wide ? 32u : 16u;
+                const uint32_t groups = (a.shared_rows + per_group - 1) / per_group;
+                const uint32_t want = (rgrid.x * rgrid.y + groups - 1) / groups;
+                sh.tiles_per_slice = (tiles + want - 1) / want;
+                sh.slices = (tiles + sh.tiles_per_slice - 1) / sh.tiles_per_slice;
+            }
             if (wide) {
                 auto kernel = expert_resident_kernel<TYPE, DT, 2>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, sh);
             } else {
                 auto kernel = expert_resident_kernel<TYPE, DT, 1>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, sh);
             }
             return;
         }

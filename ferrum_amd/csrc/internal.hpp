@@ -166,6 +166,13 @@ struct GemmArgs {
     // gather_metadata[3a + 1], as expert_assign would have copied it
     const float* gather_metadata;
     uint32_t x_rows;
+    // that kernel can carry a shared expert: tokens 0 .. shared_rows - 1 on the dense matrix
+    // shared_w [n, k], reading row t of shared_x (null: row t of x, which then holds token
+    // rows) and writing row t of shared_y
+    const void* shared_w;
+    uint32_t shared_rows;
+    const void* shared_x;
+    void* shared_y;
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

@@ -689,8 +689,9 @@ public:
         Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
         if (shared_input_) {
             const size_t tokens = dims[0], a = tokens * routing_.top_k;
-            if (fuse_inputs && shared_rides_ && a <= fused_max_assignments) {
-                // decode: four launches, the shared expert's rows are batch entries of the routed ones
+            if (fuse_inputs && shared_rides_ && (a <= fused_max_assignments || hidden.dtype() != DType::F32)) {
+                // four launches: the shared expert's rows are batch entries of the routed ones in
+                // decode and further token groups of the grouped kernel beyond it
                 auto up = device_.expert_project_with_shared(hidden, meta, input_, *shared_input_, tokens, FH_INPUT_GATHER);
                 auto down = device_.expert_project_with_shared(up.first, meta, output_, *shared_output_, tokens,
                                                                FH_INPUT_SILU_MUL, &up.second);

@@ -450,7 +450,7 @@ def _shared_case(api, d, dtype, tokens, seed):
          "sin": api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, packed["sin"]),
          "sout": api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, packed["sout"])}
     dt = getattr(api.DType, dtype)
-    x = synth.activations(tokens, hidden, seed=seed + 4, f16=True) * np.float32(2.0 ** -4)
+    x = synth.activations(tokens, hidden, seed=seed + 4, f16=True) * np.float32(2.0 ** -6)
     logits = synth.rng(seed + 5).standard_normal((tokens, experts)).astype(np.float32)
     xt = api.Tensor.from_f32(d, x.shape, dt, x)
     lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
@@ -507,9 +507,10 @@ def test_shared_expert_projection_rejects_what_it_cannot_run(api, d):
     assert call(1, ov, sv) == 0
 
 
-@pytest.mark.parametrize("tokens,gated", [(1, False), (3, True), (40, True)])
+@pytest.mark.parametrize("tokens,gated", [(1, False), (3, True), (20, False), (300, True)])
 def test_sparse_moe_with_a_shared_expert(api, d, tokens, gated):
-    # one and three tokens: the shared expert rides in the routed launches; 40: separate dense calls
+    # one and three tokens: the shared expert's rows are batch entries of the per-assignment
+    # launches; 20 and 300: token groups (of 16, then of 32) of the grouped kernel
     (experts, hidden, inter, top_k), packed, w, x, logits, xt, lt = _shared_case(api, d, "F16", tokens, 191)
     moe = api.SparseMoe(d, w["win"], w["wout"], api.MoeRoutingPolicy(experts, top_k),
                         shared_input=w["sin"], shared_output=w["sout"])
@@ -535,9 +536,32 @@ def test_sparse_moe_with_a_shared_expert(api, d, tokens, gated):
     sdown = oracle.round_storage(oracle.project(Q4_K, packed["sout"], hidden, inter,
                                                 oracle.expert_silu_mul(sup, inter, code)), code)
     want = oracle.expert_combine_shared(down, meta, tokens, hidden, top_k, sdown, gate_values, dtype=code)
+    assert np.isfinite(want).all() and np.abs(want).max() > 1e-3
     for result in (got, separate):
         assert rel_l2(result.to_f32(), want) <= 3e-3
-    assert np.abs(want).max() > 1e-3
+
+
+def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
+    # 32 rows of 2560 halves are more than the grouped kernel's LDS: the routed rows are staged and
+    # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit
+    experts, hidden, inter, top_k, tokens = 4, 2560, 2560, 2, 40
+    fmt = api.QuantizationFormat(Q4_K)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=85), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * hidden, inter, seed=86), fmt,
+                                         experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, synth.matrix(Q4_K, 2 * inter, hidden, seed=89))
+    sout = api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, synth.matrix(Q4_K, hidden, inter, seed=90))
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k), shared_input=sin, shared_output=sout)
+    x = synth.activations(tokens, hidden, seed=87, f16=True) * np.float32(2.0 ** -5)
+    logits = synth.rng(88).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    riding = moe.forward(xt, lt)
+    moe.fuse_inputs = False
+    apart = moe.forward(xt, lt)
+    assert np.array_equal(riding.raw(), apart.raw())
+    assert np.abs(riding.to_f32()).max() > 1e-3
 
 
 # ------------------------------------------------- the hybrid engine's router and combine

@@ -346,7 +346,7 @@ fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* wei
  * fh_expert_project_fused groups the assignments by expert (16-bit rows,
  * 32 assignments or more), the shared expert's tokens join the grouped
  * kernel as further groups of 16 or 32 tokens on the dense matrix (512
- * tokens: 41 us of dense tile GEMMs become +19 us in the two grouped
+ * tokens: 41 us of dense tile GEMMs become +23 us in the two grouped
  * launches); results then agree with the separate calls to the matmul
  * tolerance, not bitwise.  Rows too wide for that kernel's LDS run as the
  * separate calls. */

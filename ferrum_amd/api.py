@@ -125,6 +125,7 @@ SYMBOLS = {
     "fh_hybrid_moe_map": (_I32, [_P, _VP, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_gather": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_hybrid_project_mm_id": (_I32, [_P, _P, _VP, _VP, _U32, _VP]),
+    "fh_hybrid_project_mm_id_with_shared": (_I32, [_P, _P, _P, _VP, _VP, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_combine": (_I32, [_P, _VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32, _VP]),
     "fh_expert_assign": (_I32, [_P, _VP, _U32, _U32, _VP, _U32, _VP]),
     "fh_expert_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP, _VP]),
@@ -784,6 +785,24 @@ class Device:
         _check(_lib.fh_hybrid_project_mm_id(self._handle, _handle_of(weight), ctypes.byref(xv), ctypes.byref(fv),
                                             dims[0], ctypes.byref(yv)))
         return y
+
+    def hybrid_project_mm_id_with_shared(self, weight: "QuantizedExpertMatrix", shared_weight: "QuantizedMatrix",
+                                         x: Tensor, offsets: Tensor, shared_x: Tensor):
+        """``hybrid_project_mm_id`` and, in the same launch, the shared expert's dense projection of
+        ``shared_x`` [tokens, K].  Returns (y [routes, N], shared_y [tokens, N])."""
+        dims, sd = x.shape(), shared_x.shape()
+        if (len(dims) != 2 or dims[0] == 0 or dims[1] != weight.columns() or offsets.shape() != (weight.experts() + 1,)
+                or len(sd) != 2 or sd[0] == 0 or sd[1] != dims[1] or shared_x.dtype != x.dtype
+                or shared_weight.rows() != weight.rows_per_expert() or shared_weight.columns() != weight.columns()
+                or shared_weight.format().ggml_type() != weight.format().ggml_type()):
+            raise ShapeError("expert projection geometry")
+        y = Tensor.zeros(self, (dims[0], weight.rows_per_expert()), x.dtype)
+        ys = Tensor.zeros(self, (sd[0], weight.rows_per_expert()), x.dtype)
+        xv, fv, sxv, yv, ysv = x._view(), offsets._view(), shared_x._view(), y._view(), ys._view()
+        _check(_lib.fh_hybrid_project_mm_id_with_shared(
+            self._handle, _handle_of(weight), _handle_of(shared_weight), ctypes.byref(xv), ctypes.byref(fv), dims[0],
+            sd[0], ctypes.byref(sxv), ctypes.byref(yv), ctypes.byref(ysv)))
+        return y, ys
 
     def hybrid_moe_combine(self, down: Tensor, weights: Tensor, position: Tensor | None, shared: Tensor,
                            shared_gate: Tensor, used: int) -> Tensor:

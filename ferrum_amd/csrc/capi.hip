@@ -897,8 +897,11 @@ fh_status fh_hybrid_moe_gather(fh_device* device, const fh_view* x, const fh_vie
     return FH_OK;
 }
 
-fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
-                                  const fh_view* offsets, uint32_t routes, const fh_view* y) {
+namespace {
+
+fh_status hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                               const fh_view* offsets, uint32_t routes, const fh_view* y,
+                               const SharedExpert* shared) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device || routes == 0 || weight->experts > 1024 || offsets == nullptr ||
         offsets->dtype != FH_F32 || x == nullptr || y == nullptr)
@@ -913,14 +916,47 @@ fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, c
     if ((st = resolve(device, offsets, weight->experts + 1, "expert offsets", &fr, 4)) != FH_OK) return st;
     if ((st = resolve(device, y, (uint64_t)routes * rows, "expert output", &yr)) != FH_OK) return st;
     if (overlaps(xr, yr) || overlaps(fr, yr)) return fail(FH_ERR_RANGE, "expert output aliases an input");
+    Range sxr{nullptr, 0}, syr{nullptr, 0};
+    if (shared != nullptr) {
+        const fh_qmatrix* sw = shared->weight;
+        if (sw == nullptr || shared->x == nullptr || shared->y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+        if (sw->device != device) {
+            g_last_error = "weight belongs to another device";
+            return FH_ERR_DEVICE_MISMATCH;
+        }
+        if (sw->experts != 1 || sw->rows != rows || sw->cols != k || sw->ggml_type != weight->ggml_type)
+            return fail(FH_ERR_SHAPE, "the shared expert's matrix must have one expert's shape and format");
+        if (shared->tokens == 0 || !fits_u32((uint64_t)shared->tokens * rows) || !fits_u32((uint64_t)shared->tokens * k))
+            return fail(FH_ERR_SHAPE, "the shared expert runs once per token");
+        if (shared->y->dtype != y->dtype || shared->x->dtype != x->dtype)
+            return fail(FH_ERR_DTYPE, "the shared expert's tensors differ in dtype from the routed ones");
+        if ((st = resolve(device, shared->x, (uint64_t)shared->tokens * k, "shared expert input", &sxr)) != FH_OK) return st;
+        if ((st = resolve(device, shared->y, (uint64_t)shared->tokens * rows, "shared expert output", &syr)) != FH_OK)
+            return st;
+        if (overlaps(sxr, syr) || overlaps(sxr, yr) || overlaps(xr, syr) || overlaps(fr, syr) || overlaps(yr, syr))
+            return fail(FH_ERR_RANGE, "shared expert output aliases another tensor");
+        if (!expert_rows_fit_lds((uint32_t)k, routes, (uint32_t)weight->experts)) {
+            // rows too wide for the kernel that carries the shared expert: the two run apart
+            st = hybrid_project_mm_id(device, weight, x, offsets, routes, y, nullptr);
+            if (st != FH_OK) return st;
+            return project(device, shared->weight, shared->x, shared->tokens, shared->y, false, 5);
+        }
+    }
     // the tiles are f16 / bf16, as the reference's h_mm_id kernels make theirs; f32 rows are rounded to f16 first
     const void* tile_x = xr.begin;
+    const void* shared_tile_x = sxr.begin;
     if (x->dtype == FH_F32) {
-        st = ensure_scratch(device, (size_t)routes * k * sizeof(uint16_t));
+        const size_t shared_elements = shared != nullptr ? (size_t)shared->tokens * k : 0;
+        st = ensure_scratch(device, ((size_t)routes * k + shared_elements) * sizeof(uint16_t));
         if (st != FH_OK) return st;
         uint16_t* x16 = reinterpret_cast<uint16_t*>(scratch_data(device));
         launch_round_to_f16(device->stream, reinterpret_cast<const float*>(xr.begin), x16, (size_t)routes * k);
         tile_x = x16;
+        if (shared != nullptr) {
+            launch_round_to_f16(device->stream, reinterpret_cast<const float*>(sxr.begin), x16 + (size_t)routes * k,
+                                shared_elements);
+            shared_tile_x = x16 + (size_t)routes * k;
+        }
     }
     GemmArgs g{};
     g.ggml_type = weight->ggml_type;
@@ -936,6 +972,12 @@ fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, c
     g.experts = (uint32_t)weight->experts;
     g.expert_offsets = reinterpret_cast<const uint32_t*>(fr.begin);
     g.expert_order = nullptr;   // rows are already expert-sorted
+    if (shared != nullptr) {
+        g.shared_w = shared->weight->ptr;
+        g.shared_rows = shared->tokens;
+        g.shared_x = shared_tile_x;
+        g.shared_y = const_cast<uint8_t*>(syr.begin);
+    }
     launch_gemm_skinny(device->stream, g);
     device->last_operation = weight->ggml_type == kQ4K     ? "h_mm_id_q4_k"
                              : weight->ggml_type == kQ5K   ? "h_mm_id_q5_k"
@@ -944,6 +986,27 @@ fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, c
                                                            : "h_mm_id_iq4_xs";
     FH_HIP(hipGetLastError());
     return FH_OK;
+}
+
+}  // namespace
+
+fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                  const fh_view* offsets, uint32_t routes, const fh_view* y) {
+    return hybrid_project_mm_id(device, weight, x, offsets, routes, y, nullptr);
+}
+
+fh_status fh_hybrid_project_mm_id_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                              const fh_qmatrix* shared_weight, const fh_view* x,
+                                              const fh_view* offsets, uint32_t routes, uint32_t tokens,
+                                              const fh_view* shared_x, const fh_view* y, const fh_view* shared_y) {
+    if (shared_weight == nullptr || shared_x == nullptr || shared_y == nullptr)
+        return fail(FH_ERR_PARAMETER, "null argument");
+    SharedExpert shared;
+    shared.weight = shared_weight;
+    shared.tokens = tokens;
+    shared.x = shared_x;
+    shared.y = shared_y;
+    return hybrid_project_mm_id(device, weight, x, offsets, routes, y, &shared);
 }
 
 fh_status fh_hybrid_moe_combine(fh_device* device, const fh_view* down, const fh_view* weights,

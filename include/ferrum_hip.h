@@ -298,6 +298,19 @@ fh_status fh_hybrid_moe_gather(fh_device* device, const fh_view* x, const fh_vie
                                uint32_t used, uint32_t routes, const fh_view* out);
 fh_status fh_hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
                                   const fh_view* offsets, uint32_t routes, const fh_view* y);
+/* fh_hybrid_project_mm_id with the shared expert's projection in the same
+ * launch: moe_ffn's prompt branch runs the shared expert's dense FFN
+ * (engine.rs:2925) as three more tile GEMMs next to the three project_mm_id
+ * calls.  Here row t of shared_x [tokens, K] is multiplied by the dense
+ * shared_weight (one expert's rows, columns and format) into row t of
+ * shared_y [tokens, rows] by the workgroups of the routed kernel, after their
+ * own expert's rows; f32 rows are rounded to f16 like the routed ones.  Same
+ * results as fh_hybrid_project_mm_id plus fh_hybrid_project to the matmul
+ * tolerance; rows too wide for the kernel's LDS run as those two calls. */
+fh_status fh_hybrid_project_mm_id_with_shared(fh_device* device, const fh_qmatrix* weight,
+                                              const fh_qmatrix* shared_weight, const fh_view* x,
+                                              const fh_view* offsets, uint32_t routes, uint32_t tokens,
+                                              const fh_view* shared_x, const fh_view* y, const fh_view* shared_y);
 fh_status fh_hybrid_moe_combine(fh_device* device, const fh_view* down, const fh_view* weights,
                                 const fh_view* position, const fh_view* shared, const fh_view* shared_gate,
                                 uint32_t hidden, uint32_t used, uint32_t tokens, const fh_view* out);

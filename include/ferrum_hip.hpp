@@ -521,6 +521,24 @@ public:
         check(fh_hybrid_project_mm_id(handle_->raw, w.matrix().raw(), &xv, &fv, (uint32_t)dims[0], &yv));
         return y;
     }
+    // project_mm_id with the shared expert's dense projection of shared_x [tokens, K] in the same launch.
+    // Returns {y [routes, N], shared_y [tokens, N]}.
+    std::pair<Tensor, Tensor> hybrid_project_mm_id_with_shared(const QuantizedExpertMatrix& w, const QuantizedMatrix& shared_w,
+                                                               const Tensor& x, const Tensor& offsets,
+                                                               const Tensor& shared_x) const {
+        const auto& dims = x.shape();
+        const auto& sd = shared_x.shape();
+        if (dims.size() != 2 || dims[0] == 0 || dims[1] != w.columns() || offsets.numel() != w.experts() + 1 ||
+            sd.size() != 2 || sd[0] == 0 || sd[1] != dims[1] || shared_x.dtype() != x.dtype() ||
+            shared_w.rows() != w.rows_per_expert() || shared_w.columns() != w.columns() || shared_w.format() != w.format())
+            throw Error(ErrorKind::Shape, "expert projection geometry");
+        Tensor y = zeros({dims[0], w.rows_per_expert()}, x.dtype());
+        Tensor ys = zeros({sd[0], w.rows_per_expert()}, x.dtype());
+        fh_view xv = x.c_view(), fv = offsets.c_view(), sxv = shared_x.c_view(), yv = y.c_view(), ysv = ys.c_view();
+        check(fh_hybrid_project_mm_id_with_shared(handle_->raw, w.matrix().raw(), shared_w.raw(), &xv, &fv, (uint32_t)dims[0],
+                                                  (uint32_t)sd[0], &sxv, &yv, &ysv));
+        return {y, ys};
+    }
     // h_moe_combine (f32): weighted sum of each token's routed rows through `position` (or the routes
     // themselves when null) plus shared_gate[t] * shared[t]
     Tensor hybrid_moe_combine(const Tensor& down, const Tensor& weights, const Tensor* position, const Tensor& shared,

@@ -132,6 +132,39 @@ def test_project_id_carries_the_shared_expert(api, d, ggml):
         d.hybrid_project_id_with_shared(w, other, x, ids, routes, used, tokens)
 
 
+@pytest.mark.parametrize("dtype,tokens", [("F32", 24), ("F16", 100), ("F32", 7)])
+def test_project_mm_id_carries_the_shared_expert(api, d, dtype, tokens):
+    # the prompt branch with its shared expert (src/hybrid/engine.rs:2925): routed rows are those of
+    # project_mm_id bit for bit, shared rows are the dense projection of f16-rounded rows
+    experts, used, rows, cols = 16, 4, 96, 512
+    fmt = api.QuantizationFormat(Q4_K)
+    packed_shared = synth.matrix(Q4_K, rows, cols, seed=432)
+    w = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * rows, cols, seed=431), fmt, experts, rows, cols)
+    sw = api.QuantizedMatrix.from_bytes(d, rows, cols, fmt, packed_shared)
+    dt = getattr(api.DType, dtype)
+    rng = synth.rng(433, tokens)
+    routes = tokens * used
+    ids = rng.integers(0, experts, routes).astype(np.uint32)
+    offsets, order, _ = d.hybrid_moe_map(carrier(api, d, ids), experts)
+    x = (rng.standard_normal((tokens, cols)) * 2.0 ** -3).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+    xg = d.hybrid_moe_gather(xt, order, used) if dtype == "F32" else \
+        api.Tensor.from_f32(d, (routes, cols), dt, x[u32(order) // used])
+    y, ys = d.hybrid_project_mm_id_with_shared(w, sw, xg, offsets, xt)
+    assert d.last_operation() == "h_mm_id_q4_k"
+    assert np.array_equal(y.raw(), d.hybrid_project_mm_id(w, xg, offsets).raw())
+    want = oracle.project(Q4_K, packed_shared, rows, cols, oracle.round_storage(x, oracle.F16), accumulate="f64",
+                          weight_round=oracle.F16)
+    got = ys.to_f32()
+    if dtype == "F32":
+        assert_matmul_parity(got, want, "shared rows")
+    else:   # the output itself is stored in f16
+        assert_matmul_parity(got, want, "shared rows", max_rel_tol=2e-3, l2_tol=1e-3)
+    with pytest.raises(api.ShapeError):
+        other = api.QuantizedMatrix.from_bytes(d, rows, 2 * cols, fmt, synth.matrix(Q4_K, rows, 2 * cols, seed=434))
+        d.hybrid_project_mm_id_with_shared(w, other, xg, offsets, xt)
+
+
 def test_prompt_chain_map_gather_mm_id_combine_matches_the_decode_chain_and_the_oracle(api, d):
     # HybridModel::moe_ffn's two branches (src/hybrid/engine.rs:3030-3075): per-route GEMVs with
     # `identity` rows, or map -> gather -> expert GEMM over sorted rows -> combine through position

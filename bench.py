@@ -235,7 +235,7 @@ def moe_case(api, synth, dev, tokens, steps):
     return {
         "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
         "operation": ("moe_route + 2 x (expert_project with the shared expert riding) + combine" if tokens * top_k <= 31
-                      else "moe_route + 2 x expert_project (grouped) + silu_mul + shared FFN + combine"),
+                      else "moe_route + 2 x (expert_project grouped, shared expert pieces inside) + 2 x silu_mul + combine"),
         "us": round(best * 1e6, 2),
         "GB/s": round(nbytes / best / 1e9, 1),
         "frac_hbm": round(nbytes / best / 1e9 / HBM_PEAK_GBS, 4),

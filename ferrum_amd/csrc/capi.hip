@@ -184,6 +184,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
+    d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
@@ -248,6 +249,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
     } else if (k == "gemm_min_rows") {
         ok = value >= 2;
+    } else if (k == "gemm_resident") {
+        ok = value == 0 || value == 1;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {
@@ -533,6 +536,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.cu_count = device->props.multiProcessorCount;
         a.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
         a.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
+        a.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, a);
     } else {
         GemvArgs a{};
@@ -1155,6 +1159,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.cu_count = device->props.multiProcessorCount;
         g.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
         g.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
+        g.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, g);
         FH_HIP(hipGetLastError());
         return FH_OK;

@@ -462,8 +462,9 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t r = lane & 15u, g = lane >> 4;
     const uint32_t k = nb * 256, ld = k + 8;
-    const uint32_t expert_first = offsets[blockIdx.y];
-    const uint32_t count = offsets[blockIdx.y + 1] - expert_first;
+    // no offsets: a dense product, all of it shared-expert pieces
+    const uint32_t expert_first = offsets != nullptr ? offsets[blockIdx.y] : 0;
+    const uint32_t count = offsets != nullptr ? offsets[blockIdx.y + 1] - expert_first : 0;
     const uint32_t tiles = (n + 15) / 16;
     const uint32_t pieces = k / 8;  // 16-byte pieces per activation row
 
@@ -623,6 +624,40 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
     const uint32_t nb = a.k / 256;
+    if (a.rows_resident && a.expert_offsets == nullptr && a.m > (uint32_t)a.skinny_max_rows) {
+        // dense product with the activation rows resident in LDS: (32-row group, row-tile slice)
+        // pieces, about one per compute unit
+        const bool wide = a.m > 16 && (size_t)32 * (a.k + 8) * 2 <= 150u * 1024;
+        const uint32_t per_group = wide ? 32u : 16u;
+        const size_t lds = (size_t)per_group * (a.k + 8) * 2;
+        const uint32_t tiles = (a.n + 15) / 16;
+        const uint32_t cus = a.cu_count > 0 ? (uint32_t)a.cu_count : 256u;
+        const uint32_t groups = (a.m + per_group - 1) / per_group;
+        const uint32_t want = (cus + groups - 1) / groups;
+        ResidentShared sh{};
+        sh.w = w;
+        sh.x = nullptr;
+        sh.y = a.y;
+        sh.tokens = a.m;
+        sh.tiles_per_slice = (tiles + want - 1) / want;
+        sh.slices = (tiles + sh.tiles_per_slice - 1) / sh.tiles_per_slice;
+        const uint32_t pieces = groups * sh.slices;
+        const dim3 rgrid(pieces < cus ? pieces : cus, 1);
+        if (wide) {
+            auto kernel = expert_resident_kernel<TYPE, DT, 2>;
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, nullptr, x, nullptr, a.n, nb, a.y_dtype,
+                               nullptr, nullptr, 0u, nullptr, 0u, sh);
+        } else {
+            auto kernel = expert_resident_kernel<TYPE, DT, 1>;
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, nullptr, x, nullptr, a.n, nb, a.y_dtype,
+                               nullptr, nullptr, 0u, nullptr, 0u, sh);
+        }
+        return;
+    }
     if (a.expert_offsets != nullptr) {
         const bool wide = a.m > 8 * a.experts;   // mean tokens per expert > 8: 32 tokens a pass
         const size_t lds = (size_t)(wide ? 32 : 16) * (a.k + 8) * 2;
@@ -698,6 +733,18 @@ bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts) {
 
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
     const bool grouped = a.expert_offsets != nullptr;
+    if (!grouped && a.rows_resident && a.m > (uint32_t)a.skinny_max_rows) {
+        static const char* const names[5] = {"q4_k_gemm_mfma_resident", "q5_k_gemm_mfma_resident",
+                                             "q6_k_gemm_mfma_resident", "iq4_xs_gemm_mfma_resident",
+                                             "q8_0_gemm_mfma_resident"};
+        const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : a.ggml_type == kQ6K ? 2 : a.ggml_type == kIQ4XS ? 3 : 4;
+#define FH_RES(TYPE) \
+    if (a.x_dtype == FH_F16) launch_tt<TYPE, 1>(s, a); else launch_tt<TYPE, 2>(s, a)
+        if (f == 0) { FH_RES(kQ4K); } else if (f == 1) { FH_RES(kQ5K); } else if (f == 2) { FH_RES(kQ6K); }
+        else if (f == 3) { FH_RES(kIQ4XS); } else { FH_RES(kQ8_0); }
+#undef FH_RES
+        return names[f];
+    }
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) launch_tt<kQ4K, 1>(s, a); else launch_tt<kQ4K, 2>(s, a);
         return grouped ? "expert_project_q4_k_grouped_mfma" : "q4_k_gemm_mfma_skinny";

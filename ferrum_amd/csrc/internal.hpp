@@ -173,6 +173,8 @@ struct GemmArgs {
     uint32_t shared_rows;
     const void* shared_x;
     void* shared_y;
+    // dense product through that kernel: the activation rows stay in LDS for the whole K
+    bool rows_resident;
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

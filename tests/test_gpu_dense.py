@@ -206,7 +206,11 @@ def test_tile_gemm_both_tile_sizes_match_the_f16_tile_oracle(api, d, ggml, dtype
     for n in (16000, 1000):
         packed = synth.matrix(ggml, n, k, seed=92 + n)
         w = qm(api, d, ggml, n, k, packed)
-        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        d.set_tuning("gemm_resident", 0)   # rows this short would otherwise stay in LDS (tested below)
+        try:
+            out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        finally:
+            d.set_tuning("gemm_resident", 1)
         assert out.operation == ("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
         got = out.tensor.to_f32()
         rows = np.unique(np.concatenate([np.arange(0, 130), np.arange(n - 70, n),
@@ -521,7 +525,11 @@ def test_q5_k_tile_kernels_match_the_rounded_weight_oracle(api, d, m, n, dtype_n
     packed = synth.matrix(Q5_K, n, k, seed=201 + n)
     w = qm(api, d, Q5_K, n, k, packed)
     x = oracle.round_storage(synth.activations(m, k, seed=202), code).reshape(m, k)
-    out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    d.set_tuning("gemm_resident", 0)       # the square tiles, which rows longer than LDS still take
+    try:
+        out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_resident", 1)
     want_name = {8: "q5_k_gemm_mfma_skinny", 20: "q5_k_gemm_mfma_skinny", 130: "q5_k_gemm_mfma",
                  300: "q5_k_gemm_mfma_m256"}[m]
     assert out.operation == want_name
@@ -558,3 +566,38 @@ def test_q5_k_expert_projection_and_validation(api, d):
         api.QuantizedMatrix.from_bytes(d, experts * rows, cols, api.QuantizationFormat(Q5_K), bad)
     with pytest.raises(api.Error):
         api.QuantizedMatrix.from_bytes(d, experts * rows, cols, api.QuantizationFormat(Q5_K), packed[:-1])
+
+
+IQ4_XS, Q8_0 = 23, 8
+
+
+# Rows that fit LDS for their whole length (K <= 2392 for groups of 32 rows, K <= 4792 for groups
+# of 16) and more than 64 of them: the kernel that keeps a group of rows resident and streams the
+# weights past them.  Ragged row groups, ragged row tiles, more pieces than compute units, both
+# group sizes, every format, both 16-bit dtypes.
+@pytest.mark.parametrize("ggml,m,n,k,dtype_name", [
+    (Q4_K, 70, 1000, 768, "F16"), (Q4_K, 200, 50, 4096, "BF16"), (Q4_K, 2000, 1000, 256, "F16"),
+    (Q5_K, 130, 1000, 512, "BF16"), (Q6_K, 97, 530, 1024, "F16"), (Q6_K, 65, 40, 2560, "F16"),
+    (IQ4_XS, 300, 300, 512, "F16"), (Q8_0, 129, 260, 1280, "BF16")])
+def test_rows_resident_gemm_matches_the_rounded_weight_oracle(api, d, ggml, m, n, k, dtype_name):
+    dtype = api.DType[dtype_name]
+    code = oracle.F16 if dtype_name == "F16" else oracle.BF16
+    packed = synth.matrix(ggml, n, k, seed=301 + n + m)
+    w = qm(api, d, ggml, n, k, packed)
+    x = oracle.round_storage(synth.activations(m, k, seed=302 + m), code).reshape(m, k)
+    xt = api.Tensor.from_f32(d, x.shape, dtype, x)
+    out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    assert out.operation.endswith("_gemm_mfma_resident")
+    rows = np.unique(np.concatenate([np.arange(0, min(n, 48)), np.arange(max(0, n - 40), n),
+                                     synth.rng(303).integers(0, n, 32)]))
+    want = oracle_columns(ggml, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+    got = out.tensor.to_f32()
+    assert_matmul_parity(got[:, rows], want, f"rows-resident m={m} n={n} k={k}")
+    # every row group and tile was written: the square tiles give the same product
+    d.set_tuning("gemm_resident", 0)
+    try:
+        tiles = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_resident", 1)
+    assert not tiles.operation.endswith("_resident")
+    assert rel_l2(got, tiles.tensor.to_f32()) <= 1e-5

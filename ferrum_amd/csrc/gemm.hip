@@ -861,10 +861,21 @@ void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
 }  // namespace
 
 const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
-    if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
     // the 256-row tile pays off only when its workgroups cover at least half the chip
     const uint64_t wide_wgs = (uint64_t)((a.m + kWM - 1) / kWM) * ((a.n + 127) / 128);
-    if (a.m >= (uint32_t)a.wide_min_rows && wide_wgs * 2 >= (uint64_t)a.cu_count) {
+    const bool wide_pays = a.m >= (uint32_t)a.wide_min_rows && wide_wgs * 2 >= (uint64_t)a.cu_count;
+    // Rows that fit LDS for their whole length take the kernel that keeps them there and streams
+    // the weights past them through registers.  Against the register-dequant kernel that stages
+    // the rows slab by slab (up to 64 rows) it is 15% faster at 2 - 16 rows and up to twice at 64
+    // (64 x 4096 x 4096: 14.1 against 29.7 us), except for 512-long rows in 16-row batches or
+    // less, where a launch is 4 us either way; against the square tiles 1.4 - 2.2 times
+    // (512 x 1024 x 2048: 11.5 against 22.8 us).  The 256-row tile keeps what it fills.
+    if (a.rows_resident) {
+        const bool few = a.m <= (uint32_t)a.skinny_max_rows;
+        if (few ? !(a.k <= 512 && a.m <= 16) : !wide_pays) return launch_gemm_resident(s, a);
+    }
+    if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
+    if (wide_pays) {
         const WidePlan plan = wide_plan(a.m, a.n, a.cu_count);
         if (a.ggml_type == kQ4K) {
             if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan); else launch_wide_nt<kQ4K, 2>(s, a, plan);
@@ -885,10 +896,6 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
         if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
         return "q6_k_gemm_mfma_m256";
     }
-    // Below that, rows that fit LDS for their whole length take the kernel that keeps them
-    // there and streams the weights past them through registers: 1.4 - 2.2 times the square
-    // tiles' rate on every such shape measured (512 x 1024 x 2048: 11.5 against 22.8 us).
-    if (a.rows_resident) return launch_gemm_skinny(s, a);
     // 128 x 128 tiles, or 64 x 64 when those would leave most of the chip idle
     const uint64_t big_wgs = (uint64_t)((a.n + kBN - 1) / kBN) * ((a.m + kBM - 1) / kBM);
     const bool small = big_wgs * 2 < (uint64_t)a.cu_count;

@@ -624,7 +624,7 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
     const uint32_t nb = a.k / 256;
-    if (a.rows_resident && a.expert_offsets == nullptr && a.m > (uint32_t)a.skinny_max_rows) {
+    if (a.use_resident) {
         // dense product with the activation rows resident in LDS: (32-row group, row-tile slice)
         // pieces, about one per compute unit
         const bool wide = a.m > 16 && (size_t)32 * (a.k + 8) * 2 <= 150u * 1024;
@@ -731,9 +731,11 @@ bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts) {
     return (size_t)(m > 8 * experts ? 32 : 16) * (k + 8) * 2 <= 150u * 1024;
 }
 
-const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
-    const bool grouped = a.expert_offsets != nullptr;
-    if (!grouped && a.rows_resident && a.m > (uint32_t)a.skinny_max_rows) {
+const char* launch_gemm_resident(hipStream_t s, const GemmArgs& dense) {
+    GemmArgs a = dense;
+    a.use_resident = true;
+    a.expert_offsets = nullptr;
+    {
         static const char* const names[5] = {"q4_k_gemm_mfma_resident", "q5_k_gemm_mfma_resident",
                                              "q6_k_gemm_mfma_resident", "iq4_xs_gemm_mfma_resident",
                                              "q8_0_gemm_mfma_resident"};
@@ -745,6 +747,10 @@ const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
 #undef FH_RES
         return names[f];
     }
+}
+
+const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a) {
+    const bool grouped = a.expert_offsets != nullptr;
     if (a.ggml_type == kQ4K) {
         if (a.x_dtype == FH_F16) launch_tt<kQ4K, 1>(s, a); else launch_tt<kQ4K, 2>(s, a);
         return grouped ? "expert_project_q4_k_grouped_mfma" : "q4_k_gemm_mfma_skinny";

@@ -173,13 +173,17 @@ struct GemmArgs {
     uint32_t shared_rows;
     const void* shared_x;
     void* shared_y;
-    // dense product through that kernel: the activation rows stay in LDS for the whole K
+    // dense product: the rows are short enough to stay in LDS for the whole K (launch_gemm
+    // then weighs launch_gemm_resident against the other kernels)
     bool rows_resident;
+    bool use_resident;    // set by launch_gemm_resident only
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 
 // gemm_skinny.hip
 const char* launch_gemm_skinny(hipStream_t s, const GemmArgs& a);
+// dense [m, k] x [n, k]^T with 16 or 32 rows at a time resident in LDS; needs expert_rows_fit_lds(k, 1, 1)
+const char* launch_gemm_resident(hipStream_t s, const GemmArgs& a);
 // whether the routed form keeps an expert's activation rows of width k in LDS,
 // which is the kernel that takes the gathered input form
 bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts);

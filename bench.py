@@ -334,6 +334,9 @@ def main():
             dev.set_tuning("gemm_f32_min_rows", 5)   # the hybrid engine's tiering: f16 tiles from 5 rows on
             timed(Q4_K, 17408, 5120, 512, f32, "Q4_K GEMM M=512 K=5120 N=17408 f32 x (rounded to f16 for the tiles)", 120)
             dev.set_tuning("gemm_f32_min_rows", 0)
+        # rows short enough to stay in LDS (an A3B-sized model's attention projections)
+        for m in (8, 64, 512):
+            timed(Q4_K, 4096, 2048, m, f16, f"Q4_K GEMM M={m} K=2048 N=4096 f16 x", 400)
         if not args.only or args.only in "MoE FFN T=1":
             cases.append(moe_case(api, synth, dev, 1, 200))
         if not args.only or args.only in "MoE FFN T=512":

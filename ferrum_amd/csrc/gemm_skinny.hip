@@ -419,13 +419,14 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
 // further barrier: wave w takes row tiles w, w+4, ... of the workgroup's share
 // and walks (tile, super-block) units through a register ring, so the prefetch
 // runs across tile boundaries.  blockIdx.y = expert, blockIdx.x = which share
-// of the expert's rows.  Dynamic LDS: 16*TT rows of (K + 8) halfs.
+// of the expert's rows.  Dynamic LDS: 16*TT rows of K halfs.
 //
 // The rows are [A, K] rows or, with metadata given, the row of the assignment's
 // token in [tokens, K]: expert_assign folded into the gather.  (SiLU * up is not
 // folded in: it is bound by its exponentials and divisions, and one workgroup
 // per compute unit doing them ahead of its first MFMA costs more than the
 // launch that spreads them over the whole chip: +11 us against -5 us.)
+constexpr size_t kResLdsBytes = 160u * 1024;   // a workgroup may take all of a compute unit's LDS
 constexpr int kResRing = 6;
 constexpr int kResWaves = 8;                    // two waves per SIMD hide each other's decode and MFMA waits
 constexpr int kResThreads = 64 * kResWaves;
@@ -461,7 +462,10 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t r = lane & 15u, g = lane >> 4;
-    const uint32_t k = nb * 256, ld = k + 8;
+    // Rows are not padded: 16 rows of 5120 halves are all of LDS.  The 16-byte piece p of row t
+    // sits at piece p ^ (t & 15) instead, so the sixteen rows a B-operand read touches at one k
+    // (and the sixteen consecutive pieces a gather write covers) fall on different banks.
+    const uint32_t k = nb * 256, ld = k;
     // no offsets: a dense product, all of it shared-expert pieces
     const uint32_t expert_first = offsets != nullptr ? offsets[blockIdx.y] : 0;
     const uint32_t count = offsets != nullptr ? offsets[blockIdx.y + 1] - expert_first : 0;
@@ -503,7 +507,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
             for (int j = 0; j < 8; ++j) {
                 const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
                 const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
-                dst[j] = tok * ld + 8 * pc;
+                dst[j] = tok * ld + 8 * (pc ^ (tok & 15u));
                 const uint32_t slot = first_token + tok;
                 uint32_t row = slot;  // a shared group's slots are its tokens
                 if (!shared) {
@@ -532,7 +536,7 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
         }
         uint32_t kl[8];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) kl[s] = Quarter<TYPE>::klocal(g, s);
+        for (int s = 0; s < 8; ++s) kl[s] = (((Quarter<TYPE>::klocal(g, s) >> 3) ^ r) << 3);  // row 16t + r: swizzle r
 
         // units = (tile, super-block) pairs of this wave, in order
         const uint32_t my_tiles = (tile_end - tile_begin + kResWaves - 1) / kResWaves;
@@ -627,9 +631,9 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     if (a.use_resident) {
         // dense product with the activation rows resident in LDS: (32-row group, row-tile slice)
         // pieces, about one per compute unit
-        const bool wide = a.m > 16 && (size_t)32 * (a.k + 8) * 2 <= 150u * 1024;
+        const bool wide = a.m > 16 && (size_t)32 * a.k * 2 <= kResLdsBytes;
         const uint32_t per_group = wide ? 32u : 16u;
-        const size_t lds = (size_t)per_group * (a.k + 8) * 2;
+        const size_t lds = (size_t)per_group * a.k * 2;
         const uint32_t tiles = (a.n + 15) / 16;
         const uint32_t cus = a.cu_count > 0 ? (uint32_t)a.cu_count : 256u;
         const uint32_t groups = (a.m + per_group - 1) / per_group;
@@ -660,7 +664,7 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
     }
     if (a.expert_offsets != nullptr) {
         const bool wide = a.m > 8 * a.experts;   // mean tokens per expert > 8: 32 tokens a pass
-        const size_t lds = (size_t)(wide ? 32 : 16) * (a.k + 8) * 2;
+        const size_t lds = (size_t)(wide ? 32 : 16) * a.k * 2;
         if (expert_rows_fit_lds(a.k, a.m, a.experts)) {
             // the expert's rows are cut into shares so that about one workgroup per compute unit
             // exists: every share gathers the expert's tokens again, and at 256 experts one share
@@ -728,7 +732,7 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
 
 bool expert_rows_fit_lds(uint32_t k, uint32_t m, uint32_t experts) {
     // more than 8 tokens per expert on average: 32 tokens a pass, else 16
-    return (size_t)(m > 8 * experts ? 32 : 16) * (k + 8) * 2 <= 150u * 1024;
+    return (size_t)(m > 8 * experts ? 32 : 16) * k * 2 <= kResLdsBytes;
 }
 
 const char* launch_gemm_resident(hipStream_t s, const GemmArgs& dense) {

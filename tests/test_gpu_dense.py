@@ -575,13 +575,13 @@ def test_q5_k_expert_projection_and_validation(api, d):
 IQ4_XS, Q8_0 = 23, 8
 
 
-# Rows that fit LDS for their whole length (K <= 2392 for groups of 32 rows, K <= 4792 for groups
+# Rows that fit LDS for their whole length (K <= 2560 for groups of 32 rows, K <= 5120 for groups
 # of 16), two rows or more: the kernel that keeps a group of rows resident and streams the
 # weights past them.  Ragged row groups, ragged row tiles, more pieces than compute units, both
 # group sizes, every format, both 16-bit dtypes.
 @pytest.mark.parametrize("ggml,m,n,k,dtype_name", [
     (Q4_K, 70, 1000, 768, "F16"), (Q4_K, 200, 50, 4096, "BF16"), (Q4_K, 2000, 1000, 256, "F16"),
-    (Q4_K, 2, 1000, 768, "F16"), (Q4_K, 16, 100, 4096, "BF16"), (Q6_K, 17, 530, 1024, "F16"), (Q5_K, 64, 1000, 512, "F16"),
+    (Q4_K, 40, 300, 5120, "F16"), (Q4_K, 2, 1000, 768, "F16"), (Q4_K, 16, 100, 4096, "BF16"), (Q6_K, 17, 530, 1024, "F16"), (Q5_K, 64, 1000, 512, "F16"),
     (Q5_K, 130, 1000, 512, "BF16"), (Q6_K, 97, 530, 1024, "F16"), (Q6_K, 65, 40, 2560, "F16"),
     (IQ4_XS, 300, 300, 512, "F16"), (Q8_0, 129, 260, 1280, "BF16")])
 def test_rows_resident_gemm_matches_the_rounded_weight_oracle(api, d, ggml, m, n, k, dtype_name):

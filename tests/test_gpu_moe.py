@@ -417,9 +417,9 @@ def test_sparse_moe_fused_inputs_match_the_separate_steps(api, d, tokens):
 
 @pytest.mark.parametrize("dtype", ["F16", "BF16"])
 def test_grouped_input_forms_when_an_experts_rows_do_not_fit_lds(api, d, dtype):
-    # 32 rows of 2560 halves are more than the kernel's LDS: the library writes the gathered
+    # 32 rows of 2816 halves are more than the kernel's LDS: the library writes the gathered
     # and the activated rows out itself and the result is still that of the separate steps
-    experts, hidden, inter, top_k, tokens = 4, 2560, 2560, 2, 40
+    experts, hidden, inter, top_k, tokens = 4, 2816, 2816, 2, 40
     fmt = api.QuantizationFormat(Q4_K)
     win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=85), fmt,
                                         experts, 2 * inter, hidden)
@@ -542,9 +542,9 @@ def test_sparse_moe_with_a_shared_expert(api, d, tokens, gated):
 
 
 def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
-    # 32 rows of 2560 halves are more than the grouped kernel's LDS: the routed rows are staged and
+    # 32 rows of 2816 halves are more than the grouped kernel's LDS: the routed rows are staged and
     # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit
-    experts, hidden, inter, top_k, tokens = 4, 2560, 2560, 2, 40
+    experts, hidden, inter, top_k, tokens = 4, 2816, 2816, 2, 40
     fmt = api.QuantizationFormat(Q4_K)
     win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=85), fmt,
                                         experts, 2 * inter, hidden)

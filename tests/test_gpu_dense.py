@@ -598,6 +598,10 @@ def test_rows_resident_gemm_matches_the_rounded_weight_oracle(api, d, ggml, m, n
     want = oracle_columns(ggml, packed, n, k, rows, x, weight_round=code, accumulate="f64")
     got = out.tensor.to_f32()
     assert_matmul_parity(got[:, rows], want, f"rows-resident m={m} n={n} k={k}")
+    # stored in the activation dtype (packed stores where rows allow, element stores on ragged ones)
+    stored = d.project_quantized(xt, w)
+    assert stored.operation == out.operation
+    assert np.array_equal(bits(stored.tensor.to_f32()), bits(oracle.round_storage(got, code).reshape(m, n)))
     # every row group and tile was written: the square tiles give the same product
     d.set_tuning("gemm_resident", 0)
     try:

@@ -870,15 +870,21 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     // (64 x 4096 x 4096: 14.1 against 29.7 us; 64 x 17408 x 5120: 52.8 against 74.0 us, the same
     // bits), except for 512-long rows in 16-row batches or
     // less, where a launch is 4 us either way; against the square tiles 1.4 - 2.2 times
-    // (512 x 1024 x 2048: 11.5 against 22.8 us).  The 256-row tile keeps what it fills.
+    // (512 x 1024 x 2048: 11.5 against 22.8 us).
     // Rows longer than 2560 fit only 16 at a time, and every weight is then decoded M / 16 times:
     // that still wins up to 256 rows (256 x 5120 x 5120: 51 against 86 us) and loses at 512 (95
     // against 84 us).
     if (a.rows_resident) {
         const bool few = a.m <= (uint32_t)a.skinny_max_rows;
         const bool groups_of_32 = (size_t)32 * a.k * 2 <= 160u * 1024;
-        if (few ? !(a.k <= 512 && a.m <= 16) : !wide_pays && (groups_of_32 || a.m <= 256))
-            return launch_gemm_resident(s, a);
+        // Where the 256-row tile would pay, it is mostly empty below 256 rows while this kernel's
+        // cost grows with the row count: 65 x 17408 x 5120 takes 67 against 82 us and 128 rows
+        // 87 against 87; with groups of 32 (K = 2048) 128 rows take 30 against 41 us and 256
+        // rows 49 against 49.
+        const bool take = few          ? !(a.k <= 512 && a.m <= 16)
+                          : wide_pays ? a.m <= (groups_of_32 ? 192u : 96u)
+                                      : groups_of_32 || a.m <= 256;
+        if (take) return launch_gemm_resident(s, a);
     }
     if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
     if (wide_pays) {

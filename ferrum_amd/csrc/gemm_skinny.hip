@@ -637,7 +637,8 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
         const uint32_t tiles = (a.n + 15) / 16;
         const uint32_t cus = a.cu_count > 0 ? (uint32_t)a.cu_count : 256u;
         const uint32_t groups = (a.m + per_group - 1) / per_group;
-        const uint32_t want = (cus + groups - 1) / groups;
+        // never a few pieces more than workgroups: those would make a second round
+        const uint32_t want = cus / groups > 0 ? cus / groups : 1;
         ResidentShared sh{};
         sh.w = w;
         sh.x = nullptr;
@@ -685,7 +686,7 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                 // about one piece per workgroup: a token group's rows are cut into as many slices
                 const uint32_t per_group = wide ? 32u : 16u;
                 const uint32_t groups = (a.shared_rows + per_group - 1) / per_group;
-                const uint32_t want = (rgrid.x * rgrid.y + groups - 1) / groups;
+                const uint32_t want = rgrid.x * rgrid.y / groups > 0 ? rgrid.x * rgrid.y / groups : 1;
                 sh.tiles_per_slice = (tiles + want - 1) / want;
                 sh.slices = (tiles + sh.tiles_per_slice - 1) / sh.tiles_per_slice;
             }

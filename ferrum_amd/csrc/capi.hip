@@ -1190,14 +1190,13 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
             } else if (form == FH_INPUT_GATHER) {
                 launch_expert_assign(device->stream, xr.begin, reinterpret_cast<const float*>(mr.begin), rows_x,
                                      assignments, (uint32_t)(k * sizeof(uint16_t)), x_rows);
+            } else if (shared != nullptr) {
+                shared_rows_x = rows_x + (size_t)assignments * k * sizeof(uint16_t);
+                launch_expert_silu_mul_pair(device->stream, xr.begin, sxr.begin, rows_x, assignments, shared->tokens,
+                                            (uint32_t)k, x->dtype);
             } else {
                 launch_expert_silu_mul(device->stream, xr.begin, rows_x, assignments, (uint32_t)k, x->dtype,
                                        x->dtype);
-                if (shared != nullptr) {
-                    shared_rows_x = rows_x + (size_t)assignments * k * sizeof(uint16_t);
-                    launch_expert_silu_mul(device->stream, sxr.begin, shared_rows_x, shared->tokens, (uint32_t)k,
-                                           x->dtype, x->dtype);
-                }
             }
             tile_x = rows_x;
         }

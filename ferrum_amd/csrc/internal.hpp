@@ -218,6 +218,8 @@ const char* launch_expert_assign(hipStream_t s, const void* hidden, const float*
                                  void* out, uint32_t assignments, uint32_t row_bytes, uint32_t tokens);
 const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uint32_t assignments,
                                    uint32_t intermediate, uint32_t in_dtype, uint32_t out_dtype);
+void launch_expert_silu_mul_pair(hipStream_t s, const void* in, const void* in2, void* out, uint32_t rows,
+                                 uint32_t rows2, uint32_t intermediate, uint32_t dtype);
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,
                                   uint32_t tokens, uint32_t hidden, uint32_t top_k,
                                   uint32_t in_dtype, uint32_t out_dtype, const void* shared,

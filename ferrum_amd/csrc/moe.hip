@@ -316,6 +316,32 @@ __global__ __launch_bounds__(256) void expert_silu_mul8_kernel(const void* __res
     }
 }
 
+// expert_silu_mul8_kernel over two inputs whose outputs follow one another: rows of `in`
+// first, then rows of `in2` (a shared expert's rows behind the routed ones), in one launch.
+__global__ __launch_bounds__(256) void expert_silu_mul8_pair_kernel(const void* __restrict__ in,
+                                                                    const void* __restrict__ in2,
+                                                                    void* __restrict__ out, uint32_t rows,
+                                                                    uint32_t rows2, uint32_t intermediate,
+                                                                    uint32_t dtype) {
+    const size_t total = (size_t)(rows + rows2) * intermediate / 8;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t a = (i * 8) / intermediate;
+        const size_t column = (i * 8) % intermediate;
+        const void* src = in;
+        if (a >= rows) {
+            a -= rows;
+            src = in2;
+        }
+        float gate[8], up[8], result[8];
+        load8(src, a * 2 * intermediate + column, dtype, gate);
+        load8(src, a * 2 * intermediate + intermediate + column, dtype, up);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) result[j] = round_storage(silu_stable(gate[j]), dtype) * up[j];
+        store8(out, i * 8, dtype, result);
+    }
+}
+
 // The dtypes are template parameters: with one token the kernel is a single short
 // dependent instruction stream, and every runtime dtype switch lengthens it.
 template <uint32_t in_dtype, uint32_t out_dtype>
@@ -638,6 +664,21 @@ const char* launch_expert_silu_mul(hipStream_t s, const void* in, void* out, uin
                            dim3(256), 0, s, in, out, assignments, intermediate, in_dtype, out_dtype);
     }
     return "expert_silu_mul";
+}
+
+// rows of `in` then rows2 of `in2`, [.., 2 * intermediate] each, into out [rows + rows2, intermediate]
+void launch_expert_silu_mul_pair(hipStream_t s, const void* in, const void* in2, void* out, uint32_t rows,
+                                 uint32_t rows2, uint32_t intermediate, uint32_t dtype) {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(in2) |
+                           reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    if (intermediate % 8 == 0 && aligned) {
+        hipLaunchKernelGGL(expert_silu_mul8_pair_kernel, dim3(grid_for((size_t)(rows + rows2) * intermediate / 8)),
+                           dim3(256), 0, s, in, in2, out, rows, rows2, intermediate, dtype);
+        return;
+    }
+    launch_expert_silu_mul(s, in, out, rows, intermediate, dtype, dtype);
+    launch_expert_silu_mul(s, in2, static_cast<uint8_t*>(out) + (size_t)rows * intermediate * 2, rows2, intermediate,
+                           dtype, dtype);
 }
 
 const char* launch_expert_combine(hipStream_t s, const void* in, const float* metadata, void* out,

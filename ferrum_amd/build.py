@@ -17,7 +17,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libferrum_hip.so")
 
-SOURCES = ["capi.hip", "dequant.hip", "gemv.hip", "gemm.hip", "gemm_skinny.hip", "moe.hip", "norm.hip"]
+SOURCES = ["capi.hip", "dequant.hip", "gemv.hip", "gemv_stream.hip", "gemm.hip", "gemm_skinny.hip", "moe.hip", "norm.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",
@@ -50,7 +50,7 @@ def _compile(src: str, extra: list[str]) -> str:
     return obj
 
 
-def build(extra_flags: list[str] | None = None, jobs: int = 5, output: str | None = None) -> str:
+def build(extra_flags: list[str] | None = None, jobs: int = 8, output: str | None = None) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     extra = list(extra_flags or [])

@@ -114,12 +114,21 @@ fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
 // Frees device memory now, or after the recording in progress has ended.
 void release_memory(fh_device* d, void* ptr) {
     if (ptr == nullptr) return;
+    if (d != nullptr && d->closed) {
+        (void)hipFree(ptr);   // synchronizes by itself; the stream no longer exists
+        return;
+    }
     if (d != nullptr && d->capturing) {
         d->deferred_frees.push_back(ptr);
         return;
     }
     if (d != nullptr) (void)hipStreamSynchronize(d->stream);
     (void)hipFree(ptr);
+}
+
+// One object created on the device is gone (or the caller's handle is); the last one frees it.
+void drop_device_handle(fh_device* d) {
+    if (d != nullptr && --d->handles == 0) delete d;
 }
 
 void drain_deferred(fh_device* d) {
@@ -185,6 +194,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
+    d->tuning["gemv_stream"] = 1;           // dense Q4_K rows that fit LDS take the streamed matrix-core GEMV (0 = the FMA kernel)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
@@ -199,13 +209,25 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
 void fh_device_destroy(fh_device* device) {
     if (device == nullptr) return;
     (void)hipSetDevice(device->ordinal);
+    if (device->closed) return;
+    // what was put off during a recording goes first, while the stream it waits on exists
+    if (device->capturing) {
+        hipGraph_t abandoned = nullptr;
+        (void)hipStreamEndCapture(device->stream, &abandoned);
+        if (abandoned) (void)hipGraphDestroy(abandoned);
+        device->capturing = false;
+    }
+    drain_deferred(device);
     if (device->stream) {
         (void)hipStreamSynchronize(device->stream);
         (void)hipStreamDestroy(device->stream);
+        device->stream = nullptr;
     }
-    drain_deferred(device);
     if (device->scratch) (void)hipFree(device->scratch);
-    delete device;
+    device->scratch = nullptr;
+    device->scratch_bytes = 0;
+    device->closed = true;
+    drop_device_handle(device);
 }
 
 fh_status fh_device_properties(const fh_device* device, fh_device_props* out) {
@@ -249,7 +271,7 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
     } else if (k == "gemm_min_rows") {
         ok = value >= 2;
-    } else if (k == "gemm_resident") {
+    } else if (k == "gemm_resident" || k == "gemv_stream") {
         ok = value == 0 || value == 1;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
@@ -296,6 +318,7 @@ fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out) {
         return fail(FH_ERR_ALLOCATION, "out of host memory");
     }
     b->device = device;
+    ++device->handles;
     b->ptr = p;
     b->bytes = bytes;
     *out = b;
@@ -305,6 +328,7 @@ fh_status fh_buffer_alloc(fh_device* device, size_t bytes, fh_buffer** out) {
 void fh_buffer_free(fh_buffer* buffer) {
     if (buffer == nullptr) return;
     release_memory(buffer->device, buffer->ptr);
+    drop_device_handle(buffer->device);
     delete buffer;
 }
 
@@ -314,6 +338,7 @@ void* fh_buffer_device_ptr(fh_buffer* buffer) { return buffer ? buffer->ptr : nu
 fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, size_t bytes) {
     if (buffer && buffer->device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (buffer == nullptr || (src == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
+    if (buffer->device->closed) return fail(FH_ERR_DEVICE_MISMATCH, "the buffer's device has been destroyed");
     if (offset > buffer->bytes || bytes > buffer->bytes - offset)
         return fail(FH_ERR_RANGE, "upload [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
                     buffer->bytes);
@@ -328,6 +353,7 @@ fh_status fh_buffer_upload(fh_buffer* buffer, size_t offset, const void* src, si
 fh_status fh_buffer_download(const fh_buffer* buffer, size_t offset, void* dst, size_t bytes) {
     if (buffer && buffer->device->capturing) return fail(FH_ERR_SYNCHRONIZATION, "not available while an execution is being recorded");
     if (buffer == nullptr || (dst == nullptr && bytes)) return fail(FH_ERR_PARAMETER, "null argument");
+    if (buffer->device->closed) return fail(FH_ERR_DEVICE_MISMATCH, "the buffer's device has been destroyed");
     if (offset > buffer->bytes || bytes > buffer->bytes - offset)
         return fail(FH_ERR_RANGE, "download [%zu, +%zu) exceeds buffer of %zu bytes", offset, bytes,
                     buffer->bytes);
@@ -414,6 +440,7 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
         return fail(FH_ERR_ALLOCATION, "out of host memory");
     }
     m->device = device;
+    ++device->handles;
     m->ptr = dptr;
     m->bytes = packed_len;
     m->ggml_type = ggml_type;
@@ -427,6 +454,7 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
 void fh_qmatrix_destroy(fh_qmatrix* matrix) {
     if (matrix == nullptr) return;
     release_memory(matrix->device, matrix->ptr);
+    drop_device_handle(matrix->device);
     delete matrix;
 }
 
@@ -552,6 +580,8 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.metadata = nullptr;
         a.experts = 1;
         a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
+        a.stream = tuning(device, "gemv_stream") != 0;
+        a.cu_count = device->props.multiProcessorCount;
         a.x_mode = silu_mul ? kXSiluMul : kXPlain;
         a.x_rows = m;
         st = prepare_gemv(device, a);
@@ -1385,6 +1415,7 @@ fh_status fh_execution_end(fh_device* device, fh_graph** out) {
         return fail(FH_ERR_ALLOCATION, "out of host memory");
     }
     g->device = device;
+    ++device->handles;
     g->graph = graph;
     g->exec = exec;
     *out = g;
@@ -1393,6 +1424,7 @@ fh_status fh_execution_end(fh_device* device, fh_graph** out) {
 
 fh_status fh_graph_launch(fh_graph* graph) {
     if (graph == nullptr) return fail(FH_ERR_PARAMETER, "null graph");
+    if (graph->device->closed) return fail(FH_ERR_DEVICE_MISMATCH, "the graph's device has been destroyed");
     if (graph->device->capturing) return fail(FH_ERR_DISPATCH, "cannot replay while recording");
     FH_HIP(hipGraphLaunch(graph->exec, graph->device->stream));
     return FH_OK;
@@ -1400,13 +1432,14 @@ fh_status fh_graph_launch(fh_graph* graph) {
 
 void fh_graph_destroy(fh_graph* graph) {
     if (graph == nullptr) return;
-    if (graph->device->capturing) {
+    if (!graph->device->closed && graph->device->capturing) {
         graph->device->deferred_graphs.emplace_back(graph->exec, graph->graph);
     } else {
-        (void)hipStreamSynchronize(graph->device->stream);
+        if (!graph->device->closed) (void)hipStreamSynchronize(graph->device->stream);
         (void)hipGraphExecDestroy(graph->exec);
         (void)hipGraphDestroy(graph->graph);
     }
+    drop_device_handle(graph->device);
     delete graph;
 }
 
@@ -1423,6 +1456,7 @@ fh_status fh_event_create(fh_device* device, fh_event** out) {
         return hip_fail(e, "hipEventCreate");
     }
     ev->device = device;
+    ++device->handles;
     *out = ev;
     return FH_OK;
 }
@@ -1430,11 +1464,13 @@ fh_status fh_event_create(fh_device* device, fh_event** out) {
 void fh_event_destroy(fh_event* event) {
     if (event == nullptr) return;
     (void)hipEventDestroy(event->event);
+    drop_device_handle(event->device);
     delete event;
 }
 
 fh_status fh_event_record(fh_event* event) {
     if (event == nullptr) return fail(FH_ERR_PARAMETER, "null event");
+    if (event->device->closed) return fail(FH_ERR_DEVICE_MISMATCH, "the event's device has been destroyed");
     FH_HIP(hipEventRecord(event->event, event->device->stream));
     return FH_OK;
 }

@@ -532,6 +532,11 @@ GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
 }
 
 const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
+    if (a.stream && a.ggml_type == kQ4K && a.metadata == nullptr && a.x_mode == kXPlain && a.shared_w == nullptr &&
+        a.ksplit == 0) {
+        const StreamPlan stream = gemv_stream_plan(a.n, a.k, a.m, a.cu_count);
+        if (stream.ok) return launch_gemv_stream(s, a, stream);
+    }
     const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
     Params p{};
     p.w = static_cast<const uint8_t*>(a.w);

@@ -14,6 +14,10 @@
 #include "../../include/ferrum_hip.h"
 
 struct fh_device {
+    // The device object lives until fh_device_destroy has been called and the last buffer,
+    // matrix, graph or event created on it is gone: their release functions read it.
+    int handles = 1;       // the caller's own handle, plus one per live object
+    bool closed = false;   // fh_device_destroy has run: the stream is gone, memory is freed directly
     int ordinal = 0;
     hipStream_t stream = nullptr;
     hipDeviceProp_t props{};
@@ -134,6 +138,9 @@ struct GemvArgs {
     uint32_t shared_rows;
     const void* shared_x;
     void* shared_y;
+    // the streamed matrix-core kernel may take the launch (dense Q4_K, plain rows, rows that fit LDS)
+    bool stream;
+    int cu_count;
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
 };
@@ -143,6 +150,18 @@ struct GemvPlan {
 };
 GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments);
 const char* launch_gemv(hipStream_t s, const GemvArgs& a);
+
+// gemv_stream.hip: the Q4_K GEMV with LDS-direct weight loads and matrix-core dot products
+struct StreamPlan {
+    bool ok;              // the row length fits the kernel (LDS and per-wave block budget)
+    uint32_t tile_rows;   // weight rows per workgroup (1..16)
+    uint32_t tiles;
+    uint32_t waves;       // waves per workgroup
+    uint32_t row_stride;  // bytes between a tile's rows in LDS
+    uint32_t lds_bytes;
+};
+StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count);
+const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPlan& plan);
 
 // gemm.hip
 struct GemmArgs {

@@ -1,4 +1,6 @@
 """Shared helpers for the parity tests."""
+import contextlib
+
 import numpy as np
 
 import oracle
@@ -40,3 +42,15 @@ def oracle_columns(ggml_type, packed, n, k, rows, x, **kw):
     row_bytes = (k // 256) * bb
     sub = np.ascontiguousarray(packed.reshape(n, row_bytes)[rows]).reshape(-1)
     return oracle.project(ggml_type, sub, len(rows), k, x, **kw)
+
+
+@contextlib.contextmanager
+def fma_gemv(d):
+    """Dense Q4_K GEMVs inside the block take the FMA kernel, the one the fused and
+    per-assignment launches run on, so results can be compared with them bit for bit (the
+    streamed matrix-core GEMV sums in another order and agrees to the matmul tolerance)."""
+    d.set_tuning("gemv_stream", 0)
+    try:
+        yield
+    finally:
+        d.set_tuning("gemv_stream", 1)

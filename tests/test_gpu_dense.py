@@ -12,7 +12,7 @@ import pytest
 
 import ferrum_fixtures as fx
 import oracle
-from helpers import assert_matmul_parity, bits, oracle_columns, rel_l2
+from helpers import assert_matmul_parity, bits, fma_gemv, oracle_columns, rel_l2
 from ferrum_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -288,6 +288,56 @@ def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):
     # the reference's sequential-f32 answer, whose own rounding error grows with K
     assert_matmul_parity(got, want32, f"gemv {ggml} {n}x{k} vs f32seq", l2_tol=l2_tol)
     assert l2 <= rel_l2(want32, want64) * 1.5 + 1e-7, "GPU is less accurate than the sequential CPU sum"
+
+
+# The streamed matrix-core GEMV (dense Q4_K rows of up to 48 super-blocks): row lengths on both
+# sides of its per-wave block budgets, tile heights 1..16, every activation dtype, batched rows.
+@pytest.mark.parametrize("n,k", [(37, 256), (133, 2560), (300, 4864), (1100, 5120), (4100, 2048), (70, 6144),
+                                 (33, 8192), (20, 12288)])
+@pytest.mark.parametrize("dtype", ["F32", "F16", "BF16"])
+def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
+    code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
+    packed = synth.matrix(Q4_K, n, k, seed=n + k)
+    w = qm(api, d, Q4_K, n, k, packed)
+    for m in ((1, 3) if dtype == "F32" else (1,)):   # 16-bit rows beyond the first take the tile kernels
+        x = oracle.round_storage(synth.activations(m, k, seed=7 * n + m), code).reshape(m, k)
+        xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
+        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        assert out.operation == ("q4_k_gemv_factored" if m == 1 else "q4_k_gemm")
+        want = oracle.project(Q4_K, packed, n, k, x, accumulate="f64")
+        assert_matmul_parity(out.tensor.to_f32(), want, f"streamed gemv {n}x{k} {dtype} m={m}")
+        with fma_gemv(d):
+            other = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+        assert rel_l2(out.tensor.to_f32(), other) <= 1e-5 and not np.array_equal(bits(out.tensor.to_f32()), bits(other))
+
+
+def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
+    # activations whose 64-value chunks differ by dozens of orders of magnitude, zero chunks, one
+    # value per chunk: the per-chunk power-of-two scale keeps 22 bits of each
+    n, k = 64, 2048
+    packed = synth.matrix(Q4_K, n, k, seed=91)
+    w = qm(api, d, Q4_K, n, k, packed)
+    x = synth.activations(1, k, seed=92).reshape(k // 64, 64)
+    x *= np.float32(10.0) ** np.linspace(-30, 30, k // 64, dtype=np.float32)[:, None]
+    x[3] = 0
+    x[5, 1:] = 0
+    x = x.reshape(1, k)
+    got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, x), w).tensor.to_f32()
+    want = oracle.project(Q4_K, packed, n, k, x, accumulate="f64")
+    assert rel_l2(got, want) <= 1e-5
+    # each chunk alone: what the huge chunks would hide
+    for chunk in (0, 5, 16, 31):
+        part = np.zeros_like(x).reshape(k // 64, 64)
+        part[chunk] = x.reshape(k // 64, 64)[chunk]
+        part = part.reshape(1, k)
+        got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, part), w).tensor.to_f32()
+        want = oracle.project(Q4_K, packed, n, k, part, accumulate="f64")
+        assert rel_l2(got, want) <= 1e-5, chunk
+    # non-finite activations reach the rows they touch
+    bad = x.copy()
+    bad[0, 7] = np.inf
+    got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, bad), w).tensor.to_f32()
+    assert not np.isfinite(got).any()
 
 
 def test_config0_q4_k_gemv_4096(api, d):

@@ -8,7 +8,7 @@ import pytest
 
 import ferrum_fixtures as fx
 import oracle
-from helpers import assert_matmul_parity, bits, rel_l2
+from helpers import assert_matmul_parity, bits, fma_gemv, rel_l2
 from ferrum_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -379,9 +379,12 @@ def test_dense_projection_with_silu_mul_input_matches_the_two_calls(api, d, dtyp
     w = api.QuantizedMatrix.from_bytes(d, n, k, api.QuantizationFormat(Q4_K), packed)
     gate_up = oracle.round_storage(synth.activations(m, 2 * k, seed=72), code).reshape(m, 2 * k)
     t = api.Tensor.from_f32(d, gate_up.shape, dt, gate_up)
-    two = d.project_quantized(d.expert_silu_mul(t, k), w).tensor
+    with fma_gemv(d):   # the fused form runs on the FMA kernel
+        two = d.project_quantized(d.expert_silu_mul(t, k), w).tensor
     one = d.project_quantized(t, w, silu_mul=True).tensor
     assert np.array_equal(one.raw(), two.raw())
+    streamed = d.project_quantized(d.expert_silu_mul(t, k), w).tensor
+    assert rel_l2(streamed.to_f32(), one.to_f32()) <= (1e-5 if dtype == "F32" else 2e-3)
     want = oracle.project(Q4_K, packed, n, k, oracle.expert_silu_mul(gate_up, k, code), accumulate="f64")
     assert rel_l2(one.to_f32(), want) <= (1e-5 if dtype == "F32" else 2e-3)
     with pytest.raises(api.ShapeError):
@@ -468,7 +471,8 @@ def test_shared_expert_rides_in_the_routed_launch(api, d, dtype, tokens):
         assert d.last_operation() == "expert_project_q4_k_factored"
         assert np.array_equal(up.raw(), d.expert_project_quantized(xt, meta, w["win"], hidden, experts,
                                                                    form="gather").raw())
-        assert np.array_equal(shared_up.raw(), d.project_quantized(xt, w["sin"]).tensor.raw())
+        with fma_gemv(d):
+            assert np.array_equal(shared_up.raw(), d.project_quantized(xt, w["sin"]).tensor.raw())
         down, shared_down = d.expert_project_with_shared(up, meta, w["wout"], w["sout"], tokens, "silu_mul",
                                                          shared_input=shared_up)
         assert np.array_equal(down.raw(), d.expert_project_quantized(up, meta, w["wout"], inter, experts,

@@ -194,10 +194,11 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
-    d->tuning["gemv_stream"] = 1;           // dense Q4_K rows that fit LDS take the streamed matrix-core GEMV (0 = the FMA kernel)
+    d->tuning["gemv_stream"] = 1;           // dense Q4_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st != FH_OK) {
+        if (d->scratch) (void)hipFree(d->scratch);
         (void)hipStreamDestroy(d->stream);
         delete d;
         return st;
@@ -271,8 +272,10 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
     } else if (k == "gemm_min_rows") {
         ok = value >= 2;
-    } else if (k == "gemm_resident" || k == "gemv_stream") {
+    } else if (k == "gemm_resident") {
         ok = value == 0 || value == 1;
+    } else if (k == "gemv_stream") {
+        ok = value >= 0 && value <= 2;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {
@@ -580,7 +583,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.metadata = nullptr;
         a.experts = 1;
         a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
-        a.stream = tuning(device, "gemv_stream") != 0;
+        a.stream = (int)tuning(device, "gemv_stream");
         a.cu_count = device->props.multiProcessorCount;
         a.x_mode = silu_mul ? kXSiluMul : kXPlain;
         a.x_rows = m;

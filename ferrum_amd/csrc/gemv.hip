@@ -532,9 +532,9 @@ GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
 }
 
 const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
-    if (a.stream && a.ggml_type == kQ4K && a.metadata == nullptr && a.x_mode == kXPlain && a.shared_w == nullptr &&
+    if (a.stream != 0 && a.ggml_type == kQ4K && a.metadata == nullptr && a.x_mode == kXPlain && a.shared_w == nullptr &&
         a.ksplit == 0) {
-        const StreamPlan stream = gemv_stream_plan(a.n, a.k, a.m, a.cu_count);
+        const StreamPlan stream = gemv_stream_plan(a.n, a.k, a.m, a.cu_count, a.stream == 2);
         if (stream.ok) return launch_gemv_stream(s, a, stream);
     }
     const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);

@@ -261,7 +261,7 @@ void gemv_stream_q4k(const StreamParams p) {
 
 // Tile height that spreads the rows evenly: the fewest 16-row rounds per compute unit, then the
 // smallest height that still fits them.
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count) {
+StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size) {
     StreamPlan plan{};
     const uint32_t nb = k / 256u;
     const uint32_t cus = cu_count > 0 ? (uint32_t)cu_count : 256u;
@@ -278,7 +278,8 @@ StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count) {
     plan.tiles = (n + h - 1u) / h;
     plan.waves = 8u;
     plan.lds_bytes = h * plan.row_stride + plan.waves * kSlotBytes + plan.waves * 64u;
-    plan.ok = nb >= 1 && nb <= 48u && h >= 1u && plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u;
+    // matrices of a megabyte or two finish sooner on the FMA kernel's smaller workgroups
+    plan.ok = nb >= 1 && nb <= 48u && h >= 1u && (any_size || (uint64_t)n * nb >= 16384u) && plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u;
     return plan;
 }
 

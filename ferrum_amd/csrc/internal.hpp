@@ -139,7 +139,7 @@ struct GemvArgs {
     const void* shared_x;
     void* shared_y;
     // the streamed matrix-core kernel may take the launch (dense Q4_K, plain rows, rows that fit LDS)
-    bool stream;
+    int stream;           // 0 never, 1 where it is the faster kernel, 2 wherever it can run
     int cu_count;
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
@@ -160,7 +160,8 @@ struct StreamPlan {
     uint32_t row_stride;  // bytes between a tile's rows in LDS
     uint32_t lds_bytes;
 };
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count);
+// any_size: also matrices so small that the FMA kernel is the faster one
+StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size);
 const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPlan& plan);
 
 // gemm.hip

@@ -49,8 +49,9 @@ def fma_gemv(d):
     """Dense Q4_K GEMVs inside the block take the FMA kernel, the one the fused and
     per-assignment launches run on, so results can be compared with them bit for bit (the
     streamed matrix-core GEMV sums in another order and agrees to the matmul tolerance)."""
+    before = d.get_tuning("gemv_stream")
     d.set_tuning("gemv_stream", 0)
     try:
         yield
     finally:
-        d.set_tuning("gemv_stream", 1)
+        d.set_tuning("gemv_stream", before)

@@ -299,6 +299,7 @@ def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
     code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
     packed = synth.matrix(Q4_K, n, k, seed=n + k)
     w = qm(api, d, Q4_K, n, k, packed)
+    d.set_tuning("gemv_stream", 2)   # also where the matrix is small enough for the FMA kernel to win
     for m in ((1, 3) if dtype == "F32" else (1,)):   # 16-bit rows beyond the first take the tile kernels
         x = oracle.round_storage(synth.activations(m, k, seed=7 * n + m), code).reshape(m, k)
         xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
@@ -309,6 +310,7 @@ def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
         with fma_gemv(d):
             other = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
         assert rel_l2(out.tensor.to_f32(), other) <= 1e-5 and not np.array_equal(bits(out.tensor.to_f32()), bits(other))
+    d.set_tuning("gemv_stream", 1)
 
 
 def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
@@ -317,6 +319,7 @@ def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
     n, k = 64, 2048
     packed = synth.matrix(Q4_K, n, k, seed=91)
     w = qm(api, d, Q4_K, n, k, packed)
+    d.set_tuning("gemv_stream", 2)
     x = synth.activations(1, k, seed=92).reshape(k // 64, 64)
     x *= np.float32(10.0) ** np.linspace(-30, 30, k // 64, dtype=np.float32)[:, None]
     x[3] = 0
@@ -338,6 +341,7 @@ def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
     bad[0, 7] = np.inf
     got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, bad), w).tensor.to_f32()
     assert not np.isfinite(got).any()
+    d.set_tuning("gemv_stream", 1)
 
 
 def test_config0_q4_k_gemv_4096(api, d):

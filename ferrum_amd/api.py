@@ -113,6 +113,7 @@ SYMBOLS = {
     "fh_dequantize": (_I32, [_P, _P, _VP]),
     "fh_embedding_gather_quantized": (_I32, [_P, _P, ctypes.POINTER(_U32), _SZ, _VP]),
     "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
+    "fh_project_quantized_no_alloc": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_add_rmsnorm": (_I32, [_P, _VP, _VP, _VP, _U32, _U32, ctypes.c_float, _VP, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
@@ -593,6 +594,17 @@ class Device:
         xv, yv = a._view(), out._view()
         call = _lib.fh_project_silu_mul_quantized if silu_mul else _lib.fh_project_quantized
         _check(call(self._handle, _handle_of(weight), ctypes.byref(xv), m, ctypes.byref(yv)))
+        return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
+
+    def project_quantized_no_alloc(self, a: Tensor, weight, out: Tensor) -> Output:
+        """fh_project_quantized_no_alloc: the per-row GEMV kernels with the library's fixed
+        scratch; the caller brings the output, nothing is allocated on the device."""
+        dims = a.shape()
+        if len(dims) != 2 or dims[1] != weight.columns() or out.shape() != (dims[0], weight.rows()):
+            raise ShapeError("quantized projection requires [M,K] matching [N,K]")
+        xv, yv = a._view(), out._view()
+        _check(_lib.fh_project_quantized_no_alloc(self._handle, _handle_of(weight), ctypes.byref(xv), dims[0],
+                                                  ctypes.byref(yv)))
         return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
 
     def argmax_rows(self, logits: Tensor) -> Tensor:

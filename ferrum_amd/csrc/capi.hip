@@ -153,6 +153,14 @@ int64_t tuning(const fh_device* d, const char* key) {
 
 using namespace fh;
 
+// Scratch of the entry point that allocates nothing: the K-segment partial sums and the
+// row-tile counters of the GEMV.  Every device the library runs on holds its own copy of
+// the array at its own address for the life of the process; `scratch` itself is only the
+// host-side name of the symbol, the device address comes from hipGetSymbolAddress.
+constexpr size_t kFixedCounterWords = 4096;
+constexpr size_t kFixedScratchBytes = 1u << 20;   // 16 KiB of counters, then partial sums
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+
 static_assert(kXDivide > FH_INPUT_SILU_MUL, "the row-divide mode is internal: it has no public input form");
 static_assert(kXPlain == FH_INPUT_ROWS && kXGather == FH_INPUT_GATHER && kXSiluMul == FH_INPUT_SILU_MUL,
               "the kernel's input modes are the ABI's input forms");
@@ -197,6 +205,15 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemv_stream"] = 1;           // dense Q4_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
+    if (st == FH_OK) {
+        // this device's address of the fixed scratch (the device is current), counters at zero
+        void* fixed = nullptr;
+        e = hipGetSymbolAddress(&fixed, HIP_SYMBOL(scratch));
+        if (e == hipSuccess) e = hipMemsetAsync(fixed, 0, kFixedCounterWords * sizeof(uint32_t), d->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(d->stream);
+        if (e != hipSuccess) st = hip_fail(e, "fixed scratch");
+        d->fixed_scratch = fixed;
+    }
     if (st != FH_OK) {
         if (d->scratch) (void)hipFree(d->scratch);
         (void)hipStreamDestroy(d->stream);
@@ -612,6 +629,58 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
 fh_status fh_project_silu_mul_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* packed,
                                         uint32_t m, const fh_view* y) {
     return project(device, weight, packed, m, y, true);
+}
+
+// fh_project_quantized through the per-row GEMV kernels only, with the kernel's scratch in the
+// library's fixed array: no hipMalloc, hipFree or synchronisation on any path.
+fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
+                                        uint32_t m, const fh_view* y) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device) return fail(FH_ERR_DEVICE_MISMATCH, "weight belongs to another device");
+    if (device->fixed_scratch == nullptr) return fail(FH_ERR_DISPATCH, "the fixed scratch is not set up");
+    const uint64_t n = weight->rows * weight->experts, k = weight->cols;
+    if (m == 0 || k > 0xffffffffull - 32)
+        return fail(FH_ERR_SHAPE, "quantized projection requires [M,K] matching [N,K]");
+    if (!fits_u32((uint64_t)m * k) || !fits_u32((uint64_t)m * n) || !fits_u32(n) || m > 65535u)
+        return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+    Range xr, yr;
+    fh_status st = resolve(device, x, (uint64_t)m * k, "projection input", &xr);
+    if (st != FH_OK) return st;
+    st = resolve(device, y, (uint64_t)m * n, "projection output", &yr);
+    if (st != FH_OK) return st;
+    if (overlaps(xr, yr)) return fail(FH_ERR_RANGE, "projection output aliases its input");
+    GemvArgs a{};
+    a.ggml_type = weight->ggml_type;
+    a.w = weight->ptr;
+    a.x = xr.begin;
+    a.y = const_cast<uint8_t*>(yr.begin);
+    a.n = (uint32_t)n;
+    a.k = (uint32_t)k;
+    a.m = m;
+    a.x_dtype = x->dtype;
+    a.y_dtype = y->dtype;
+    a.experts = 1;
+    a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
+    a.stream = (int)tuning(device, "gemv_stream");
+    a.cu_count = device->props.multiProcessorCount;
+    a.x_mode = kXPlain;
+    a.x_rows = m;
+    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    if (plan.segments > 1) {
+        const uint64_t counters = (uint64_t)plan.tiles * m;
+        const uint64_t partial_bytes = (uint64_t)plan.segments * m * n * sizeof(float);
+        if (counters > kFixedCounterWords || partial_bytes > kFixedScratchBytes - kFixedCounterWords * sizeof(uint32_t))
+            return fail(FH_ERR_SHAPE,
+                        "projection needs %llu counters and %llu bytes of partial sums; the fixed scratch holds %zu and %zu",
+                        (unsigned long long)counters, (unsigned long long)partial_bytes, kFixedCounterWords,
+                        kFixedScratchBytes - kFixedCounterWords * sizeof(uint32_t));
+        uint8_t* const base = static_cast<uint8_t*>(device->fixed_scratch);
+        a.counters = reinterpret_cast<uint32_t*>(base);
+        a.partials = reinterpret_cast<float*>(base + kFixedCounterWords * sizeof(uint32_t));
+    }
+    device->last_operation = launch_gemv(device->stream, a);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
 }
 
 // ---- mixture of experts -------------------------------------------------------------

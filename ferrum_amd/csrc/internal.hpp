@@ -27,6 +27,8 @@ struct fh_device {
     // scratch owned by the device: [counter words | floats / ids]
     void* scratch = nullptr;
     size_t scratch_bytes = 0;
+    // this device's copy of the library's fixed scratch array (fh_project_quantized_no_alloc)
+    void* fixed_scratch = nullptr;
     static constexpr size_t kCounterWords = 1u << 16;
     // Releases asked for while an execution is being recorded wait for its end:
     // freeing or synchronizing inside a stream capture would invalidate it.

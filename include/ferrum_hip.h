@@ -168,6 +168,19 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
 fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
                                uint32_t m, const fh_view* y);
 
+/* fh_project_quantized for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Every row of x goes through the GEMV kernels (any m,
+ * any dtype; same results as fh_project_quantized whenever that takes those kernels),
+ * and the partial sums and row-tile counters a long-K launch needs live in a fixed 1 MiB
+ * array inside the library, one copy per GPU, held until the process ends.  The call
+ * makes no hipMalloc / hipFree and does not synchronise.  FH_ERR_SHAPE when a launch
+ * would need more than 4096 counters (row tiles x m) or 1032192 bytes of partial sums
+ * (K segments x m x N x 4); nothing is launched then.  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams, two threads) race. */
+fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* weight,
+                                        const fh_view* x, uint32_t m, const fh_view* y);
+
 /* MetalDevice::argmax_rows (src/ops/transformer.rs:768-792, kernel
  * src/metal/shaders/ops.metal:2438-2464): greedy selection over the rows of a
  * logits matrix, the step after the lm_head projection.  out is an f32 carrier

@@ -638,7 +638,10 @@ __device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int 
     }
 }
 
-constexpr int kWideThreads = 512;
+// Waves that multiply: each owns 16 * kWideRowTiles rows of the 256-row tile; four more waves decode.
+constexpr int kWideConsumers = 4;   // eight (two multiplying waves per SIMD) measured the same at M = 512 and slower for the heavier decoders
+constexpr int kWideRowTiles = 16 / kWideConsumers;
+constexpr int kWideThreads = (kWideConsumers + 4) * 64;
 
 template <uint32_t TYPE, int DT, int NT>
 __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* __restrict__ w,
@@ -668,9 +671,9 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
     const uint32_t k = nb << 8;
     const uint32_t steps = nb * 4;
 
-    if (wave >= 4) {
+    if (wave >= kWideConsumers) {
         // ---- producers: global -> registers -> (decode) -> LDS, two slabs ahead ----
-        const uint32_t pt = tid - 256, pw = wave - 4;
+        const uint32_t pt = tid - kWideConsumers * 64, pw = wave - kWideConsumers;
         const uint32_t wr = pt >> 1, wh = pt & 1u;
         const uint8_t* wsrc = w + (size_t)(n0 + (wr < ncols ? wr : ncols - 1)) * nb * kBlockBytes;
         // rows 128.. of a 136-column tile: 8 rows x 2 halves x 4 quarter pieces, one per lane
@@ -717,9 +720,9 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
     }
 
     // ---- consumers: LDS fragments -> MFMA ----
-    float4v acc[4][NT];
+    float4v acc[kWideRowTiles][NT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kWideRowTiles; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[i][j] = float4v{0.f, 0.f, 0.f, 0.f};
 
@@ -729,18 +732,18 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
     // through a ring of three register sets, loaded two K halves ahead.
     const uint32_t g = lane >> 4;
     // rows past m are clamped: they only feed outputs that are never stored
-    const uint16_t* asrc[4];
+    const uint16_t* asrc[kWideRowTiles];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        uint32_t row = m0 + wave * 64 + 16 * i + (lane & 15u);
+    for (int i = 0; i < kWideRowTiles; ++i) {
+        uint32_t row = m0 + wave * (16 * kWideRowTiles) + 16 * i + (lane & 15u);
         asrc[i] = x + (size_t)(row < m ? row : m - 1) * k + 8 * g;
     }
-    auto load_a = [&](uint4 (&a)[4], uint32_t u) {
+    auto load_a = [&](uint4 (&a)[kWideRowTiles], uint32_t u) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const uint4*>(asrc[i] + (size_t)u * 32);
+        for (int i = 0; i < kWideRowTiles; ++i) a[i] = *reinterpret_cast<const uint4*>(asrc[i] + (size_t)u * 32);
     };
     const uint32_t frag_off = (lane & 15u) * kLd + 8 * g;
-    auto mma_half = [&](const uint4 (&a)[4], uint32_t u) {
+    auto mma_half = [&](const uint4 (&a)[kWideRowTiles], uint32_t u) {
         const uint16_t* ws = lds + ((u >> 1) & 1u) * kStage + frag_off + (u & 1u) * 32;
         // B fragments through a ring of four so three LDS reads stay in flight
         uint4 b[4];
@@ -750,21 +753,21 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
         for (int j = 0; j < NT; ++j) {
             if (j + 3 < NT) b[(j + 3) % 4] = *reinterpret_cast<const uint4*>(ws + 16 * (j + 3) * kLd);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i][j] = mfma16<DT>(a[i], b[j % 4], acc[i][j]);
+            for (int i = 0; i < kWideRowTiles; ++i) acc[i][j] = mfma16<DT>(a[i], b[j % 4], acc[i][j]);
         }
         // issue order for the scheduler (0x100 = DS read, 0x008 = MFMA)
         __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
         for (int j = 0; j < NT - 3; ++j) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, kWideRowTiles, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, 12, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 3 * kWideRowTiles, 0);
     };
     const uint32_t halves = steps * 2;
     constexpr int kRing = 4;               // A register sets: loads run kRing - 1 halves ahead
     static_assert(kRing % 2 == 0, "the slab barrier falls on even halves of the ring");
-    uint4 a[kRing][4];
+    uint4 a[kRing][kWideRowTiles];
 #pragma unroll
     for (int i = 0; i < kRing - 1; ++i)
         if ((uint32_t)i < halves) load_a(a[i], i);
@@ -795,13 +798,13 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
     __builtin_amdgcn_s_setprio(0);
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kWideRowTiles; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             const uint32_t lc = 16 * j + (lane & 15u);
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const uint32_t row = m0 + wave * 64 + 16 * i + 4 * (lane >> 4) + v;
+                const uint32_t row = m0 + wave * (16 * kWideRowTiles) + 16 * i + 4 * (lane >> 4) + v;
                 if (row < m && lc < ncols)
                     store_from_f32(y, (size_t)row * n + n0 + lc, y_dtype, acc[i][j][v]);
             }
@@ -813,13 +816,14 @@ struct WidePlan {
     uint32_t cols, tiles_m, tiles_n;
 };
 
-// Columns per workgroup: 128, 136 or 144, whichever wastes the least of the
-// chip's `cus` compute units (whole rounds of workgroups) and of the MFMA tile.
+// Columns per workgroup: 128 or 136, whichever wastes the least of the chip's `cus`
+// compute units (whole rounds of workgroups) and of the MFMA tile.  The ninth column
+// tile is decoded eight rows deep (LDS rows 128..135), so 136 is the widest.
 WidePlan wide_plan(uint32_t m, uint32_t n, int cus) {
     WidePlan best{};
     double best_cost = 1e300;
     const uint32_t tiles_m = (m + kWM - 1) / kWM;
-    for (uint32_t cols : {128u, 136u, 144u}) {
+    for (uint32_t cols : {128u, 136u}) {
         const int nt = cols > 128 ? 9 : 8;
         const uint32_t tiles_n = (n + cols - 1) / cols;
         const uint64_t wgs = (uint64_t)tiles_m * tiles_n;

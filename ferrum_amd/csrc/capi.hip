@@ -73,14 +73,25 @@ fh_status resolve(const fh_device* device, const fh_view* view, uint64_t element
 bool fits_u32(uint64_t v) { return v <= 0xffffffffull; }
 
 // Device scratch: kCounterWords zeroed counter words followed by a data area
-// of at least `data_bytes`.  Growing it waits for the stream first.
+// of at least `data_bytes`.  Growing it waits for the stream first.  Recorded executions
+// carry the scratch address in their kernel arguments, so a block that is outgrown while
+// any of them is alive is kept (they replay on it unchanged) and freed with the last one.
 fh_status ensure_scratch(fh_device* d, size_t data_bytes) {
     const size_t counter_bytes = fh_device::kCounterWords * sizeof(uint32_t);
     if (d->scratch != nullptr && d->scratch_bytes >= counter_bytes + data_bytes) return FH_OK;
     if (d->capturing)
         return fail(FH_ERR_SYNCHRONIZATION, "device scratch must grow: run the operator once before recording it");
     FH_HIP(hipStreamSynchronize(d->stream));
-    if (d->scratch) (void)hipFree(d->scratch);
+    // at least twice the old data area, so the blocks kept for recordings add up to less than the live one
+    const size_t old_data = d->scratch_bytes > counter_bytes ? d->scratch_bytes - counter_bytes : 0;
+    if (data_bytes < 2 * old_data) data_bytes = 2 * old_data;
+    if (d->scratch) {
+        if (d->live_graphs > 0) {
+            d->retired_scratch.push_back(d->scratch);
+        } else {
+            (void)hipFree(d->scratch);
+        }
+    }
     d->scratch = nullptr;
     d->scratch_bytes = 0;
     size_t cap = counter_bytes + (data_bytes < (16u << 20) ? (16u << 20) : data_bytes);
@@ -107,6 +118,45 @@ fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
         if (st != FH_OK) return st;
         a.partials = reinterpret_cast<float*>(scratch_data(d));
         a.counters = scratch_counters(d);
+    }
+    return FH_OK;
+}
+
+// Runs a GEMV launch of any batch size: the batch is cut into runs that fit the grid's z
+// extent and, where K is cut into segments, the counter words (one per row tile and batch
+// entry).  A launch that carries a shared expert is not cut.
+fh_status run_gemv(fh_device* d, GemvArgs a, const char** name) {
+    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    uint64_t most = 65535u;
+    if (plan.segments > 1 && plan.tiles > 0) most = std::min<uint64_t>(most, fh_device::kCounterWords / plan.tiles);
+    if (a.x_mode == kXDivide && a.x_div > 1) most -= most % a.x_div;   // the routes of a token stay together
+    if (a.m <= most || a.shared_w != nullptr || most == 0) {
+        fh_status st = prepare_gemv(d, a);
+        if (st != FH_OK) return st;
+        if (a.m > 65535u) return fail(FH_ERR_SHAPE, "batch of %u entries exceeds the launch grid", a.m);
+        *name = launch_gemv(d->stream, a);
+        return FH_OK;
+    }
+    const uint32_t total = a.m;
+    const size_t x_row = (size_t)a.k * dtype_bytes(a.x_dtype) * (a.x_mode == kXSiluMul ? 2 : 1);
+    const size_t y_row = (size_t)a.n * dtype_bytes(a.y_dtype);
+    const uint32_t stride = a.meta_stride == 0 ? 3u : a.meta_stride;
+    for (uint32_t first = 0; first < total; first += (uint32_t)most) {
+        GemvArgs part = a;
+        part.m = std::min<uint32_t>((uint32_t)most, total - first);
+        part.y = static_cast<uint8_t*>(a.y) + first * y_row;
+        if (a.metadata != nullptr) part.metadata = a.metadata + (size_t)first * stride;
+        if (a.x_mode == kXPlain || a.x_mode == kXSiluMul) {
+            part.x = static_cast<const uint8_t*>(a.x) + first * x_row;
+            part.x_rows = part.m;
+        } else if (a.x_mode == kXDivide) {
+            const uint32_t div = a.x_div == 0 ? 1u : a.x_div;
+            part.x = static_cast<const uint8_t*>(a.x) + (size_t)(first / div) * x_row;
+            part.x_rows = part.m / div;
+        }   // kXGather reads the token row named by each entry's metadata: x stays whole
+        fh_status st = prepare_gemv(d, part);
+        if (st != FH_OK) return st;
+        *name = launch_gemv(d->stream, part);
     }
     return FH_OK;
 }
@@ -242,6 +292,8 @@ void fh_device_destroy(fh_device* device) {
         device->stream = nullptr;
     }
     if (device->scratch) (void)hipFree(device->scratch);
+    for (void* old : device->retired_scratch) (void)hipFree(old);
+    device->retired_scratch.clear();
     device->scratch = nullptr;
     device->scratch_bytes = 0;
     device->closed = true;
@@ -604,9 +656,9 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.cu_count = device->props.multiProcessorCount;
         a.x_mode = silu_mul ? kXSiluMul : kXPlain;
         a.x_rows = m;
-        st = prepare_gemv(device, a);
+        const char* name = "";
+        st = run_gemv(device, a, &name);
         if (st != FH_OK) return st;
-        const char* name = launch_gemv(device->stream, a);
         if (m > 1)
             name = weight->ggml_type == kQ4K   ? "q4_k_gemm"
                    : weight->ggml_type == kQ5K ? "q5_k_gemm"
@@ -930,9 +982,9 @@ fh_status hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const f
         a.shared_x = sxr.begin;
         a.shared_y = const_cast<uint8_t*>(syr.begin);
     }
-    st = prepare_gemv(device, a);
+    const char* unused = "";
+    st = run_gemv(device, a, &unused);
     if (st != FH_OK) return st;
-    launch_gemv(device->stream, a);
     device->last_operation = weight->ggml_type == kQ4K     ? "h_mv_id_q4_k"
                              : weight->ggml_type == kQ5K   ? "h_mv_id_q5_k"
                              : weight->ggml_type == kQ6K   ? "h_mv_id_q6_k"
@@ -1354,9 +1406,10 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         a.shared_x = sxr.begin;
         a.shared_y = const_cast<uint8_t*>(syr.begin);
     }
-    st = prepare_gemv(device, a);
+    const char* name = "";
+    st = run_gemv(device, a, &name);
     if (st != FH_OK) return st;
-    device->last_operation = launch_gemv(device->stream, a);
+    device->last_operation = name;
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -1488,6 +1541,7 @@ fh_status fh_execution_end(fh_device* device, fh_graph** out) {
     }
     g->device = device;
     ++device->handles;
+    ++device->live_graphs;
     g->graph = graph;
     g->exec = exec;
     *out = g;
@@ -1510,6 +1564,11 @@ void fh_graph_destroy(fh_graph* graph) {
         if (!graph->device->closed) (void)hipStreamSynchronize(graph->device->stream);
         (void)hipGraphExecDestroy(graph->exec);
         (void)hipGraphDestroy(graph->graph);
+    }
+    if (--graph->device->live_graphs == 0 && !graph->device->capturing) {
+        // nothing can replay on the outgrown scratch blocks any more
+        for (void* old : graph->device->retired_scratch) release_memory(graph->device, old);
+        graph->device->retired_scratch.clear();
     }
     drop_device_handle(graph->device);
     delete graph;

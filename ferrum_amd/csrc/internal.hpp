@@ -32,6 +32,10 @@ struct fh_device {
     static constexpr size_t kCounterWords = 1u << 16;
     // Releases asked for while an execution is being recorded wait for its end:
     // freeing or synchronizing inside a stream capture would invalidate it.
+    // scratch blocks that were outgrown while recorded executions (which carry their address)
+    // were alive: freed with the last of those
+    std::vector<void*> retired_scratch;
+    int live_graphs = 0;
     std::vector<void*> deferred_frees;
     std::vector<std::pair<hipGraphExec_t, hipGraph_t>> deferred_graphs;
 };

@@ -459,6 +459,100 @@ def test_recorded_execution_replays_bitwise_with_eager_work_in_between(api, d):
         d.synchronize()
 
 
+def test_a_recorded_execution_survives_the_growth_of_the_scratch(api, d):
+    # a recorded long-K GEMV carries the address of the device scratch (partial sums, counters);
+    # an eager call that outgrows the scratch afterwards must not take that memory away
+    n, k = 2048, 17408
+    w = qm(api, d, Q4_K, n, k, synth.matrix(Q4_K, n, k, seed=121))
+    x = api.Tensor.from_f32(d, (1, k), api.DType.F32, synth.activations(1, k, seed=122))
+    y = api.Tensor.zeros(d, (1, n), api.DType.F32)
+    eager = d.project_quantized(x, w)
+    assert eager.operation == "q4_k_gemv_ksplit"
+    with d.execution() as ex:
+        d.project_quantized(x, w, out=y)
+    ex.graph.launch()
+    assert np.array_equal(y.raw(), eager.tensor.raw())
+    # 3000 x 5120 f32 rows rounded to f16 in the scratch: 30 MB, beyond the 16 MB it starts with
+    kb, nbig, mb = 5120, 256, 3000
+    wb = qm(api, d, Q4_K, nbig, kb, synth.matrix(Q4_K, nbig, kb, seed=123))
+    xb = api.Tensor.from_f32(d, (mb, kb), api.DType.F32, synth.activations(mb, kb, seed=124))
+    d.set_tuning("gemm_f32_min_rows", 2)
+    try:
+        big = d.project_quantized(xb, wb)
+    finally:
+        d.set_tuning("gemm_f32_min_rows", 0)
+    assert "mfma" in big.operation
+    for _ in range(2):
+        y.buffer.upload(0, np.zeros(n, np.float32))
+        ex.graph.launch()
+        assert np.array_equal(y.raw(), eager.tensor.raw())
+        d.project_quantized(x, w)          # eager work on the new scratch in between
+        d.synchronize()
+
+
+def test_f32_batches_of_any_size_run_through_the_long_k_gemv(api, d):
+    # q4_k_gemm accepts any M (src/metal/shaders/ops.metal:1102-1121): a long-K projection of 110 f32
+    # rows needs more row-tile counters than one launch has, so the batch is cut into runs
+    n, k, m = 5120, 17408, 110
+    packed = synth.matrix(Q4_K, n, k, seed=131)
+    w = qm(api, d, Q4_K, n, k, packed)
+    x = synth.activations(m, k, seed=132)
+    out = d.project_quantized(api.Tensor.from_f32(d, (m, k), api.DType.F32, x), w)
+    assert out.operation == "q4_k_gemm"
+    got = out.tensor.to_f32()
+    first = d.project_quantized(api.Tensor.from_f32(d, (60, k), api.DType.F32, x[:60]), w).tensor.to_f32()
+    last = d.project_quantized(api.Tensor.from_f32(d, (50, k), api.DType.F32, x[60:]), w).tensor.to_f32()
+    assert np.array_equal(bits(got[:60]), bits(first)) and np.array_equal(bits(got[60:]), bits(last))
+    rows = np.unique(synth.rng(133).integers(0, n, 48))
+    picked = [0, 59, 60, 101, 102, 103, 109]
+    want = oracle_columns(Q4_K, packed, n, k, rows, x[picked], accumulate="f64")
+    assert_matmul_parity(got[picked][:, rows], want, "f32 batch through the K-split GEMV")
+
+
+def test_wide_gemm_covers_every_column_of_its_tiles(api, d):
+    # 300 rows x 36864 columns: the 256-row tile kernel with 136 columns per workgroup; the last
+    # columns of a workgroup's tile (the ninth MFMA column tile) are the ones checked
+    n, k, m = 36864, 512, 300
+    packed = synth.matrix(Q4_K, n, k, seed=141)
+    w = qm(api, d, Q4_K, n, k, packed)
+    x = synth.activations(m, k, seed=142, f16=True)
+    out = d.project_quantized(api.Tensor.from_f32(d, (m, k), api.DType.F16, x), w, out_dtype=api.DType.F32)
+    assert out.operation == "q4_k_gemm_mfma_m256"
+    got = out.tensor.to_f32()
+    for width in (128, 136, 144):      # whichever width the plan chose, its tiles' last 16 columns
+        rows = np.concatenate([np.arange(t * width + width - 16, t * width + width) for t in (0, 1, 100, n // width - 1)])
+        rows = rows[rows < n]
+        want = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", weight_round=oracle.F16)
+        assert_matmul_parity(got[:, rows], want, f"columns at the end of {width}-wide tiles")
+    rows = np.arange(n - 40, n)
+    want = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", weight_round=oracle.F16)
+    assert_matmul_parity(got[:, rows], want, "last columns")
+
+
+def test_objects_may_outlive_their_device(api):
+    # buffers, matrices and recorded executions hold the device object: releasing them after
+    # fh_device_destroy (any order a garbage collector may pick) is safe
+    import gc
+    dev = api.Device.new()
+    n, k = 64, 512
+    w = qm(api, dev, Q4_K, n, k, synth.matrix(Q4_K, n, k, seed=151))
+    x = api.Tensor.from_f32(dev, (1, k), api.DType.F32, synth.activations(1, k, seed=152))
+    y = api.Tensor.zeros(dev, (1, n), api.DType.F32)
+    with dev.execution() as ex:
+        dev.project_quantized(x, w, out=y)
+    ex.graph.launch()
+    want = y.to_f32().copy()
+    handle, dev._handle = dev._handle, None
+    api._lib.fh_device_destroy(handle)
+    with pytest.raises(api.Error):
+        y.to_f32()                                  # the device is gone: a clear error, not a crash
+    with pytest.raises(api.Error):
+        ex.graph.launch()
+    del ex, w, x, y
+    gc.collect()
+    assert np.abs(want).max() > 0
+
+
 def test_releases_asked_for_while_recording_wait_for_its_end(api, d):
     import gc
     n, k = 512, 1024

@@ -387,6 +387,31 @@ def test_config3_q4_k_gemm_5120_17408(api, d, m):
             assert_matmul_parity(half.tensor.to_f32(), got[: m // 2], f"gemm M={m // 2} vs M={m}")
 
 
+@pytest.mark.parametrize("m", [8, 512])
+def test_config3_every_column_against_a_closed_form(api, d, m):
+    # All 17408 columns, which a sample of columns cannot vouch for: row n keeps one super-block,
+    # number n % 20, and zero blocks (d = dmin = 0) elsewhere, so y[:, n] is a 256-term product the
+    # host evaluates for every column.
+    n, k = 17408, 5120
+    nb = k // 256
+    blocks = synth.matrix(Q4_K, n, 256, seed=401).reshape(n, 144)
+    packed = np.zeros((n, nb, 144), np.uint8)
+    keep = np.arange(n) % nb
+    packed[np.arange(n), keep] = blocks
+    x = synth.activations(m, k, seed=402, f16=True)
+    w = qm(api, d, Q4_K, n, k, packed.reshape(-1))
+    out = d.project_quantized(api.Tensor.from_f32(d, (m, k), api.DType.F16, x), w, out_dtype=api.DType.F32)
+    got = out.tensor.to_f32()
+    dense = oracle.round_storage(oracle.dequantize(Q4_K, blocks.reshape(-1), n, 256), oracle.F16).astype(np.float64)
+    want = np.empty((m, n), np.float64)
+    for b in range(nb):
+        rows = np.nonzero(keep == b)[0]
+        want[:, rows] = x[:, 256 * b:256 * (b + 1)].astype(np.float64) @ dense[rows].T
+    assert_matmul_parity(got, want, f"every column at M={m} ({out.operation})")
+    worst = np.abs(got - want).max(axis=0)
+    assert worst.max() <= 1e-3 * np.abs(want).max(), int(worst.argmax())
+
+
 # ------------------------------------------------------------ error behaviour
 
 def test_project_rejects_bad_geometry_and_foreign_buffers(api, d):

@@ -322,6 +322,77 @@ def test_a3b_style_ffn_with_shared_expert(api, d, tokens):
     assert np.abs(got - want).max() <= 4e-3 * np.abs(want).max()
 
 
+def _scaled_d(blocks, power):
+    """Q4_K blocks [.., 144] with every block's f16 d multiplied by 2^power (exponent bits)."""
+    out = blocks.copy()
+    d = out[..., 0:2].copy().view(np.uint16)
+    assert ((d >> 10) & 31).min() >= 1 and ((d >> 10) & 31).max() + power < 31
+    out[..., 0:2] = (d + np.uint16(power << 10)).view(np.uint8)
+    return out
+
+
+@pytest.mark.parametrize("tokens", [1, 512])
+def test_a3b_ffn_as_benchmarked_with_256_distinct_experts(api, d, tokens):
+    # The path bench.py times: SparseMoe.forward with the shared expert riding in the routed launches,
+    # hidden 2048, 256 experts of intermediate 512, top-8, f16.  Every expert is different, every
+    # token is checked, and the host side still evaluates one expert per token: expert e is the base
+    # expert with (a) its output rows rotated by 8e, (b) its up rows scaled by 2^((e / 2) % 4), an exact
+    # scaling because the minimums are zero, and (c) for odd e the gate / up rows rotated by 256, with the
+    # down projection's two column blocks swapped to match.  So routed_e(x) = 2^c roll(routed_base(x)).
+    hidden, inter, experts, top_k = 2048, 512, 256, 8
+    fmt = api.QuantizationFormat.Q4_K
+    base_in = synth.matrix(Q4_K, 2 * inter, hidden, seed=201).reshape(2 * inter, hidden // 256, 144).copy()
+    base_out = synth.matrix(Q4_K, hidden, inter, seed=202).reshape(hidden, inter // 256, 144).copy()
+    for blocks in (base_in, base_out):
+        blocks[..., 2:4] = 0                                     # dmin = 0
+        small = blocks[..., 0:2].copy().view(np.uint16) < (1 << 10)
+        blocks[..., 0:2] = np.where(small, np.uint16(0x2000), blocks[..., 0:2].copy().view(np.uint16)).view(np.uint8)
+    w_in = np.empty((experts,) + base_in.shape, np.uint8)
+    w_out = np.empty((experts,) + base_out.shape, np.uint8)
+    power = lambda e: (e // 2) % 4
+    for e in range(experts):
+        s = 256 * (e % 2)
+        w_in[e, :inter] = np.roll(base_in[:inter], -s, axis=0)
+        w_in[e, inter:] = _scaled_d(np.roll(base_in[inter:], -s, axis=0), power(e))
+        w_out[e] = np.roll(np.roll(base_out, -8 * e, axis=0), -(s // 256), axis=1)
+    s_in = synth.matrix(Q4_K, 2 * inter, hidden, seed=203)
+    s_out = synth.matrix(Q4_K, hidden, inter, seed=204)
+    x = synth.activations(tokens, hidden, seed=205, f16=True) * np.float32(2.0 ** -9)
+    logits = synth.rng(206).standard_normal((tokens, experts)).astype(np.float32)
+
+    win = api.QuantizedExpertMatrix.new(d, w_in.reshape(-1), fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, w_out.reshape(-1), fmt, experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, s_in)
+    sout = api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, s_out)
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k), shared_input=sin, shared_output=sout)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
+    got = moe.forward(xt, api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)).to_f32()
+    assert d.last_operation() in ("expert_combine", "h_moe_combine", "expert_combine_shared")
+
+    code = oracle.F16
+    tile = code if tokens > 1 else 0                # one token runs on exact f32 weights
+    meta = oracle.select_routes(logits, experts, top_k)
+    up = oracle.round_storage(oracle.project(Q4_K, base_in.reshape(-1), 2 * inter, hidden, x, accumulate="f64",
+                                             weight_round=tile, threads=8), code)
+    act = oracle.expert_silu_mul(up, inter, code)
+    down = oracle.round_storage(oracle.project(Q4_K, base_out.reshape(-1), hidden, inter, act, accumulate="f64",
+                                               weight_round=tile, threads=8), code)
+    ids = meta[:, 0].copy().view(np.uint32)
+    toks = meta[:, 1].copy().view(np.uint32)
+    rows = np.stack([np.float32(2.0 ** power(int(e))) * np.roll(down[t], -8 * int(e)) for e, t in zip(ids, toks)])
+    sup = oracle.round_storage(oracle.project(Q4_K, s_in, 2 * inter, hidden, x, accumulate="f64", weight_round=tile,
+                                              threads=8), code)
+    sdown = oracle.round_storage(oracle.project(Q4_K, s_out, hidden, inter, oracle.expert_silu_mul(sup, inter, code),
+                                                accumulate="f64", weight_round=tile, threads=8), code)
+    want = oracle.expert_combine_shared(rows, meta, tokens, hidden, top_k, sdown, None, dtype=code)
+    assert np.isfinite(want).all() and np.abs(want).max() > 1e-3
+    if tokens > 1:
+        assert len(np.unique(ids)) == experts       # every expert is hit
+    assert rel_l2(got, want) <= 3e-3
+    per_token = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
+    assert per_token.max() <= 1e-2, int(per_token.argmax())
+
+
 # ------------------------------------------------------- decode-sized fusions
 
 @pytest.mark.parametrize("ggml,dtype", [(Q4_K, "F32"), (Q4_K, "F16"), (Q4_K, "BF16"), (Q6_K, "F16"), (Q6_K, "F32")])

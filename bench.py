@@ -9,14 +9,26 @@ recorded once into a HIP graph and replayed, so the timed region holds kernel
 launches only; HIP events on the library's own stream bracket it.
 
 ``value`` is algorithmic bytes per step / time per step.  ``roofline`` prices the
-GEMV kernel against the 8 TB/s HBM peak.  ``cases`` carries the other shapes of
-the dense-decode, Q6_K, small-M / prefill GEMM workloads (GB/s and TFLOP/s
-against both peaks), and ``cpu_baseline`` is the CPU oracle's sequential-fp32
-GEMV on the host's cores over a bounded number of repeats of the same step.
+GEMV kernel against the 8 TB/s HBM peak; its ``traffic`` is read from the HBM
+counter summary under ``profiles/`` when that summary was taken from the kernel
+sources as they are now, and is null otherwise.  ``cases`` carries the other
+shapes of the dense-decode, Q6_K, small-M / prefill GEMM and MoE workloads
+(GB/s and TFLOP/s against both peaks).  ``cpu_baseline`` is the CPU oracle on
+the host's cores over a bounded sample: the sequential-fp32 GEMV beside the
+metric, dequantize-once + blocked sgemm beside ``gemm_m512``, and the routed
+FFN chain beside the two MoE cases.
+
+``--cases read`` times a plain 128-bit read of the same rotating matrices (the
+HBM rate a kernel gets that does nothing with the bytes) and ``--cases mfma``
+times MFMA issue loops from registers (the matrix-core rate per instruction
+shape); ``--cases copy`` launches a row copy of known size, the calibration of
+the HBM counters.
 """
 from __future__ import annotations
 
 import argparse
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -34,10 +46,48 @@ Q8_0, Q4_K, Q5_K, Q6_K, IQ4_XS = 8, 12, 13, 14, 23
 BLOCK_BYTES = {Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}    # per 256 weights
 ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
 
-# HBM bytes per launch of the headline GEMV kernel from rocprofv3 counter runs:
-# FETCH_SIZE 24723.1 KiB x 1.94485 + WRITE_SIZE 68.0 KiB x 1.0, the factors being
-# known bytes / counter reading for the row-copy kernel of `--cases copy`.
-MEASURED_TRAFFIC_BYTES = 49319405
+CSRC = os.path.join(ROOT, "ferrum_amd", "csrc")
+GEMV_SOURCES = ("gemv_stream.hip", "gemv.hip", "device_utils.hpp")
+GEMM_SOURCES = ("gemm.hip", "tile_decode.hpp", "device_utils.hpp")
+
+
+def sources_digest(names):
+    """First 16 hex digits of the SHA-256 over the named kernel sources, in order."""
+    h = hashlib.sha256()
+    for name in names:
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload_key, names):
+    """HBM bytes per launch from the counter summaries under profiles/: a line
+    `traffic: workload=<key> sources=<digest> bytes=<n>` counts only while the
+    digest equals that of the kernel sources here, so a figure taken from an
+    older kernel is never reported for a newer one."""
+    digest = sources_digest(names)
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_counters.txt"))):
+        with open(path) as f:
+            for text in f:
+                if not text.startswith("traffic:"):
+                    continue
+                fields = dict(part.split("=", 1) for part in text.split()[1:] if "=" in part)
+                if fields.get("workload") == workload_key and fields.get("sources") == digest:
+                    return int(fields["bytes"])
+    return None
+
+
+def host_info():
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for text in f:
+                if text.lower().startswith("model name"):
+                    model = text.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "cpu_count": os.cpu_count()}
 
 
 def algorithmic_bytes(ggml, n, k, m, x_size, y_size):
@@ -130,20 +180,30 @@ def report(case, seconds_per_step):
     }
 
 
-def cpu_baseline(case, budget_seconds=12.0):
-    """The CPU oracle's sequential-fp32 GEMV on the same tensors, all host threads."""
-    import oracle
-    threads = max(1, min(16, os.cpu_count() or 1))
-    packed = case.packed.reshape(-1)
-    x = case.x_host
-    oracle.project(case.ggml, packed, case.n, case.k, x, threads=threads)  # page in
+def host_threads():
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def _repeat(fn, budget_seconds, limit=20000):
+    fn()   # page in
     runs, spent = 0, 0.0
-    while spent < budget_seconds and runs < 20000:
+    while spent < budget_seconds and runs < limit:
         t0 = time.perf_counter()
-        oracle.project(case.ggml, packed, case.n, case.k, x, threads=threads)
+        fn()
         spent += time.perf_counter() - t0
         runs += 1
-    per = spent / runs
+    return runs, spent / runs
+
+
+def cpu_baseline(case, budget_seconds=8.0):
+    """The CPU oracle's sequential-fp32 GEMV on the same tensors: all host threads
+    (`value`) and one thread."""
+    import oracle
+    threads = host_threads()
+    packed = case.packed.reshape(-1)
+    x = case.x_host
+    runs, per = _repeat(lambda: oracle.project(case.ggml, packed, case.n, case.k, x, threads=threads), budget_seconds)
+    runs1, per1 = _repeat(lambda: oracle.project(case.ggml, packed, case.n, case.k, x, threads=1), 4.0)
     return {
         "value": round(case.bytes / per / 1e9, 3),
         "unit": "GB/s",
@@ -151,7 +211,84 @@ def cpu_baseline(case, budget_seconds=12.0):
         "kind": "port",
         "sample": f"{runs} repeats of the same {case.label} step ({per * 1e3:.1f} ms each), "
                   f"dequant + sequential fp32 dot, rows split over {threads} threads",
+        "one_thread": {"value": round(case.bytes / per1 / 1e9, 3), "unit": "GB/s", "cores": 1,
+                       "sample": f"{runs1} repeats ({per1 * 1e3:.1f} ms each)"},
     }
+
+
+def cpu_baseline_gemm(case, sample_columns=1024):
+    """CPU figures for the prefill GEMM on the same tensors.  `value`: every
+    weight dequantized once by the oracle, then numpy's blocked sgemm over the
+    whole [M,K] x [K,N] product.  `oracle_sequential`: the oracle's own product
+    (each row dequantized once, then M sequential-fp32 dots) on a sample of the
+    output columns."""
+    import oracle
+    threads = host_threads()
+    blas_threads = None
+    try:
+        from threadpoolctl import threadpool_info
+        blas = [p.get("num_threads") for p in threadpool_info() if p.get("user_api") == "blas"]
+        blas_threads = blas[0] if blas else None
+    except Exception:
+        pass
+    x = np.ascontiguousarray(case.x_host, dtype=np.float32).reshape(case.m, case.k)
+    t0 = time.perf_counter()
+    w = oracle.dequantize(case.ggml, case.packed.reshape(-1), case.n, case.k)
+    t_dequant = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    y = x @ w.T
+    t_gemm = time.perf_counter() - t0
+    del w, y
+    total = t_dequant + t_gemm
+    cols = np.linspace(0, case.n - 1, sample_columns).astype(np.int64)
+    sub = np.ascontiguousarray(case.packed[cols]).reshape(-1)
+    t0 = time.perf_counter()
+    oracle.project(case.ggml, sub, len(cols), case.k, x, threads=threads)
+    t_seq = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    few = cols[: max(1, sample_columns // 8)]
+    oracle.project(case.ggml, np.ascontiguousarray(case.packed[few]).reshape(-1), len(few), case.k, x, threads=1)
+    t_seq1 = time.perf_counter() - t0
+    return {
+        "value": round(case.flops / total / 1e9, 1),
+        "unit": "GFLOP/s",
+        "cores": blas_threads or threads,
+        "kind": "port",
+        "sample": f"one whole {case.label} product: oracle dequantize of all {case.n}x{case.k} weights on one thread "
+                  f"({t_dequant:.2f} s) + numpy sgemm on {blas_threads or '?'} BLAS threads ({t_gemm:.2f} s)",
+        "sgemm_alone": {"value": round(case.flops / t_gemm / 1e9, 1), "unit": "GFLOP/s"},
+        "oracle_sequential": {
+            "value": round(2.0 * case.m * len(cols) * case.k / t_seq / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
+            "sample": f"{len(cols)} of {case.n} output columns, all {case.m} rows ({t_seq:.2f} s), "
+                      f"row dequantized once then sequential fp32 dots",
+            "one_thread": {"value": round(2.0 * case.m * len(few) * case.k / t_seq1 / 1e9, 2), "unit": "GFLOP/s",
+                           "cores": 1, "sample": f"{len(few)} columns ({t_seq1:.2f} s)"},
+        },
+    }
+
+
+def gemm_distance(api, dev, case, sample_columns=96):
+    """How far the tile GEMM's output is from the oracle on a sample of columns:
+    against the product with weights rounded to f16 first (what the tiles multiply)
+    and against the unrounded product, both accumulated in f64."""
+    import oracle
+    dev.project_quantized(case.x, case.weights[0], out=case.y)
+    dev.synchronize()
+    got = case.y.to_f32().reshape(case.m, case.n)
+    cols = np.unique(np.concatenate([np.linspace(0, case.n - 1, sample_columns).astype(np.int64),
+                                     np.arange(case.n - 8, case.n)]))
+    sub = np.ascontiguousarray(case.packed[cols]).reshape(-1)
+    x = np.ascontiguousarray(case.x_host, dtype=np.float32).reshape(case.m, case.k)
+    out = {}
+    for name, rounding in (("tile_rounded_oracle", oracle.F16), ("unrounded_oracle", 0)):
+        want = oracle.project(case.ggml, sub, len(cols), case.k, x, accumulate="f64", weight_round=rounding,
+                              threads=host_threads()).astype(np.float64)
+        diff = got[:, cols].astype(np.float64) - want
+        floor = float(np.sqrt(np.mean(want * want)))
+        out[name] = {"rel_l2": float(np.linalg.norm(diff) / np.linalg.norm(want)),
+                     "max_rel": float(np.max(np.abs(diff) / np.maximum(np.abs(want), floor)))}
+    out["sample"] = f"{len(cols)} of {case.n} columns, all {case.m} rows; max_rel = |err| / max(|ref|, rms(ref))"
+    return out
 
 
 def layer_case(api, synth, dev, steps, layers=4):
@@ -192,7 +329,7 @@ def layer_case(api, synth, dev, steps, layers=4):
     }
 
 
-def moe_case(api, synth, dev, tokens, steps):
+def moe_case(api, synth, dev, tokens, steps, cpu=True):
     """A3B-style routed FFN: hidden 2048, 256 experts x intermediate 512 in Q4_K,
     top-8 softmax routing with renormalised weights, plus one shared expert
     whose output the combine adds; f16 activations.  One step =
@@ -204,20 +341,24 @@ def moe_case(api, synth, dev, tokens, steps):
     f16, f32 = api.DType.F16, api.DType.F32
     eight_in = synth.matrix(Q4_K, 8 * 2 * inter, hidden, seed=11).reshape(8, -1)
     eight_out = synth.matrix(Q4_K, 8 * hidden, inter, seed=12).reshape(8, -1)
-    win = api.QuantizedExpertMatrix.new(dev, np.tile(eight_in, (experts // 8, 1)).reshape(-1), fmt,
-                                        experts, 2 * inter, hidden)
-    wout = api.QuantizedExpertMatrix.new(dev, np.tile(eight_out, (experts // 8, 1)).reshape(-1), fmt,
-                                         experts, hidden, inter)
-    sin = api.QuantizedMatrix.from_bytes(dev, 2 * inter, hidden, fmt, synth.matrix(Q4_K, 2 * inter, hidden, seed=13))
-    sout = api.QuantizedMatrix.from_bytes(dev, hidden, inter, fmt, synth.matrix(Q4_K, hidden, inter, seed=14))
+    packed_in = np.tile(eight_in, (experts // 8, 1)).reshape(-1)
+    packed_out = np.tile(eight_out, (experts // 8, 1)).reshape(-1)
+    shared_in = synth.matrix(Q4_K, 2 * inter, hidden, seed=13)
+    shared_out = synth.matrix(Q4_K, hidden, inter, seed=14)
+    win = api.QuantizedExpertMatrix.new(dev, packed_in, fmt, experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(dev, packed_out, fmt, experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(dev, 2 * inter, hidden, fmt, shared_in)
+    sout = api.QuantizedMatrix.from_bytes(dev, hidden, inter, fmt, shared_out)
     moe = api.SparseMoe(dev, win, wout, api.MoeRoutingPolicy(experts, top_k), shared_input=sin, shared_output=sout)
     moe.workspace(tokens, f16)
-    x = api.Tensor.from_f32(dev, (tokens, hidden), f16,
-                            synth.activations(tokens, hidden, seed=15, f16=True) * np.float32(2.0 ** -6))
+    x_host = synth.activations(tokens, hidden, seed=15, f16=True) * np.float32(2.0 ** -6)
+    x = api.Tensor.from_f32(dev, (tokens, hidden), f16, x_host)
     variants = 16
-    logit_sets, hit = [], []
+    logit_sets, hit, first_logits = [], [], None
     for i in range(variants):
         values = synth.rng(16, i).standard_normal((tokens, experts)).astype(np.float32)
+        if first_logits is None:
+            first_logits = values
         logit_sets.append(api.Tensor.from_f32(dev, values.shape, f32, values))
         hit.append(len(np.unique(np.argsort(-values, axis=1)[:, :top_k])))
     names = []
@@ -232,7 +373,36 @@ def moe_case(api, synth, dev, tokens, steps):
     act_bytes = tokens * hidden * 2 * 2 + tokens * experts * 4
     nbytes = mean_hit * per_expert + per_expert + act_bytes
     flops = 2 * tokens * (top_k + 1) * (2 * inter * hidden + hidden * inter)
+    cpu_line = None
+    if cpu:
+        # the same step on the CPU oracle, one thread, for a bounded number of the tokens
+        import oracle
+        sample = min(tokens, 8)
+        code = oracle.F16
+        xs = oracle.round_storage(x_host.reshape(tokens, hidden)[:sample], code).reshape(sample, hidden)
+
+        def chain():
+            meta = oracle.select_routes(first_logits[:sample], experts, top_k)
+            up = oracle.round_storage(oracle.expert_project(Q4_K, packed_in, experts, 2 * inter, hidden,
+                                                            oracle.expert_assign(xs, meta), meta), code)
+            down = oracle.round_storage(oracle.expert_project(Q4_K, packed_out, experts, hidden, inter,
+                                                              oracle.expert_silu_mul(up, inter, code), meta), code)
+            sup = oracle.round_storage(oracle.project(Q4_K, shared_in, 2 * inter, hidden, xs), code)
+            sdown = oracle.round_storage(oracle.project(Q4_K, shared_out, hidden, inter,
+                                                        oracle.expert_silu_mul(sup, inter, code)), code)
+            return oracle.expert_combine_shared(down, meta, sample, hidden, top_k, sdown, None, dtype=code)
+
+        runs, per = _repeat(chain, 4.0, limit=50)
+        per_token = per / sample
+        cpu_line = {
+            "value": round(flops / tokens / per_token / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "us_per_step": round(per_token * tokens * 1e6, 1),
+            "sample": f"{runs} repeats of the oracle chain (route, gate|up, SiLU*up, down, shared expert, combine) "
+                      f"over {sample} of the step's {tokens} tokens ({per * 1e3:.1f} ms each), scaled by tokens; "
+                      f"every assignment dequantizes its expert's rows, sequential fp32 dots, one thread",
+        }
     return {
+        "cpu_baseline": cpu_line,
         "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
         "operation": ("moe_route + 2 x (expert_project with the shared expert riding) + combine" if tokens * top_k <= 31
                       else "moe_route + 2 x (expert_project grouped, shared expert pieces inside) + 2 x silu_mul + combine"),
@@ -266,14 +436,59 @@ def copy_calibration(api, dev, rows=65536, width=1024, launches=10):
                       "copied_correctly": bool(same)}), flush=True)
 
 
+def read_probe_case(api, synth, dev, steps, warmup):
+    """The headline's rotating matrices read by a kernel that only loads them."""
+    head = Case(api, synth, dev, Q4_K, 17408, 5120, 1, api.DType.F32, "plain 128-bit read of the 17408x5120 Q4_K matrices")
+    head.enqueue = lambda i: dev.probe_read(head.weights[i % len(head.weights)])
+    _, event = measure(dev, head, steps, warmup)
+    per = event / steps
+    gemv = Case.__new__(Case)
+    gemv.__dict__.update(head.__dict__)
+    gemv.label = "Q4_K GEMV M=1 K=5120 N=17408 f32 x"
+    gemv.enqueue = lambda i: dev.project_quantized(gemv.x, gemv.weights[i % len(gemv.weights)], out=gemv.y)
+    _, gevent = measure(dev, gemv, steps, warmup)
+    gper = gevent / steps
+    print(json.dumps({
+        "read_probe": {"kernel": head.operation, "bytes_per_launch": head.weight_bytes, "us": round(per * 1e6, 3),
+                       "GB/s": round(head.weight_bytes / per / 1e9, 1),
+                       "frac_hbm": round(head.weight_bytes / per / 1e9 / HBM_PEAK_GBS, 4)},
+        "gemv_same_run": {"kernel": gemv.operation, "us": round(gper * 1e6, 3),
+                          "GB/s": round(gemv.bytes / gper / 1e9, 1),
+                          "frac_hbm": round(gemv.bytes / gper / 1e9 / HBM_PEAK_GBS, 4)},
+        "gemv_over_read": round(gper / per, 3),
+        "weight_copies_rotated": len(head.weights), "steps": steps}), flush=True)
+
+
+def mfma_probe_case(dev, steps):
+    """MFMA issue loops from registers, four waves per workgroup, four workgroups per CU."""
+    props = dev.properties()
+    groups = 4 * int(props.get("compute_units") or 256)
+    iterations = 4096
+    out = {}
+    for shape, name in ((0, "v_mfma_f32_16x16x32_f16"), (1, "v_mfma_f32_32x32x16_f16")):
+        flops = [0.0]
+
+        def enqueue(i):
+            flops[0] = dev.probe_mfma(shape, groups, iterations)
+
+        best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(3)) / steps
+        out[name] = {"kernel": dev.last_operation(), "us": round(best * 1e6, 2),
+                     "TFLOP/s": round(flops[0] / best / 1e12, 1),
+                     "frac_published_peak": round(flops[0] / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+    print(json.dumps({"mfma_probe": out, "workgroups": groups, "waves_per_workgroup": 4,
+                      "independent_chains_per_wave": 8, "iterations": iterations}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2400)
     ap.add_argument("--warmup", type=int, default=240)
-    ap.add_argument("--cases", choices=["headline", "all", "copy"], default="all",
+    ap.add_argument("--cases", choices=["headline", "all", "copy", "read", "mfma"], default="all",
                     help="'headline' times only the metric's GEMV; 'all' adds the other shapes; "
-                         "'copy' launches a plain row copy of known size (counter calibration)")
+                         "'copy' launches a plain row copy of known size (counter calibration); "
+                         "'read' times a plain read of the metric's matrices beside the GEMV; "
+                         "'mfma' times matrix-core issue loops")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="with --cases all: run only the cases whose label contains this text")
     ap.add_argument("--eager", action="store_true",
@@ -292,6 +507,10 @@ def main():
     f32, f16 = api.DType.F32, api.DType.F16
     if args.cases == "copy":
         return copy_calibration(api, dev)
+    if args.cases == "read":
+        return read_probe_case(api, synth, dev, args.steps, args.warmup)
+    if args.cases == "mfma":
+        return mfma_probe_case(dev, min(args.steps, 20))
 
     head = Case(api, synth, dev, Q4_K, 17408, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=17408 f32 x")
     wall, event = measure(dev, head, args.steps, args.warmup)
@@ -304,15 +523,24 @@ def main():
     cases = [head_report]
     gemm = None
     if args.cases == "all":
-        def timed(ggml, n, k, m, xd, label, steps, copies=None):
+        def timed(ggml, n, k, m, xd, label, steps, copies=None, after=None):
             if args.only and args.only not in label:
                 return None
             c = Case(api, synth, dev, ggml, n, k, m, xd, label, copies)
             _, ev = measure(dev, c, steps, min(args.warmup, len(c.weights)), repeats=2)
             r = report(c, ev / steps)
             cases.append(r)
+            if after is not None:
+                after(c)
             del c
             return r
+
+        gemm_extra = {}
+
+        def gemm_checks(c):
+            gemm_extra["distance_to_oracle"] = gemm_distance(api, dev, c)
+            if not args.no_cpu:
+                gemm_extra["cpu_baseline"] = cpu_baseline_gemm(c)
 
         timed(Q4_K, 4096, 4096, 1, f32, "Q4_K GEMV M=1 K=4096 N=4096", 1200)
         timed(Q4_K, 5120, 5120, 1, f32, "Q4_K GEMV M=1 K=5120 N=5120", 1200)
@@ -326,7 +554,7 @@ def main():
         timed(Q6_K, 151936, 5120, 1, f32, "Q6_K GEMV M=1 K=5120 N=151936", 40, copies=2)
         for m in (8, 16, 128):
             timed(Q4_K, 17408, 5120, m, f16, f"Q4_K GEMM M={m} K=5120 N=17408 f16 x", 240)
-        gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240)
+        gemm = timed(Q4_K, 17408, 5120, 512, f16, "Q4_K GEMM M=512 K=5120 N=17408 f16 x", 240, after=gemm_checks)
         for m in (8, 512):
             timed(IQ4_XS, 17408, 5120, m, f16, f"IQ4_XS GEMM M={m} K=5120 N=17408 f16 x", 240)
             timed(Q8_0, 17408, 5120, m, f16, f"Q8_0 GEMM M={m} K=5120 N=17408 f16 x", 240)
@@ -338,9 +566,9 @@ def main():
         for m in (8, 64, 512):
             timed(Q4_K, 4096, 2048, m, f16, f"Q4_K GEMM M={m} K=2048 N=4096 f16 x", 400)
         if not args.only or args.only in "MoE FFN T=1":
-            cases.append(moe_case(api, synth, dev, 1, 200))
+            cases.append(moe_case(api, synth, dev, 1, 200, cpu=not args.no_cpu))
         if not args.only or args.only in "MoE FFN T=512":
-            cases.append(moe_case(api, synth, dev, 512, 20))
+            cases.append(moe_case(api, synth, dev, 512, 20, cpu=not args.no_cpu))
 
     line = {
         "metric": "Q4_K GEMV GB/s at M=1, K=5120, N=17408",
@@ -361,14 +589,17 @@ def main():
             "weight_copies_rotated": len(head.weights),
             "bytes_per_step": head.bytes,
             "device": props.get("name") or props.get("arch"),
+            "arch": props.get("arch"),
+            "compute_units": props.get("compute_units"),
         },
+        "host": host_info(),
         "roofline": {
             "bound": "hbm",
             "achieved": round(kernel_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(kernel_gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES,
+            "traffic": measured_traffic("gemv_q4k_n17408_k5120_m1", GEMV_SOURCES),
             "kernel": head.operation,
             "kernel_us": round(step_event * 1e6, 3),
         },
@@ -378,8 +609,11 @@ def main():
             "value": gemm["TFLOP/s"],
             "unit": "TFLOP/s",
             "roofline": {"bound": "mfma", "achieved": gemm["TFLOP/s"], "peak": MFMA_F16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": gemm["frac_mfma_f16"], "traffic": None,
+                         "unit": "TFLOP/s", "frac": gemm["frac_mfma_f16"],
+                         "traffic": measured_traffic("gemm_q4k_n17408_k5120_m512", GEMM_SOURCES),
                          "kernel": gemm["operation"], "kernel_us": gemm["us"]},
+            "cpu_baseline": gemm_extra.get("cpu_baseline"),
+            "distance_to_oracle": gemm_extra.get("distance_to_oracle"),
         },
         "cases": cases,
     }

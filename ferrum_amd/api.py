@@ -114,6 +114,8 @@ SYMBOLS = {
     "fh_embedding_gather_quantized": (_I32, [_P, _P, ctypes.POINTER(_U32), _SZ, _VP]),
     "fh_project_quantized": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_project_quantized_no_alloc": (_I32, [_P, _P, _VP, _U32, _VP]),
+    "fh_probe_read": (_I32, [_P, _P]),
+    "fh_probe_mfma": (_I32, [_P, _U32, _U32, _U32, ctypes.POINTER(ctypes.c_double)]),
     "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_add_rmsnorm": (_I32, [_P, _VP, _VP, _VP, _U32, _U32, ctypes.c_float, _VP, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
@@ -606,6 +608,18 @@ class Device:
         _check(_lib.fh_project_quantized_no_alloc(self._handle, _handle_of(weight), ctypes.byref(xv), dims[0],
                                                   ctypes.byref(yv)))
         return Output(out, self.last_operation(), a.byte_size() + weight.byte_size(), out.byte_size())
+
+    def probe_read(self, weight) -> None:
+        """fh_probe_read: reads every byte of a resident matrix with 128-bit loads and
+        writes nothing (a measurement kernel; the reference has none)."""
+        _check(_lib.fh_probe_read(self._handle, _handle_of(weight)))
+
+    def probe_mfma(self, shape: int, groups: int, iterations: int) -> float:
+        """fh_probe_mfma: an MFMA issue loop from registers (shape 0 = 16x16x32 f16,
+        1 = 32x32x16 f16); returns the floating-point operations of the launch."""
+        flops = ctypes.c_double()
+        _check(_lib.fh_probe_mfma(self._handle, shape, groups, iterations, ctypes.byref(flops)))
+        return float(flops.value)
 
     def argmax_rows(self, logits: Tensor) -> Tensor:
         """[rows, 2] F32 carrier of u32 bits: first maximal index and a non-finite flag

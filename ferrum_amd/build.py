@@ -17,7 +17,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libferrum_hip.so")
 
-SOURCES = ["capi.hip", "dequant.hip", "gemv.hip", "gemv_stream.hip", "gemm.hip", "gemm_skinny.hip", "moe.hip", "norm.hip"]
+SOURCES = ["capi.hip", "dequant.hip", "gemv.hip", "gemv_stream.hip", "probe.hip", "gemm.hip", "gemm_skinny.hip", "moe.hip", "norm.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

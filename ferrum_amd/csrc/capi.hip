@@ -304,6 +304,9 @@ fh_status fh_device_properties(const fh_device* device, fh_device_props* out) {
     if (device == nullptr || out == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     std::memset(out, 0, sizeof(*out));
     std::snprintf(out->name, sizeof(out->name), "%s", device->props.name);
+    if (out->name[0] == '\0')   // some driver stacks leave the marketing name empty
+        std::snprintf(out->name, sizeof(out->name), "%.40s, %d CUs, %.0f GiB", device->props.gcnArchName,
+                      device->props.multiProcessorCount, (double)device->props.totalGlobalMem / (1 << 30));
     std::snprintf(out->arch, sizeof(out->arch), "%s", device->props.gcnArchName);
     out->compute_units = device->props.multiProcessorCount;
     out->wavefront = device->props.warpSize;
@@ -731,6 +734,31 @@ fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* wei
         a.partials = reinterpret_cast<float*>(base + kFixedCounterWords * sizeof(uint32_t));
     }
     device->last_operation = launch_gemv(device->stream, a);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+// ---- measurement ----------------------------------------------------------------------
+
+fh_status fh_probe_read(fh_device* device, const fh_qmatrix* weight) {
+    if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (weight->device != device) return fail(FH_ERR_PARAMETER, "matrix belongs to another device");
+    fh_status st = ensure_scratch(device, 0);
+    if (st != FH_OK) return st;
+    device->last_operation = launch_read_probe(device->stream, weight->ptr, weight->bytes,
+                                               reinterpret_cast<uint32_t*>(scratch_data(device)));
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_probe_mfma(fh_device* device, uint32_t shape, uint32_t groups, uint32_t iterations, double* flops) {
+    if (device == nullptr || flops == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (shape > 1 || groups == 0 || groups > 65535 || iterations == 0)
+        return fail(FH_ERR_SHAPE, "mfma probe: shape 0 or 1, 1..65535 workgroups, at least one iteration");
+    fh_status st = ensure_scratch(device, (size_t)groups * 256 * sizeof(float));
+    if (st != FH_OK) return st;
+    device->last_operation = launch_mfma_probe(device->stream, (int)shape, groups, iterations,
+                                               reinterpret_cast<float*>(scratch_data(device)), flops);
     FH_HIP(hipGetLastError());
     return FH_OK;
 }

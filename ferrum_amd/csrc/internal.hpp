@@ -106,6 +106,11 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                                     const uint32_t* ids_dev, size_t count, void* out,
                                     uint32_t out_dtype);
 
+// probe.hip: measurement kernels (a plain 128-bit read of a buffer; an MFMA issue loop)
+const char* launch_read_probe(hipStream_t s, const void* data, size_t bytes, uint32_t* sink);
+const char* launch_mfma_probe(hipStream_t s, int shape, uint32_t groups, uint32_t iterations, float* sink,
+                              double* flops);
+
 // norm.hip
 // residual = round(a + b), normed = rmsnorm(residual) * weight; all operands of one dtype,
 // no output overlapping an operand or the other output.

@@ -1,0 +1,104 @@
+// Measurement kernels: what the device does with no operator attached.
+//
+//  * read_probe: every lane loads 8 x 16 bytes that its wave covers contiguously and
+//    xors them; nothing is written.  Its time over a buffer is what HBM delivers to a
+//    kernel that does nothing with the bytes, the figure a streaming GEMV is read
+//    against.
+//  * mfma_probe: every wave issues `iterations` rounds of eight independent MFMA
+//    chains on register operands and stores one float at the end.  Its rate is what the
+//    matrix cores sustain for one instruction shape, the figure a tile GEMM is read
+//    against.
+//
+// Neither has a counterpart in the reference; both are launched by the benchmark only.
+#include "internal.hpp"
+
+namespace fh {
+namespace {
+
+constexpr int kReadUnroll = 8;
+
+__global__ __launch_bounds__(256) void read_probe(const uint4* __restrict__ p, size_t n16,
+                                                  uint32_t* __restrict__ sink) {
+    const size_t base = (size_t)blockIdx.x * 256 * kReadUnroll + threadIdx.x;
+    uint4 v[kReadUnroll];
+#pragma unroll
+    for (int i = 0; i < kReadUnroll; ++i) {
+        const size_t idx = base + (size_t)i * 256;
+        v[i] = idx < n16 ? p[idx] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t a = 0;
+#pragma unroll
+    for (int i = 0; i < kReadUnroll; ++i) a ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    // the store keeps the loads alive; one lane in 2^32 takes it on random data, into scratch
+    if (a == 0x9e3779b9u) sink[0] = a;
+}
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kChains = 8;
+
+// SHAPE 0: v_mfma_f32_16x16x32_f16 (16384 flop), SHAPE 1: v_mfma_f32_32x32x16_f16 (32768 flop)
+template <int SHAPE>
+__global__ __launch_bounds__(256) void mfma_probe(uint32_t iterations, float seed, float* __restrict__ sink) {
+    half8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a[i] = (_Float16)(seed * (float)((threadIdx.x + i) & 7));
+        b[i] = (_Float16)(seed * (float)((threadIdx.x * 3 + i) & 7));
+    }
+    float total = 0.0f;
+    if constexpr (SHAPE == 0) {
+        float4v acc[kChains];
+#pragma unroll
+        for (int c = 0; c < kChains; ++c) acc[c] = float4v{0, 0, 0, 0};
+        for (uint32_t it = 0; it < iterations; ++it) {
+#pragma unroll
+            for (int c = 0; c < kChains; ++c)
+                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < kChains; ++c) total += acc[c][0] + acc[c][1] + acc[c][2] + acc[c][3];
+    } else {
+        float16v acc[kChains];
+#pragma unroll
+        for (int c = 0; c < kChains; ++c)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[c][j] = 0.0f;
+        for (uint32_t it = 0; it < iterations; ++it) {
+#pragma unroll
+            for (int c = 0; c < kChains; ++c)
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < kChains; ++c)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) total += acc[c][j];
+    }
+    sink[blockIdx.x * 256 + threadIdx.x] = total;
+}
+
+}  // namespace
+
+const char* launch_read_probe(hipStream_t stream, const void* data, size_t bytes, uint32_t* sink) {
+    const size_t n16 = bytes / 16;
+    const size_t per_group = (size_t)256 * kReadUnroll;
+    const unsigned groups = (unsigned)((n16 + per_group - 1) / per_group);
+    read_probe<<<dim3(groups), dim3(256), 0, stream>>>(static_cast<const uint4*>(data), n16, sink);
+    return "read_probe";
+}
+
+const char* launch_mfma_probe(hipStream_t stream, int shape, uint32_t groups, uint32_t iterations,
+                              float* sink, double* flops) {
+    const double per = shape == 0 ? 2.0 * 16 * 16 * 32 : 2.0 * 32 * 32 * 16;
+    *flops = per * kChains * (double)iterations * 4.0 * groups;
+    if (shape == 0) {
+        mfma_probe<0><<<dim3(groups), dim3(256), 0, stream>>>(iterations, 0x1p-10f, sink);
+        return "mfma_probe_16x16x32_f16";
+    }
+    mfma_probe<1><<<dim3(groups), dim3(256), 0, stream>>>(iterations, 0x1p-10f, sink);
+    return "mfma_probe_32x32x16_f16";
+}
+
+}  // namespace fh

@@ -23,6 +23,7 @@ import enum
 import math
 import os
 import sys
+import time
 from dataclasses import dataclass
 
 import numpy as np
@@ -457,6 +458,34 @@ class MoeRoutingPolicy:
                        self.routed_scaling_factor)
 
 
+@dataclass
+class MoeStats:
+    """What SparseMoe.forward did since the last take_stats (MoeStats, src/nn/moe.rs:75-116).
+    Durations are host seconds spent enqueueing; routing runs on the device, so the set of
+    active experts is never read back and `active_experts_known` turns false with the first
+    forward pass."""
+    router_projection_enqueue: float = 0.0
+    routing: float = 0.0
+    routing_boundary_wait: float = 0.0
+    expert_dispatch: float = 0.0
+    combine_dispatch: float = 0.0
+    active_experts: int = 0
+    active_experts_known: bool = True
+    assignments: int = 0
+    peak_temporary_bytes: int = 0
+
+    def merge(self, other: "MoeStats") -> None:
+        self.router_projection_enqueue += other.router_projection_enqueue
+        self.routing += other.routing
+        self.routing_boundary_wait += other.routing_boundary_wait
+        self.expert_dispatch += other.expert_dispatch
+        self.combine_dispatch += other.combine_dispatch
+        self.active_experts += other.active_experts
+        self.active_experts_known = self.active_experts_known and other.active_experts_known
+        self.assignments += other.assignments
+        self.peak_temporary_bytes = max(self.peak_temporary_bytes, other.peak_temporary_bytes)
+
+
 class Event:
     def __init__(self, device: "Device"):
         handle = ctypes.c_void_p()
@@ -552,6 +581,14 @@ class Device:
 
     def set_k_quant_gemv_ksplit(self, simds: int):
         self.set_tuning("k_quant_gemv_ksplit", simds)
+
+    def set_moe_routing_temporary_limit(self, nbytes: int):
+        """Bound on the routing temporaries of one SparseMoe chunk
+        (set_moe_routing_temporary_limit, src/metal/legacy.rs:520-534; 128 MiB at first)."""
+        self.set_tuning("moe_routing_temporary_limit", nbytes)
+
+    def moe_routing_temporary_limit(self) -> int:
+        return self.get_tuning("moe_routing_temporary_limit")
 
     def event(self) -> Event:
         return Event(self)
@@ -1010,6 +1047,7 @@ class SparseMoe:
                               and shared_input.format().ggml_type() == input_experts.format().ggml_type()
                               and shared_output.format().ggml_type() == output_experts.format().ggml_type())
         self._ws = None
+        self._stats = MoeStats()
         # most f32 assignments that take the fused per-assignment kernels (f32 rows have no
         # grouped form by default, and the per-assignment SiLU is recomputed by every workgroup);
         # also the most assignments whose shared expert rides in the routed launches
@@ -1034,17 +1072,64 @@ class SparseMoe:
                              "shared_output": Tensor.zeros(d, (tokens, h), dtype)})
         return self._ws
 
+    def take_stats(self) -> MoeStats:
+        """The statistics gathered since the last call, which start afresh (take_stats,
+        src/nn/moe.rs:218-220)."""
+        taken, self._stats = self._stats, MoeStats()
+        return taken
+
+    def temporary_bytes(self, tokens: int, dtype: DType) -> int:
+        """Routing temporaries of `tokens` tokens as the reference counts them
+        (src/nn/moe.rs:232-249, :306-316): per assignment the assigned row, the gate|up
+        row, the activated row and the projected output row plus one routing record; per
+        token its logits and its combined row."""
+        per_assignment = (2 * self.hidden_size + 3 * self.intermediate_size) * dtype.size_bytes() + 12
+        per_token = per_assignment * self.routing.top_k + (self.expert_count + self.hidden_size) * dtype.size_bytes()
+        return tokens * per_token
+
     def forward(self, hidden: Tensor, router_logits: Tensor, shared_gate: Tensor | None = None) -> Tensor:
+        """Tokens are taken in chunks whose routing temporaries stay under the device's
+        moe_routing_temporary_limit (src/nn/moe.rs:250-256); every chunk's combine writes its
+        rows of one output tensor, so nothing is read back between chunks."""
         dims = hidden.shape()
         if len(dims) != 2 or dims[1] != self.hidden_size or dims[0] == 0:
             raise ShapeError("sparse expert input requires [tokens,hidden]")
         if hidden.buffer.device is not self.device:
             raise DeviceMismatch("tensor belongs to another device")
+        if router_logits.shape() != (dims[0], self.expert_count):
+            raise ShapeError("router logits require [tokens,experts]")
+        if shared_gate is not None and shared_gate.numel() != dims[0]:
+            raise ShapeError("shared gate requires one value per token")
+        tokens = dims[0]
+        per_token = self.temporary_bytes(1, hidden.dtype)
+        chunk_tokens = min(tokens, max(1, self.device.moe_routing_temporary_limit() // per_token))
+        stats = MoeStats(active_experts_known=False)
+        if chunk_tokens == tokens:
+            ws = self._ws if self._ws and self._ws["tokens"] == tokens and self._ws["dtype"] == hidden.dtype else {}
+            out = self._forward_chunk(hidden, router_logits, shared_gate, ws, None, stats)
+        else:
+            out = Tensor.zeros(self.device, (tokens, self.hidden_size), hidden.dtype)
+            for start in range(0, tokens, chunk_tokens):
+                count = min(chunk_tokens, tokens - start)
+                gate = None if shared_gate is None else shared_gate.view(start, (count,))
+                self._forward_chunk(hidden.view(start * self.hidden_size, (count, self.hidden_size)),
+                                    router_logits.view(start * self.expert_count, (count, self.expert_count)),
+                                    gate, {}, out.view(start * self.hidden_size, (count, self.hidden_size)), stats)
+        self._stats.merge(stats)
+        return out
+
+    def _forward_chunk(self, hidden, router_logits, shared_gate, ws, out, stats):
+        dims = hidden.shape()
         d, k = self.device, self.routing.top_k
-        ws = self._ws if self._ws and self._ws["tokens"] == dims[0] and self._ws["dtype"] == hidden.dtype else {}
+        stats.assignments += dims[0] * k
+        stats.peak_temporary_bytes = max(stats.peak_temporary_bytes, self.temporary_bytes(dims[0], hidden.dtype))
+        combined = out if out is not None else ws.get("combined")
+        t0 = time.perf_counter()
         metadata = d.moe_route(router_logits, self.selection_bias, self.routing, out=ws.get("metadata"))
+        t1 = time.perf_counter()
+        stats.routing += t1 - t0
         if self.shared_input is not None:
-            return self._forward_with_shared(hidden, metadata, shared_gate, ws)
+            return self._forward_with_shared(hidden, metadata, shared_gate, ws, combined, stats, t1)
         if self.fuse_inputs and (dims[0] * k <= self.fused_max_assignments or hidden.dtype != DType.F32):
             # the copy and the activation ride inside the projections: per assignment in
             # decode, and in the grouped kernel's gather of an expert's rows beyond it
@@ -1061,10 +1146,13 @@ class SparseMoe:
             expert_output = d.expert_project_quantized(activated, metadata, self.output_experts,
                                                        self.intermediate_size, self.expert_count,
                                                        out=ws.get("expert_output"))
-        return d.expert_combine(expert_output, metadata, dims[0], self.hidden_size, k,
-                                out=ws.get("combined"))
+        t2 = time.perf_counter()
+        stats.expert_dispatch += t2 - t1
+        result = d.expert_combine(expert_output, metadata, dims[0], self.hidden_size, k, out=combined)
+        stats.combine_dispatch += time.perf_counter() - t2
+        return result
 
-    def _forward_with_shared(self, hidden, metadata, shared_gate, ws):
+    def _forward_with_shared(self, hidden, metadata, shared_gate, ws, combined, stats, t1):
         d, k, tokens = self.device, self.routing.top_k, hidden.shape()[0]
         a = tokens * k
         if self.fuse_inputs and self._shared_rides and (a <= self.fused_max_assignments or hidden.dtype != DType.F32):
@@ -1101,8 +1189,12 @@ class SparseMoe:
                                                      out=ws.get("shared_activated"))
                 shared_output = d.project_quantized(shared_activated, self.shared_output,
                                                     out=ws.get("shared_output")).tensor
-        return d.expert_combine_shared(expert_output, metadata, tokens, self.hidden_size, k, shared_output,
-                                       shared_gate, out=ws.get("combined"))
+        t2 = time.perf_counter()
+        stats.expert_dispatch += t2 - t1
+        result = d.expert_combine_shared(expert_output, metadata, tokens, self.hidden_size, k, shared_output,
+                                         shared_gate, out=combined)
+        stats.combine_dispatch += time.perf_counter() - t2
+        return result
 
 
 def _handle_of(weight):

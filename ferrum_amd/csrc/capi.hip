@@ -253,6 +253,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
     d->tuning["gemv_stream"] = 1;           // dense Q4_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
+    d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
     fh_status st = ensure_scratch(d, 0);
     if (st == FH_OK) {
@@ -356,6 +357,9 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 0;
     } else if (k == "gemm_f32_min_rows") {
         ok = value == 0 || value >= 2;
+    } else if (k == "moe_routing_temporary_limit") {
+        // set_moe_routing_temporary_limit (src/metal/legacy.rs:523-531): positive, on an idle device
+        ok = value > 0 && !device->capturing;
     }
     if (!ok) return fail(FH_ERR_PARAMETER, "value %lld is out of range for %s", (long long)value, key);
     it->second = value;

@@ -297,8 +297,10 @@ __global__ __launch_bounds__(kSkThreads) void gemm_skinny_kernel(const uint8_t* 
     uint32_t first_token = 0, count = m;
     size_t expert_row = 0;
     if constexpr (GROUPED) {
-        first_token = offsets[blockIdx.y];
-        count = offsets[blockIdx.y + 1] - first_token;
+        // a damaged offsets table reads wrong rows, never rows outside the m assignments
+        first_token = min(offsets[blockIdx.y], m);
+        const uint32_t upto = min(offsets[blockIdx.y + 1], m);
+        count = upto > first_token ? upto - first_token : 0;
         expert_row = (size_t)blockIdx.y * n;
     }
     const uint8_t* wrow = w + (expert_row + row) * nb * kBB;
@@ -455,7 +457,8 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
                                                                      const uint32_t* __restrict__ order,
                                                                      uint32_t tiles_per_wg,
                                                                      const float* __restrict__ metadata,
-                                                                     uint32_t x_rows, const ResidentShared sh) {
+                                                                     uint32_t x_rows, uint32_t routes,
+                                                                     const ResidentShared sh) {
     constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
     constexpr int kTokens = 16 * TT;
     extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
@@ -467,8 +470,10 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
     // (and the sixteen consecutive pieces a gather write covers) fall on different banks.
     const uint32_t k = nb * 256, ld = k;
     // no offsets: a dense product, all of it shared-expert pieces
-    const uint32_t expert_first = offsets != nullptr ? offsets[blockIdx.y] : 0;
-    const uint32_t count = offsets != nullptr ? offsets[blockIdx.y + 1] - expert_first : 0;
+    // a damaged offsets table reads wrong rows, never rows outside the `routes` assignments
+    const uint32_t expert_first = offsets != nullptr ? min(offsets[blockIdx.y], routes) : 0;
+    const uint32_t expert_upto = offsets != nullptr ? min(offsets[blockIdx.y + 1], routes) : 0;
+    const uint32_t count = expert_upto > expert_first ? expert_upto - expert_first : 0;
     const uint32_t tiles = (n + 15) / 16;
     const uint32_t pieces = k / 8;  // 16-byte pieces per activation row
 
@@ -653,13 +658,13 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, nullptr, x, nullptr, a.n, nb, a.y_dtype,
-                               nullptr, nullptr, 0u, nullptr, 0u, sh);
+                               nullptr, nullptr, 0u, nullptr, 0u, 0u, sh);
         } else {
             auto kernel = expert_resident_kernel<TYPE, DT, 1>;
             (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, nullptr, x, nullptr, a.n, nb, a.y_dtype,
-                               nullptr, nullptr, 0u, nullptr, 0u, sh);
+                               nullptr, nullptr, 0u, nullptr, 0u, 0u, sh);
         }
         return;
     }
@@ -695,13 +700,13 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, sh);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, a.m, sh);
             } else {
                 auto kernel = expert_resident_kernel<TYPE, DT, 1>;
                 (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
                 hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), lds, s, w, x, a.y, a.n, nb, a.y_dtype,
-                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, sh);
+                                   a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, a.m, sh);
             }
             return;
         }

@@ -58,7 +58,12 @@ enum { FH_F32 = 0, FH_F16 = 1, FH_BF16 = 2 };
  * and Q8_0 are the hybrid engine's Format::Iq4Xs and Format::Q8_0,
  * src/hybrid/weights.rs:29-60: 136-byte blocks of 256 weights and 34-byte
  * blocks of 32, src/loader/gguf.rs:91-121).  Rows are a multiple of 256
- * weights long in every format; for Q8_0 that is eight blocks, 272 bytes. */
+ * weights long in every format; for Q8_0 that is eight blocks, 272 bytes.
+ * The reference takes Q8_0 rows of any multiple of 32 weights
+ * (src/hybrid/weights.rs:29-51); this library refuses the ones that are not a
+ * multiple of 256 long: fh_qmatrix_create returns FH_ERR_SHAPE for them and
+ * nothing is uploaded.  Every model dimension the reference's loaders produce
+ * is a multiple of 256. */
 enum { FH_GGML_Q8_0 = 8, FH_GGML_Q4_K = 12, FH_GGML_Q5_K = 13, FH_GGML_Q6_K = 14, FH_GGML_IQ4_XS = 23 };
 
 typedef struct fh_device fh_device;

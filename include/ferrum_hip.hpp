@@ -13,6 +13,8 @@
 #ifndef FERRUM_HIP_HPP
 #define FERRUM_HIP_HPP
 
+#include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -263,6 +265,15 @@ public:
     std::string last_operation() const { return fh_last_operation(handle_->raw); }
     void set_k_quant_gemv_ksplit(int64_t simds) const { check(fh_set_tuning(handle_->raw, "k_quant_gemv_ksplit", simds)); }
     void set_tuning(const char* key, int64_t value) const { check(fh_set_tuning(handle_->raw, key, value)); }
+    int64_t get_tuning(const char* key) const {
+        int64_t value = 0;
+        check(fh_get_tuning(handle_->raw, key, &value));
+        return value;
+    }
+    // Bound on the routing temporaries of one SparseMoe chunk (set_moe_routing_temporary_limit,
+    // src/metal/legacy.rs:520-534; 128 MiB at first).
+    void set_moe_routing_temporary_limit(size_t bytes) const { set_tuning("moe_routing_temporary_limit", (int64_t)bytes); }
+    size_t moe_routing_temporary_limit() const { return (size_t)get_tuning("moe_routing_temporary_limit"); }
     bool owns(const Tensor& t) const { return t.buffer_ && t.buffer_->owner == handle_; }
 
     // ---- tensors ----
@@ -673,6 +684,29 @@ private:
     std::shared_ptr<detail::DeviceHandle> handle_;
 };
 
+// What SparseMoe::forward did since the last take_stats (MoeStats, src/nn/moe.rs:75-116).
+// Durations are host seconds spent enqueueing.  Routing runs on the device, so the set of
+// active experts is never read back and active_experts_known turns false with the first pass.
+struct MoeStats {
+    double router_projection_enqueue = 0, routing = 0, routing_boundary_wait = 0, expert_dispatch = 0,
+           combine_dispatch = 0;
+    size_t active_experts = 0;
+    bool active_experts_known = true;
+    size_t assignments = 0;
+    size_t peak_temporary_bytes = 0;
+    void merge(const MoeStats& other) {
+        router_projection_enqueue += other.router_projection_enqueue;
+        routing += other.routing;
+        routing_boundary_wait += other.routing_boundary_wait;
+        expert_dispatch += other.expert_dispatch;
+        combine_dispatch += other.combine_dispatch;
+        active_experts += other.active_experts;
+        active_experts_known = active_experts_known && other.active_experts_known;
+        assignments += other.assignments;
+        peak_temporary_bytes = std::max(peak_temporary_bytes, other.peak_temporary_bytes);
+    }
+};
+
 // SparseMoe::forward without the router's own dense layer: the caller passes
 // the router logits (that layer is outside the quantized path).
 class SparseMoe {
@@ -698,33 +732,49 @@ public:
         shared_input_ = std::move(input);
         shared_output_ = std::move(output);
     }
+    // Routing temporaries of `tokens` tokens as the reference counts them (src/nn/moe.rs:232-249,
+    // :306-316): per assignment the assigned, gate|up, activated and output rows plus one routing
+    // record; per token its logits and its combined row.
+    size_t temporary_bytes(size_t tokens, DType dtype) const {
+        const size_t h = input_.columns(), i = input_.rows_per_expert() / 2, e = input_.experts();
+        const size_t per_assignment = (2 * h + 3 * i) * size_bytes(dtype) + 3 * sizeof(float);
+        return tokens * (per_assignment * routing_.top_k + (e + h) * size_bytes(dtype));
+    }
+    // The statistics gathered since the last call, which start afresh (take_stats, src/nn/moe.rs:218-220).
+    MoeStats take_stats() const {
+        MoeStats taken = stats_;
+        stats_ = MoeStats{};
+        return taken;
+    }
+    // Tokens are taken in chunks whose routing temporaries stay under the device's
+    // moe_routing_temporary_limit (src/nn/moe.rs:250-256); every chunk's combine writes its rows of
+    // one output tensor, so nothing is read back between chunks.
     Tensor forward(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias = nullptr,
                    const Tensor* shared_gate = nullptr) const {
         const auto& dims = hidden.shape();
-        const size_t h = input_.columns(), i = input_.rows_per_expert() / 2, e = input_.experts();
+        const size_t h = input_.columns(), e = input_.experts();
         if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
             throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
-        Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
-        if (shared_input_) {
-            const size_t tokens = dims[0], a = tokens * routing_.top_k;
-            if (fuse_inputs && shared_rides_ && (a <= fused_max_assignments || hidden.dtype() != DType::F32)) {
-                // four launches: the shared expert's rows are batch entries of the routed ones in
-                // decode and further token groups of the grouped kernel beyond it
-                auto up = device_.expert_project_with_shared(hidden, meta, input_, *shared_input_, tokens, FH_INPUT_GATHER);
-                auto down = device_.expert_project_with_shared(up.first, meta, output_, *shared_output_, tokens,
-                                                               FH_INPUT_SILU_MUL, &up.second);
-                return device_.expert_combine_shared(down.first, meta, tokens, h, routing_.top_k, down.second, shared_gate);
-            }
-            Tensor expert_output = routed(hidden, meta, h, i, e);
-            Tensor shared_projected = device_.project_quantized(hidden, *shared_input_).tensor;
-            Tensor shared_output =
-                fuse_inputs && tokens <= fused_max_assignments
-                    ? device_.project_silu_mul_quantized(shared_projected, *shared_output_).tensor
-                    : device_.project_quantized(device_.expert_silu_mul(shared_projected, shared_output_->columns()),
-                                                *shared_output_).tensor;
-            return device_.expert_combine_shared(expert_output, meta, tokens, h, routing_.top_k, shared_output, shared_gate);
+        if (router_logits.shape() != std::vector<size_t>{dims[0], e})
+            throw Error(ErrorKind::Shape, "router logits require [tokens,experts]");
+        const size_t tokens = dims[0];
+        const size_t per_token = temporary_bytes(1, hidden.dtype());
+        const size_t limit = (size_t)device_.get_tuning("moe_routing_temporary_limit");
+        const size_t chunk = std::min(tokens, std::max<size_t>(1, limit / per_token));
+        MoeStats stats;
+        stats.active_experts_known = false;
+        Tensor out = chunk == tokens ? forward_chunk(hidden, router_logits, selection_bias, shared_gate, nullptr, stats)
+                                     : device_.zeros({tokens, h}, hidden.dtype());
+        for (size_t start = 0; chunk != tokens && start < tokens; start += chunk) {
+            const size_t count = std::min(chunk, tokens - start);
+            Tensor rows = out.view(start * h, {count, h});
+            Tensor gate;
+            if (shared_gate) gate = shared_gate->view(start, {count});
+            forward_chunk(hidden.view(start * h, {count, h}), router_logits.view(start * e, {count, e}), selection_bias,
+                          shared_gate ? &gate : nullptr, &rows, stats);
         }
-        return device_.expert_combine(routed(hidden, meta, h, i, e), meta, dims[0], h, routing_.top_k);
+        stats_.merge(stats);
+        return out;
     }
 
     // most f32 assignments that take the fused per-assignment kernels (f32 rows have no
@@ -735,6 +785,52 @@ public:
     bool fuse_inputs = true;
 
 private:
+    Tensor forward_chunk(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias,
+                         const Tensor* shared_gate, const Tensor* out, MoeStats& stats) const {
+        using clock = std::chrono::steady_clock;
+        const auto seconds = [](clock::time_point a, clock::time_point b) {
+            return std::chrono::duration<double>(b - a).count();
+        };
+        const auto& dims = hidden.shape();
+        const size_t h = input_.columns(), i = input_.rows_per_expert() / 2, e = input_.experts();
+        const size_t tokens = dims[0], a = tokens * routing_.top_k;
+        stats.assignments += a;
+        stats.peak_temporary_bytes = std::max(stats.peak_temporary_bytes, temporary_bytes(tokens, hidden.dtype()));
+        const auto t0 = clock::now();
+        Tensor meta = device_.moe_route(router_logits, selection_bias, routing_);
+        const auto t1 = clock::now();
+        stats.routing += seconds(t0, t1);
+        Tensor expert_output, shared_output;
+        if (shared_input_) {
+            if (fuse_inputs && shared_rides_ && (a <= fused_max_assignments || hidden.dtype() != DType::F32)) {
+                // four launches: the shared expert's rows are batch entries of the routed ones in
+                // decode and further token groups of the grouped kernel beyond it
+                auto up = device_.expert_project_with_shared(hidden, meta, input_, *shared_input_, tokens, FH_INPUT_GATHER);
+                auto down = device_.expert_project_with_shared(up.first, meta, output_, *shared_output_, tokens,
+                                                               FH_INPUT_SILU_MUL, &up.second);
+                expert_output = down.first;
+                shared_output = down.second;
+            } else {
+                expert_output = routed(hidden, meta, h, i, e);
+                Tensor shared_projected = device_.project_quantized(hidden, *shared_input_).tensor;
+                shared_output =
+                    fuse_inputs && tokens <= fused_max_assignments
+                        ? device_.project_silu_mul_quantized(shared_projected, *shared_output_).tensor
+                        : device_.project_quantized(device_.expert_silu_mul(shared_projected, shared_output_->columns()),
+                                                    *shared_output_).tensor;
+            }
+        } else {
+            expert_output = routed(hidden, meta, h, i, e);
+        }
+        const auto t2 = clock::now();
+        stats.expert_dispatch += seconds(t1, t2);
+        Tensor combined = shared_input_ ? device_.expert_combine_shared(expert_output, meta, tokens, h, routing_.top_k,
+                                                                        shared_output, shared_gate, out)
+                                        : device_.expert_combine(expert_output, meta, tokens, h, routing_.top_k, out);
+        stats.combine_dispatch += seconds(t2, clock::now());
+        return combined;
+    }
+
     // the routed experts' outputs [A, H], before the combine
     Tensor routed(const Tensor& hidden, const Tensor& meta, size_t h, size_t i, size_t e) const {
         const auto& dims = hidden.shape();
@@ -755,6 +851,7 @@ private:
     MoeRoutingPolicy routing_;
     std::optional<QuantizedMatrix> shared_input_, shared_output_;
     bool shared_rides_ = false;
+    mutable MoeStats stats_;
 };
 
 }  // namespace ferrum

@@ -255,6 +255,34 @@ int main() {
         }
         report("a shared expert whose output matrix does not fit is Error::Config", refused);
 
+        // chunks: 80 f16 tokens, twenty to a chunk (enough assignments for the grouped kernels), against the pass that is not cut (src/nn/moe.rs:467-520)
+        {
+            const size_t many = 80;
+            std::vector<float> xm(many * hidden), lm(many * experts);
+            for (size_t t = 0; t < many; ++t) {
+                std::copy(x.begin() + (t % tokens) * hidden, x.begin() + (t % tokens + 1) * hidden, xm.begin() + t * hidden);
+                for (size_t j = 0; j < experts; ++j) lm[t * experts + j] = logits[(t % tokens) * experts + (j + t) % experts];
+            }
+            Tensor xt = d.from_f32({many, hidden}, DType::F16, xm), lt = d.from_f32({many, experts}, DType::F32, lm);
+            std::vector<float> gates(many);
+            for (size_t t = 0; t < many; ++t) gates[t] = 0.25f + 0.01f * (float)t;
+            Tensor gt = d.from_f32({many}, DType::F32, gates);
+            moe.fuse_inputs = true;
+            (void)moe.take_stats();
+            const auto whole = moe.forward(xt, lt, nullptr, &gt).to_f32();
+            const MoeStats ws = moe.take_stats();
+            const size_t before = d.moe_routing_temporary_limit(), per_token = moe.temporary_bytes(1, DType::F16);
+            d.set_moe_routing_temporary_limit(20 * per_token + 1);
+            const auto cut = moe.forward(xt, lt, nullptr, &gt).to_f32();
+            const MoeStats cs = moe.take_stats();
+            d.set_moe_routing_temporary_limit(before);
+            report("SparseMoe::forward in chunks gives the bits of the whole pass",
+                   before == (size_t(128) << 20) && std::memcmp(cut.data(), whole.data(), cut.size() * 4) == 0 &&
+                       ws.assignments == many * top_k && cs.assignments == many * top_k && !cs.active_experts_known &&
+                       ws.peak_temporary_bytes == many * per_token && cs.peak_temporary_bytes == 20 * per_token &&
+                       moe.take_stats().assignments == 0);
+        }
+
         Device other(0);
         bool threw = false;
         try {

@@ -168,6 +168,30 @@ def test_project_mm_id_carries_the_shared_expert(api, d, dtype, tokens):
         d.hybrid_project_mm_id_with_shared(w, other, xg, offsets, xt)
 
 
+@pytest.mark.parametrize("cols", [512, 6144])
+def test_project_mm_id_keeps_inside_its_rows_whatever_the_offsets_say(api, d, cols):
+    # offsets past the number of routes (a table made for another batch) are cut to it: the experts
+    # before the damage give their usual rows, the damaged one takes what is left, none reads or
+    # writes beyond the routes.  512 columns stay in LDS (the resident kernel), 6144 do not.
+    experts, rows, routes = 8, 64, 200
+    fmt = api.QuantizationFormat(Q4_K)
+    w = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * rows, cols, seed=441), fmt, experts, rows, cols)
+    ids = synth.rng(442).integers(0, experts, routes).astype(np.uint32)
+    offsets, order, _ = d.hybrid_moe_map(carrier(api, d, ids), experts)
+    x = api.Tensor.from_f32(d, (routes, cols), api.DType.F16, synth.activations(routes, cols, seed=443, f16=True))
+    good = d.hybrid_project_mm_id(w, x, offsets).to_f32()
+    table = u32(offsets).copy()
+    table[experts // 2 + 1:] = 0xFFFFFFF0
+    damaged = d.hybrid_project_mm_id(w, x, carrier(api, d, table)).to_f32()
+    intact = int(table[experts // 2])
+    assert 0 < intact < routes
+    assert np.array_equal(bits(damaged[:intact]), bits(good[:intact]))
+    assert np.isfinite(damaged).all()
+    table[1:] = table[:-1][::-1].copy()          # descending pairs are empty experts
+    table[0] = 0
+    assert np.isfinite(d.hybrid_project_mm_id(w, x, carrier(api, d, table)).to_f32()).all()
+
+
 def test_prompt_chain_map_gather_mm_id_combine_matches_the_decode_chain_and_the_oracle(api, d):
     # HybridModel::moe_ffn's two branches (src/hybrid/engine.rs:3030-3075): per-route GEMVs with
     # `identity` rows, or map -> gather -> expert GEMM over sorted rows -> combine through position

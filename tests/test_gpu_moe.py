@@ -616,6 +616,51 @@ def test_sparse_moe_with_a_shared_expert(api, d, tokens, gated):
         assert rel_l2(result.to_f32(), want) <= 3e-3
 
 
+@pytest.mark.parametrize("dtype,shared", [("F16", True), ("F16", False), ("F32", False)])
+def test_chunked_forward_gives_the_bits_of_the_unchunked_one(api, d, dtype, shared):
+    # the reference's chunk test (src/nn/moe.rs:467-520) compares two ways of assembling
+    # the chunks; here every chunk's combine writes its rows of the one output, and the
+    # comparison is with the pass that was not cut at all.  Chunks of 64 tokens leave a
+    # last one of 44: every chunk has enough assignments for the kernels the whole batch
+    # takes (grouped tiles for f16, the per-assignment GEMV for f32), whose rows do not
+    # depend on their neighbours.
+    tokens = 300
+    (experts, hidden, inter, top_k), packed, w, x, logits, xt, lt = _shared_case(api, d, dtype, tokens, 201)
+    kw = dict(shared_input=w["sin"], shared_output=w["sout"]) if shared else {}
+    moe = api.SparseMoe(d, w["win"], w["wout"], api.MoeRoutingPolicy(experts, top_k), **kw)
+    gate = api.Tensor.from_f32(d, (tokens,), api.DType.F32,
+                               (0.25 + 0.5 * synth.rng(202).random(tokens)).astype(np.float32)) if shared else None
+    before = d.moe_routing_temporary_limit()
+    assert before == 128 << 20       # src/metal/legacy.rs:95
+    whole = moe.forward(xt, lt, shared_gate=gate)
+    stats = moe.take_stats()
+    assert stats.assignments == tokens * top_k and not stats.active_experts_known
+    assert stats.peak_temporary_bytes == moe.temporary_bytes(tokens, xt.dtype)
+    per_token = moe.temporary_bytes(1, xt.dtype)
+    assert per_token == ((2 * hidden + 3 * inter) * xt.dtype.size_bytes() + 12) * top_k \
+        + (experts + hidden) * xt.dtype.size_bytes()
+    try:
+        d.set_moe_routing_temporary_limit(64 * per_token + per_token // 2)
+        cut = moe.forward(xt, lt, shared_gate=gate)
+        cut_stats = moe.take_stats()
+        d.set_moe_routing_temporary_limit(1)          # one token per chunk: the per-assignment kernels
+        single = moe.forward(xt, lt, shared_gate=gate)
+        single_stats = moe.take_stats()
+        with pytest.raises(api.ParameterError):
+            d.set_moe_routing_temporary_limit(0)
+        with d.execution():
+            with pytest.raises(api.ParameterError):
+                d.set_moe_routing_temporary_limit(1 << 20)
+    finally:
+        d.set_moe_routing_temporary_limit(before)
+    assert np.array_equal(cut.raw(), whole.raw())
+    assert cut_stats.assignments == tokens * top_k
+    assert cut_stats.peak_temporary_bytes == 64 * per_token <= 64 * per_token + per_token // 2
+    assert single_stats.peak_temporary_bytes == per_token and single_stats.assignments == tokens * top_k
+    assert rel_l2(single.to_f32(), whole.to_f32()) <= (1e-6 if dtype == "F32" else 2e-3)
+    assert moe.take_stats() == api.MoeStats()
+
+
 def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
     # 32 rows of 2816 halves are more than the grouped kernel's LDS: the routed rows are staged and
     # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit

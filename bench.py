@@ -460,23 +460,38 @@ def read_probe_case(api, synth, dev, steps, warmup):
 
 
 def mfma_probe_case(dev, steps):
-    """MFMA issue loops from registers, four waves per workgroup, four workgroups per CU."""
-    props = dev.properties()
-    groups = 4 * int(props.get("compute_units") or 256)
+    """Matrix-core rates: MFMA issue loops from registers with one and with four waves per
+    SIMD, and an MFMA wave beside a VALU wave on the same SIMD."""
+    cus = int(dev.properties().get("compute_units") or 256)
     iterations = 4096
     out = {}
     for shape, name in ((0, "v_mfma_f32_16x16x32_f16"), (1, "v_mfma_f32_32x32x16_f16")):
-        flops = [0.0]
+        for waves in (1, 4):
+            flops = [0.0]
 
+            def enqueue(i):
+                flops[0] = dev.probe_mfma(shape, waves * cus, iterations)
+
+            best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(3)) / steps
+            out[f"{name}, {waves} wave(s) per SIMD"] = {
+                "kernel": dev.last_operation(), "us": round(best * 1e6, 2),
+                "TFLOP/s": round(flops[0] / best / 1e12, 1),
+                "frac_published_peak": round(flops[0] / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+    together = {}
+
+    def timed(mfma, rounds):
         def enqueue(i):
-            flops[0] = dev.probe_mfma(shape, groups, iterations)
+            dev.probe_coissue(cus, iterations, mfma, rounds)
+        return min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(3)) / steps * 1e6
 
-        best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(3)) / steps
-        out[name] = {"kernel": dev.last_operation(), "us": round(best * 1e6, 2),
-                     "TFLOP/s": round(flops[0] / best / 1e12, 1),
-                     "frac_published_peak": round(flops[0] / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
-    print(json.dumps({"mfma_probe": out, "workgroups": groups, "waves_per_workgroup": 4,
-                      "independent_chains_per_wave": 8, "iterations": iterations}), flush=True)
+    together["mfma_wave_alone_us"] = round(timed(True, 0), 1)
+    for rounds in (1, 2, 4, 8):
+        alone, both = timed(False, rounds), timed(True, rounds)
+        together[f"valu_{8 * rounds}_fma_per_8_mfma"] = {
+            "valu_wave_alone_us": round(alone, 1), "both_us": round(both, 1),
+            "sum_us": round(alone + together["mfma_wave_alone_us"], 1)}
+    print(json.dumps({"mfma_probe": out, "independent_chains_per_wave": 8, "iterations": iterations,
+                      "mfma_and_valu_waves_on_one_simd": together}), flush=True)
 
 
 def main():

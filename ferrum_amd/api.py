@@ -117,6 +117,7 @@ SYMBOLS = {
     "fh_project_quantized_no_alloc": (_I32, [_P, _P, _VP, _U32, _VP]),
     "fh_probe_read": (_I32, [_P, _P]),
     "fh_probe_mfma": (_I32, [_P, _U32, _U32, _U32, ctypes.POINTER(ctypes.c_double)]),
+    "fh_probe_coissue": (_I32, [_P, _U32, _U32, _U32, _U32]),
     "fh_argmax_rows": (_I32, [_P, _VP, _U32, _U32, _VP]),
     "fh_add_rmsnorm": (_I32, [_P, _VP, _VP, _VP, _U32, _U32, ctypes.c_float, _VP, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
@@ -657,6 +658,10 @@ class Device:
         flops = ctypes.c_double()
         _check(_lib.fh_probe_mfma(self._handle, shape, groups, iterations, ctypes.byref(flops)))
         return float(flops.value)
+
+    def probe_coissue(self, groups: int, iterations: int, mfma: bool, valu_rounds: int) -> None:
+        """fh_probe_coissue: an MFMA wave and a VALU wave on every SIMD, either or both."""
+        _check(_lib.fh_probe_coissue(self._handle, groups, iterations, int(mfma), valu_rounds))
 
     def argmax_rows(self, logits: Tensor) -> Tensor:
         """[rows, 2] F32 carrier of u32 bits: first maximal index and a non-finite flag

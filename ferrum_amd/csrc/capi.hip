@@ -248,6 +248,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     }
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
+    d->tuning["gemm_wide_shape"] = 1;       // matrix instruction of the 256-row tile: 0 = 16x16x32, 1 = 32x32x16 where it wins, 2 = 32x32x16 always
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
@@ -348,6 +349,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
     } else if (k == "gemm_resident") {
         ok = value == 0 || value == 1;
     } else if (k == "gemv_stream") {
+        ok = value >= 0 && value <= 2;
+    } else if (k == "gemm_wide_shape") {
         ok = value >= 0 && value <= 2;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
@@ -642,6 +645,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.y_dtype = y->dtype;
         a.cu_count = device->props.multiProcessorCount;
         a.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
+        a.wide_shape = (int)tuning(device, "gemm_wide_shape");
         a.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         a.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, a);
@@ -763,6 +767,19 @@ fh_status fh_probe_mfma(fh_device* device, uint32_t shape, uint32_t groups, uint
     if (st != FH_OK) return st;
     device->last_operation = launch_mfma_probe(device->stream, (int)shape, groups, iterations,
                                                reinterpret_cast<float*>(scratch_data(device)), flops);
+    FH_HIP(hipGetLastError());
+    return FH_OK;
+}
+
+fh_status fh_probe_coissue(fh_device* device, uint32_t groups, uint32_t iterations, uint32_t mfma,
+                           uint32_t valu_rounds) {
+    if (device == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (groups == 0 || groups > 65535 || iterations == 0 || (mfma == 0 && valu_rounds == 0))
+        return fail(FH_ERR_SHAPE, "co-issue probe: 1..65535 workgroups, at least one iteration, something to run");
+    fh_status st = ensure_scratch(device, (size_t)groups * 512 * sizeof(float));
+    if (st != FH_OK) return st;
+    device->last_operation = launch_coissue_probe(device->stream, groups, iterations, mfma, valu_rounds,
+                                                  reinterpret_cast<float*>(scratch_data(device)));
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
@@ -1344,6 +1361,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.y_dtype = y->dtype;
         g.cu_count = device->props.multiProcessorCount;
         g.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
+        g.wide_shape = (int)tuning(device, "gemm_wide_shape");
         g.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         g.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, g);

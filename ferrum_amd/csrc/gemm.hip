@@ -11,6 +11,8 @@
 // Tile: 128 (M) x 128 (N) x 64 (K) per 256-thread workgroup; four waves in a
 // 2 x 2 arrangement, each owning 64 x 64 outputs as 2 x 2 MFMA 32x32x16 tiles.
 // LDS rows are padded to 72 halfs so 128-bit fragment reads are conflict free.
+#include <type_traits>
+
 #include "device_utils.hpp"
 #include "tile_decode.hpp"
 #include "internal.hpp"
@@ -386,6 +388,13 @@ __device__ __forceinline__ void decode_to_lds(const RawW<TYPE>& raw, uint32_t c,
 // input dword (4 quant bytes) of slab c into tile values: Q4_K gives two
 // dwords for k = 16h + 4t .. (low nibbles) and two for k = 32 + 16h + 4t ..
 // (high nibbles); Q6_K gives two dwords for k = 32h + 4t ...
+// component t of a register quad; t may differ between lanes (two selects), and folds away
+// when it is a constant
+__device__ __forceinline__ uint32_t pick4(const uint4& q, int t) {
+    const uint32_t lo = (t & 1) ? q.y : q.x, hi = (t & 1) ? q.w : q.z;
+    return (t & 2) ? hi : lo;
+}
+
 template <uint32_t TYPE>
 struct BlockW;
 
@@ -407,10 +416,7 @@ struct BlockW<kQ4K> {
         // d*sc and dmin*m are exact in f32; the powers of two undo the subnormal encoding
         return {(d * sc0) * 16777216.f, (d * sc1) * 1048576.f, -(dmin * mn0), -(dmin * mn1)};
     }
-    __device__ __forceinline__ uint32_t dword(int c, int t) const {
-        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
-        return v[t];
-    }
+    __device__ __forceinline__ uint32_t dword(int c, int t) const { return pick4(q[c], t); }
     // out[0..1]: low-nibble pair dwords, out[2..3]: high-nibble pair dwords
     template <int DT>
     __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
@@ -443,10 +449,8 @@ struct BlockW<kQ5K> {
     // low nibble | fifth bit << 4 reads as q * 2^-24; high nibble in place | fifth bit << 8 as 16q * 2^-24
     template <int DT>
     __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
-        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
-        const uint32_t p[4] = {qh.x, qh.y, qh.z, qh.w};
-        const uint32_t w0 = v[t], w1 = w0 >> 8;
-        const uint32_t p0 = p[t] >> (2 * c), p1 = p0 >> 8;
+        const uint32_t w0 = pick4(q[c], t), w1 = w0 >> 8;
+        const uint32_t p0 = pick4(qh, t) >> (2 * c), p1 = p0 >> 8;
         const uint32_t l02 = (w0 & 0x000f000fu) | ((p0 & 0x00010001u) << 4);
         const uint32_t l13 = (w1 & 0x000f000fu) | ((p1 & 0x00010001u) << 4);
         const uint32_t h02 = (w0 & 0x00f000f0u) | ((p0 & 0x00020002u) << 7);
@@ -476,8 +480,8 @@ struct BlockW<kIQ4XS> {
     }
     template <int DT>
     __device__ __forceinline__ void decode(int c, uint32_t, int t, const Scales& s, uint32_t (&out)[4]) const {
-        const uint32_t v[4] = {q[c].x, q[c].y, q[c].z, q[c].w};
-        const uint32_t l = iq4_lookup4(v[t]), u = iq4_lookup4(v[t] >> 4);
+        const uint32_t v = pick4(q[c], t);
+        const uint32_t l = iq4_lookup4(v), u = iq4_lookup4(v >> 4);
         const uint32_t l01 = bytes01_as_halves(l), l23 = bytes23_as_halves(l);
         const uint32_t u01 = bytes01_as_halves(u), u23 = bytes23_as_halves(u);
         out[0] = fma_pair<DT>(lo_half(l01), hi_half(l01), s.a_lo, s.b_lo);
@@ -620,9 +624,7 @@ __device__ __forceinline__ void decode_block_piece(const BlockW<TYPE>& blk, int 
     const auto s = blk.scales(c, h);
     if constexpr (!kEightDwords<TYPE>) {
         uint32_t out[4];
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
-            if (tt == t) blk.template decode<DT>(c, h, tt, s, out);
+        blk.template decode<DT>(c, h, t, s, out);   // the dword is selected, the arithmetic runs once
         *reinterpret_cast<uint2*>(wrow_lds + k_lo_of<TYPE>(h) + 4 * t) = make_uint2(out[0], out[1]);
         *reinterpret_cast<uint2*>(wrow_lds + k_hi_of<TYPE>(h) + 4 * t) = make_uint2(out[2], out[3]);
     } else {
@@ -811,6 +813,239 @@ __global__ __launch_bounds__(kWideThreads) void gemm_wide_kernel(const uint8_t* 
         }
 }
 
+// ---- the 256-row tile on the 32x32x16 matrix instruction --------------------------------
+// Same division of labour as gemm_wide_kernel (four waves decode weight rows into a double
+// buffered LDS slab of 64 K, four waves multiply, each owning 64 of the tile's 256 activation
+// rows), but the multiplying waves issue v_mfma_f32_32x32x16, which does twice the work per
+// issue slot of the 16x16x32 form.  A wave's tile is 2 x NT blocks of 32 x 32 (NT = 4 or 5:
+// 128 or 160 weight rows per workgroup).  Within a slab lane group kg = lane / 32 multiplies
+// K 32 kg .. 32 kg + 31, eight at a step, so a lane's activations for one slab are 64
+// contiguous bytes of its row.
+template <int DT>
+__device__ __forceinline__ float16v mfma32(uint4 a, uint4 b, float16v c) {
+    if constexpr (DT == 1) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
+                                                      __builtin_bit_cast(half8, b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+}
+
+// LDS of the 32x32x16 form: four activation rings of 16 KB (one per multiplying wave, two
+// stages of 64 rows x 64 K), then the two weight slabs.  The rings come first: an LDS-direct
+// load takes its LDS address from M0, which holds 16 bits.
+constexpr uint32_t kWide32RingBytes = 16384;
+constexpr uint32_t kWide32WeightsAt = 4 * kWide32RingBytes;
+
+// LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
+__device__ __forceinline__ void lds_direct16(const void* g, uint32_t lds_addr) {
+    const uint32_t a = __builtin_amdgcn_readfirstlane(lds_addr);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
+}
+
+template <uint32_t TYPE, int DT, int NT>
+__global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restrict__ w,
+                                                          const uint16_t* __restrict__ x,
+                                                          void* __restrict__ y, uint32_t m, uint32_t n,
+                                                          uint32_t nb, uint32_t y_dtype, uint32_t cols,
+                                                          uint32_t tiles_m, uint32_t tiles_n) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
+    constexpr uint32_t kRowsW = 32 * NT;
+    constexpr uint32_t kStage = kRowsW * kLd;  // halfs per buffer
+    constexpr bool kExtra = NT > 4;            // rows 128 .. 159 are a second decode task
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    // XCD-aware tile order: ids r, r+8, r+16, .. of a group share the XCD (id mod 8)
+    uint32_t tile_m, tile_n;
+    {
+        const uint32_t group_ids = 8 * tiles_m, id = blockIdx.x;
+        const uint32_t g = id / group_ids, r = id % group_ids;
+        tile_n = g * 8 + (r & 7u);
+        tile_m = r >> 3;
+        if (tile_n >= tiles_n) return;
+    }
+    const uint32_t n0 = tile_n * cols, m0 = tile_m * kWM;
+    const uint32_t ncols = n - n0 < cols ? n - n0 : cols;
+    const uint32_t k = nb << 8;
+
+    if (wave >= 4) {
+        // ---- producers: global -> registers -> (decode) -> LDS, blocks ahead ----
+        const uint32_t pt = tid - 256, pw = wave - 4;
+        const uint32_t wr = pt >> 1, wh = pt & 1u;
+        const uint8_t* wsrc = w + (size_t)(n0 + (wr < ncols ? wr : ncols - 1)) * nb * kBlockBytes;
+        // rows 128 .. 159: every wave takes eight of them, a lane one quarter of a (row, half) task
+        // of every slab, so all slabs cost the same
+        const uint32_t er = 128 + 8 * pw + (lane >> 3), eh = (lane >> 2) & 1u, et = lane & 3u;
+        const uint8_t* esrc = w + (size_t)(n0 + (er < ncols ? er : ncols - 1)) * nb * kBlockBytes;
+        constexpr bool kDeep = !kEightDwords<TYPE>;   // Q6_K and Q8_0 sets are twice as large: one block ahead
+        BlockW<TYPE> cur, n1, n2, ecur, en1, en2;
+        auto store_slab = [&](int c) {
+            uint16_t* ws = lds + kWide32WeightsAt / 2 + (c & 1) * kStage;
+            decode_block_slab<TYPE, DT>(cur, c, wh, ws + wr * kLd);
+            if (kExtra) decode_block_piece<TYPE, DT>(ecur, c, eh, (int)et, ws + er * kLd);
+        };
+        cur.load(wsrc, wh);
+        if (kExtra) ecur.load(esrc, eh);
+        if (nb > 1) {
+            n1.load(wsrc + kBlockBytes, wh);
+            if (kExtra) en1.load(esrc + kBlockBytes, eh);
+        }
+        if (kDeep && nb > 2) {
+            n2.load(wsrc + 2 * (size_t)kBlockBytes, wh);
+            if (kExtra) en2.load(esrc + 2 * (size_t)kBlockBytes, eh);
+        }
+        store_slab(0);
+        // The register set that the shift after a block's last slab frees is loaded with the block
+        // `ahead` blocks on: rows 0 .. 127 at once, rows 128 .. two slabs later, so the load
+        // instructions are spread over the slabs.
+        constexpr uint32_t ahead = kDeep ? 3 : 2;
+        for (uint32_t b = 0; b < nb; ++b) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                __syncthreads();  // slab 4b + c is visible; the other buffer is free
+                if (c < 3) {
+                    store_slab(c + 1);
+                    if (c == 1 && kExtra && b >= 1 && b + ahead - 1 < nb) {
+                        if (kDeep) en2.load(esrc + (size_t)(b + ahead - 1) * kBlockBytes, eh);
+                        else en1.load(esrc + (size_t)(b + ahead - 1) * kBlockBytes, eh);
+                    }
+                } else if (b + 1 < nb) {
+                    cur = n1;
+                    if (kDeep) {
+                        ecur = en1;
+                        n1 = n2;
+                        en1 = en2;
+                        if (b + 3 < nb) n2.load(wsrc + (size_t)(b + 3) * kBlockBytes, wh);
+                    } else {
+                        ecur = en1;
+                        if (b + 2 < nb) n1.load(wsrc + (size_t)(b + 2) * kBlockBytes, wh);
+                    }
+                    store_slab(0);
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- consumers: own activation rows by LDS-direct loads, weights from LDS -> MFMA ----
+    float16v acc[2][NT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const uint32_t r32 = lane & 31u, kg = lane >> 5;
+    // The wave's 64 activation rows travel through a ring of its own in LDS, one slab (64 K,
+    // 8 KB) per stage, two stages: no other wave reads them, so no barrier is involved, only the
+    // wave's own count of outstanding loads.  A stage is two halves of 32 K; in a half the
+    // 16-byte piece q of local row r sits at unit 4 r + (q ^ ((r >> 2) & 3)), which spreads
+    // the sixteen rows a fragment read touches over all banks.  One load instruction fills
+    // 1 KB: 16 rows x 4 pieces, lane l = (row 16 t + l / 4, unit l % 4).
+    const uint32_t a_ring = wave * kWide32RingBytes;   // stage s of the ring is a_ring + 8192 (s & 1)
+    const uint16_t* adma[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const uint32_t r = 16 * t + (lane >> 2);
+        const uint32_t q = (lane & 3u) ^ ((r >> 2) & 3u);
+        const uint32_t row = m0 + wave * 64 + r;
+        // rows past m are clamped: they only feed outputs that are never stored
+        adma[t] = x + (size_t)(row < m ? row : m - 1) * k + 8 * q;
+    }
+    // load instruction i (0..7) of a slab: half i / 4, rows 16 (i % 4) ..
+    auto dma_piece = [&](uint32_t slab, int i) {
+        lds_direct16(adma[i & 3] + (size_t)slab * 64 + 32 * (i >> 2),
+                     a_ring + (slab & 1u) * 8192u + (uint32_t)(i >> 2) * 4096u + (uint32_t)(i & 3) * 1024u);
+    };
+    auto dma_slab = [&](uint32_t slab) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dma_piece(slab, i);
+    };
+    // fragment addresses: activations of row tile i at step s (0..3) of the slab, weights of column tile j
+    const uint32_t sw = (r32 >> 2) & 3u;
+    const uint32_t a_off0 = (4 * r32 + ((2 * kg) ^ sw)) * 16, a_off1 = (4 * r32 + ((2 * kg + 1) ^ sw)) * 16;
+    const uint8_t* const lds_bytes = reinterpret_cast<const uint8_t*>(lds);
+    const uint32_t b_off = kWide32WeightsAt + (r32 * kLd + 16 * kg) * 2;
+    constexpr int kFrags = 2 + NT;   // fragments of a step: two of activations, NT of weights
+    struct Frags {
+        uint4 v[kFrags];
+    };
+    auto read_frag = [&](Frags& f, uint32_t slab, int s, int t) {
+        if (t < 2) {
+            f.v[t] = *reinterpret_cast<const uint4*>(lds_bytes + a_ring + (slab & 1u) * 8192u + (s >> 1) * 4096u +
+                                                      ((s & 1) ? a_off1 : a_off0) + t * 2048);
+        } else {
+            f.v[t] = *reinterpret_cast<const uint4*>(lds_bytes + b_off + (slab & 1u) * (kStage * 2) + (s >> 1) * 64 +
+                                                      (s & 1) * 16 + (t - 2) * (32 * kLd * 2));
+        }
+    };
+    // One step: 2 NT multiplications on `cur`, and between them, one at a time so that each
+    // hides behind a multiplication in flight, the reads of step (slab, s)'s fragments into
+    // `next` and, with DMA set, the eight load instructions of activation slab `dma`.
+    auto step = [&](const Frags& cur, Frags& next, uint32_t slab, int s, auto with_reads, auto with_dma, uint32_t dma) {
+#pragma unroll
+        for (int idx = 0; idx < 2 * NT; ++idx) {
+            if constexpr (decltype(with_reads)::value)
+                if (idx < kFrags) read_frag(next, slab, s, idx);
+            if constexpr (decltype(with_dma)::value)
+                if (idx < 8) dma_piece(dma, idx);
+            acc[idx & 1][idx >> 1] = mfma32<DT>(cur.v[idx & 1], cur.v[2 + (idx >> 1)], acc[idx & 1][idx >> 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    constexpr std::true_type yes{};
+    constexpr std::false_type no{};
+    // Software pipeline, one step deep: the fragments of step s + 1 are read while step s
+    // multiplies, also across the slab boundary.  The barrier that opens slab c + 1 therefore
+    // sits before the last step of slab c, whose fragments are in registers by then.
+    const uint32_t slabs = nb * 4;   // at least four
+    Frags f0, f1;
+    dma_slab(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();               // the weights of slab 0 are visible
+    dma_slab(1);
+#pragma unroll
+    for (int t = 0; t < kFrags; ++t) read_frag(f0, 0, 0, t);
+    __builtin_amdgcn_s_setprio(2);  // the MFMA wave goes first when both waves of a SIMD can issue
+    // the loop body is one straight run of code, so the counts of outstanding LDS reads are exact
+    for (uint32_t c = 0; c + 1 < slabs; ++c) {
+        step(f0, f1, c, 1, yes, no, 0u);
+        step(f1, f0, c, 2, yes, no, 0u);
+        step(f0, f1, c, 3, yes, no, 0u);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the activations of slab c + 1 have landed
+        __syncthreads();           // its weights are visible; slab c is in registers, its buffers are free
+        __builtin_amdgcn_sched_barrier(0);
+        // past the end the last slab is loaded once more, into the stage nobody reads
+        step(f1, f0, c + 1, 0, yes, yes, c + 2 < slabs ? c + 2 : slabs - 1);
+    }
+    {
+        const uint32_t c = slabs - 1;
+        step(f0, f1, c, 1, yes, no, 0u);
+        step(f1, f0, c, 2, yes, no, 0u);
+        step(f0, f1, c, 3, yes, no, 0u);
+        step(f1, f0, c, 0, no, no, 0u);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the spare load of the last slab
+    }
+    __builtin_amdgcn_s_setprio(0);
+
+    // element v of a lane's block: row 8 (v / 4) + 4 kg + v % 4, column r32
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const uint32_t lc = 32 * j + r32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t row = m0 + wave * 64 + 32 * i + 8 * (v >> 2) + 4 * kg + (v & 3);
+                if (row < m && lc < ncols)
+                    store_from_f32(y, (size_t)row * n + n0 + lc, y_dtype, acc[i][j][v]);
+            }
+        }
+}
+
 struct WidePlan {
     int nt;
     uint32_t cols, tiles_m, tiles_n;
@@ -837,6 +1072,41 @@ WidePlan wide_plan(uint32_t m, uint32_t n, int cus) {
     return best;
 }
 
+// Columns per workgroup of the 32x32x16 form: 128 or 160.
+WidePlan wide32_plan(uint32_t m, uint32_t n, int cus) {
+    WidePlan best{};
+    double best_cost = 1e300;
+    const uint32_t tiles_m = (m + kWM - 1) / kWM;
+    for (uint32_t cols : {128u, 160u}) {
+        const int nt = (int)cols / 32;
+        const uint32_t tiles_n = (n + cols - 1) / cols;
+        const uint64_t wgs = (uint64_t)tiles_m * tiles_n;
+        const uint64_t rounds = (wgs + cus - 1) / cus;
+        const double cost = (double)rounds * nt;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = {nt, cols, tiles_m, tiles_n};
+        }
+    }
+    return best;
+}
+
+template <uint32_t TYPE, int DT, int NT>
+void launch_wide32(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
+    const size_t lds = kWide32WeightsAt + 2 * (size_t)(32 * NT) * kLd * sizeof(uint16_t);
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wide32_kernel<TYPE, DT, NT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        configured = true;
+    }
+    const uint32_t groups = (plan.tiles_n + 7) / 8;
+    dim3 grid(groups * 8 * plan.tiles_m);
+    hipLaunchKernelGGL((gemm_wide32_kernel<TYPE, DT, NT>), grid, dim3(512), lds, s,
+                       static_cast<const uint8_t*>(a.w), static_cast<const uint16_t*>(a.x), a.y, a.m, a.n,
+                       a.k / 256, a.y_dtype, plan.cols, plan.tiles_m, plan.tiles_n);
+}
+
 template <uint32_t TYPE, int DT, int NT>
 void launch_wide(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
     const size_t lds = 2 * (size_t)(16 * NT) * kLd * sizeof(uint16_t);
@@ -855,6 +1125,24 @@ void launch_wide(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
 
 template <uint32_t TYPE, int DT>
 void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
+    // The 32x32x16 form does a sixth more work per column and cycle, but its tiles are 160 or
+    // 128 columns wide and fill the chip less evenly.  It is taken where its workgroups run as
+    // one round on at least four fifths of the compute units (512 x 17408 x 5120: 218
+    // workgroups, 112 against 114 us); over several rounds the 16x16x32 form overlaps one
+    // workgroup's stores with the next one's loop better (2048 rows: 443 against 468 us).
+    // wide_shape 2 takes it always.
+    if (a.wide_shape != 0) {
+        const WidePlan p32 = wide32_plan(a.m, a.n, a.cu_count);
+        const uint64_t wgs = (uint64_t)p32.tiles_m * p32.tiles_n;
+        if (a.wide_shape == 2 || (wgs <= (uint64_t)a.cu_count && wgs * 5 >= (uint64_t)a.cu_count * 4)) {
+            if (p32.nt == 5) {
+                launch_wide32<TYPE, DT, 5>(s, a, p32);
+            } else {
+                launch_wide32<TYPE, DT, 4>(s, a, p32);
+            }
+            return;
+        }
+    }
     if (plan.nt == 9) {
         launch_wide<TYPE, DT, 9>(s, a, plan);
     } else {

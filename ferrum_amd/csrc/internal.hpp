@@ -110,6 +110,8 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
 const char* launch_read_probe(hipStream_t s, const void* data, size_t bytes, uint32_t* sink);
 const char* launch_mfma_probe(hipStream_t s, int shape, uint32_t groups, uint32_t iterations, float* sink,
                               double* flops);
+const char* launch_coissue_probe(hipStream_t s, uint32_t groups, uint32_t iterations, uint32_t mfma,
+                                 uint32_t valu_rounds, float* sink);
 
 // norm.hip
 // residual = round(a + b), normed = rmsnorm(residual) * weight; all operands of one dtype,
@@ -185,6 +187,7 @@ struct GemmArgs {
     uint32_t x_dtype, y_dtype;
     int cu_count;
     int wide_min_rows;   // smallest M that takes the 256-row tile
+    int wide_shape;      // matrix instruction of the 256-row tile: 0 = 16x16x32, 1 = 32x32x16 where it wins, 2 = always
     int skinny_max_rows; // largest M that takes the register-dequant kernel
     // routed-expert form of the register-dequant kernel: w is [experts, n, k],
     // x and y rows are assignments, m is their count; tokens of expert e are

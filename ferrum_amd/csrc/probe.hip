@@ -8,8 +8,14 @@
 //    chains on register operands and stores one float at the end.  Its rate is what the
 //    matrix cores sustain for one instruction shape, the figure a tile GEMM is read
 //    against.
+//  * coissue_probe: workgroups of eight waves, two per SIMD.  Waves 0..3 issue
+//    v_mfma_f32_32x32x16_f16 (when `mfma` is set), waves 4..7 issue rounds of eight
+//    independent v_fma_f32 (when `valu_rounds` is not zero).  Timed alone and
+//    together, it shows whether matrix and vector arithmetic of two waves on one
+//    SIMD overlap: what a kernel that decodes weights next to its multiplications
+//    can hope for.
 //
-// Neither has a counterpart in the reference; both are launched by the benchmark only.
+// None has a counterpart in the reference; all are launched by the benchmark only.
 #include "internal.hpp"
 
 namespace fh {
@@ -79,7 +85,56 @@ __global__ __launch_bounds__(256) void mfma_probe(uint32_t iterations, float see
     sink[blockIdx.x * 256 + threadIdx.x] = total;
 }
 
+__global__ __launch_bounds__(512) void coissue_probe(uint32_t iterations, uint32_t mfma, uint32_t valu_rounds,
+                                                     float* __restrict__ sink) {
+    const uint32_t wave = threadIdx.x >> 6;
+    float total = 0.0f;
+    if (wave < 4) {
+        if (mfma == 0) return;
+        half8 a, b;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = (_Float16)(0x1p-10f * (float)((threadIdx.x + i) & 7));
+            b[i] = (_Float16)(0x1p-10f * (float)((threadIdx.x * 3 + i) & 7));
+        }
+        float16v acc[kChains];
+#pragma unroll
+        for (int c = 0; c < kChains; ++c)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[c][j] = 0.0f;
+        for (uint32_t it = 0; it < iterations; ++it) {
+#pragma unroll
+            for (int c = 0; c < kChains; ++c)
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < kChains; ++c)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) total += acc[c][j];
+    } else {
+        if (valu_rounds == 0) return;
+        float x[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = 0x1p-10f * (float)(threadIdx.x + i);
+        const float scale = 1.0001f, step = 0.5f;
+        for (uint32_t it = 0; it < iterations; ++it)
+            for (uint32_t r = 0; r < valu_rounds; ++r) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = __builtin_fmaf(x[i], scale, step);
+            }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) total += x[i];
+    }
+    sink[blockIdx.x * 512 + threadIdx.x] = total;
+}
+
 }  // namespace
+
+const char* launch_coissue_probe(hipStream_t stream, uint32_t groups, uint32_t iterations, uint32_t mfma,
+                                 uint32_t valu_rounds, float* sink) {
+    coissue_probe<<<dim3(groups), dim3(512), 0, stream>>>(iterations, mfma, valu_rounds, sink);
+    return mfma != 0 && valu_rounds != 0 ? "coissue_probe_mfma_and_valu" : mfma != 0 ? "coissue_probe_mfma" : "coissue_probe_valu";
+}
 
 const char* launch_read_probe(hipStream_t stream, const void* data, size_t bytes, uint32_t* sink) {
     const size_t n16 = bytes / 16;

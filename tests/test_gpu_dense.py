@@ -377,14 +377,23 @@ def test_config3_q4_k_gemm_5120_17408(api, d, m):
     plain = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", threads=8)
     # distance to the unrounded CPU reference: only the f16 tile rounding
     assert rel_l2(got[:, rows], plain) <= 4e-4
-    # linearity in M: row i of the product depends only on row i of X
+    # linearity in M: row i of the product depends only on row i of X.  The 256-row tile has two
+    # forms that sum in different orders and are chosen by shape, so each is held fixed in turn.
     if m >= 16:
         xt2 = api.Tensor.from_f32(d, (m // 2, k), api.DType.F16, x[: m // 2])
-        half = d.project_quantized(xt2, w, out_dtype=api.DType.F32)
-        if half.operation == full.operation:
-            assert np.array_equal(half.tensor.to_f32(), got[: m // 2])
-        else:  # another kernel, another summation order
-            assert_matmul_parity(half.tensor.to_f32(), got[: m // 2], f"gemm M={m // 2} vs M={m}")
+        before = d.get_tuning("gemm_wide_shape")
+        try:
+            for shape in (0, 2):
+                d.set_tuning("gemm_wide_shape", shape)
+                whole = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+                half = d.project_quantized(xt2, w, out_dtype=api.DType.F32)
+                if half.operation == whole.operation:
+                    assert np.array_equal(half.tensor.to_f32(), whole.tensor.to_f32()[: m // 2])
+                else:  # another kernel, another summation order
+                    assert_matmul_parity(half.tensor.to_f32(), got[: m // 2], f"gemm M={m // 2} vs M={m}")
+                assert_matmul_parity(whole.tensor.to_f32()[:, rows], tile, f"gemm M={m}, tile form {shape}")
+        finally:
+            d.set_tuning("gemm_wide_shape", before)
 
 
 @pytest.mark.parametrize("m", [8, 512])
@@ -552,6 +561,34 @@ def test_wide_gemm_covers_every_column_of_its_tiles(api, d):
     rows = np.arange(n - 40, n)
     want = oracle_columns(Q4_K, packed, n, k, rows, x, accumulate="f64", weight_round=oracle.F16)
     assert_matmul_parity(got[:, rows], want, "last columns")
+
+
+@pytest.mark.parametrize("ggml", [12, 13, 14, 23, 8], ids=["q4_k", "q5_k", "q6_k", "iq4_xs", "q8_0"])
+@pytest.mark.parametrize("dtype,cols", [("F16", 160), ("BF16", 160), ("F16", 128)])
+def test_wide_gemm_on_the_32x32x16_instruction(api, d, ggml, dtype, cols):
+    # the 256-row tile built on v_mfma_f32_32x32x16: 300 rows (a second, partly empty row tile) and a
+    # column count that leaves the last workgroup 40 of its 160 (or 8 of its 128) columns; every
+    # output is checked.  17000 columns plan 160-wide tiles (one round of 214 workgroups where
+    # 128-wide ones would need two), 8072 columns 128-wide ones.
+    n, k, m = (17000, 512, 300) if cols == 160 else (8072, 512, 300)
+    packed = synth.matrix(ggml, n, k, seed=171)
+    w = qm(api, d, ggml, n, k, packed)
+    code = oracle.F16 if dtype == "F16" else oracle.BF16
+    x = oracle.round_storage(synth.activations(m, k, seed=172), code).reshape(m, k)
+    xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
+    before = d.get_tuning("gemm_wide_shape")
+    try:
+        d.set_tuning("gemm_wide_shape", 2)
+        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        d.set_tuning("gemm_wide_shape", 0)
+        other = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_wide_shape", before)
+    assert out.operation.endswith("_gemm_mfma_m256") and other.operation == out.operation
+    got = out.tensor.to_f32()
+    want = oracle.project(ggml, packed, n, k, x, accumulate="f64", weight_round=code, threads=8)
+    assert_matmul_parity(got, want, "every output of the 32x32x16 tiles")
+    assert_matmul_parity(got, other.tensor.to_f32(), "against the 16x16x32 tiles", l2_tol=2e-6)
 
 
 def test_objects_may_outlive_their_device(api):

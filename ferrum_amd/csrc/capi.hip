@@ -109,7 +109,7 @@ uint8_t* scratch_data(fh_device* d) {
 // Points a GEMV launch that cuts K into segments at the device scratch
 // (partial sums and one zeroed counter word per row tile and batch row).
 fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
-    GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    const GemvScratch plan = gemv_scratch(a);
     if (plan.segments > 1) {
         if ((uint64_t)plan.tiles * a.m > fh_device::kCounterWords)
             return fail(FH_ERR_SHAPE, "projection needs %llu row tiles, more than the K-split scratch holds",
@@ -126,7 +126,7 @@ fh_status prepare_gemv(fh_device* d, GemvArgs& a) {
 // extent and, where K is cut into segments, the counter words (one per row tile and batch
 // entry).  A launch that carries a shared expert is not cut.
 fh_status run_gemv(fh_device* d, GemvArgs a, const char** name) {
-    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    const GemvScratch plan = gemv_scratch(a);
     uint64_t most = 65535u;
     if (plan.segments > 1 && plan.tiles > 0) most = std::min<uint64_t>(most, fh_device::kCounterWords / plan.tiles);
     if (a.x_mode == kXDivide && a.x_div > 1) most -= most % a.x_div;   // the routes of a token stay together
@@ -728,7 +728,7 @@ fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* wei
     a.cu_count = device->props.multiProcessorCount;
     a.x_mode = kXPlain;
     a.x_rows = m;
-    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    const GemvScratch plan = gemv_scratch(a);
     if (plan.segments > 1) {
         const uint64_t counters = (uint64_t)plan.tiles * m;
         const uint64_t partial_bytes = (uint64_t)plan.segments * m * n * sizeof(float);

@@ -531,12 +531,24 @@ GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
     return plan;
 }
 
+bool gemv_takes_stream(const GemvArgs& a, StreamPlan* plan) {
+    if (a.stream == 0 || a.ggml_type != kQ4K || a.metadata != nullptr || a.x_mode != kXPlain || a.shared_w != nullptr ||
+        a.ksplit != 0)
+        return false;
+    *plan = gemv_stream_plan(a.n, a.k, a.m, a.cu_count, a.stream == 2);
+    return plan->ok;
+}
+
+GemvScratch gemv_scratch(const GemvArgs& a) {
+    StreamPlan stream;
+    if (gemv_takes_stream(a, &stream)) return {stream.segments, stream.tiles};
+    const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
+    return {plan.segments, plan.tiles};
+}
+
 const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
-    if (a.stream != 0 && a.ggml_type == kQ4K && a.metadata == nullptr && a.x_mode == kXPlain && a.shared_w == nullptr &&
-        a.ksplit == 0) {
-        const StreamPlan stream = gemv_stream_plan(a.n, a.k, a.m, a.cu_count, a.stream == 2);
-        if (stream.ok) return launch_gemv_stream(s, a, stream);
-    }
+    StreamPlan stream;
+    if (gemv_takes_stream(a, &stream)) return launch_gemv_stream(s, a, stream);
     const GemvPlan plan = gemv_plan(a.n, a.k, a.m, a.ksplit);
     Params p{};
     p.w = static_cast<const uint8_t*>(a.w);

@@ -56,6 +56,10 @@ struct StreamParams {
     uint32_t tile_rows;   // rows per workgroup, 1..16
     uint32_t row_stride;  // bytes between rows of the tile in LDS
     uint32_t x_dtype, y_dtype;
+    // rows longer than a tile can hold: grid.y K segments of seg_blocks super-blocks each
+    uint32_t segments, seg_blocks, m;
+    float* partials;      // [segments][m][n]
+    uint32_t* counters;   // one per (row tile, batch row), zero between launches
 };
 
 // LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
@@ -134,8 +138,11 @@ void gemv_stream_q4k(const StreamParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nb = p.nb;
-    const uint32_t row_bytes = nb * kQ4Bytes;
+    // this workgroup's K segment: super-blocks first .. first + nb - 1 of the rows
+    const uint32_t first = blockIdx.y * p.seg_blocks;
+    const uint32_t nb = min(p.seg_blocks, p.nb - first);
+    const uint32_t row_bytes = nb * kQ4Bytes;          // of the segment
+    const uint32_t full_row_bytes = p.nb * kQ4Bytes;
     const uint32_t row0 = blockIdx.x * p.tile_rows;
     const uint32_t rows = min(p.tile_rows, p.n - row0);
 
@@ -144,7 +151,7 @@ void gemv_stream_q4k(const StreamParams p) {
     float* const rsum = reinterpret_cast<float*>(tile + p.tile_rows * p.row_stride + kSWaves * kSlotBytes);
 
     // 1. this wave's activation blocks are requested first
-    const size_t xrow = (size_t)blockIdx.z * nb * 256u;
+    const size_t xrow = ((size_t)blockIdx.z * p.nb + first) * 256u;
     typename std::conditional<DT == FH_F32, u32x4, u32x2>::type xraw[MAXB];
 #pragma unroll
     for (int i = 0; i < MAXB; ++i) {
@@ -163,13 +170,13 @@ void gemv_stream_q4k(const StreamParams p) {
     // 2. the tile: instruction i covers kilobyte (i % per_row) of row (i / per_row)
     const uint32_t per_row = (row_bytes + 1023u) >> 10;
     const uint32_t total = rows * per_row;
-    const uint8_t* const wbase = p.w + (size_t)row0 * row_bytes + lane * 16u;
+    const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kQ4Bytes + lane * 16u;
     const uint32_t tile_addr = (uint32_t)(uintptr_t)tile;
     uint32_t issued = 0;
     for (uint32_t i = wave; i < total; i += kSWaves) {
         const uint32_t r = i / per_row, c = i - r * per_row;
         if (c * 1024u + lane * 16u < row_bytes)
-            lds_load16(wbase + (size_t)r * row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
+            lds_load16(wbase + (size_t)r * full_row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
         ++issued;
     }
     if (lane < 4u) reinterpret_cast<uint32_t*>(slot + 1024u + 64u)[lane] = 0u;
@@ -249,11 +256,40 @@ void gemv_stream_q4k(const StreamParams p) {
     acc += __shfl_xor(acc, 32, 64);
     if (lane < 16u) rsum[wave * 16u + lane] = acc;
     __syncthreads();
+    float total_sum = 0.f;
     if (tid < rows) {
-        float total_sum = 0.f;
 #pragma unroll
         for (int w = 0; w < kSWaves; ++w) total_sum += rsum[w * 16 + tid];
-        store_from_f32(p.y, (size_t)blockIdx.z * p.n + row0 + tid, p.y_dtype, total_sum);
+    }
+    if (p.segments == 1) {
+        if (tid < rows) store_from_f32(p.y, (size_t)blockIdx.z * p.n + row0 + tid, p.y_dtype, total_sum);
+        return;
+    }
+    // 6. K segments meet in the scratch buffer and the last workgroup of a tile adds them in segment
+    // order (device-scope relaxed atomics, coherent across the L2 slices; src/metal/shaders/ops.metal:1031-1070
+    // has the same two-stage shape)
+    const uint32_t mrow = blockIdx.z;
+    if (tid < rows)
+        __hip_atomic_store(&p.partials[((size_t)blockIdx.y * p.m + mrow) * p.n + row0 + tid], total_sum, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stores above have completed
+    __syncthreads();
+    uint32_t* const flag = reinterpret_cast<uint32_t*>(rsum);   // the row sums have been read
+    if (tid == 0) {
+        uint32_t* counter = p.counters + (size_t)mrow * gridDim.x + blockIdx.x;
+        const uint32_t ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t last = ticket == p.segments - 1 ? 1u : 0u;
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last;
+    }
+    __syncthreads();
+    if (*flag == 0) return;
+    if (tid < rows) {
+        float total = 0.f;
+        for (uint32_t sg = 0; sg < p.segments; ++sg)
+            total += __hip_atomic_load(&p.partials[((size_t)sg * p.m + mrow) * p.n + row0 + tid], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        store_from_f32(p.y, (size_t)mrow * p.n + row0 + tid, p.y_dtype, total);
     }
 }
 
@@ -269,17 +305,36 @@ StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bo
     uint32_t h = (n + cus * rounds - 1u) / (cus * rounds);
     if (h > 16u) h = 16u;
     if (h < 1u) h = 1u;
-    uint32_t units = 9u * nb;          // row bytes / 16
-    if ((units & 1u) == 0) ++units;    // odd number of 16-byte units: 16 rows start in 16 different bank groups
-    plan.row_stride = units * 16u;
-    // an LDS-direct load names its LDS address in 16 bits of M0: the tile stays below 64 KB
+    // An LDS-direct load names its LDS address in 16 bits of M0, so a tile stays below 64 KB, and
+    // a wave owns at most six super-blocks: longer rows are cut into K segments of equal length.
+    auto stride_of = [](uint32_t blocks) {
+        uint32_t units = 9u * blocks;      // bytes / 16
+        if ((units & 1u) == 0) ++units;    // odd number of 16-byte units: 16 rows start in 16 different bank groups
+        return units * 16u;
+    };
+    // ... and, where it must be cut anyway, short enough that three workgroups share a compute
+    // unit's LDS (the headline's uncut 14 x 2896 bytes do)
+    const uint32_t budget = (160u * 1024u) / 3u - 8u * kSlotBytes - 8u * 64u;
+    // (the segments then spread the work, so the tiles are as tall as the matrix instruction)
+    if (nb > 48u || h * stride_of(nb) > 65536u) h = n < 16u ? n : 16u;
+    uint32_t segments = 1, seg = nb;
+    while (seg > 48u || h * stride_of(seg) > (segments == 1 ? 65536u : budget)) {
+        ++segments;
+        seg = (nb + segments - 1u) / segments;
+        if (seg <= 1u) break;
+    }
+    segments = (nb + seg - 1u) / seg;
+    plan.segments = segments;
+    plan.seg_blocks = seg;
+    plan.row_stride = stride_of(seg);
     if (h * plan.row_stride > 65536u) h = 65536u / plan.row_stride;
     plan.tile_rows = h;
     plan.tiles = (n + h - 1u) / h;
     plan.waves = 8u;
     plan.lds_bytes = h * plan.row_stride + plan.waves * kSlotBytes + plan.waves * 64u;
     // matrices of a megabyte or two finish sooner on the FMA kernel's smaller workgroups
-    plan.ok = nb >= 1 && nb <= 48u && h >= 1u && (any_size || (uint64_t)n * nb >= 16384u) && plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u;
+    plan.ok = nb >= 1 && seg >= 1u && seg <= 48u && segments <= 65535u && h >= 1u && (any_size || (uint64_t)n * nb >= 16384u) &&
+              plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u;
     return plan;
 }
 
@@ -294,6 +349,11 @@ const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPla
     p.row_stride = plan.row_stride;
     p.x_dtype = a.x_dtype;
     p.y_dtype = a.y_dtype;
+    p.segments = plan.segments;
+    p.seg_blocks = plan.seg_blocks;
+    p.m = a.m;
+    p.partials = a.partials;
+    p.counters = a.counters;
     typedef void (*Kernel)(const StreamParams);
     // [dtype][blocks per wave: 2, 3, 6]
     static const Kernel kernels[3][3] = {
@@ -309,9 +369,9 @@ const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPla
                                           160 * 1024);
         raised = true;
     }
-    const int shape = p.nb <= 16u ? 0 : p.nb <= 24u ? 1 : 2;
-    hipLaunchKernelGGL(kernels[a.x_dtype][shape], dim3(plan.tiles, 1, a.m), dim3(plan.waves * kWave), plan.lds_bytes, s, p);
-    return "q4_k_gemv_factored";
+    const int shape = plan.seg_blocks <= 16u ? 0 : plan.seg_blocks <= 24u ? 1 : 2;
+    hipLaunchKernelGGL(kernels[a.x_dtype][shape], dim3(plan.tiles, plan.segments, a.m), dim3(plan.waves * kWave), plan.lds_bytes, s, p);
+    return plan.segments > 1 ? "q4_k_gemv_ksplit" : "q4_k_gemv_factored";
 }
 
 }  // namespace fh

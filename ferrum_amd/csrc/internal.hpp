@@ -172,10 +172,20 @@ struct StreamPlan {
     uint32_t waves;       // waves per workgroup
     uint32_t row_stride;  // bytes between a tile's rows in LDS
     uint32_t lds_bytes;
+    // rows too long for one tile are cut into K segments (grid.y), met through the scratch
+    // partials and counters exactly as the FMA kernel's segments are
+    uint32_t segments, seg_blocks;
 };
 // any_size: also matrices so small that the FMA kernel is the faster one
 StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size);
 const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPlan& plan);
+// whether launch_gemv hands this launch to the streamed kernel, and its plan
+bool gemv_takes_stream(const GemvArgs& a, StreamPlan* plan);
+// K segments and row tiles of the kernel launch_gemv will run: what sizes the scratch
+struct GemvScratch {
+    uint32_t segments, tiles;
+};
+GemvScratch gemv_scratch(const GemvArgs& a);
 
 // gemm.hip
 struct GemmArgs {

@@ -290,10 +290,11 @@ def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):
     assert l2 <= rel_l2(want32, want64) * 1.5 + 1e-7, "GPU is less accurate than the sequential CPU sum"
 
 
-# The streamed matrix-core GEMV (dense Q4_K rows of up to 48 super-blocks): row lengths on both
-# sides of its per-wave block budgets, tile heights 1..16, every activation dtype, batched rows.
+# The streamed matrix-core GEMV (dense Q4_K): row lengths on both sides of its per-wave block
+# budgets, tile heights 1..16, every activation dtype, batched rows; rows too long for one tile
+# (more than 48 super-blocks, or 16 rows of them past 64 KB) are cut into 2 to 6 K segments.
 @pytest.mark.parametrize("n,k", [(37, 256), (133, 2560), (300, 4864), (1100, 5120), (4100, 2048), (70, 6144),
-                                 (33, 8192), (20, 12288)])
+                                 (33, 8192), (20, 12288), (100, 12544), (777, 14336), (530, 17408), (64, 34816)])
 @pytest.mark.parametrize("dtype", ["F32", "F16", "BF16"])
 def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
     code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
@@ -304,9 +305,13 @@ def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
         x = oracle.round_storage(synth.activations(m, k, seed=7 * n + m), code).reshape(m, k)
         xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
         out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
-        assert out.operation == ("q4_k_gemv_factored" if m == 1 else "q4_k_gemm")
+        segmented = k > 12288
+        assert out.operation == (("q4_k_gemv_ksplit" if segmented else "q4_k_gemv_factored") if m == 1 else "q4_k_gemm")
         want = oracle.project(Q4_K, packed, n, k, x, accumulate="f64")
         assert_matmul_parity(out.tensor.to_f32(), want, f"streamed gemv {n}x{k} {dtype} m={m}")
+        if segmented:   # the segments are added in a fixed order
+            again = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+            assert np.array_equal(bits(again), bits(out.tensor.to_f32()))
         with fma_gemv(d):
             other = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
         assert rel_l2(out.tensor.to_f32(), other) <= 1e-5 and not np.array_equal(bits(out.tensor.to_f32()), bits(other))

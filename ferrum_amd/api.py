@@ -122,6 +122,7 @@ SYMBOLS = {
     "fh_add_rmsnorm": (_I32, [_P, _VP, _VP, _VP, _U32, _U32, ctypes.c_float, _VP, _VP]),
     "fh_moe_route": (_I32, [_P, _VP, _U32, _VP, ctypes.POINTER(_Policy), _VP]),
     "fh_moe_route_ranked": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP]),
+    "fh_moe_ffn": (_I32, [_P, _VP, _VP, _U32, _VP, ctypes.POINTER(_Policy), _P, _P, _P, _P, _VP, _VP]),
     "fh_expert_combine_shared": (_I32, [_P, _VP, _VP, _U32, _U32, _U32, _VP, _VP, _VP]),
     "fh_hybrid_moe_route": (_I32, [_P, _VP, _U32, ctypes.POINTER(_Policy), _VP, _VP, _U32, _VP, _VP, _VP]),
     "fh_hybrid_project": (_I32, [_P, _P, _VP, _U32, _VP, _U32]),
@@ -1076,6 +1077,30 @@ class SparseMoe:
                              "shared_activated": Tensor.zeros(d, (tokens, si), dtype),
                              "shared_output": Tensor.zeros(d, (tokens, h), dtype)})
         return self._ws
+
+    def forward_in_one_call(self, hidden: Tensor, router_logits: Tensor, shared_gate: Tensor | None = None,
+                            out: Tensor | None = None) -> Tensor:
+        """fh_moe_ffn: the steps of ``forward`` (inputs folded into the projections) enqueued by
+        one library call, temporaries in the library's workspace; the same bits."""
+        dims = hidden.shape()
+        if len(dims) != 2 or dims[1] != self.hidden_size or dims[0] == 0:
+            raise ShapeError("sparse expert input requires [tokens,hidden]")
+        if router_logits.shape() != (dims[0], self.expert_count):
+            raise ShapeError("router logits require [tokens,experts]")
+        if shared_gate is not None and shared_gate.numel() != dims[0]:
+            raise ShapeError("shared gate requires one value per token")
+        if out is None:
+            out = Tensor.zeros(self.device, dims, hidden.dtype)
+        hv, lv, ov, pc = hidden._view(), router_logits._view(), out._view(), self.routing._c()
+        bv = self.selection_bias._view() if self.selection_bias is not None else None
+        gv = shared_gate._view() if shared_gate is not None else None
+        ref = lambda v: ctypes.byref(v) if v is not None else None
+        _check(_lib.fh_moe_ffn(self.device._handle, ctypes.byref(hv), ctypes.byref(lv), dims[0], ref(bv), ctypes.byref(pc),
+                               self.input_experts._handle, self.output_experts._handle,
+                               _handle_of(self.shared_input) if self.shared_input is not None else None,
+                               _handle_of(self.shared_output) if self.shared_output is not None else None,
+                               ref(gv), ctypes.byref(ov)))
+        return out
 
     def take_stats(self) -> MoeStats:
         """The statistics gathered since the last call, which start afresh (take_stats,

@@ -294,6 +294,11 @@ void fh_device_destroy(fh_device* device) {
         device->stream = nullptr;
     }
     if (device->scratch) (void)hipFree(device->scratch);
+    if (device->workspace) {
+        if (device->workspace->ptr) (void)hipFree(device->workspace->ptr);
+        delete device->workspace;
+        device->workspace = nullptr;
+    }
     for (void* old : device->retired_scratch) (void)hipFree(old);
     device->retired_scratch.clear();
     device->scratch = nullptr;
@@ -1556,6 +1561,156 @@ fh_status fh_expert_combine_shared(fh_device* device, const fh_view* in, const f
                                    const fh_view* shared_gate, const fh_view* out) {
     if (shared == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     return combine(device, in, metadata, tokens, hidden, top_k, shared, shared_gate, out);
+}
+
+// ---- the routed FFN in one call ------------------------------------------------------------
+
+namespace {
+
+// The workspace: a buffer object the library owns (it holds no count on the device), grown
+// like the scratch: outside recordings only, by at least 2x, old blocks kept for the recorded
+// executions that carry their address.
+fh_status ensure_workspace(fh_device* d, size_t bytes) {
+    if (d->workspace != nullptr && d->workspace->bytes >= bytes) return FH_OK;
+    if (d->capturing)
+        return fail(FH_ERR_SYNCHRONIZATION, "the routed FFN's workspace must grow: run the call once before recording it");
+    FH_HIP(hipStreamSynchronize(d->stream));
+    if (d->workspace == nullptr) {
+        d->workspace = new (std::nothrow) fh_buffer();
+        if (d->workspace == nullptr) return fail(FH_ERR_ALLOCATION, "out of host memory");
+        d->workspace->device = d;
+    }
+    if (bytes < 2 * d->workspace->bytes) bytes = 2 * d->workspace->bytes;
+    if (d->workspace->ptr) {
+        if (d->live_graphs > 0) d->retired_scratch.push_back(d->workspace->ptr);
+        else (void)hipFree(d->workspace->ptr);
+    }
+    d->workspace->ptr = nullptr;
+    d->workspace->bytes = 0;
+    hipError_t e = hipMalloc(&d->workspace->ptr, bytes);
+    if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+    d->workspace->bytes = bytes;
+    return FH_OK;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* router_logits, uint32_t tokens,
+                     const fh_view* selection_bias, const fh_routing_policy* policy,
+                     const fh_qmatrix* input_experts, const fh_qmatrix* output_experts,
+                     const fh_qmatrix* shared_input, const fh_qmatrix* shared_output,
+                     const fh_view* shared_gate, const fh_view* out) {
+    if (device == nullptr || hidden == nullptr || router_logits == nullptr || policy == nullptr ||
+        input_experts == nullptr || output_experts == nullptr || out == nullptr)
+        return fail(FH_ERR_PARAMETER, "null argument");
+    // SparseMoe::new's geometry checks (src/nn/moe.rs:137-181)
+    const uint64_t e = input_experts->experts, two_i = input_experts->rows, h = input_experts->cols;
+    if (tokens == 0 || two_i == 0 || two_i % 2 != 0 || output_experts->experts != e || output_experts->rows != h ||
+        output_experts->cols * 2 != two_i || policy->experts != e || policy->top_k == 0 || policy->top_k > e ||
+        input_experts->device != device || output_experts->device != device)
+        return fail(FH_ERR_SHAPE, "invalid sparse expert weight geometry");
+    const bool shared = shared_input != nullptr;
+    if ((shared_input == nullptr) != (shared_output == nullptr) ||
+        (shared && (shared_input->cols != h || shared_output->rows != h || shared_input->rows == 0 ||
+                    shared_input->rows != 2 * shared_output->cols || shared_input->experts != 1 ||
+                    shared_output->experts != 1 || shared_input->device != device || shared_output->device != device)))
+        return fail(FH_ERR_SHAPE, "invalid shared expert weight geometry");
+    if (!shared && shared_gate != nullptr) return fail(FH_ERR_PARAMETER, "a shared gate without a shared expert");
+    if (out->dtype != hidden->dtype) return fail(FH_ERR_DTYPE, "the routed FFN writes the activation dtype");
+    const uint32_t k = policy->top_k, dt = hidden->dtype;
+    const size_t es = dtype_bytes(dt), inter = (size_t)two_i / 2, si = shared ? (size_t)shared_output->cols : 0;
+    const bool rides = shared && shared_input->rows == two_i && shared_input->ggml_type == input_experts->ggml_type &&
+                       shared_output->ggml_type == output_experts->ggml_type;
+
+    // tokens are taken in chunks whose routing temporaries stay under the limit (src/nn/moe.rs:232-256)
+    const size_t per_assignment = (2 * (size_t)h + 3 * inter) * es + 3 * sizeof(float);
+    const size_t per_token = per_assignment * k + ((size_t)e + (size_t)h) * es;
+    const size_t limit = (size_t)tuning(device, "moe_routing_temporary_limit");
+    const uint32_t chunk = (uint32_t)std::min<size_t>(tokens, std::max<size_t>(1, limit / per_token));
+
+    // workspace layout for one chunk
+    const size_t a_max = (size_t)chunk * k;
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        const size_t here = at;
+        at += align256(bytes);
+        return here;
+    };
+    const size_t meta_at = take(a_max * 3 * sizeof(float));
+    const size_t assigned_at = take(a_max * h * es);
+    const size_t projected_at = take(a_max * two_i * es);
+    const size_t activated_at = take(a_max * inter * es);
+    const size_t expert_out_at = take(a_max * h * es);
+    const size_t sproj_at = take(shared ? (size_t)chunk * 2 * si * es : 0);
+    const size_t sact_at = take(shared ? (size_t)chunk * si * es : 0);
+    const size_t sout_at = take(shared ? (size_t)chunk * h * es : 0);
+    fh_status st = ensure_workspace(device, at);
+    if (st != FH_OK) return st;
+    fh_buffer* ws = device->workspace;
+    auto view = [&](size_t offset, uint32_t dtype) { return fh_view{ws, offset, dtype}; };
+
+    for (uint32_t start = 0; start < tokens; start += chunk) {
+        const uint32_t count = std::min(chunk, tokens - start);
+        const uint32_t a = count * k;
+        const fh_view x = {hidden->buffer, hidden->offset + (size_t)start * h * es, dt};
+        const fh_view logits = {router_logits->buffer,
+                                router_logits->offset + (size_t)start * e * dtype_bytes(router_logits->dtype),
+                                router_logits->dtype};
+        const fh_view y = {out->buffer, out->offset + (size_t)start * h * es, dt};
+        fh_view gate{};
+        if (shared_gate) gate = {shared_gate->buffer, shared_gate->offset + (size_t)start * sizeof(float), shared_gate->dtype};
+        const fh_view meta = view(meta_at, FH_F32), assigned = view(assigned_at, dt), projected = view(projected_at, dt),
+                      activated = view(activated_at, dt), expert_out = view(expert_out_at, dt),
+                      sproj = view(sproj_at, dt), sact = view(sact_at, dt), sout = view(sout_at, dt);
+        st = fh_moe_route(device, &logits, count, selection_bias, policy, &meta);
+        if (st != FH_OK) return st;
+        // the copy and the activation ride inside the projections: per assignment in decode, in
+        // the grouped kernel's gather of an expert's rows beyond it (f32 rows have no grouped form)
+        const bool fused = a <= 31 || dt != FH_F32;
+        if (shared && rides && fused) {
+            st = fh_expert_project_with_shared(device, input_experts, shared_input, &x, count, FH_INPUT_GATHER, a, &meta,
+                                               nullptr, &projected, &sproj);
+            if (st != FH_OK) return st;
+            st = fh_expert_project_with_shared(device, output_experts, shared_output, &projected, count,
+                                               FH_INPUT_SILU_MUL, a, &meta, &sproj, &expert_out, &sout);
+            if (st != FH_OK) return st;
+        } else {
+            if (fused) {
+                st = fh_expert_project_fused(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected);
+                if (st != FH_OK) return st;
+                st = fh_expert_project_fused(device, output_experts, &projected, a, FH_INPUT_SILU_MUL, a, &meta, &expert_out);
+                if (st != FH_OK) return st;
+            } else {
+                st = fh_expert_assign(device, &x, count, (uint32_t)h, &meta, k, &assigned);
+                if (st != FH_OK) return st;
+                st = fh_expert_project_quantized(device, input_experts, &assigned, a, &meta, &projected);
+                if (st != FH_OK) return st;
+                st = fh_expert_silu_mul(device, &projected, a, (uint32_t)inter, &activated);
+                if (st != FH_OK) return st;
+                st = fh_expert_project_quantized(device, output_experts, &activated, a, &meta, &expert_out);
+                if (st != FH_OK) return st;
+            }
+            if (shared) {
+                st = fh_project_quantized(device, shared_input, &x, count, &sproj);
+                if (st != FH_OK) return st;
+                if (count <= 31) {
+                    st = fh_project_silu_mul_quantized(device, shared_output, &sproj, count, &sout);
+                } else {
+                    st = fh_expert_silu_mul(device, &sproj, count, (uint32_t)si, &sact);
+                    if (st != FH_OK) return st;
+                    st = fh_project_quantized(device, shared_output, &sact, count, &sout);
+                }
+                if (st != FH_OK) return st;
+            }
+        }
+        st = shared ? fh_expert_combine_shared(device, &expert_out, &meta, count, (uint32_t)h, k, &sout,
+                                               shared_gate ? &gate : nullptr, &y)
+                    : fh_expert_combine(device, &expert_out, &meta, count, (uint32_t)h, k, &y);
+        if (st != FH_OK) return st;
+    }
+    return FH_OK;
 }
 
 // ---- batched execution ---------------------------------------------------------------

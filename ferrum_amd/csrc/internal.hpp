@@ -35,6 +35,8 @@ struct fh_device {
     // scratch blocks that were outgrown while recorded executions (which carry their address)
     // were alive: freed with the last of those
     std::vector<void*> retired_scratch;
+    // temporaries of fh_moe_ffn: one block, grown like the scratch and retired with it
+    fh_buffer* workspace = nullptr;
     int live_graphs = 0;
     std::vector<void*> deferred_frees;
     std::vector<std::pair<hipGraphExec_t, hipGraph_t>> deferred_graphs;

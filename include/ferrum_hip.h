@@ -413,6 +413,24 @@ fh_status fh_expert_silu_mul(fh_device* device, const fh_view* in, uint32_t assi
 fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view* metadata,
                             uint32_t tokens, uint32_t hidden, uint32_t top_k, const fh_view* out);
 
+/* SparseMoe::forward (src/nn/moe.rs:222-390) in one call: route, gate|up projection, SiLU*up,
+ * down projection and weighted combine of `tokens` rows, with the hybrid engine's shared expert
+ * (HybridModel::moe_ffn, src/hybrid/engine.rs:2881-3092) when shared_input [2*I_s, H] (gate rows
+ * first) and shared_output [H, I_s] are given; shared_gate (may be NULL) [tokens] f32 scales its
+ * rows.  hidden [tokens, H], router_logits [tokens, experts] (the router's own dense layer is the
+ * caller's), selection_bias as in fh_moe_route, out [tokens, H] in the activation dtype.  The
+ * steps are exactly those the calls above would make one by one, with expert_assign and
+ * expert_silu_mul folded into the projections and the shared expert riding in the routed launches
+ * where fh_expert_project_with_shared allows, so the result has their bits.  Tokens are taken in
+ * chunks whose routing temporaries stay under the tuning value moe_routing_temporary_limit
+ * (src/nn/moe.rs:232-256); the temporaries live in a workspace the library keeps per device,
+ * which grows outside recordings only (run the call once before recording it). */
+fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* router_logits, uint32_t tokens,
+                     const fh_view* selection_bias, const fh_routing_policy* policy,
+                     const fh_qmatrix* input_experts, const fh_qmatrix* output_experts,
+                     const fh_qmatrix* shared_input, const fh_qmatrix* shared_output,
+                     const fh_view* shared_gate, const fh_view* out);
+
 /* ---- batched execution ---------------------------------------------------------
  * MetalDevice::execution_with_shared_encoder / Execution::finish
  * (src/metal/mod.rs:263-278, 563-572): operator calls between begin and end

@@ -777,6 +777,29 @@ public:
         return out;
     }
 
+    // fh_moe_ffn: the steps of forward() with the inputs folded into the projections, enqueued by one
+    // library call with its temporaries in the library's workspace; the same bits.
+    Tensor forward_in_one_call(const Tensor& hidden, const Tensor& router_logits, const Tensor* selection_bias = nullptr,
+                               const Tensor* shared_gate = nullptr) const {
+        const auto& dims = hidden.shape();
+        const size_t h = input_.columns(), e = input_.experts();
+        if (dims.size() != 2 || dims[1] != h || dims[0] == 0)
+            throw Error(ErrorKind::Shape, "sparse expert input requires [tokens,hidden]");
+        if (router_logits.shape() != std::vector<size_t>{dims[0], e})
+            throw Error(ErrorKind::Shape, "router logits require [tokens,experts]");
+        Tensor out = device_.zeros({dims[0], h}, hidden.dtype());
+        fh_view hv = hidden.c_view(), lv = router_logits.c_view(), ov = out.c_view(), bv{}, gv{};
+        if (selection_bias) bv = selection_bias->c_view();
+        if (shared_gate) gv = shared_gate->c_view();
+        const fh_routing_policy pc = routing_.c();
+        check(fh_moe_ffn(device_.raw(), &hv, &lv, (uint32_t)dims[0], selection_bias ? &bv : nullptr, &pc,
+                                        input_.matrix().raw(), output_.matrix().raw(),
+                                        shared_input_ ? shared_input_->raw() : nullptr,
+                                        shared_output_ ? shared_output_->raw() : nullptr,
+                                        shared_gate ? &gv : nullptr, &ov));
+        return out;
+    }
+
     // most f32 assignments that take the fused per-assignment kernels (f32 rows have no
     // grouped form by default, and the per-assignment SiLU is recomputed by every workgroup);
     // also the most assignments whose shared expert rides in the routed launches

@@ -276,6 +276,8 @@ int main() {
             const auto cut = moe.forward(xt, lt, nullptr, &gt).to_f32();
             const MoeStats cs = moe.take_stats();
             d.set_moe_routing_temporary_limit(before);
+            const auto one_call = moe.forward_in_one_call(xt, lt, nullptr, &gt).to_f32();
+            report("fh_moe_ffn gives the bits of SparseMoe::forward", std::memcmp(one_call.data(), whole.data(), whole.size() * 4) == 0);
             report("SparseMoe::forward in chunks gives the bits of the whole pass",
                    before == (size_t(128) << 20) && std::memcmp(cut.data(), whole.data(), cut.size() * 4) == 0 &&
                        ws.assignments == many * top_k && cs.assignments == many * top_k && !cs.active_experts_known &&

@@ -661,6 +661,45 @@ def test_chunked_forward_gives_the_bits_of_the_unchunked_one(api, d, dtype, shar
     assert moe.take_stats() == api.MoeStats()
 
 
+@pytest.mark.parametrize("dtype,tokens,shared,gated", [("F16", 1, True, True), ("F16", 3, True, False), ("F16", 300, True, True),
+                                                       ("F16", 20, False, False), ("F32", 5, True, True), ("F32", 40, True, False),
+                                                       ("F32", 40, False, False), ("BF16", 70, True, False)])
+def test_the_ffn_in_one_call_gives_the_bits_of_the_separate_calls(api, d, dtype, tokens, shared, gated):
+    # fh_moe_ffn enqueues the steps SparseMoe.forward makes one by one (per-assignment and grouped
+    # kernels, the shared expert riding or apart, f32 rows through assign / silu_mul launches of
+    # their own), with its temporaries in the library's workspace; also cut into chunks, and
+    # recorded into an execution once the workspace has its size
+    (experts, hidden, inter, top_k), packed, w, x, logits, xt, lt = _shared_case(api, d, dtype, tokens, 301)
+    kw = dict(shared_input=w["sin"], shared_output=w["sout"]) if shared else {}
+    moe = api.SparseMoe(d, w["win"], w["wout"], api.MoeRoutingPolicy(experts, top_k), **kw)
+    gate = api.Tensor.from_f32(d, (tokens,), api.DType.F32,
+                               (0.25 + 0.5 * synth.rng(302).random(tokens)).astype(np.float32)) if gated else None
+    want = moe.forward(xt, lt, shared_gate=gate)
+    got = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+    assert np.abs(want.to_f32()).max() > 1e-3
+    assert np.array_equal(got.raw(), want.raw())
+    out = api.Tensor.zeros(d, (tokens, hidden), xt.dtype)
+    with d.execution() as ex:
+        moe.forward_in_one_call(xt, lt, shared_gate=gate, out=out)
+    for _ in range(2):
+        ex.graph.launch()
+        d.synchronize()
+        assert np.array_equal(out.raw(), want.raw())
+        api._check(api._lib.fh_buffer_fill_zero(out.buffer._handle, 0, out.byte_size()))
+        d.synchronize()
+    if tokens >= 40:
+        before = d.moe_routing_temporary_limit()
+        try:
+            d.set_moe_routing_temporary_limit(16 * moe.temporary_bytes(1, xt.dtype))
+            cut = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+            stepwise = moe.forward(xt, lt, shared_gate=gate)
+        finally:
+            d.set_moe_routing_temporary_limit(before)
+        assert np.array_equal(cut.raw(), stepwise.raw())
+    with pytest.raises(api.ShapeError):
+        moe.forward_in_one_call(xt, api.Tensor.zeros(d, (tokens, experts + 1), api.DType.F32))
+
+
 def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
     # 32 rows of 2816 halves are more than the grouped kernel's LDS: the routed rows are staged and
     # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit

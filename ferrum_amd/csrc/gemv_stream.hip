@@ -297,7 +297,7 @@ void gemv_stream_q4k(const StreamParams p) {
 
 // Tile height that spreads the rows evenly: the fewest 16-row rounds per compute unit, then the
 // smallest height that still fits them.
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size) {
+StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size, int forced_segments) {
     StreamPlan plan{};
     const uint32_t nb = k / 256u;
     const uint32_t cus = cu_count > 0 ? (uint32_t)cu_count : 256u;
@@ -316,8 +316,10 @@ StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bo
     // unit's LDS (the headline's uncut 14 x 2896 bytes do)
     const uint32_t budget = (160u * 1024u) / 3u - 8u * kSlotBytes - 8u * 64u;
     // (the segments then spread the work, so the tiles are as tall as the matrix instruction)
-    if (nb > 48u || h * stride_of(nb) > 65536u) h = n < 16u ? n : 16u;
-    uint32_t segments = 1, seg = nb;
+    // the reference's K-split switch asks for at least that many segments, as far as whole blocks go
+    const uint32_t wanted = forced_segments > 1 ? ((uint32_t)forced_segments < nb ? (uint32_t)forced_segments : nb) : 1u;
+    if (wanted > 1u || nb > 48u || h * stride_of(nb) > 65536u) h = n < 16u ? n : 16u;
+    uint32_t segments = wanted, seg = (nb + wanted - 1u) / wanted;
     while (seg > 48u || h * stride_of(seg) > (segments == 1 ? 65536u : budget)) {
         ++segments;
         seg = (nb + segments - 1u) / segments;

@@ -179,7 +179,7 @@ struct StreamPlan {
     uint32_t segments, seg_blocks;
 };
 // any_size: also matrices so small that the FMA kernel is the faster one
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size);
+StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size, int forced_segments);
 const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPlan& plan);
 // whether launch_gemv hands this launch to the streamed kernel, and its plan
 bool gemv_takes_stream(const GemvArgs& a, StreamPlan* plan);

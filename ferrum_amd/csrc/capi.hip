@@ -248,7 +248,8 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     }
     d->tuning["k_quant_gemv_ksplit"] = 0;   // 0 = automatic
     d->tuning["gemm_min_rows"] = 2;         // smallest M that takes the MFMA tile path
-    d->tuning["gemm_wide_shape"] = 1;       // matrix instruction of the 256-row tile: 0 = 16x16x32, 1 = 32x32x16 where it wins, 2 = 32x32x16 always
+    d->tuning["gemm_wide_shape"] = 1;       // matrix instruction of the 128- and 256-row tiles: 0 = 16x16x32, 1 = whichever is estimated faster, 2 = 32x32x16
+    d->tuning["gemm_wide32_tile"] = 0;      // 0 = by shape; 12, 14, 15 (128-row tile x 64, 128, 160 columns), 24, 25 (256-row tile)
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
@@ -357,6 +358,8 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 0 && value <= 2;
     } else if (k == "gemm_wide_shape") {
         ok = value >= 0 && value <= 2;
+    } else if (k == "gemm_wide32_tile") {
+        ok = value == 0 || value == 12 || value == 14 || value == 15 || value == 24 || value == 25;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {
@@ -651,6 +654,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.cu_count = device->props.multiProcessorCount;
         a.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
         a.wide_shape = (int)tuning(device, "gemm_wide_shape");
+        a.wide32_tile = (int)tuning(device, "gemm_wide32_tile");
         a.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         a.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, a);
@@ -1367,6 +1371,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.cu_count = device->props.multiProcessorCount;
         g.wide_min_rows = (int)tuning(device, "gemm_wide_min_rows");
         g.wide_shape = (int)tuning(device, "gemm_wide_shape");
+        g.wide32_tile = (int)tuning(device, "gemm_wide32_tile");
         g.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         g.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
         device->last_operation = launch_gemm(device->stream, g);

@@ -835,8 +835,17 @@ __device__ __forceinline__ float16v mfma32(uint4 a, uint4 b, float16v c) {
 // LDS of the 32x32x16 form: four activation rings of 16 KB (one per multiplying wave, two
 // stages of 64 rows x 64 K), then the two weight slabs.  The rings come first: an LDS-direct
 // load takes its LDS address from M0, which holds 16 bits.
-constexpr uint32_t kWide32RingBytes = 16384;
-constexpr uint32_t kWide32WeightsAt = 4 * kWide32RingBytes;
+// (RT = row tiles of 32 per multiplying wave: 2 for the 256-row tile, 1 for a 128-row tile)
+template <int RT>
+struct Wide32 {
+    static constexpr uint32_t kWaveRows = 32 * RT;
+    static constexpr uint32_t kTileRows = 4 * kWaveRows;
+    static constexpr uint32_t kHalfBytes = kWaveRows * 64;          // a wave's rows x 32 K
+    static constexpr uint32_t kStageBytes = 2 * kHalfBytes;         // one slab
+    static constexpr uint32_t kRingBytes = 2 * kStageBytes;         // two stages
+    static constexpr uint32_t kWeightsAt = 4 * kRingBytes;
+    static constexpr int kDmaPieces = 4 * RT;                       // load instructions per slab and wave
+};
 
 // LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
 __device__ __forceinline__ void lds_direct16(const void* g, uint32_t lds_addr) {
@@ -844,7 +853,7 @@ __device__ __forceinline__ void lds_direct16(const void* g, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
 }
 
-template <uint32_t TYPE, int DT, int NT>
+template <uint32_t TYPE, int DT, int NT, int RT>
 __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restrict__ w,
                                                           const uint16_t* __restrict__ x,
                                                           void* __restrict__ y, uint32_t m, uint32_t n,
@@ -852,6 +861,7 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
                                                           uint32_t tiles_m, uint32_t tiles_n) {
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
+    using Geo = Wide32<RT>;
     constexpr uint32_t kRowsW = 32 * NT;
     constexpr uint32_t kStage = kRowsW * kLd;  // halfs per buffer
     constexpr bool kExtra = NT > 4;            // rows 128 .. 159 are a second decode task
@@ -866,7 +876,7 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
         tile_m = r >> 3;
         if (tile_n >= tiles_n) return;
     }
-    const uint32_t n0 = tile_n * cols, m0 = tile_m * kWM;
+    const uint32_t n0 = tile_n * cols, m0 = tile_m * Geo::kTileRows;
     const uint32_t ncols = n - n0 < cols ? n - n0 : cols;
     const uint32_t k = nb << 8;
 
@@ -881,19 +891,23 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
         const uint8_t* esrc = w + (size_t)(n0 + (er < ncols ? er : ncols - 1)) * nb * kBlockBytes;
         constexpr bool kDeep = !kEightDwords<TYPE>;   // Q6_K and Q8_0 sets are twice as large: one block ahead
         BlockW<TYPE> cur, n1, n2, ecur, en1, en2;
+        const bool has_row = kRowsW >= 128 || wr < kRowsW;   // narrow tiles leave some decoding lanes without a row
         auto store_slab = [&](int c) {
-            uint16_t* ws = lds + kWide32WeightsAt / 2 + (c & 1) * kStage;
-            decode_block_slab<TYPE, DT>(cur, c, wh, ws + wr * kLd);
+            uint16_t* ws = lds + Geo::kWeightsAt / 2 + (c & 1) * kStage;
+            if (has_row) decode_block_slab<TYPE, DT>(cur, c, wh, ws + wr * kLd);
             if (kExtra) decode_block_piece<TYPE, DT>(ecur, c, eh, (int)et, ws + er * kLd);
         };
-        cur.load(wsrc, wh);
+        auto load_main = [&](BlockW<TYPE>& set, uint32_t b) {
+            if (has_row) set.load(wsrc + (size_t)b * kBlockBytes, wh);
+        };
+        load_main(cur, 0);
         if (kExtra) ecur.load(esrc, eh);
         if (nb > 1) {
-            n1.load(wsrc + kBlockBytes, wh);
+            load_main(n1, 1);
             if (kExtra) en1.load(esrc + kBlockBytes, eh);
         }
         if (kDeep && nb > 2) {
-            n2.load(wsrc + 2 * (size_t)kBlockBytes, wh);
+            load_main(n2, 2);
             if (kExtra) en2.load(esrc + 2 * (size_t)kBlockBytes, eh);
         }
         store_slab(0);
@@ -917,10 +931,10 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
                         ecur = en1;
                         n1 = n2;
                         en1 = en2;
-                        if (b + 3 < nb) n2.load(wsrc + (size_t)(b + 3) * kBlockBytes, wh);
+                        if (b + 3 < nb) load_main(n2, b + 3);
                     } else {
                         ecur = en1;
-                        if (b + 2 < nb) n1.load(wsrc + (size_t)(b + 2) * kBlockBytes, wh);
+                        if (b + 2 < nb) load_main(n1, b + 2);
                     }
                     store_slab(0);
                 }
@@ -930,9 +944,9 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
     }
 
     // ---- consumers: own activation rows by LDS-direct loads, weights from LDS -> MFMA ----
-    float16v acc[2][NT];
+    float16v acc[RT][NT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j)
 #pragma unroll
@@ -945,54 +959,59 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
     // 16-byte piece q of local row r sits at unit 4 r + (q ^ ((r >> 2) & 3)), which spreads
     // the sixteen rows a fragment read touches over all banks.  One load instruction fills
     // 1 KB: 16 rows x 4 pieces, lane l = (row 16 t + l / 4, unit l % 4).
-    const uint32_t a_ring = wave * kWide32RingBytes;   // stage s of the ring is a_ring + 8192 (s & 1)
-    const uint16_t* adma[4];
+    const uint32_t a_ring = wave * Geo::kRingBytes;   // stage s of the ring is a_ring + kStageBytes (s & 1)
+    const uint16_t* adma[2 * RT];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2 * RT; ++t) {
         const uint32_t r = 16 * t + (lane >> 2);
         const uint32_t q = (lane & 3u) ^ ((r >> 2) & 3u);
-        const uint32_t row = m0 + wave * 64 + r;
+        const uint32_t row = m0 + wave * Geo::kWaveRows + r;
         // rows past m are clamped: they only feed outputs that are never stored
         adma[t] = x + (size_t)(row < m ? row : m - 1) * k + 8 * q;
     }
-    // load instruction i (0..7) of a slab: half i / 4, rows 16 (i % 4) ..
+    // load instruction i of a slab: half i / (2 RT), rows 16 (i % (2 RT)) ..
     auto dma_piece = [&](uint32_t slab, int i) {
-        lds_direct16(adma[i & 3] + (size_t)slab * 64 + 32 * (i >> 2),
-                     a_ring + (slab & 1u) * 8192u + (uint32_t)(i >> 2) * 4096u + (uint32_t)(i & 3) * 1024u);
+        lds_direct16(adma[i % (2 * RT)] + (size_t)slab * 64 + 32 * (i / (2 * RT)),
+                     a_ring + (slab & 1u) * Geo::kStageBytes + (uint32_t)(i / (2 * RT)) * Geo::kHalfBytes +
+                         (uint32_t)(i % (2 * RT)) * 1024u);
     };
     auto dma_slab = [&](uint32_t slab) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dma_piece(slab, i);
+        for (int i = 0; i < Geo::kDmaPieces; ++i) dma_piece(slab, i);
     };
     // fragment addresses: activations of row tile i at step s (0..3) of the slab, weights of column tile j
     const uint32_t sw = (r32 >> 2) & 3u;
     const uint32_t a_off0 = (4 * r32 + ((2 * kg) ^ sw)) * 16, a_off1 = (4 * r32 + ((2 * kg + 1) ^ sw)) * 16;
     const uint8_t* const lds_bytes = reinterpret_cast<const uint8_t*>(lds);
-    const uint32_t b_off = kWide32WeightsAt + (r32 * kLd + 16 * kg) * 2;
-    constexpr int kFrags = 2 + NT;   // fragments of a step: two of activations, NT of weights
+    const uint32_t b_off = Geo::kWeightsAt + (r32 * kLd + 16 * kg) * 2;
+    constexpr int kFrags = RT + NT;   // fragments of a step: RT of activations, NT of weights
     struct Frags {
         uint4 v[kFrags];
     };
     auto read_frag = [&](Frags& f, uint32_t slab, int s, int t) {
-        if (t < 2) {
-            f.v[t] = *reinterpret_cast<const uint4*>(lds_bytes + a_ring + (slab & 1u) * 8192u + (s >> 1) * 4096u +
-                                                      ((s & 1) ? a_off1 : a_off0) + t * 2048);
+        if (t < RT) {
+            f.v[t] = *reinterpret_cast<const uint4*>(lds_bytes + a_ring + (slab & 1u) * Geo::kStageBytes +
+                                                      (s >> 1) * Geo::kHalfBytes + ((s & 1) ? a_off1 : a_off0) + t * 2048);
         } else {
             f.v[t] = *reinterpret_cast<const uint4*>(lds_bytes + b_off + (slab & 1u) * (kStage * 2) + (s >> 1) * 64 +
-                                                      (s & 1) * 16 + (t - 2) * (32 * kLd * 2));
+                                                      (s & 1) * 16 + (t - RT) * (32 * kLd * 2));
         }
     };
     // One step: 2 NT multiplications on `cur`, and between them, one at a time so that each
     // hides behind a multiplication in flight, the reads of step (slab, s)'s fragments into
     // `next` and, with DMA set, the eight load instructions of activation slab `dma`.
     auto step = [&](const Frags& cur, Frags& next, uint32_t slab, int s, auto with_reads, auto with_dma, uint32_t dma) {
+        constexpr int kMul = RT * NT;
+        constexpr int kSlots = kMul > kFrags ? (kMul > Geo::kDmaPieces ? kMul : Geo::kDmaPieces)
+                                             : (kFrags > Geo::kDmaPieces ? kFrags : Geo::kDmaPieces);
 #pragma unroll
-        for (int idx = 0; idx < 2 * NT; ++idx) {
+        for (int idx = 0; idx < kSlots; ++idx) {
             if constexpr (decltype(with_reads)::value)
                 if (idx < kFrags) read_frag(next, slab, s, idx);
             if constexpr (decltype(with_dma)::value)
-                if (idx < 8) dma_piece(dma, idx);
-            acc[idx & 1][idx >> 1] = mfma32<DT>(cur.v[idx & 1], cur.v[2 + (idx >> 1)], acc[idx & 1][idx >> 1]);
+                if (idx < Geo::kDmaPieces) dma_piece(dma, idx);
+            if (idx < kMul)
+                acc[idx % RT][idx / RT] = mfma32<DT>(cur.v[idx % RT], cur.v[RT + idx / RT], acc[idx % RT][idx / RT]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -1033,13 +1052,13 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
 
     // element v of a lane's block: row 8 (v / 4) + 4 kg + v % 4, column r32
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             const uint32_t lc = 32 * j + r32;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const uint32_t row = m0 + wave * 64 + 32 * i + 8 * (v >> 2) + 4 * kg + (v & 3);
+                const uint32_t row = m0 + wave * Geo::kWaveRows + 32 * i + 8 * (v >> 2) + 4 * kg + (v & 3);
                 if (row < m && lc < ncols)
                     store_from_f32(y, (size_t)row * n + n0 + lc, y_dtype, acc[i][j][v]);
             }
@@ -1049,6 +1068,7 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
 struct WidePlan {
     int nt;
     uint32_t cols, tiles_m, tiles_n;
+    int rt;   // 32x32x16 form: row tiles of 32 per multiplying wave (2: 256-row tile, 1: 128-row tile)
 };
 
 // Columns per workgroup: 128 or 136, whichever wastes the least of the chip's `cus`
@@ -1072,37 +1092,93 @@ WidePlan wide_plan(uint32_t m, uint32_t n, int cus) {
     return best;
 }
 
-// Columns per workgroup of the 32x32x16 form: 128 or 160.
-WidePlan wide32_plan(uint32_t m, uint32_t n, int cus) {
+// What a round of workgroups of one 32x32x16 tile takes over rows of 5120, in us: one workgroup per
+// compute unit (`alone`), or two where LDS and registers hold two, from the first pair
+// (`pair_first`) to a pair everywhere (`pair_all`; 0 = the tile runs alone).  Measured on
+// 17408 / 34816 / 8192 / 5120 columns at 48 - 2048 rows; two 128 x 128 tiles on a compute unit take
+// 88 - 108 us where one takes 64, so a pair does a fifth to a half more per microsecond.
+struct Wide32Tile {
+    int rt, nt;
+    double alone, pair_first, pair_all;
+};
+constexpr Wide32Tile kWide32Tiles[] = {
+    {1, 2, 49.0, 61.0, 71.0}, {1, 4, 64.0, 88.0, 108.0}, {1, 5, 79.0, 0.0, 0.0},
+    {2, 4, 90.0, 0.0, 0.0},   {2, 5, 108.0, 0.0, 0.0},
+};
+// an eighth of a tile's time is its prologue and its stores, the rest goes with the length of a row
+inline double wide_row_length_factor(uint32_t k) { return 0.125 + 0.875 * (double)k / 5120.0; }
+
+WidePlan wide32_make(uint32_t m, uint32_t n, int rt, int nt) {
+    const uint32_t rows = 128u * (uint32_t)rt, cols = 32u * (uint32_t)nt;
+    return WidePlan{nt, cols, (m + rows - 1) / rows, (n + cols - 1) / cols, rt};
+}
+
+double wide32_estimate(const Wide32Tile& t, uint64_t wgs, uint64_t cus) {
+    if (wgs <= cus) return t.alone;
+    if (t.pair_first == 0.0) return (double)((wgs + cus - 1) / cus) * t.alone;
+    const uint64_t full = wgs / (2 * cus), rest = wgs % (2 * cus);
+    double us = (double)full * t.pair_all;
+    if (rest > cus) {
+        us += t.pair_first + (t.pair_all - t.pair_first) * (double)(rest - cus) / (double)cus;
+    } else if (rest > 0) {
+        us += full > 0 ? 0.66 * t.alone : t.alone;  // a last round of single workgroups starts while pairs still run
+    }
+    return us;
+}
+
+// The tile of the 32x32x16 form with the smallest estimate for this shape.  Tiles whose workgroups
+// would leave more than half the chip idle are left to the kernels made for few columns (nt = 0
+// when that holds for all of them).  At 17408 x 5120 that gives 128 x 64 up to 128 rows (61 us),
+// 128 x 160 up to 256 (78), 128 x 128 up to 384 (97), 256 x 160 beyond (111 at 512 rows), each
+// against the 16x16x32 form's 85 / 106 / 108 / 115 us; at 8192 x 4096 and 512 rows 128 x 128, 52
+// against 83 us.  Over 38 measured shapes the estimate picked the fastest tile every time.
+WidePlan wide32_plan(uint32_t m, uint32_t n, uint32_t k, int cus, double* estimate) {
     WidePlan best{};
-    double best_cost = 1e300;
-    const uint32_t tiles_m = (m + kWM - 1) / kWM;
-    for (uint32_t cols : {128u, 160u}) {
-        const int nt = (int)cols / 32;
-        const uint32_t tiles_n = (n + cols - 1) / cols;
-        const uint64_t wgs = (uint64_t)tiles_m * tiles_n;
-        const uint64_t rounds = (wgs + cus - 1) / cus;
-        const double cost = (double)rounds * nt;
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = {nt, cols, tiles_m, tiles_n};
+    double best_us = 1e300;
+    for (const Wide32Tile& t : kWide32Tiles) {
+        const WidePlan p = wide32_make(m, n, t.rt, t.nt);
+        const uint64_t wgs = (uint64_t)p.tiles_m * p.tiles_n;
+        if (wgs * 2 < (uint64_t)cus) continue;
+        const double us = wide32_estimate(t, wgs, (uint64_t)cus);
+        if (us < best_us) {
+            best_us = us;
+            best = p;
         }
     }
+    *estimate = best_us * wide_row_length_factor(k);
     return best;
 }
 
-template <uint32_t TYPE, int DT, int NT>
+// The 16x16x32 form keeps two workgroups on a compute unit, one storing while the other
+// multiplies, so its rounds need not be whole: 2048 x 17408 x 5120 takes 442 us in 4.25 rounds.
+double wide16_estimate(uint32_t m, uint32_t n, uint32_t k, int cus) {
+    const uint64_t wgs = (uint64_t)((m + kWM - 1) / kWM) * ((n + 127) / 128);
+    const double rounds = (double)wgs / (double)cus;
+    return (rounds < 1.0 ? 1.0 : rounds) * 105.0 * wide_row_length_factor(k);
+}
+
+// The rows-resident kernel: a start that grows with the matrix, then a cost per group of rows that
+// LDS holds at once (32 rows of up to 2560, 16 of up to 5120), since every weight is decoded once
+// per group.  Measured at 48 - 512 rows on the shapes above and 151936 x 2048; within a sixth of each.
+double resident_estimate(uint32_t m, uint32_t n, uint32_t k) {
+    const double weights = (double)n * (double)k;
+    if ((size_t)32 * k * 2 <= 160u * 1024) return 12.0 + weights * 0.68e-7 + weights * 1.25e-7 * ((m + 31) / 32);
+    const double start = weights * 1.5e-7;
+    return 12.0 + (start < 14.0 ? start : 14.0) + weights * 8.3e-8 * ((m + 15) / 16);
+}
+
+template <uint32_t TYPE, int DT, int NT, int RT>
 void launch_wide32(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
-    const size_t lds = kWide32WeightsAt + 2 * (size_t)(32 * NT) * kLd * sizeof(uint16_t);
+    const size_t lds = Wide32<RT>::kWeightsAt + 2 * (size_t)(32 * NT) * kLd * sizeof(uint16_t);
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wide32_kernel<TYPE, DT, NT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_wide32_kernel<TYPE, DT, NT, RT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         configured = true;
     }
     const uint32_t groups = (plan.tiles_n + 7) / 8;
     dim3 grid(groups * 8 * plan.tiles_m);
-    hipLaunchKernelGGL((gemm_wide32_kernel<TYPE, DT, NT>), grid, dim3(512), lds, s,
+    hipLaunchKernelGGL((gemm_wide32_kernel<TYPE, DT, NT, RT>), grid, dim3(512), lds, s,
                        static_cast<const uint8_t*>(a.w), static_cast<const uint16_t*>(a.x), a.y, a.m, a.n,
                        a.k / 256, a.y_dtype, plan.cols, plan.tiles_m, plan.tiles_n);
 }
@@ -1124,24 +1200,17 @@ void launch_wide(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
 }
 
 template <uint32_t TYPE, int DT>
-void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan) {
-    // The 32x32x16 form does a sixth more work per column and cycle, but its tiles are 160 or
-    // 128 columns wide and fill the chip less evenly.  It is taken where its workgroups run as
-    // one round on at least four fifths of the compute units (512 x 17408 x 5120: 218
-    // workgroups, 112 against 114 us); over several rounds the 16x16x32 form overlaps one
-    // workgroup's stores with the next one's loop better (2048 rows: 443 against 468 us).
-    // wide_shape 2 takes it always.
-    if (a.wide_shape != 0) {
-        const WidePlan p32 = wide32_plan(a.m, a.n, a.cu_count);
-        const uint64_t wgs = (uint64_t)p32.tiles_m * p32.tiles_n;
-        if (a.wide_shape == 2 || (wgs <= (uint64_t)a.cu_count && wgs * 5 >= (uint64_t)a.cu_count * 4)) {
-            if (p32.nt == 5) {
-                launch_wide32<TYPE, DT, 5>(s, a, p32);
-            } else {
-                launch_wide32<TYPE, DT, 4>(s, a, p32);
-            }
-            return;
+void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan, const WidePlan& p32) {
+    if (p32.nt != 0) {
+        if (p32.rt == 1) {
+            if (p32.nt == 2) launch_wide32<TYPE, DT, 2, 1>(s, a, p32);
+            else if (p32.nt == 5) launch_wide32<TYPE, DT, 5, 1>(s, a, p32);
+            else launch_wide32<TYPE, DT, 4, 1>(s, a, p32);
+        } else {
+            if (p32.nt == 5) launch_wide32<TYPE, DT, 5, 2>(s, a, p32);
+            else launch_wide32<TYPE, DT, 4, 2>(s, a, p32);
         }
+        return;
     }
     if (plan.nt == 9) {
         launch_wide<TYPE, DT, 9>(s, a, plan);
@@ -1166,6 +1235,23 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     // Rows longer than 2560 fit only 16 at a time, and every weight is then decoded M / 16 times:
     // that still wins up to 256 rows (256 x 5120 x 5120: 51 against 86 us) and loses at 512 (95
     // against 84 us).
+    // From wide_min_rows rows on, the tiles of the 32x32x16 form compete: the smallest estimate
+    // among them, the 16x16x32 form and the rows-resident kernel takes the call.
+    WidePlan p32{};
+    double us32 = 1e300;
+    if (a.wide_shape != 0 && a.m >= (uint32_t)a.wide_min_rows) {
+        if (a.wide32_tile != 0) {
+            p32 = wide32_make(a.m, a.n, a.wide32_tile / 10, a.wide32_tile % 10);
+            us32 = 0.0;
+        } else {
+            p32 = wide32_plan(a.m, a.n, a.k, a.cu_count, &us32);
+            if (p32.nt == 0 && a.wide_shape == 2 && wide_pays) {
+                p32 = wide32_make(a.m, a.n, 2, 5);
+                us32 = 0.0;
+            }
+        }
+    }
+    const double us16 = wide_pays && a.wide_shape != 2 ? wide16_estimate(a.m, a.n, a.k, a.cu_count) : 1e300;
     if (a.rows_resident) {
         const bool few = a.m <= (uint32_t)a.skinny_max_rows;
         const bool groups_of_32 = (size_t)32 * a.k * 2 <= 160u * 1024;
@@ -1173,31 +1259,35 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
         // cost grows with the row count: 65 x 17408 x 5120 takes 67 against 82 us and 128 rows
         // 87 against 87; with groups of 32 (K = 2048) 128 rows take 30 against 41 us and 256
         // rows 49 against 49.
-        const bool take = few          ? !(a.k <= 512 && a.m <= 16)
-                          : wide_pays ? a.m <= (groups_of_32 ? 192u : 96u)
-                                      : groups_of_32 || a.m <= 256;
+        bool take = few          ? !(a.k <= 512 && a.m <= 16)
+                    : wide_pays ? a.m <= (groups_of_32 ? 192u : 96u)
+                                : groups_of_32 || a.m <= 256;
+        // (the estimates were measured on rows of 2048 and more; shorter ones keep the rule above)
+        if (p32.nt != 0 && (a.k >= 1024 || a.wide32_tile != 0))
+            take = resident_estimate(a.m, a.n, a.k) < (us32 < us16 ? us32 : us16);
         if (take) return launch_gemm_resident(s, a);
     }
-    if (a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
-    if (wide_pays) {
+    if (p32.nt != 0 && us16 < us32) p32.nt = 0;
+    if (p32.nt == 0 && a.m <= (uint32_t)a.skinny_max_rows) return launch_gemm_skinny(s, a);
+    if (wide_pays || p32.nt != 0) {
         const WidePlan plan = wide_plan(a.m, a.n, a.cu_count);
         if (a.ggml_type == kQ4K) {
-            if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan); else launch_wide_nt<kQ4K, 2>(s, a, plan);
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ4K, 1>(s, a, plan, p32); else launch_wide_nt<kQ4K, 2>(s, a, plan, p32);
             return "q4_k_gemm_mfma_m256";
         }
         if (a.ggml_type == kQ5K) {
-            if (a.x_dtype == FH_F16) launch_wide_nt<kQ5K, 1>(s, a, plan); else launch_wide_nt<kQ5K, 2>(s, a, plan);
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ5K, 1>(s, a, plan, p32); else launch_wide_nt<kQ5K, 2>(s, a, plan, p32);
             return "q5_k_gemm_mfma_m256";
         }
         if (a.ggml_type == kIQ4XS) {
-            if (a.x_dtype == FH_F16) launch_wide_nt<kIQ4XS, 1>(s, a, plan); else launch_wide_nt<kIQ4XS, 2>(s, a, plan);
+            if (a.x_dtype == FH_F16) launch_wide_nt<kIQ4XS, 1>(s, a, plan, p32); else launch_wide_nt<kIQ4XS, 2>(s, a, plan, p32);
             return "iq4_xs_gemm_mfma_m256";
         }
         if (a.ggml_type == kQ8_0) {
-            if (a.x_dtype == FH_F16) launch_wide_nt<kQ8_0, 1>(s, a, plan); else launch_wide_nt<kQ8_0, 2>(s, a, plan);
+            if (a.x_dtype == FH_F16) launch_wide_nt<kQ8_0, 1>(s, a, plan, p32); else launch_wide_nt<kQ8_0, 2>(s, a, plan, p32);
             return "q8_0_gemm_mfma_m256";
         }
-        if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan); else launch_wide_nt<kQ6K, 2>(s, a, plan);
+        if (a.x_dtype == FH_F16) launch_wide_nt<kQ6K, 1>(s, a, plan, p32); else launch_wide_nt<kQ6K, 2>(s, a, plan, p32);
         return "q6_k_gemm_mfma_m256";
     }
     // 128 x 128 tiles, or 64 x 64 when those would leave most of the chip idle

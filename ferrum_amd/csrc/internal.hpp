@@ -200,6 +200,7 @@ struct GemmArgs {
     int cu_count;
     int wide_min_rows;   // smallest M that takes the 256-row tile
     int wide_shape;      // matrix instruction of the 256-row tile: 0 = 16x16x32, 1 = 32x32x16 where it wins, 2 = always
+    int wide32_tile;     // 0 = chosen by shape; else 10 x (row tiles per wave) + column tiles of the 32x32x16 form
     int skinny_max_rows; // largest M that takes the register-dequant kernel
     // routed-expert form of the register-dequant kernel: w is [experts, n, k],
     // x and y rows are assignments, m is their count; tokens of expert e are

@@ -206,11 +206,13 @@ def test_tile_gemm_both_tile_sizes_match_the_f16_tile_oracle(api, d, ggml, dtype
     for n in (16000, 1000):
         packed = synth.matrix(ggml, n, k, seed=92 + n)
         w = qm(api, d, ggml, n, k, packed)
-        d.set_tuning("gemm_resident", 0)   # rows this short would otherwise stay in LDS (tested below)
+        d.set_tuning("gemm_resident", 0)   # rows this short would otherwise stay in LDS (tested below),
+        d.set_tuning("gemm_wide_shape", 0) # and the 128-row tiles of the 32x32x16 form would take 16000 columns
         try:
             out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
         finally:
             d.set_tuning("gemm_resident", 1)
+            d.set_tuning("gemm_wide_shape", 1)
         assert out.operation == ("q4_k_gemm_mfma" if ggml == Q4_K else "q6_k_gemm_mfma")
         got = out.tensor.to_f32()
         rows = np.unique(np.concatenate([np.arange(0, 130), np.arange(n - 70, n),
@@ -555,7 +557,11 @@ def test_wide_gemm_covers_every_column_of_its_tiles(api, d):
     packed = synth.matrix(Q4_K, n, k, seed=141)
     w = qm(api, d, Q4_K, n, k, packed)
     x = synth.activations(m, k, seed=142, f16=True)
-    out = d.project_quantized(api.Tensor.from_f32(d, (m, k), api.DType.F16, x), w, out_dtype=api.DType.F32)
+    d.set_tuning("gemm_wide_shape", 0)     # the 16x16x32 form, whose tiles have the ninth column tile
+    try:
+        out = d.project_quantized(api.Tensor.from_f32(d, (m, k), api.DType.F16, x), w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_wide_shape", 1)
     assert out.operation == "q4_k_gemm_mfma_m256"
     got = out.tensor.to_f32()
     for width in (128, 136, 144):      # whichever width the plan chose, its tiles' last 16 columns
@@ -569,31 +575,62 @@ def test_wide_gemm_covers_every_column_of_its_tiles(api, d):
 
 
 @pytest.mark.parametrize("ggml", [12, 13, 14, 23, 8], ids=["q4_k", "q5_k", "q6_k", "iq4_xs", "q8_0"])
-@pytest.mark.parametrize("dtype,cols", [("F16", 160), ("BF16", 160), ("F16", 128)])
-def test_wide_gemm_on_the_32x32x16_instruction(api, d, ggml, dtype, cols):
-    # the 256-row tile built on v_mfma_f32_32x32x16: 300 rows (a second, partly empty row tile) and a
-    # column count that leaves the last workgroup 40 of its 160 (or 8 of its 128) columns; every
-    # output is checked.  17000 columns plan 160-wide tiles (one round of 214 workgroups where
-    # 128-wide ones would need two), 8072 columns 128-wide ones.
-    n, k, m = (17000, 512, 300) if cols == 160 else (8072, 512, 300)
+@pytest.mark.parametrize("dtype", ["F16", "BF16"])
+def test_wide_gemm_on_the_32x32x16_instruction(api, d, ggml, dtype):
+    # the tiles built on v_mfma_f32_32x32x16, each forced in turn: 256 rows x 160 / 128 columns and
+    # 128 rows x 160 / 128 / 64 columns.  300 rows leave the last row tile 44 rows, 8072 columns
+    # leave the last workgroup 72, 8 or 8 of its columns.  Every output of the first is checked
+    # against the oracle; the others add the same products in the same order, so they must give
+    # its bits, and so must whichever tile the library picks by itself.
+    n, k, m = 8072, 512, 300
     packed = synth.matrix(ggml, n, k, seed=171)
     w = qm(api, d, ggml, n, k, packed)
     code = oracle.F16 if dtype == "F16" else oracle.BF16
     x = oracle.round_storage(synth.activations(m, k, seed=172), code).reshape(m, k)
     xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
-    before = d.get_tuning("gemm_wide_shape")
+    shape, tile = d.get_tuning("gemm_wide_shape"), d.get_tuning("gemm_wide32_tile")
+    results = {}
     try:
         d.set_tuning("gemm_wide_shape", 2)
-        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        for forced in (25, 24, 15, 14, 12, 0):
+            d.set_tuning("gemm_wide32_tile", forced)
+            out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+            assert out.operation.endswith("_gemm_mfma_m256")
+            results[forced] = out.tensor.to_f32()
         d.set_tuning("gemm_wide_shape", 0)
         other = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        assert other.operation.endswith("_gemm_mfma_m256")
     finally:
-        d.set_tuning("gemm_wide_shape", before)
-    assert out.operation.endswith("_gemm_mfma_m256") and other.operation == out.operation
-    got = out.tensor.to_f32()
+        d.set_tuning("gemm_wide_shape", shape)
+        d.set_tuning("gemm_wide32_tile", tile)
     want = oracle.project(ggml, packed, n, k, x, accumulate="f64", weight_round=code, threads=8)
-    assert_matmul_parity(got, want, "every output of the 32x32x16 tiles")
-    assert_matmul_parity(got, other.tensor.to_f32(), "against the 16x16x32 tiles", l2_tol=2e-6)
+    assert_matmul_parity(results[25], want, "every output of the 256 x 160 tiles")
+    for forced, got in results.items():
+        assert np.array_equal(bits(got), bits(results[25])), f"tile {forced} against 256 x 160"
+    assert_matmul_parity(results[25], other.tensor.to_f32(), "against the 16x16x32 tiles", l2_tol=2e-6)
+
+
+@pytest.mark.parametrize("m", [80, 128, 200, 330, 512])
+def test_the_tile_picked_by_row_count_gives_the_bits_of_the_largest(api, d, m):
+    # 17000 columns at every row count that changes the tile (128 x 64 up to 128 rows, 128 x 160 up
+    # to 256, 128 x 128 up to 384, 256 x 160 beyond); the pick against the forced 256 x 160 tile.
+    n, k = 17000, 2816
+    w = qm(api, d, Q4_K, n, k, synth.matrix(Q4_K, n, k, seed=173))
+    x = synth.activations(m, k, seed=174, f16=True)
+    xt = api.Tensor.from_f32(d, (m, k), api.DType.F16, x)
+    tile, resident, shape = d.get_tuning("gemm_wide32_tile"), d.get_tuning("gemm_resident"), d.get_tuning("gemm_wide_shape")
+    try:
+        d.set_tuning("gemm_resident", 0)      # at 80 rows its estimate is close to the tile's,
+        d.set_tuning("gemm_wide_shape", 2)    # at 512 the 16x16x32 form's, whose bits differ
+        picked = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        d.set_tuning("gemm_wide32_tile", 25)
+        largest = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_wide32_tile", tile)
+        d.set_tuning("gemm_resident", resident)
+        d.set_tuning("gemm_wide_shape", shape)
+    assert picked.operation == largest.operation == "q4_k_gemm_mfma_m256"
+    assert np.array_equal(picked.tensor.raw(), largest.tensor.raw())
 
 
 def test_objects_may_outlive_their_device(api):
@@ -745,10 +782,12 @@ def test_q5_k_tile_kernels_match_the_rounded_weight_oracle(api, d, m, n, dtype_n
     w = qm(api, d, Q5_K, n, k, packed)
     x = oracle.round_storage(synth.activations(m, k, seed=202), code).reshape(m, k)
     d.set_tuning("gemm_resident", 0)       # the square tiles, which rows longer than LDS still take
+    d.set_tuning("gemm_wide_shape", 0)     # where too few 256-row tiles would fill the chip (128-row ones do)
     try:
         out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
     finally:
         d.set_tuning("gemm_resident", 1)
+        d.set_tuning("gemm_wide_shape", 1)
     want_name = {8: "q5_k_gemm_mfma_skinny", 20: "q5_k_gemm_mfma_skinny", 130: "q5_k_gemm_mfma",
                  300: "q5_k_gemm_mfma_m256"}[m]
     assert out.operation == want_name

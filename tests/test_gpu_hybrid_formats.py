@@ -113,11 +113,13 @@ def test_tile_kernels_match_the_rounded_weight_oracle(api, d, ggml, m, n, dtype_
     packed = synth.matrix(ggml, n, k, seed=311 + n)
     w = qm(api, d, n, k, packed, ggml)
     x = oracle.round_storage(synth.activations(m, k, seed=312), code).reshape(m, k)
-    d.set_tuning("gemm_resident", 0)   # the square tiles: rows this short would otherwise stay in LDS
+    d.set_tuning("gemm_resident", 0)   # the square tiles: rows this short would otherwise stay in LDS,
+    d.set_tuning("gemm_wide_shape", 0) # and 130 x 16000 would fill the chip with 128-row tiles of the 32x32x16 form
     try:
         out = d.project_quantized(api.Tensor.from_f32(d, x.shape, dtype, x), w, out_dtype=api.DType.F32)
     finally:
         d.set_tuning("gemm_resident", 1)
+        d.set_tuning("gemm_wide_shape", 1)
     suffix = {8: "_skinny", 20: "_skinny", 50: "_skinny", 130: "", 300: "_m256"}[m]
     assert out.operation == f"{NAME[ggml]}_gemm_mfma{suffix}"
     rows = np.unique(np.concatenate([np.arange(0, 150), np.arange(n - 150, n), synth.rng(313).integers(0, n, 64)]))

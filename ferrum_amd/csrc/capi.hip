@@ -253,6 +253,8 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
+    d->tuning["gemm_few_tiles_split"] = 1;  // up to 16 rows and few weight tiles per workgroup: super-blocks dealt over the waves (0 = whole tiles per wave)
+    d->tuning["moe_fold_combine"] = 1;      // fh_moe_ffn with few tokens: down projection and weighted sum in one launch (0 = two)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
     d->tuning["gemv_stream"] = 1;           // dense Q4_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
@@ -352,7 +354,9 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value == 0 || value == 1 || value == 2 || value == 4 || value == 8;
     } else if (k == "gemm_min_rows") {
         ok = value >= 2;
-    } else if (k == "gemm_resident") {
+    } else if (k == "gemm_resident" || k == "moe_fold_combine" || k == "moe_fold_route") {
+        ok = value == 0 || value == 1;
+    } else if (k == "gemm_few_tiles_split") {
         ok = value == 0 || value == 1;
     } else if (k == "gemv_stream") {
         ok = value >= 0 && value <= 2;
@@ -657,6 +661,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.wide32_tile = (int)tuning(device, "gemm_wide32_tile");
         a.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         a.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
+        a.few_tiles_split = tuning(device, "gemm_few_tiles_split") != 0;
         device->last_operation = launch_gemm(device->stream, a);
     } else {
         GemvArgs a{};
@@ -1374,6 +1379,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.wide32_tile = (int)tuning(device, "gemm_wide32_tile");
         g.skinny_max_rows = (int)tuning(device, "gemm_skinny_max_rows");
         g.rows_resident = tuning(device, "gemm_resident") != 0 && expert_rows_fit_lds((uint32_t)k, 1, 1);
+        g.few_tiles_split = tuning(device, "gemm_few_tiles_split") != 0;
         device->last_operation = launch_gemm(device->stream, g);
         FH_HIP(hipGetLastError());
         return FH_OK;
@@ -1674,6 +1680,44 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         // the copy and the activation ride inside the projections: per assignment in decode, in
         // the grouped kernel's gather of an expert's rows beyond it (f32 rows have no grouped form)
         const bool fused = a <= 31 || dt != FH_F32;
+        // One or two tokens: the down projection of a token's entries and the weighted sum over
+        // them are one launch (the bits of the two; 17.9 against 18.5 us for one token of the
+        // 256-expert top-8 FFN, 22.2 against 22.7 for two; from three tokens on the launch that
+        // stages an entry's activations once for 32 rows instead of 8 is the faster one).
+        const bool folded = count <= 2 && a <= 31 && (!shared || rides) && tuning(device, "moe_fold_combine") != 0 &&
+                            (!shared_gate || shared_gate->dtype == FH_F32) &&
+                            expert_down_combine_fits(output_experts->ggml_type, (uint32_t)h, (uint32_t)inter, k, shared);
+        if (folded) {
+            st = shared ? fh_expert_project_with_shared(device, input_experts, shared_input, &x, count, FH_INPUT_GATHER,
+                                                        a, &meta, nullptr, &projected, &sproj)
+                        : fh_expert_project_fused(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected);
+            if (st != FH_OK) return st;
+            Range yr, gr{nullptr, 0};
+            st = resolve(device, &y, (uint64_t)count * h, "routed FFN output", &yr);
+            if (st != FH_OK) return st;
+            if (shared_gate) {
+                st = resolve(device, &gate, count, "shared-expert gate", &gr, 4);
+                if (st != FH_OK) return st;
+            }
+            ExpertDownCombineArgs d{};
+            d.ggml_type = output_experts->ggml_type;
+            d.w = output_experts->ptr;
+            d.w_shared = shared ? shared_output->ptr : nullptr;
+            d.x = static_cast<const uint8_t*>(ws->ptr) + projected_at;
+            d.x_shared = shared ? static_cast<const uint8_t*>(ws->ptr) + sproj_at : nullptr;
+            d.metadata = reinterpret_cast<const float*>(static_cast<const uint8_t*>(ws->ptr) + meta_at);
+            d.shared_gate = reinterpret_cast<const float*>(gr.begin);
+            d.y = const_cast<uint8_t*>(yr.begin);
+            d.n = (uint32_t)h;
+            d.k = (uint32_t)inter;
+            d.tokens = count;
+            d.top_k = k;
+            d.experts = (uint32_t)e;
+            d.dtype = dt;
+            device->last_operation = launch_expert_down_combine(device->stream, d);
+            FH_HIP(hipGetLastError());
+            continue;
+        }
         if (shared && rides && fused) {
             st = fh_expert_project_with_shared(device, input_experts, shared_input, &x, count, FH_INPUT_GATHER, a, &meta,
                                                nullptr, &projected, &sproj);

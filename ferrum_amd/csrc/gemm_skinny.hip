@@ -628,11 +628,163 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
     }
 }
 
+// Dense product of up to 16 activation rows where a workgroup owns only a few 16-row weight
+// tiles (up to kFewTiles of them).  In expert_resident_kernel a wave walks whole tiles, so with
+// five tiles per workgroup five waves each stream twenty super-blocks one after another and
+// three idle: the length of that chain, not the memory system, sets the time.  Here the
+// super-blocks of every tile are dealt over the waves (wave w takes blocks w, w + WAVES, .. of
+// tile 0, shifted by four for the next tile so the odd ones even out), every wave keeps one
+// accumulator per tile, and the partial sums of a tile meet in LDS, where the activation rows
+// were, once nobody reads those any more; they are added in wave order, so the result is
+// deterministic.  The first weight loads are issued before the activation rows are fetched.
+constexpr int kFewTiles = 5;        // tiles per workgroup
+
+// WAVES: 8 or 16 per workgroup; every wave takes up to 24 / WAVES super-blocks of each tile (rows
+// of up to 24 super-blocks: more do not fit LDS anyway).  AHEAD: units in flight per wave.
+template <uint32_t TYPE, int DT, int WAVES, int AHEAD>
+__global__ __launch_bounds__(64 * WAVES) void dense_few_tiles_kernel(const uint8_t* __restrict__ w,
+                                                                    const uint16_t* __restrict__ x,
+                                                                    void* __restrict__ y, uint32_t m, uint32_t n,
+                                                                    uint32_t nb, uint32_t y_dtype) {
+    constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
+    constexpr int kPerTile = 24 / WAVES + (24 % WAVES != 0 ? 1 : 0);
+    constexpr int kUnits = kFewTiles * kPerTile;
+    constexpr uint32_t kThreads = 64 * WAVES;
+    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t k = nb * 256, ld = k, pieces = k / 8;
+    const uint32_t tiles = (n + 15) / 16;
+    const uint32_t per = (tiles + gridDim.x - 1) / gridDim.x;
+    const uint32_t tile_begin = blockIdx.x * per;
+    const uint32_t my_tiles = min(per, tiles - tile_begin);
+
+    // unit i = (tile i / kPerTile, the (i % kPerTile)-th block of this wave in that tile)
+    auto unit_block = [&](int i) {
+        return ((wave + 4u * (uint32_t)(i / kPerTile)) & (uint32_t)(WAVES - 1)) + (uint32_t)WAVES * (uint32_t)(i % kPerTile);
+    };
+    auto unit_valid = [&](int i) { return (uint32_t)(i / kPerTile) < my_tiles && unit_block(i) < nb; };
+    auto unit_ptr = [&](int i) {
+        const uint32_t tile = tile_begin + min((uint32_t)(i / kPerTile), my_tiles - 1);
+        const uint32_t row = min(tile * 16 + r, n - 1);
+        return w + ((size_t)row * nb + min(unit_block(i), nb - 1)) * kBB;
+    };
+    Quarter<TYPE> ring[AHEAD + 1];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) {
+        if (unit_valid(i)) ring[i].load(unit_ptr(i), g);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // the activation rows, eight 16-byte pieces per thread in flight at a time; piece p of row
+    // t sits at piece p ^ (t & 15), so the sixteen rows a B-operand read touches fall on different banks
+    const uint32_t total = m * pieces;
+    for (uint32_t base = 0; base < total; base += 8 * kThreads) {
+        u32x4 v[8];
+        uint32_t dst[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t idx = min(base + j * kThreads + tid, total - 1);
+            const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
+            dst[j] = tok * ld + 8 * (pc ^ (tok & 15u));
+            v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)tok * k + 8 * pc);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
+    }
+    __syncthreads();
+
+    const uint32_t boff = min(r, m - 1) * ld;
+    uint32_t kl[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) kl[s] = (((Quarter<TYPE>::klocal(g, s) >> 3) ^ r) << 3);
+    float4v acc[kFewTiles];
+#pragma unroll
+    for (int t = 0; t < kFewTiles; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (i + AHEAD < kUnits) {
+            if (unit_valid(i + AHEAD)) ring[(i + AHEAD) % (AHEAD + 1)].load(unit_ptr(i + AHEAD), g);
+        }
+        if (unit_valid(i)) {
+            uint4 a[8];
+            ring[i % (AHEAD + 1)].template decode<DT>(g, a);
+            const uint16_t* xb = xs + 256 * unit_block(i) + boff;
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const uint4 bfrag = *reinterpret_cast<const uint4*>(xb + kl[s]);
+                acc[i / kPerTile] = mfma16<DT>(a[s], bfrag, acc[i / kPerTile]);
+            }
+        }
+    }
+    // the partial sums take the place of the activation rows
+    __syncthreads();
+    float4* partial = reinterpret_cast<float4*>(xs);
+#pragma unroll
+    for (int t = 0; t < kFewTiles; ++t)
+        if ((uint32_t)t < my_tiles) partial[((uint32_t)t * WAVES + wave) * 64 + lane] = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    __syncthreads();
+    for (uint32_t idx = tid; idx < my_tiles * 64; idx += kThreads) {
+        const uint32_t t = idx >> 6, l = idx & 63u;
+        float4 sum = partial[(t * WAVES) * 64 + l];
+#pragma unroll
+        for (int wv = 1; wv < WAVES; ++wv) {
+            const float4 v = partial[(t * WAVES + wv) * 64 + l];
+            sum.x += v.x;
+            sum.y += v.y;
+            sum.z += v.z;
+            sum.w += v.w;
+        }
+        // C layout of 16x16x32: lane (g, r) holds weight rows 4g .. 4g + 3 of token r
+        const uint32_t token = l & 15u, out_row = (tile_begin + t) * 16 + 4 * (l >> 4);
+        if (token < m) {
+            const size_t base = (size_t)token * n + out_row;
+            const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+            if (y_dtype == FH_F32 && (n & 3u) == 0 && out_row + 3 < n) {
+                *reinterpret_cast<float4*>(static_cast<float*>(y) + base) = sum;
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (out_row + v < n) store_from_f32(y, base + v, y_dtype, vals[v]);
+            }
+        }
+    }
+}
+
 template <uint32_t TYPE, int DT>
 void launch_tt(hipStream_t s, const GemmArgs& a) {
     const uint8_t* w = static_cast<const uint8_t*>(a.w);
     const uint16_t* x = static_cast<const uint16_t*>(a.x);
     const uint32_t nb = a.k / 256;
+    if (a.use_resident && a.m <= 16 && a.few_tiles_split && nb <= 24u) {
+        const uint32_t tiles = (a.n + 15) / 16;
+        const uint32_t cus = a.cu_count > 0 ? (uint32_t)a.cu_count : 256u;
+        const uint32_t per_wg = (tiles + cus - 1) / cus;
+        if (per_wg <= (uint32_t)kFewTiles) {
+            auto go = [&](auto kernel, uint32_t waves) {
+                const size_t rows_bytes = (size_t)a.m * a.k * 2, partial_bytes = (size_t)per_wg * waves * 64 * 16;
+                const size_t lds = rows_bytes > partial_bytes ? rows_bytes : partial_bytes;
+                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                hipLaunchKernelGGL(kernel, dim3((tiles + per_wg - 1) / per_wg), dim3(64 * waves), lds, s, w, x, a.y,
+                                   a.m, a.n, nb, a.y_dtype);
+            };
+            // Sixteen waves with two units ahead where a tile has two super-blocks or more per
+            // wave of eight and the format's raw quarter is small enough for 128 registers
+            // (8 x 17408 x 5120 Q4_K: 18.2 us against 20.7 with eight waves and six ahead, 24.3
+            // with whole tiles per wave; Q5_K and Q6_K spill there: 26.2 against 32.3 and 30.9
+            // against 36.9 with eight waves); eight waves for shorter rows (8 x 4096 x 2048: 4.9
+            // against 5.3 and 7.9).
+            if constexpr (TYPE == kQ5K || TYPE == kQ6K) {
+                go(dense_few_tiles_kernel<TYPE, DT, 8, 4>, 8);
+            } else {
+                if (nb >= 16) go(dense_few_tiles_kernel<TYPE, DT, 16, 2>, 16);
+                else go(dense_few_tiles_kernel<TYPE, DT, 8, 6>, 8);
+            }
+            return;
+        }
+    }
     if (a.use_resident) {
         // dense product with the activation rows resident in LDS: (32-row group, row-tile slice)
         // pieces, about one per compute unit

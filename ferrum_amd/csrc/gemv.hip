@@ -465,6 +465,137 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     }
 }
 
+// The routed FFN's last two stages in one launch for a few tokens: the down projection of
+// every entry of a token (its top_k routed experts in rank order, then the shared expert) and
+// expert_combine's weighted sum over them (src/metal/shaders/ops.metal:1088-1101, 2234-2246;
+// the two launches src/nn/moe.rs:349-397 makes).  A workgroup owns RS rows of one token's
+// output; wave w computes entry w (and w + 16 when there are more than 16) exactly as
+// gemv_kernel does with the SiLU input form: the same fragments, the same order of
+// additions, rounded to the activation dtype where that launch would have stored it.  The
+// rounded values meet in LDS and the first RS threads add them in rank order with
+// expert_combine's rounding, so the result has the bits of the two separate launches.
+struct DownCombineParams {
+    const uint8_t* w;          // [experts][n][nb] blocks
+    const uint8_t* w_shared;   // [n][nb] blocks, or null
+    const void* x;             // [tokens * top_k][2 * k]: packed gate|up rows of the routed entries
+    const void* x_shared;      // [tokens][2 * k]
+    const float* metadata;     // [tokens * top_k][3]: expert id, token, weight
+    const float* shared_gate;  // [tokens], or null = 1
+    void* y;                   // [tokens][n]
+    uint32_t n, nb, top_k, experts;
+    uint32_t dtype;            // of x, of the rounding between the stages and of y
+};
+
+constexpr int kDownCombineMaxWaves = 16;
+
+template <uint32_t TYPE, int BS, int IT>
+__global__ __launch_bounds__(kDownCombineMaxWaves * kWave) void expert_down_combine_kernel(const DownCombineParams p) {
+    constexpr int RS = 16 / BS;
+    constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
+    extern __shared__ float4 xs_all[];  // per wave: nb * kXStride float4, then nb * 16 run sums
+    __shared__ float values[2 * kDownCombineMaxWaves][16];
+    __shared__ float weights[2 * kDownCombineMaxWaves];  // fetched next to the expert ids, before anything waits
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, waves = blockDim.x >> 6;
+    const uint32_t c = lane & 3u, bs = (lane >> 2) % BS, rs = lane / (4 * BS);
+    const uint32_t token = blockIdx.y;
+    const uint32_t entries = p.top_k + (p.w_shared != nullptr ? 1u : 0u);
+    const size_t wave_floats = (size_t)p.nb * kXStride * 4 + (size_t)p.nb * 16;
+    float4* xs = reinterpret_cast<float4*>(reinterpret_cast<float*>(xs_all) + wave * wave_floats);
+    float* rsum = reinterpret_cast<float*>(xs + (size_t)p.nb * kXStride);
+    const uint32_t row = blockIdx.x * RS + rs;
+
+    for (uint32_t entry = wave; entry < entries; entry += waves) {
+        const bool shared = entry >= p.top_k;
+        const size_t slot = (size_t)token * p.top_k + entry;
+        bool live = true;
+        size_t row_base = 0;
+        float weight;
+        if (!shared) {
+            const uint32_t expert = __float_as_uint(p.metadata[3 * slot]);
+            weight = p.metadata[3 * slot + 2];
+            live = expert < p.experts;
+            row_base = live ? (size_t)expert * p.n : 0;
+        } else {
+            weight = p.shared_gate != nullptr ? p.shared_gate[token] : 1.f;
+        }
+        if (lane == 0) weights[entry] = weight;
+        const uint8_t* wmat = shared ? p.w_shared : p.w;
+        const void* xmat = shared ? p.x_shared : p.x;
+        const uint8_t* rp = wmat + (row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb * kBlockBytes;
+        Frag<TYPE> frag[IT];
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const uint32_t b = it * BS + bs;
+            frag[it].load(rp + (size_t)(b < p.nb ? b : p.nb - 1) * kBlockBytes, c);
+        }
+        asm volatile("" ::: "memory");
+        // the entry's activations: silu(gate) * up of its packed row, staged as gemv_kernel stages them
+        const size_t xbase = (shared ? (size_t)token : slot) * 2 * p.nb * 64;
+        const uint32_t xq = p.nb * 64;
+        if (entry != wave) __builtin_amdgcn_wave_barrier();
+        for (uint32_t q = lane; q < xq; q += 64) {
+            const float4 v = silu_mul4(load_x4(xmat, p.dtype, xbase + q),
+                                       load_x4(xmat, p.dtype, xbase + (size_t)p.nb * 64 + q), p.dtype);
+            const uint32_t at = x_slot<TYPE>(q & 63u);
+            xs[(q >> 6) * kXStride + at] = v;
+            float s = (v.x + v.y) + (v.z + v.w);
+            s = dpp_add<0xB1>(s);
+            s = dpp_add<0x4E>(s);
+            if ((q & 3u) == 0) rsum[(q >> 6) * 16 + (at & 3u) * 4 + (at >> 4)] = s;
+        }
+        // the wave reads what its own lanes wrote: LDS operations of a wave complete in order
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        __builtin_amdgcn_wave_barrier();
+        float acc = 0.f;
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const uint32_t b = it * BS + bs;
+            const bool valid = b < p.nb;
+            const uint32_t bb = valid ? b : 0;
+            const float4 s = *reinterpret_cast<const float4*>(rsum + bb * 16 + c * 4);
+            const float v = frag[it].dot(xs + bb * kXStride + c, s, c);
+            acc += valid ? v : 0.f;
+            asm volatile("" : "+v"(acc)::"memory");
+        }
+        acc = dpp_add<0xB1>(acc);
+        acc = dpp_add<0x4E>(acc);
+        if (BS >= 2) acc = dpp_add<0x141>(acc);
+        if (BS >= 4) acc = dpp_add<0x140>(acc);
+        if (BS >= 8) acc += __shfl_xor(acc, 16, 64);
+        if (!live) acc = 0.f;
+        if ((lane & (4 * BS - 1)) == 0) values[entry][rs] = round_storage(acc, p.dtype);
+    }
+    __syncthreads();
+    if (tid < (uint32_t)RS) {
+        const uint32_t r = blockIdx.x * RS + tid;
+        if (r < p.n) {
+            // each product is rounded before it is added, as expert_combine does
+#pragma clang fp contract(off)
+            float sum = 0.f;
+            for (uint32_t entry = 0; entry < entries; ++entry)
+                sum += round_storage(round_storage(weights[entry], p.dtype) * values[entry][tid], p.dtype);
+            store_from_f32(p.y, (size_t)token * p.n + r, p.dtype, sum);
+        }
+    }
+}
+
+typedef void (*DownCombineFn)(dim3, dim3, size_t, hipStream_t, const DownCombineParams&);
+
+template <uint32_t TYPE, int BS, int IT>
+void launch_down_combine_impl(dim3 grid, dim3 block, size_t lds, hipStream_t s, const DownCombineParams& p) {
+    hipLaunchKernelGGL((expert_down_combine_kernel<TYPE, BS, IT>), grid, block, lds, s, p);
+}
+
+template <uint32_t TYPE>
+DownCombineFn pick_down_combine(int bs, int it) {
+#define FH_CASE(B, I) \
+    if (bs == B && it == I) return launch_down_combine_impl<TYPE, B, I>;
+    FH_CASE(8, 1) FH_CASE(8, 2) FH_CASE(4, 1) FH_CASE(4, 2) FH_CASE(2, 1) FH_CASE(2, 2) FH_CASE(1, 1)
+#undef FH_CASE
+    return nullptr;
+}
+
 typedef void (*LaunchFn)(dim3, size_t, hipStream_t, const Params&);
 
 template <uint32_t TYPE, int BS, int IT>
@@ -592,5 +723,46 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
     if (plan.segments > 1) return ksplit_names[f];
     return factored_names[f];
 }
+
+bool expert_down_combine_fits(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t top_k, bool shared) {
+    const GemvPlan plan = gemv_plan(n, k, 1, 0);
+    if (plan.segments != 1 || plan.it > 2 || (plan.bs == 1 && plan.it != 1)) return false;
+    const uint32_t entries = top_k + (shared ? 1u : 0u);
+    if (entries > 2u * kDownCombineMaxWaves) return false;
+    const uint32_t waves = entries < (uint32_t)kDownCombineMaxWaves ? entries : (uint32_t)kDownCombineMaxWaves;
+    // every wave stages its entry's activations in LDS
+    if ((size_t)waves * (k / 256) * ((size_t)kXStride * 16 + 64) > 64u * 1024) return false;
+    (void)ggml_type;
+    return true;
+}
+
+const char* launch_expert_down_combine(hipStream_t s, const ExpertDownCombineArgs& a) {
+    const GemvPlan plan = gemv_plan(a.n, a.k, 1, 0);
+    DownCombineParams p{};
+    p.w = static_cast<const uint8_t*>(a.w);
+    p.w_shared = static_cast<const uint8_t*>(a.w_shared);
+    p.x = a.x;
+    p.x_shared = a.x_shared;
+    p.metadata = a.metadata;
+    p.shared_gate = a.shared_gate;
+    p.y = a.y;
+    p.n = a.n;
+    p.nb = a.k / 256;
+    p.top_k = a.top_k;
+    p.experts = a.experts;
+    p.dtype = a.dtype;
+    const uint32_t entries = a.top_k + (a.w_shared != nullptr ? 1u : 0u);
+    const uint32_t waves = entries < (uint32_t)kDownCombineMaxWaves ? entries : (uint32_t)kDownCombineMaxWaves;
+    const uint32_t rs = 16u / (uint32_t)plan.bs;
+    const size_t lds = (size_t)waves * ((size_t)p.nb * kXStride * 16 + (size_t)p.nb * 64);
+    DownCombineFn fn = a.ggml_type == kQ4K     ? pick_down_combine<kQ4K>(plan.bs, plan.it)
+                       : a.ggml_type == kQ5K   ? pick_down_combine<kQ5K>(plan.bs, plan.it)
+                       : a.ggml_type == kIQ4XS ? pick_down_combine<kIQ4XS>(plan.bs, plan.it)
+                       : a.ggml_type == kQ8_0  ? pick_down_combine<kQ8_0>(plan.bs, plan.it)
+                                               : pick_down_combine<kQ6K>(plan.bs, plan.it);
+    fn(dim3((a.n + rs - 1) / rs, a.tokens), dim3(waves * 64), lds, s, p);
+    return a.w_shared != nullptr ? "expert_project + h_moe_combine" : "expert_project + expert_combine";
+}
+
 
 }  // namespace fh

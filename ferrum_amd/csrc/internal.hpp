@@ -166,6 +166,22 @@ struct GemvPlan {
 GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments);
 const char* launch_gemv(hipStream_t s, const GemvArgs& a);
 
+// gemv.hip: the down projection of a token's routed entries (and its shared expert) with
+// expert_combine's weighted sum in the same launch; the bits of the two separate launches
+struct ExpertDownCombineArgs {
+    uint32_t ggml_type;
+    const void* w;          // routed experts [experts][n, k]
+    const void* w_shared;   // [n, k] or null
+    const void* x;          // [tokens * top_k][2k] packed gate|up rows
+    const void* x_shared;   // [tokens][2k]
+    const float* metadata;  // [tokens * top_k][3]
+    const float* shared_gate;
+    void* y;                // [tokens][n]
+    uint32_t n, k, tokens, top_k, experts, dtype;
+};
+bool expert_down_combine_fits(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t top_k, bool shared);
+const char* launch_expert_down_combine(hipStream_t s, const ExpertDownCombineArgs& a);
+
 // gemv_stream.hip: the Q4_K GEMV with LDS-direct weight loads and matrix-core dot products
 struct StreamPlan {
     bool ok;              // the row length fits the kernel (LDS and per-wave block budget)
@@ -224,6 +240,7 @@ struct GemmArgs {
     // then weighs launch_gemm_resident against the other kernels)
     bool rows_resident;
     bool use_resident;    // set by launch_gemm_resident only
+    bool few_tiles_split; // up to 16 rows, few weight tiles per workgroup: the tiles' super-blocks are dealt over the waves
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

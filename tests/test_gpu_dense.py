@@ -633,6 +633,38 @@ def test_the_tile_picked_by_row_count_gives_the_bits_of_the_largest(api, d, m):
     assert np.array_equal(picked.tensor.raw(), largest.tensor.raw())
 
 
+@pytest.mark.parametrize("ggml", [12, 13, 14, 23, 8], ids=["q4_k", "q5_k", "q6_k", "iq4_xs", "q8_0"])
+@pytest.mark.parametrize("m,n,k,dtype", [(2, 17000, 5120, "F16"), (9, 4100, 5120, "BF16"), (16, 17000, 4096, "F16"),
+                                         (8, 1000, 2048, "F16"), (16, 20000, 768, "BF16")])
+def test_few_rows_deal_a_tiles_super_blocks_over_the_waves(api, d, ggml, m, n, k, dtype):
+    # up to 16 rows and at most five 16-row weight tiles per compute unit: every wave of the
+    # workgroup takes some super-blocks of every tile and the partial sums meet in LDS.  Rows of 1 -
+    # 20 super-blocks (8 and 16 waves), one to five tiles per workgroup, a ragged last tile, every
+    # format; against the tile-rounded oracle on sampled columns and against the kernel that
+    # gives a wave whole tiles (the same products, added in another order).
+    packed = synth.matrix(ggml, n, k, seed=181 + m)
+    w = qm(api, d, ggml, n, k, packed)
+    code = oracle.F16 if dtype == "F16" else oracle.BF16
+    x = oracle.round_storage(synth.activations(m, k, seed=182), code).reshape(m, k)
+    xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
+    out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    assert out.operation.endswith("_gemm_mfma_resident")
+    d.set_tuning("gemm_few_tiles_split", 0)
+    try:
+        whole = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_few_tiles_split", 1)
+    assert whole.operation == out.operation
+    got = out.tensor.to_f32()
+    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), synth.rng(183).integers(0, n, 80)]))
+    want = oracle_columns(ggml, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+    assert_matmul_parity(got[:, rows], want, "dealt super-blocks against the tile-rounded oracle")
+    assert_matmul_parity(got, whole.tensor.to_f32(), "against whole tiles per wave", l2_tol=2e-6)
+    assert not np.array_equal(got, np.zeros_like(got))
+    half = d.project_quantized(xt, w, out_dtype=getattr(api.DType, dtype))      # 16-bit output: the scalar stores
+    assert np.array_equal(half.tensor.to_f32(), oracle.round_storage(got, code).reshape(m, n))
+
+
 def test_objects_may_outlive_their_device(api):
     # buffers, matrices and recorded executions hold the device object: releasing them after
     # fh_device_destroy (any order a garbage collector may pick) is safe

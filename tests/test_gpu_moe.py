@@ -700,6 +700,50 @@ def test_the_ffn_in_one_call_gives_the_bits_of_the_separate_calls(api, d, dtype,
         moe.forward_in_one_call(xt, api.Tensor.zeros(d, (tokens, experts + 1), api.DType.F32))
 
 
+@pytest.mark.parametrize("ggml,inter,top_k,tokens,shared,dtype", [
+    (Q4_K, 512, 8, 1, True, "F16"), (Q4_K, 512, 8, 2, True, "BF16"), (Q4_K, 512, 8, 2, False, "F32"),
+    (Q6_K, 768, 4, 1, True, "F16"), (Q6_K, 1024, 3, 2, False, "F16"), (synth.Q5_K, 1536, 2, 2, True, "F16"),
+    (23, 2048, 2, 1, True, "F16"), (8, 512, 6, 2, True, "BF16"), (Q4_K, 256, 16, 1, True, "F16")])
+def test_few_tokens_fold_the_weighted_sum_into_the_down_projection(api, d, ggml, inter, top_k, tokens, shared, dtype):
+    # fh_moe_ffn with one or two tokens: route, gate|up, then one launch that multiplies every entry
+    # of a token (top_k routed experts, the shared one) and adds them with expert_combine's
+    # rounding.  Against the separate launches: the same bits, for every format, for rows of 1 - 8
+    # super-blocks (all lane layouts of the kernel), with 17 entries (one wave takes two), without a
+    # shared expert and with a gate on it.
+    experts, hidden = 24, 512
+    fmt_in, fmt_out = api.QuantizationFormat(Q4_K), api.QuantizationFormat(ggml)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=401), fmt_in,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(ggml, experts * hidden, inter, seed=402), fmt_out,
+                                         experts, hidden, inter)
+    kw = {}
+    if shared:
+        kw = dict(shared_input=api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt_in,
+                                                              synth.matrix(Q4_K, 2 * inter, hidden, seed=403)),
+                  shared_output=api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt_out,
+                                                               synth.matrix(ggml, hidden, inter, seed=404)))
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k), **kw)
+    dt = getattr(api.DType, dtype)
+    x = synth.activations(tokens, hidden, seed=405, f16=True) * np.float32(2.0 ** -5)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+    lt = api.Tensor.from_f32(d, (tokens, experts), api.DType.F32,
+                             synth.rng(406).standard_normal((tokens, experts)).astype(np.float32))
+    gate = api.Tensor.from_f32(d, (tokens,), api.DType.F32,
+                               (0.25 + 0.5 * synth.rng(407).random(tokens)).astype(np.float32)) if shared else None
+    want = moe.forward(xt, lt, shared_gate=gate)
+    got = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+    assert "combine" in d.last_operation() and "expert_project" in d.last_operation()
+    assert np.abs(want.to_f32()).max() > 1e-4
+    assert np.array_equal(got.raw(), want.raw())
+    d.set_tuning("moe_fold_combine", 0)
+    try:
+        apart = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+        assert "expert_project" not in d.last_operation()
+    finally:
+        d.set_tuning("moe_fold_combine", 1)
+    assert np.array_equal(apart.raw(), want.raw())
+
+
 def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
     # 32 rows of 2816 halves are more than the grouped kernel's LDS: the routed rows are staged and
     # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit

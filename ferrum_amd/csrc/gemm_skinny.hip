@@ -669,15 +669,12 @@ __global__ __launch_bounds__(64 * WAVES) void dense_few_tiles_kernel(const uint8
         const uint32_t row = min(tile * 16 + r, n - 1);
         return w + ((size_t)row * nb + min(unit_block(i), nb - 1)) * kBB;
     };
+    // The activation rows, eight 16-byte pieces per thread in flight at a time; piece p of row
+    // t sits at piece p ^ (t & 15), so the sixteen rows a B-operand read touches fall on different
+    // banks.  The first pieces are requested first and the first weights right behind them: loads
+    // return in order, the rows come from L2 (every workgroup reads the same ones) and are in LDS
+    // while the weights are still on their way from memory.
     Quarter<TYPE> ring[AHEAD + 1];
-#pragma unroll
-    for (int i = 0; i < AHEAD; ++i) {
-        if (unit_valid(i)) ring[i].load(unit_ptr(i), g);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-
-    // the activation rows, eight 16-byte pieces per thread in flight at a time; piece p of row
-    // t sits at piece p ^ (t & 15), so the sixteen rows a B-operand read touches fall on different banks
     const uint32_t total = m * pieces;
     for (uint32_t base = 0; base < total; base += 8 * kThreads) {
         u32x4 v[8];
@@ -688,6 +685,14 @@ __global__ __launch_bounds__(64 * WAVES) void dense_few_tiles_kernel(const uint8
             const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
             dst[j] = tok * ld + 8 * (pc ^ (tok & 15u));
             v[j] = *reinterpret_cast<const u32x4*>(x + (size_t)tok * k + 8 * pc);
+        }
+        if (base == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < AHEAD; ++i) {
+                if (unit_valid(i)) ring[i].load(unit_ptr(i), g);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
@@ -772,12 +777,15 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
             };
             // Sixteen waves with two units ahead where a tile has two super-blocks or more per
             // wave of eight and the format's raw quarter is small enough for 128 registers
-            // (8 x 17408 x 5120 Q4_K: 18.2 us against 20.7 with eight waves and six ahead, 24.3
-            // with whole tiles per wave; Q5_K and Q6_K spill there: 26.2 against 32.3 and 30.9
-            // against 36.9 with eight waves); eight waves for shorter rows (8 x 4096 x 2048: 4.9
-            // against 5.3 and 7.9).
+            // (8 x 17408 x 5120 Q4_K: 17.4 us against 19.9 with eight waves and six ahead, 24.3
+            // with whole tiles per wave; one or three units ahead, or 256 workgroups of four or
+            // five tiles instead of 218 of five, each cost 0.5 - 1.5 us; Q5_K and Q6_K spill
+            // there: 26.2 against 32.3 and 30.9 against 36.9 with eight waves); eight waves for
+            // shorter rows (8 x 4096 x 2048: 4.9 against 5.3 and 7.9).
             if constexpr (TYPE == kQ5K || TYPE == kQ6K) {
                 go(dense_few_tiles_kernel<TYPE, DT, 8, 4>, 8);
+            } else if constexpr (DT != 1) {
+                go(dense_few_tiles_kernel<TYPE, DT, 8, 6>, 8);  // the bf16 rounding needs more registers than 16 waves leave
             } else {
                 if (nb >= 16) go(dense_few_tiles_kernel<TYPE, DT, 16, 2>, 16);
                 else go(dense_few_tiles_kernel<TYPE, DT, 8, 6>, 8);

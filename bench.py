@@ -369,8 +369,8 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
 
     best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(2)) / steps
     separate = None
-    if tokens <= 2:
-        # one or two tokens: the same FFN through fh_moe_ffn, which adds the weighted sum inside
+    if tokens == 1:
+        # one token: the same FFN through fh_moe_ffn, which adds the weighted sum inside
         # the down projection's launch (three launches, the same bits); the four separate calls
         # of SparseMoe.forward are reported beside it
         out = api.Tensor.zeros(dev, (tokens, hidden), f16)

@@ -1680,11 +1680,12 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         // the copy and the activation ride inside the projections: per assignment in decode, in
         // the grouped kernel's gather of an expert's rows beyond it (f32 rows have no grouped form)
         const bool fused = a <= 31 || dt != FH_F32;
-        // One or two tokens: the down projection of a token's entries and the weighted sum over
-        // them are one launch (the bits of the two; 17.9 against 18.5 us for one token of the
-        // 256-expert top-8 FFN, 22.2 against 22.7 for two; from three tokens on the launch that
-        // stages an entry's activations once for 32 rows instead of 8 is the faster one).
-        const bool folded = count <= 2 && a <= 31 && (!shared || rides) && tuning(device, "moe_fold_combine") != 0 &&
+        // One token: the down projection of its entries and the weighted sum over them are one
+        // launch (the bits of the two; 17.1 against 18.4 us for the 256-expert top-8 FFN with a
+        // shared expert).  From two tokens on the two launches are the faster way (22.1 against
+        // 23.2 us): the projection's launch stages an entry's activations once for 32 rows, this one
+        // once for 8.
+        const bool folded = count == 1 && a <= 31 && (!shared || rides) && tuning(device, "moe_fold_combine") != 0 &&
                             (!shared_gate || shared_gate->dtype == FH_F32) &&
                             expert_down_combine_fits(output_experts->ggml_type, (uint32_t)h, (uint32_t)inter, k, shared);
         if (folded) {

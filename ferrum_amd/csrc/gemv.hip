@@ -288,6 +288,22 @@ __device__ __forceinline__ float4 load_x4(const void* x, uint32_t dtype, size_t 
                        bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
 }
 
+// load_x4 in two steps, so that the load can be issued long before its value is needed
+__device__ __forceinline__ uint4 raw_x4(const void* x, uint32_t dtype, size_t quad) {
+    if (dtype == FH_F32) return static_cast<const uint4*>(x)[quad];
+    const uint2 raw = static_cast<const uint2*>(x)[quad];
+    return make_uint4(raw.x, raw.y, 0u, 0u);
+}
+__device__ __forceinline__ float4 widen_x4(uint4 raw, uint32_t dtype) {
+    if (dtype == FH_F32)
+        return make_float4(__uint_as_float(raw.x), __uint_as_float(raw.y), __uint_as_float(raw.z), __uint_as_float(raw.w));
+    if (dtype == FH_F16)
+        return make_float4(f16_bits_to_f32(raw.x & 0xffffu), f16_bits_to_f32(raw.x >> 16),
+                           f16_bits_to_f32(raw.y & 0xffffu), f16_bits_to_f32(raw.y >> 16));
+    return make_float4(bf16_bits_to_f32(raw.x & 0xffffu), bf16_bits_to_f32(raw.x >> 16),
+                       bf16_bits_to_f32(raw.y & 0xffffu), bf16_bits_to_f32(raw.y >> 16));
+}
+
 // What expert_silu_mul would have stored for four columns, rounded to the
 // activation dtype at the same two points.
 __device__ __forceinline__ float4 silu_mul4(float4 g, float4 u, uint32_t dtype) {
@@ -508,6 +524,19 @@ __global__ __launch_bounds__(kDownCombineMaxWaves * kWave) void expert_down_comb
     for (uint32_t entry = wave; entry < entries; entry += waves) {
         const bool shared = entry >= p.top_k;
         const size_t slot = (size_t)token * p.top_k + entry;
+        // the entry's packed gate|up row does not depend on the routing record: its first 512
+        // columns are requested before the record, whose expert id the weight loads wait for
+        const void* xmat = shared ? p.x_shared : p.x;
+        const size_t xbase = (shared ? (size_t)token : slot) * 2 * p.nb * 64;
+        const uint32_t xq = p.nb * 64;
+        uint4 raw_gate[2], raw_up[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t q = lane + 64 * j < xq ? lane + 64 * j : xq - 1;
+            raw_gate[j] = raw_x4(xmat, p.dtype, xbase + q);
+            raw_up[j] = raw_x4(xmat, p.dtype, xbase + (size_t)p.nb * 64 + q);
+        }
+        asm volatile("" ::: "memory");
         bool live = true;
         size_t row_base = 0;
         float weight;
@@ -521,7 +550,6 @@ __global__ __launch_bounds__(kDownCombineMaxWaves * kWave) void expert_down_comb
         }
         if (lane == 0) weights[entry] = weight;
         const uint8_t* wmat = shared ? p.w_shared : p.w;
-        const void* xmat = shared ? p.x_shared : p.x;
         const uint8_t* rp = wmat + (row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb * kBlockBytes;
         Frag<TYPE> frag[IT];
 #pragma unroll
@@ -531,12 +559,17 @@ __global__ __launch_bounds__(kDownCombineMaxWaves * kWave) void expert_down_comb
         }
         asm volatile("" ::: "memory");
         // the entry's activations: silu(gate) * up of its packed row, staged as gemv_kernel stages them
-        const size_t xbase = (shared ? (size_t)token : slot) * 2 * p.nb * 64;
-        const uint32_t xq = p.nb * 64;
         if (entry != wave) __builtin_amdgcn_wave_barrier();
-        for (uint32_t q = lane; q < xq; q += 64) {
-            const float4 v = silu_mul4(load_x4(xmat, p.dtype, xbase + q),
-                                       load_x4(xmat, p.dtype, xbase + (size_t)p.nb * 64 + q), p.dtype);
+        for (uint32_t q = lane, j = 0; q < xq; q += 64, ++j) {
+            float4 gate, up;
+            if (j < 2) {
+                gate = widen_x4(j == 0 ? raw_gate[0] : raw_gate[1], p.dtype);
+                up = widen_x4(j == 0 ? raw_up[0] : raw_up[1], p.dtype);
+            } else {
+                gate = load_x4(xmat, p.dtype, xbase + q);
+                up = load_x4(xmat, p.dtype, xbase + (size_t)p.nb * 64 + q);
+            }
+            const float4 v = silu_mul4(gate, up, p.dtype);
             const uint32_t at = x_slot<TYPE>(q & 63u);
             xs[(q >> 6) * kXStride + at] = v;
             float s = (v.x + v.y) + (v.z + v.w);

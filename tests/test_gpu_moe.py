@@ -701,11 +701,11 @@ def test_the_ffn_in_one_call_gives_the_bits_of_the_separate_calls(api, d, dtype,
 
 
 @pytest.mark.parametrize("ggml,inter,top_k,tokens,shared,dtype", [
-    (Q4_K, 512, 8, 1, True, "F16"), (Q4_K, 512, 8, 2, True, "BF16"), (Q4_K, 512, 8, 2, False, "F32"),
-    (Q6_K, 768, 4, 1, True, "F16"), (Q6_K, 1024, 3, 2, False, "F16"), (synth.Q5_K, 1536, 2, 2, True, "F16"),
-    (23, 2048, 2, 1, True, "F16"), (8, 512, 6, 2, True, "BF16"), (Q4_K, 256, 16, 1, True, "F16")])
+    (Q4_K, 512, 8, 1, True, "F16"), (Q4_K, 512, 8, 1, True, "BF16"), (Q4_K, 512, 8, 1, False, "F32"),
+    (Q6_K, 768, 4, 1, True, "F16"), (Q6_K, 1024, 3, 1, False, "F16"), (synth.Q5_K, 1536, 2, 1, True, "F16"),
+    (23, 2048, 2, 1, True, "F16"), (8, 512, 6, 1, True, "BF16"), (Q4_K, 256, 16, 1, True, "F16")])
 def test_few_tokens_fold_the_weighted_sum_into_the_down_projection(api, d, ggml, inter, top_k, tokens, shared, dtype):
-    # fh_moe_ffn with one or two tokens: route, gate|up, then one launch that multiplies every entry
+    # fh_moe_ffn with one token: route, gate|up, then one launch that multiplies every entry
     # of a token (top_k routed experts, the shared one) and adds them with expert_combine's
     # rounding.  Against the separate launches: the same bits, for every format, for rows of 1 - 8
     # super-blocks (all lane layouts of the kernel), with 17 entries (one wave takes two), without a

@@ -665,6 +665,33 @@ def test_few_rows_deal_a_tiles_super_blocks_over_the_waves(api, d, ggml, m, n, k
     assert np.array_equal(half.tensor.to_f32(), oracle.round_storage(got, code).reshape(m, n))
 
 
+@pytest.mark.parametrize("ggml,m,dtype", [(12, 130, "F16"), (12, 300, "BF16"), (14, 200, "F16"), (8, 130, "F16")],
+                         ids=["q4_k-130", "q4_k-300-bf16", "q6_k-200", "q8_0-130"])
+def test_rows_too_long_for_lds_take_the_128_row_tiles(api, d, ggml, m, dtype):
+    # K = 17408 (the 27B model's down projection): no 16 rows of it fit LDS, so from 65 rows on the
+    # choice is between the tiles only.  5120 columns are too few for 256-row tiles to fill the chip
+    # and enough for 128 x 64 ones (160 or 240 workgroups), the default; the square tiles
+    # (tuning gemm_wide_shape 0) give the reference bits of the same products in another order.
+    n, k = 5120, 17408
+    packed = synth.matrix(ggml, n, k, seed=191)
+    w = qm(api, d, ggml, n, k, packed)
+    code = oracle.F16 if dtype == "F16" else oracle.BF16
+    x = oracle.round_storage(synth.activations(m, k, seed=192), code).reshape(m, k)
+    xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
+    out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    d.set_tuning("gemm_wide_shape", 0)
+    try:
+        square = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+    finally:
+        d.set_tuning("gemm_wide_shape", 1)
+    assert out.operation.endswith("_gemm_mfma_m256") == (m > 128) and square.operation.endswith("_gemm_mfma")
+    got = out.tensor.to_f32()
+    rows = np.unique(np.concatenate([np.arange(0, 70), np.arange(n - 70, n), synth.rng(193).integers(0, n, 60)]))
+    want = oracle_columns(ggml, packed, n, k, rows, x, weight_round=code, accumulate="f64")
+    assert_matmul_parity(got[:, rows], want, "rows of 17408 on the tiles")
+    assert_matmul_parity(got, square.tensor.to_f32(), "against the square tiles", l2_tol=2e-6)
+
+
 def test_objects_may_outlive_their_device(api):
     # buffers, matrices and recorded executions hold the device object: releasing them after
     # fh_device_destroy (any order a garbage collector may pick) is safe

@@ -696,9 +696,10 @@ GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments) {
 }
 
 bool gemv_takes_stream(const GemvArgs& a, StreamPlan* plan) {
-    if (a.stream == 0 || a.ggml_type != kQ4K || a.metadata != nullptr || a.x_mode != kXPlain || a.shared_w != nullptr)
+    if (a.stream == 0 || (a.ggml_type != kQ4K && a.ggml_type != kQ6K) || a.metadata != nullptr || a.x_mode != kXPlain ||
+        a.shared_w != nullptr)
         return false;
-    *plan = gemv_stream_plan(a.n, a.k, a.m, a.cu_count, a.stream == 2, a.ksplit);
+    *plan = gemv_stream_plan(a.ggml_type, a.n, a.k, a.m, a.cu_count, a.stream == 2, a.ksplit);
     return plan->ok;
 }
 

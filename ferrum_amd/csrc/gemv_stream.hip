@@ -1,7 +1,8 @@
-// Streamed Q4_K GEMV for gfx950: y[n] = sum_k W[n,k] x[k], one activation row per grid.z entry.
+// Streamed Q4_K and Q6_K GEMV for gfx950: y[n] = sum_k W[n,k] x[k], one activation row per grid.z entry.
 //
 // Same product as q4_k_gemv_factored / q4_k_gemv_ksplit of the reference
-// (src/metal/shaders/ops.metal:983-1070) in a form built around what limits a
+// (src/metal/shaders/ops.metal:983-1070; Q6_K: q6_k_factored_rows, q6_k_gemv_ksplit and
+// q6_k_gemv_factored, :1393-1439) in a form built around what limits a
 // GEMV of this size on this chip: how the bytes are requested, and how few vector
 // instructions are spent per weight.
 //
@@ -41,7 +42,13 @@ namespace fh {
 namespace {
 
 constexpr uint32_t kQ4Bytes = 144;
+constexpr uint32_t kQ6Bytes = 210;
 constexpr uint32_t kSlotBytes = 1024u + 64u + 16u;   // A operands, {group sum, group sum, 1/s, -} per chunk, 16 zero bytes
+// Q6_K: A operands, {four group sums, four 1/s} per lane group, 16 zero bytes
+constexpr uint32_t kSlot6Bytes = 1024u + 128u + 16u;
+template <uint32_t TYPE> struct StreamFormat;
+template <> struct StreamFormat<kQ4K> { static constexpr uint32_t kBytes = kQ4Bytes, kSlot = kSlotBytes, kAux = 64u; };
+template <> struct StreamFormat<kQ6K> { static constexpr uint32_t kBytes = kQ6Bytes, kSlot = kSlot6Bytes, kAux = 128u; };
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -126,23 +133,80 @@ __device__ __forceinline__ void stage_block(float4 v, uint8_t* slot, uint32_t la
     aux[2] = __uint_as_float((e - 14u) << 23);
 }
 
+// The same for a Q6_K super-block (the layout src/metal/shaders/ops.metal:1397-1425 indexes).
+// Weight 128 h + 32 s + 16 e + j (half h, slice s, j < 16) has its low four bits in
+// nibble s / 2 of ql[64 h + 32 (s & 1) + 16 e + j] and its high two in bits 2 s of
+// qh[32 h + 16 e + j]; lane group g = 2 h + e of the B operand holds those three 16-byte pieces,
+// four scale groups of 16 weights.  Step u = 2 (s & 1) + j / 8 multiplies eight bytes of a ql
+// piece: rows 4 g + 0 / 1 of A carry the hi / lo parts of the activations under the low nibbles
+// (slice s & 1), rows 4 g + 2 / 3 those under the high nibbles (slice 2 + (s & 1)), and the same
+// operand serves the two bit planes of qh that belong to those slices.  Lane L holds activations
+// 4 L .. 4 L + 3, so L = 32 h + 8 s + 4 e + j / 4: a quad of lanes is one scale group, which gets
+// a power-of-two scale of its own.
+__device__ __forceinline__ void stage_block_q6k(float4 v, uint8_t* slot, uint32_t lane) {
+    float top = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    top = dpp_max<0xB1>(top);
+    top = dpp_max<0x4E>(top);
+    uint32_t ex = __float_as_uint(top) >> 23;
+    ex = ex < 15u ? 15u : ex > 254u ? 254u : ex;
+    const float s = __uint_as_float((268u - ex) << 23);
+    half2v h02, h13, l02, l13;
+    h02.x = (_Float16)(v.x * s);
+    h02.y = (_Float16)(v.z * s);
+    h13.x = (_Float16)(v.y * s);
+    h13.y = (_Float16)(v.w * s);
+    l02.x = (_Float16)fmaf(v.x, s, -(float)h02.x);
+    l02.y = (_Float16)fmaf(v.z, s, -(float)h02.y);
+    l13.x = (_Float16)fmaf(v.y, s, -(float)h13.x);
+    l13.y = (_Float16)fmaf(v.w, s, -(float)h13.y);
+    const uint32_t h = lane >> 5, sl = (lane >> 3) & 3u, e = (lane >> 2) & 1u, up = (lane >> 1) & 1u;
+    const uint32_t g = 2u * h + e, u = 2u * (sl & 1u) + up, i = 2u * (sl >> 1);
+    uint8_t* const dst = slot + ((u * 4u + g) * 4u + i) * 16u + 8u * (lane & 1u);
+    *reinterpret_cast<uint2*>(dst) = make_uint2(__builtin_bit_cast(uint32_t, h02), __builtin_bit_cast(uint32_t, h13));
+    *reinterpret_cast<uint2*>(dst + 16) = make_uint2(__builtin_bit_cast(uint32_t, l02), __builtin_bit_cast(uint32_t, l13));
+    float sum = (v.x + v.y) + (v.z + v.w);
+    sum = dpp_add<0xB1>(sum);
+    sum = dpp_add<0x4E>(sum);   // the four lanes of a scale group now all hold its sum
+    float* const aux = reinterpret_cast<float*>(slot + 1024u) + 8u * g;
+    aux[sl] = sum;
+    aux[4u + sl] = __uint_as_float((ex - 14u) << 23);
+}
+
+// 16 or 8 bytes of a tile in LDS that are only 2-byte aligned (Q6_K blocks are 210 bytes long)
+__device__ __forceinline__ uint4 lds_u4_unaligned(const uint8_t* p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+__device__ __forceinline__ uint2 lds_u2_unaligned(const uint8_t* p) {
+    uint2 v;
+    __builtin_memcpy(&v, p, 8);
+    return v;
+}
+
 // LDS map (bytes): [tile: tile_rows x row_stride][a slot per wave][row sums: waves x 16 f32]
 // DT: activation dtype; WAVES: waves per workgroup; MAXB: super-blocks a wave may own (row length
 // <= WAVES * MAXB * 256).  Three workgroups of eight waves share a compute unit: six waves per
 // SIMD (ten-wave workgroups were tried for 20-block rows, two blocks per wave; only two of them
 // fit a compute unit's wave slots, and the launch took a third longer).
-template <int DT, int WAVES, int MAXB>
-__global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(6, 6)))
-void gemv_stream_q4k(const StreamParams p) {
+template <uint32_t TYPE, int DT, int WAVES, int MAXB>
+__device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     constexpr uint32_t kSWaves = WAVES;
+    constexpr uint32_t kBlock = StreamFormat<TYPE>::kBytes;    // bytes of a super-block
+    constexpr uint32_t kSlotBytes = StreamFormat<TYPE>::kSlot;
+    constexpr uint32_t kAuxBytes = StreamFormat<TYPE>::kAux;
+    auto stage = [](float4 v, uint8_t* slot, uint32_t lane) {
+        if constexpr (TYPE == kQ4K) stage_block(v, slot, lane);
+        else stage_block_q6k(v, slot, lane);
+    };
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // this workgroup's K segment: super-blocks first .. first + nb - 1 of the rows
     const uint32_t first = blockIdx.y * p.seg_blocks;
     const uint32_t nb = min(p.seg_blocks, p.nb - first);
-    const uint32_t row_bytes = nb * kQ4Bytes;          // of the segment
-    const uint32_t full_row_bytes = p.nb * kQ4Bytes;
+    const uint32_t row_bytes = nb * kBlock;          // of the segment
+    const uint32_t full_row_bytes = p.nb * kBlock;
     const uint32_t row0 = blockIdx.x * p.tile_rows;
     const uint32_t rows = min(p.tile_rows, p.n - row0);
 
@@ -170,7 +234,7 @@ void gemv_stream_q4k(const StreamParams p) {
     // 2. the tile: instruction i covers kilobyte (i % per_row) of row (i / per_row)
     const uint32_t per_row = (row_bytes + 1023u) >> 10;
     const uint32_t total = rows * per_row;
-    const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kQ4Bytes + lane * 16u;
+    const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kBlock + lane * 16u;
     const uint32_t tile_addr = (uint32_t)(uintptr_t)tile;
     uint32_t issued = 0;
     for (uint32_t i = wave; i < total; i += kSWaves) {
@@ -179,7 +243,7 @@ void gemv_stream_q4k(const StreamParams p) {
             lds_load16(wbase + (size_t)r * full_row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
         ++issued;
     }
-    if (lane < 4u) reinterpret_cast<uint32_t*>(slot + 1024u + 64u)[lane] = 0u;
+    if (lane < 4u) reinterpret_cast<uint32_t*>(slot + 1024u + kAuxBytes)[lane] = 0u;
 
     // 3. the activations have arrived (the tile's loads may still be in flight)
     wait_vmcnt(issued);
@@ -198,7 +262,7 @@ void gemv_stream_q4k(const StreamParams p) {
                                 bf16_bits_to_f32(xraw[i].y & 0xffffu), bf16_bits_to_f32(xraw[i].y >> 16));
         }
     }
-    stage_block(xv[0], slot, lane);   // the first block while the tile is on its way
+    stage(xv[0], slot, lane);   // the first block while the tile is on its way
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -207,9 +271,9 @@ void gemv_stream_q4k(const StreamParams p) {
     const uint32_t nc = n < rows ? n : rows - 1u;
     const bool active = (n >> 2) == g;
     const uint8_t* const wrow = tile + nc * p.row_stride;
-    const uint8_t* const xlane = active ? slot + (g * 4u + (n & 3u)) * 16u : slot + 1024u + 64u;
+    const uint8_t* const xlane = active ? slot + (g * 4u + (n & 3u)) * 16u : slot + 1024u + kAuxBytes;
     const uint32_t xstep = active ? 256u : 0u;
-    const float* const auxp = reinterpret_cast<const float*>(slot + 1024u) + 4u * g;
+    const float* const auxp = reinterpret_cast<const float*>(slot + 1024u) + (kAuxBytes / 16u) * g;
     float acc = 0.f;
 #pragma unroll
     for (int i = 0; i < MAXB; ++i) {
@@ -220,34 +284,103 @@ void gemv_stream_q4k(const StreamParams p) {
             u32x4 xa[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) xa[u] = *reinterpret_cast<const u32x4*>(xlane + u * xstep);
-            const float4 aux = *reinterpret_cast<const float4*>(auxp);
-            const uint8_t* const blk = wrow + b * kQ4Bytes;
-            const uint4 hdr = *reinterpret_cast<const uint4*>(blk);
-            const uint4 qa = *reinterpret_cast<const uint4*>(blk + 16u + 32u * g);
-            const uint4 qb = *reinterpret_cast<const uint4*>(blk + 32u + 32u * g);
-            if (i + 1 < MAXB && b + kSWaves < nb) {
-                asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");   // the five slot reads are the oldest
-                stage_block(xv[i + 1], slot, lane);
-            }
-            const uint32_t raw[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-            floatx4 dl = {0.f, 0.f, 0.f, 0.f}, dh = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (TYPE == kQ4K) {
+                const float4 aux = *reinterpret_cast<const float4*>(auxp);
+                const uint8_t* const blk = wrow + b * kBlock;
+                const uint4 hdr = *reinterpret_cast<const uint4*>(blk);
+                const uint4 qa = *reinterpret_cast<const uint4*>(blk + 16u + 32u * g);
+                const uint4 qb = *reinterpret_cast<const uint4*>(blk + 32u + 32u * g);
+                if (i + 1 < MAXB && b + kSWaves < nb) {
+                    asm volatile("s_waitcnt lgkmcnt(3)" ::: "memory");   // the five slot reads are the oldest
+                    stage(xv[i + 1], slot, lane);
+                }
+                const uint32_t raw[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+                floatx4 dl = {0.f, 0.f, 0.f, 0.f}, dh = {0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t q0 = raw[2 * u], q1 = raw[2 * u + 1];
+                    const uint32_t s0 = q0 >> 8, s1 = q1 >> 8;
+                    const u32x4 lo = {q0 & 0x000f000fu, s0 & 0x000f000fu, q1 & 0x000f000fu, s1 & 0x000f000fu};
+                    const u32x4 hi = {q0 & 0x00f000f0u, s0 & 0x00f000f0u, q1 & 0x00f000f0u, s1 & 0x00f000f0u};
+                    const half8 a = __builtin_bit_cast(half8, xa[u]);
+                    dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, lo), dl, 0, 0, 0);
+                    dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, hi), dh, 0, 0, 0);
+                }
+                float sc_lo, sc_hi, mn_lo, mn_hi;
+                q4k_chunk_scales(hdr.y, hdr.z, hdr.w, g, sc_lo, sc_hi, mn_lo, mn_hi);
+                const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
+                // low nibbles were q * 2^-24, high nibbles 16 q * 2^-24
+                const float dots = fmaf(sc_lo * 16777216.f, dl[0] + dl[1], (sc_hi * 1048576.f) * (dh[2] + dh[3]));
+                const float mins = fmaf(mn_lo, aux.x, mn_hi * aux.y);
+                acc = fmaf(d * aux.z, dots, fmaf(-dmin, mins, acc));
+            } else {
+                const float4 sums = *reinterpret_cast<const float4*>(auxp);
+                const float4 inv = *reinterpret_cast<const float4*>(auxp + 4);
+                asm volatile("" ::: "memory");   // the slot reads are issued before the tile reads
+                const uint8_t* const blk = wrow + b * kBlock;
+                const uint32_t h = g >> 1, e = g & 1u;
+                const uint4 qa = lds_u4_unaligned(blk + 64u * h + 16u * e);
+                const uint4 qb = lds_u4_unaligned(blk + 64u * h + 32u + 16u * e);
+                const uint4 qh = lds_u4_unaligned(blk + 128u + 32u * h + 16u * e);
+                const uint2 sc8 = lds_u2_unaligned(blk + 192u + 8u * h);
+                uint16_t dbits;
+                __builtin_memcpy(&dbits, blk + 208u, 2);
+                if (i + 1 < MAXB && b + kSWaves < nb) {
+                    // the six slot reads are the oldest; at least five instructions read the tile
+                    asm volatile("s_waitcnt lgkmcnt(5)" ::: "memory");
+                    stage(xv[i + 1], slot, lane);
+                }
+                const uint32_t ql[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+                const uint32_t ph[4] = {qh.x, qh.y, qh.z, qh.w};
+                // [piece][low nibbles, high nibbles, their bit planes]
+                floatx4 dn[2][4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const uint32_t q0 = raw[2 * u], q1 = raw[2 * u + 1];
-                const uint32_t s0 = q0 >> 8, s1 = q1 >> 8;
-                const u32x4 lo = {q0 & 0x000f000fu, s0 & 0x000f000fu, q1 & 0x000f000fu, s1 & 0x000f000fu};
-                const u32x4 hi = {q0 & 0x00f000f0u, s0 & 0x00f000f0u, q1 & 0x00f000f0u, s1 & 0x00f000f0u};
-                const half8 a = __builtin_bit_cast(half8, xa[u]);
-                dl = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, lo), dl, 0, 0, 0);
-                dh = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, hi), dh, 0, 0, 0);
+                for (int pc = 0; pc < 2; ++pc)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) dn[pc][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int up = 0; up < 2; ++up) {
+                    const uint32_t p0 = ph[2 * up], p1 = ph[2 * up + 1];
+                    const uint32_t t0 = p0 >> 8, t1 = p1 >> 8;
+#pragma unroll
+                    for (int pc = 0; pc < 2; ++pc) {
+                        const uint32_t q0 = ql[4 * pc + 2 * up], q1 = ql[4 * pc + 2 * up + 1];
+                        const uint32_t s0 = q0 >> 8, s1 = q1 >> 8;
+                        // Bit planes 0 and 2 belong to the first ql piece, 1 and 3 to the second.  The matrix
+                        // core's sum keeps a fixed number of bits below the operands' exponent field, which is
+                        // the same for every subnormal, so what a dot product loses does not depend on where
+                        // in the field the bits sit, while the factor that undoes the position does: planes 0
+                        // and 1, whose values count sixteenfold, move to the top of the field (bits 8..9).
+                        const uint32_t mh = pc == 0 ? 0x00300030u : 0x00c000c0u;
+                        const u32x4 nl = {q0 & 0x000f000fu, s0 & 0x000f000fu, q1 & 0x000f000fu, s1 & 0x000f000fu};
+                        const u32x4 nh = {q0 & 0x00f000f0u, s0 & 0x00f000f0u, q1 & 0x00f000f0u, s1 & 0x00f000f0u};
+                        const u32x4 pl = pc == 0 ? u32x4{(p0 << 8) & 0x03000300u, p0 & 0x03000300u, (p1 << 8) & 0x03000300u,
+                                                         p1 & 0x03000300u}
+                                                 : u32x4{(p0 << 6) & 0x03000300u, (p0 >> 2) & 0x03000300u,
+                                                         (p1 << 6) & 0x03000300u, (p1 >> 2) & 0x03000300u};
+                        const u32x4 pw = {p0 & mh, t0 & mh, p1 & mh, t1 & mh};
+                        const half8 a = __builtin_bit_cast(half8, xa[2 * pc + up]);
+                        dn[pc][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, nl), dn[pc][0], 0, 0, 0);
+                        dn[pc][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, nh), dn[pc][1], 0, 0, 0);
+                        dn[pc][2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, pl), dn[pc][2], 0, 0, 0);
+                        dn[pc][3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(half8, pw), dn[pc][3], 0, 0, 0);
+                    }
+                }
+                // The operands were (times 2^-24): low nibble q, high nibble 16 q, planes 0 and 1 256 v, plane 2
+                // 16 v, plane 3 64 v; a weight is q + 16 v - 32.  Slices 0 and 2 come from the first piece.
+                const float s0q = fmaf(16.f, dn[0][0][0] + dn[0][0][1], dn[0][2][0] + dn[0][2][1]) * 1048576.f;
+                const float s2q = fmaf(16.f, dn[0][3][2] + dn[0][3][3], dn[0][1][2] + dn[0][1][3]) * 1048576.f;
+                const float s1q = fmaf(16.f, dn[1][0][0] + dn[1][0][1], dn[1][2][0] + dn[1][2][1]) * 1048576.f;
+                const float s3q = fmaf(4.f, dn[1][3][2] + dn[1][3][3], dn[1][1][2] + dn[1][1][3]) * 1048576.f;
+                // the lane group's int8 scales: bytes e, e + 2, e + 4, e + 6 of its half's eight
+                const uint32_t lo = sc8.x >> (8u * e), hi = sc8.y >> (8u * e);
+                const float c0 = (float)(int)(int8_t)lo, c1 = (float)(int)(int8_t)(lo >> 16);
+                const float c2 = (float)(int)(int8_t)hi, c3 = (float)(int)(int8_t)(hi >> 16);
+                const float r0 = fmaf(s0q, inv.x, -32.f * sums.x), r1 = fmaf(s1q, inv.y, -32.f * sums.y);
+                const float r2 = fmaf(s2q, inv.z, -32.f * sums.z), r3 = fmaf(s3q, inv.w, -32.f * sums.w);
+                const float total = fmaf(c0, r0, c1 * r1) + fmaf(c2, r2, c3 * r3);
+                acc = fmaf(f16_bits_to_f32(dbits), total, acc);
             }
-            float sc_lo, sc_hi, mn_lo, mn_hi;
-            q4k_chunk_scales(hdr.y, hdr.z, hdr.w, g, sc_lo, sc_hi, mn_lo, mn_hi);
-            const float d = f16_bits_to_f32(hdr.x & 0xffffu), dmin = f16_bits_to_f32(hdr.x >> 16);
-            // low nibbles were q * 2^-24, high nibbles 16 q * 2^-24
-            const float dots = fmaf(sc_lo * 16777216.f, dl[0] + dl[1], (sc_hi * 1048576.f) * (dh[2] + dh[3]));
-            const float mins = fmaf(mn_lo, aux.x, mn_hi * aux.y);
-            acc = fmaf(d * aux.z, dots, fmaf(-dmin, mins, acc));
         }
     }
 
@@ -293,12 +426,27 @@ void gemv_stream_q4k(const StreamParams p) {
     }
 }
 
+template <int DT, int WAVES, int MAXB>
+__global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(6, 6)))
+void gemv_stream_q4k(const StreamParams p) {
+    gemv_stream_body<kQ4K, DT, WAVES, MAXB>(p);
+}
+
+// Q6_K rows are 46% longer: two workgroups share a compute unit, four waves per SIMD.
+template <int DT, int WAVES, int MAXB>
+__global__ __launch_bounds__(WAVES * kWave) void gemv_stream_q6k(const StreamParams p) {
+    gemv_stream_body<kQ6K, DT, WAVES, MAXB>(p);
+}
+
 }  // namespace
 
 // Tile height that spreads the rows evenly: the fewest 16-row rounds per compute unit, then the
 // smallest height that still fits them.
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size, int forced_segments) {
+StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size,
+                            int forced_segments) {
     StreamPlan plan{};
+    const bool q6 = ggml_type == kQ6K;
+    const uint32_t block = q6 ? kQ6Bytes : kQ4Bytes, slot = q6 ? kSlot6Bytes : kSlotBytes;
     const uint32_t nb = k / 256u;
     const uint32_t cus = cu_count > 0 ? (uint32_t)cu_count : 256u;
     const uint32_t rounds = ((n + 15u) / 16u + cus - 1u) / cus;
@@ -307,23 +455,26 @@ StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bo
     if (h < 1u) h = 1u;
     // An LDS-direct load names its LDS address in 16 bits of M0, so a tile stays below 64 KB, and
     // a wave owns at most six super-blocks: longer rows are cut into K segments of equal length.
-    auto stride_of = [](uint32_t blocks) {
-        uint32_t units = 9u * blocks;      // bytes / 16
+    auto stride_of = [block](uint32_t blocks) {
+        uint32_t units = (block * blocks + 15u) / 16u;   // bytes / 16
         if ((units & 1u) == 0) ++units;    // odd number of 16-byte units: 16 rows start in 16 different bank groups
         return units * 16u;
     };
     // ... and, where it must be cut anyway, short enough that three workgroups share a compute
     // unit's LDS (the headline's uncut 14 x 2896 bytes do)
-    const uint32_t budget = (160u * 1024u) / 3u - 8u * kSlotBytes - 8u * 64u;
+    const uint32_t budget = (160u * 1024u) / 3u - 8u * slot - 8u * 64u;
     // (the segments then spread the work, so the tiles are as tall as the matrix instruction)
     // the reference's K-split switch asks for at least that many segments, as far as whole blocks go
     const uint32_t wanted = forced_segments > 1 ? ((uint32_t)forced_segments < nb ? (uint32_t)forced_segments : nb) : 1u;
     if (wanted > 1u || nb > 48u || h * stride_of(nb) > 65536u) h = n < 16u ? n : 16u;
     uint32_t segments = wanted, seg = (nb + wanted - 1u) / wanted;
+    // LDS-direct loads want dword-aligned addresses: a Q6_K segment starts on an even block
+    auto even_up = [q6](uint32_t blocks) { return q6 ? (blocks + 1u) & ~1u : blocks; };
+    if (segments > 1u) seg = even_up(seg);
     while (seg > 48u || h * stride_of(seg) > (segments == 1 ? 65536u : budget)) {
         ++segments;
-        seg = (nb + segments - 1u) / segments;
-        if (seg <= 1u) break;
+        seg = even_up((nb + segments - 1u) / segments);
+        if (seg <= (q6 ? 2u : 1u)) break;
     }
     segments = (nb + seg - 1u) / seg;
     plan.segments = segments;
@@ -333,10 +484,16 @@ StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bo
     plan.tile_rows = h;
     plan.tiles = (n + h - 1u) / h;
     plan.waves = 8u;
-    plan.lds_bytes = h * plan.row_stride + plan.waves * kSlotBytes + plan.waves * 64u;
-    // matrices of a megabyte or two finish sooner on the FMA kernel's smaller workgroups
-    plan.ok = nb >= 1 && seg >= 1u && seg <= 48u && segments <= 65535u && h >= 1u && (any_size || (uint64_t)n * nb >= 16384u) &&
-              plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u;
+    plan.lds_bytes = h * plan.row_stride + plan.waves * slot + plan.waves * 64u;
+    // Matrices of a megabyte or two finish sooner on the FMA kernel's smaller workgroups.  Q6_K costs
+    // twice the matrix instructions and half again the vector work of Q4_K per super-block, which
+    // tiles of rows of 5120 do not hide (17408 x 5120 in fourteen-row tiles: 22.6 against 21.3 us on
+    // the FMA kernel; 151936 x 5120 in fifteen-row tiles 142 - 147 against 141 - 142 us, in two K
+    // segments 168 us); rows that must be cut into segments in any case gain (5120 x 17408: 22.7
+    // against 25.0 us).
+    const bool wins = q6 ? nb > 48u : (uint64_t)n * nb >= 16384u;
+    plan.ok = nb >= 1 && seg >= 1u && seg <= 48u && segments <= 65535u && h >= 1u && (any_size || wins) &&
+              plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u && (!q6 || (nb & 1u) == 0);
     return plan;
 }
 
@@ -357,22 +514,29 @@ const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPla
     p.partials = a.partials;
     p.counters = a.counters;
     typedef void (*Kernel)(const StreamParams);
-    // [dtype][blocks per wave: 2, 3, 6]
-    static const Kernel kernels[3][3] = {
-        {gemv_stream_q4k<FH_F32, 8, 2>, gemv_stream_q4k<FH_F32, 8, 3>, gemv_stream_q4k<FH_F32, 8, 6>},
-        {gemv_stream_q4k<FH_F16, 8, 2>, gemv_stream_q4k<FH_F16, 8, 3>, gemv_stream_q4k<FH_F16, 8, 6>},
-        {gemv_stream_q4k<FH_BF16, 8, 2>, gemv_stream_q4k<FH_BF16, 8, 3>, gemv_stream_q4k<FH_BF16, 8, 6>},
+    // [format][dtype][blocks per wave: 2, 3, 6]
+    static const Kernel kernels[2][3][3] = {
+        {{gemv_stream_q4k<FH_F32, 8, 2>, gemv_stream_q4k<FH_F32, 8, 3>, gemv_stream_q4k<FH_F32, 8, 6>},
+         {gemv_stream_q4k<FH_F16, 8, 2>, gemv_stream_q4k<FH_F16, 8, 3>, gemv_stream_q4k<FH_F16, 8, 6>},
+         {gemv_stream_q4k<FH_BF16, 8, 2>, gemv_stream_q4k<FH_BF16, 8, 3>, gemv_stream_q4k<FH_BF16, 8, 6>}},
+        {{gemv_stream_q6k<FH_F32, 8, 2>, gemv_stream_q6k<FH_F32, 8, 3>, gemv_stream_q6k<FH_F32, 8, 6>},
+         {gemv_stream_q6k<FH_F16, 8, 2>, gemv_stream_q6k<FH_F16, 8, 3>, gemv_stream_q6k<FH_F16, 8, 6>},
+         {gemv_stream_q6k<FH_BF16, 8, 2>, gemv_stream_q6k<FH_BF16, 8, 3>, gemv_stream_q6k<FH_BF16, 8, 6>}},
     };
     static bool raised = false;
     if (!raised) {
-        for (const auto& row : kernels)
-            for (Kernel kernel : row)
-                (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          160 * 1024);
+        for (const auto& format : kernels)
+            for (const auto& row : format)
+                for (Kernel kernel : row)
+                    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         raised = true;
     }
     const int shape = plan.seg_blocks <= 16u ? 0 : plan.seg_blocks <= 24u ? 1 : 2;
-    hipLaunchKernelGGL(kernels[a.x_dtype][shape], dim3(plan.tiles, plan.segments, a.m), dim3(plan.waves * kWave), plan.lds_bytes, s, p);
+    const int format = a.ggml_type == kQ6K ? 1 : 0;
+    hipLaunchKernelGGL(kernels[format][a.x_dtype][shape], dim3(plan.tiles, plan.segments, a.m), dim3(plan.waves * kWave),
+                       plan.lds_bytes, s, p);
+    if (format == 1) return plan.segments > 1 ? "q6_k_gemv_ksplit" : "q6_k_gemv_factored";
     return plan.segments > 1 ? "q4_k_gemv_ksplit" : "q4_k_gemv_factored";
 }
 

@@ -153,7 +153,7 @@ struct GemvArgs {
     uint32_t shared_rows;
     const void* shared_x;
     void* shared_y;
-    // the streamed matrix-core kernel may take the launch (dense Q4_K, plain rows, rows that fit LDS)
+    // the streamed matrix-core kernel may take the launch (dense Q4_K or Q6_K, plain rows, rows that fit LDS)
     int stream;           // 0 never, 1 where it is the faster kernel, 2 wherever it can run
     int cu_count;
     float* partials;      // scratch for K segments (gemv_plan says how much)
@@ -182,7 +182,7 @@ struct ExpertDownCombineArgs {
 bool expert_down_combine_fits(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t top_k, bool shared);
 const char* launch_expert_down_combine(hipStream_t s, const ExpertDownCombineArgs& a);
 
-// gemv_stream.hip: the Q4_K GEMV with LDS-direct weight loads and matrix-core dot products
+// gemv_stream.hip: the Q4_K and Q6_K GEMV with LDS-direct weight loads and matrix-core dot products
 struct StreamPlan {
     bool ok;              // the row length fits the kernel (LDS and per-wave block budget)
     uint32_t tile_rows;   // weight rows per workgroup (1..16)
@@ -195,7 +195,8 @@ struct StreamPlan {
     uint32_t segments, seg_blocks;
 };
 // any_size: also matrices so small that the FMA kernel is the faster one
-StreamPlan gemv_stream_plan(uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size, int forced_segments);
+StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t m, int cu_count, bool any_size,
+                            int forced_segments);
 const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPlan& plan);
 // whether launch_gemv hands this launch to the streamed kernel, and its plan
 bool gemv_takes_stream(const GemvArgs& a, StreamPlan* plan);

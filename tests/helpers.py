@@ -46,7 +46,7 @@ def oracle_columns(ggml_type, packed, n, k, rows, x, **kw):
 
 @contextlib.contextmanager
 def fma_gemv(d):
-    """Dense Q4_K GEMVs inside the block take the FMA kernel, the one the fused and
+    """Dense Q4_K and Q6_K GEMVs inside the block take the FMA kernel, the one the fused and
     per-assignment launches run on, so results can be compared with them bit for bit (the
     streamed matrix-core GEMV sums in another order and agrees to the matmul tolerance)."""
     before = d.get_tuning("gemv_stream")

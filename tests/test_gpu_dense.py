@@ -292,25 +292,41 @@ def check_gemv(api, d, ggml, n, k, seed, l2_tol=1e-5):
     assert l2 <= rel_l2(want32, want64) * 1.5 + 1e-7, "GPU is less accurate than the sequential CPU sum"
 
 
-# The streamed matrix-core GEMV (dense Q4_K): row lengths on both sides of its per-wave block
-# budgets, tile heights 1..16, every activation dtype, batched rows; rows too long for one tile
-# (more than 48 super-blocks, or 16 rows of them past 64 KB) are cut into 2 to 6 K segments.
-@pytest.mark.parametrize("n,k", [(37, 256), (133, 2560), (300, 4864), (1100, 5120), (4100, 2048), (70, 6144),
-                                 (33, 8192), (20, 12288), (100, 12544), (777, 14336), (530, 17408), (64, 34816)])
+# The streamed matrix-core GEMV (dense Q4_K and Q6_K): row lengths on both sides of its per-wave
+# block budgets, tile heights 1..16, every activation dtype, batched rows; rows too long for one
+# tile (more than 48 super-blocks, or 16 rows of them past 64 KB) are cut into 2 to 6 K segments.
+# Q6_K rows take it when they hold an even number of super-blocks (their 210-byte blocks then start
+# on a dword).
+STREAM_SHAPES = [(Q4_K, n, k) for n, k in [(37, 256), (133, 2560), (300, 4864), (1100, 5120), (4100, 2048), (70, 6144),
+                                           (33, 8192), (20, 12288), (100, 12544), (777, 14336), (530, 17408),
+                                           (64, 34816)]]
+STREAM_SHAPES += [(Q6_K, n, k) for n, k in [(37, 512), (133, 2560), (300, 4608), (1100, 5120), (4100, 2048), (70, 6144),
+                                            (33, 8192), (200, 9728), (20, 12288), (100, 12800), (777, 14336),
+                                            (530, 17408), (64, 34816)]]
+
+
+@pytest.mark.parametrize("ggml,n,k", STREAM_SHAPES)
 @pytest.mark.parametrize("dtype", ["F32", "F16", "BF16"])
-def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
+def test_streamed_gemv_matches_the_oracle(api, d, ggml, n, k, dtype):
     code = {"F32": oracle.F32, "F16": oracle.F16, "BF16": oracle.BF16}[dtype]
-    packed = synth.matrix(Q4_K, n, k, seed=n + k)
-    w = qm(api, d, Q4_K, n, k, packed)
+    name = "q4_k" if ggml == Q4_K else "q6_k"
+    packed = synth.matrix(ggml, n, k, seed=n + k)
+    w = qm(api, d, ggml, n, k, packed)
     d.set_tuning("gemv_stream", 2)   # also where the matrix is small enough for the FMA kernel to win
     for m in ((1, 3) if dtype == "F32" else (1,)):   # 16-bit rows beyond the first take the tile kernels
         x = oracle.round_storage(synth.activations(m, k, seed=7 * n + m), code).reshape(m, k)
         xt = api.Tensor.from_f32(d, (m, k), getattr(api.DType, dtype), x)
         out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
-        segmented = k > 12288
-        assert out.operation == (("q4_k_gemv_ksplit" if segmented else "q4_k_gemv_factored") if m == 1 else "q4_k_gemm")
-        want = oracle.project(Q4_K, packed, n, k, x, accumulate="f64")
-        assert_matmul_parity(out.tensor.to_f32(), want, f"streamed gemv {n}x{k} {dtype} m={m}")
+        if m > 1:
+            assert out.operation == name + "_gemm"
+        elif ggml == Q4_K:
+            assert out.operation == ("q4_k_gemv_ksplit" if k > 12288 else "q4_k_gemv_factored")
+        else:
+            assert out.operation in ("q6_k_gemv_ksplit", "q6_k_gemv_factored")
+            assert k <= 12288 or out.operation == "q6_k_gemv_ksplit"
+        segmented = out.operation.endswith("ksplit")
+        want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
+        assert_matmul_parity(out.tensor.to_f32(), want, f"streamed gemv {name} {n}x{k} {dtype} m={m}")
         if segmented:   # the segments are added in a fixed order
             again = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
             assert np.array_equal(bits(again), bits(out.tensor.to_f32()))
@@ -320,12 +336,14 @@ def test_streamed_gemv_matches_the_oracle(api, d, n, k, dtype):
     d.set_tuning("gemv_stream", 1)
 
 
-def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_streamed_gemv_scales_every_chunk_by_itself(api, d, ggml):
     # activations whose 64-value chunks differ by dozens of orders of magnitude, zero chunks, one
-    # value per chunk: the per-chunk power-of-two scale keeps 22 bits of each
+    # value per chunk: the power-of-two scale of a chunk (Q6_K: of a 16-weight group) keeps 22 bits
+    # of each
     n, k = 64, 2048
-    packed = synth.matrix(Q4_K, n, k, seed=91)
-    w = qm(api, d, Q4_K, n, k, packed)
+    packed = synth.matrix(ggml, n, k, seed=91)
+    w = qm(api, d, ggml, n, k, packed)
     d.set_tuning("gemv_stream", 2)
     x = synth.activations(1, k, seed=92).reshape(k // 64, 64)
     x *= np.float32(10.0) ** np.linspace(-30, 30, k // 64, dtype=np.float32)[:, None]
@@ -333,7 +351,7 @@ def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
     x[5, 1:] = 0
     x = x.reshape(1, k)
     got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, x), w).tensor.to_f32()
-    want = oracle.project(Q4_K, packed, n, k, x, accumulate="f64")
+    want = oracle.project(ggml, packed, n, k, x, accumulate="f64")
     assert rel_l2(got, want) <= 1e-5
     # each chunk alone: what the huge chunks would hide
     for chunk in (0, 5, 16, 31):
@@ -341,8 +359,20 @@ def test_streamed_gemv_scales_every_chunk_by_itself(api, d):
         part[chunk] = x.reshape(k // 64, 64)[chunk]
         part = part.reshape(1, k)
         got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, part), w).tensor.to_f32()
-        want = oracle.project(Q4_K, packed, n, k, part, accumulate="f64")
+        want = oracle.project(ggml, packed, n, k, part, accumulate="f64")
         assert rel_l2(got, want) <= 1e-5, chunk
+    if ggml == Q6_K:
+        # sixteen-value groups of one chunk that differ as much: each has a scale of its own
+        part = np.zeros((k // 16, 16), np.float32)
+        part[8:12] = synth.activations(1, 64, seed=93).reshape(4, 16) * np.float32(10.0) ** np.array([-20, 0, 11, 25], np.float32)[:, None]
+        part = part.reshape(1, k)
+        got = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, part), w).tensor.to_f32()
+        for group in range(8, 12):
+            alone = np.zeros((k // 16, 16), np.float32)
+            alone[group] = part.reshape(k // 16, 16)[group]
+            one = d.project_quantized(api.Tensor.from_f32(d, (1, k), api.DType.F32, alone.reshape(1, k)), w).tensor.to_f32()
+            assert rel_l2(one, oracle.project(ggml, packed, n, k, alone.reshape(1, k), accumulate="f64")) <= 1e-5, group
+        assert rel_l2(got, oracle.project(ggml, packed, n, k, part, accumulate="f64")) <= 1e-5
     # non-finite activations reach the rows they touch
     bad = x.copy()
     bad[0, 7] = np.inf

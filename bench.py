@@ -418,7 +418,7 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
     return {
         "cpu_baseline": cpu_line,
         "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
-        "operation": ("fh_moe_ffn: moe_route + expert_project with the shared expert riding + (expert_project + combine)"
+        "operation": ("fh_moe_ffn: (moe_route + expert_project with the shared expert riding) + (expert_project + combine)"
                       if separate is not None else
                       "moe_route + 2 x (expert_project with the shared expert riding) + combine" if tokens * top_k <= 31
                       else "moe_route + 2 x (expert_project grouped, shared expert pieces inside) + 2 x silu_mul + combine"),

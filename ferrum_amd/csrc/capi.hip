@@ -253,6 +253,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_wide_min_rows"] = 33;   // smallest M that takes the 256-row tile (it wins from there up)
     d->tuning["gemm_skinny_max_rows"] = 64; // largest M that takes the register-dequant MFMA kernel (0 = never)
     d->tuning["expert_grouped_min_assignments"] = 32;  // fewest assignments grouped by expert (0 = never)
+    d->tuning["moe_fold_route"] = 1;        // fh_moe_ffn, one token: the gate|up launch routes the token itself (0 = a moe_route launch first)
     d->tuning["gemm_few_tiles_split"] = 1;  // up to 16 rows and few weight tiles per workgroup: super-blocks dealt over the waves (0 = whole tiles per wave)
     d->tuning["moe_fold_combine"] = 1;      // fh_moe_ffn with few tokens: down projection and weighted sum in one launch (0 = two)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
@@ -855,7 +856,7 @@ namespace {
 fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const fh_view* selection_bias,
                 const fh_routing_policy* policy, const fh_view* metadata, bool ranked, const fh_view* gate_x,
                 const fh_view* gate_w, uint32_t hidden, const fh_view* shared_gate, const fh_view* ids = nullptr,
-                const fh_view* weights = nullptr) {
+                const fh_view* weights = nullptr, RouteTokenArgs* defer = nullptr) {
     if (device == nullptr || policy == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     const fh_routing_policy& p = *policy;
     if (tokens == 0 || p.experts == 0 || p.top_k == 0 || p.top_k > 16 || p.top_k > p.experts ||
@@ -915,6 +916,23 @@ fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const
             extras.gate_w = reinterpret_cast<const float*>(wr.begin);
             extras.hidden = hidden;
         }
+    }
+    if (defer != nullptr) {
+        // checked as a launch would be; the projection that follows routes the token itself
+        RouteTokenArgs& r = *defer;
+        r = RouteTokenArgs{};
+        r.logits = lr.begin;
+        r.logits_dtype = logits->dtype;
+        r.bias = reinterpret_cast<const float*>(br.begin);
+        r.metadata = reinterpret_cast<float*>(const_cast<uint8_t*>(mr.begin));
+        r.experts = p.experts;
+        r.top_k = p.top_k;
+        r.sigmoid = p.sigmoid;
+        r.normalize = p.normalize_top_k_prob;
+        r.eps = p.normalization_epsilon;
+        r.scaling = p.routed_scaling_factor;
+        r.rank_order = extras.rank_order;
+        return FH_OK;
     }
     device->last_operation = launch_moe_route(
         device->stream, lr.begin, logits->dtype, reinterpret_cast<const float*>(br.begin),
@@ -1288,7 +1306,7 @@ namespace {
 
 fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t x_rows,
                          uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y,
-                         const SharedExpert* shared = nullptr) {
+                         const SharedExpert* shared = nullptr, const RouteTokenArgs* route = nullptr) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (form > FH_INPUT_SILU_MUL) return fail(FH_ERR_PARAMETER, "unknown input form %u", form);
     if (shared != nullptr && form == FH_INPUT_ROWS)
@@ -1350,6 +1368,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     const bool grouped = (x->dtype != FH_F32 || f32_grouped) && grouped_min > 0 &&
                          assignments >= (uint64_t)grouped_min && weight->experts <= 1024 &&
                          (rows * dtype_bytes(y->dtype)) % 4 == 0;
+    if (grouped && route != nullptr) return fail(FH_ERR_DISPATCH, "only the per-assignment launch routes its token");
     if (grouped && shared != nullptr &&
         !expert_rows_fit_lds((uint32_t)k, assignments, (uint32_t)weight->experts)) {
         // a shared expert rides in the grouped form only in the kernel that keeps rows in LDS;
@@ -1465,6 +1484,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
     a.ksplit = 0;
     a.x_mode = form;
     a.x_rows = form == FH_INPUT_GATHER ? x_rows : assignments;
+    a.route = route;
     if (shared != nullptr) {
         a.m = assignments + shared->tokens;
         a.shared_w = shared->weight->ptr;
@@ -1675,8 +1695,6 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         const fh_view meta = view(meta_at, FH_F32), assigned = view(assigned_at, dt), projected = view(projected_at, dt),
                       activated = view(activated_at, dt), expert_out = view(expert_out_at, dt),
                       sproj = view(sproj_at, dt), sact = view(sact_at, dt), sout = view(sout_at, dt);
-        st = fh_moe_route(device, &logits, count, selection_bias, policy, &meta);
-        if (st != FH_OK) return st;
         // the copy and the activation ride inside the projections: per assignment in decode, in
         // the grouped kernel's gather of an expert's rows beyond it (f32 rows have no grouped form)
         const bool fused = a <= 31 || dt != FH_F32;
@@ -1688,10 +1706,25 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         const bool folded = count == 1 && a <= 31 && (!shared || rides) && tuning(device, "moe_fold_combine") != 0 &&
                             (!shared_gate || shared_gate->dtype == FH_F32) &&
                             expert_down_combine_fits(output_experts->ggml_type, (uint32_t)h, (uint32_t)inter, k, shared);
+        // ... and so does the routing: every workgroup of the gate|up launch routes the token
+        // itself before it asks for its expert's rows, which takes a launch and the wait for its
+        // records out of the chain
+        const int64_t grouped_from = tuning(device, "expert_grouped_min_assignments");
+        const bool routes_inside = folded && tuning(device, "moe_fold_route") != 0 &&
+                                   (grouped_from <= 0 || a < (uint64_t)grouped_from) &&   // the per-assignment launch
+                                   gemv_routes((uint32_t)two_i, (uint32_t)h, (uint32_t)e, k);
+        RouteTokenArgs inside{};
+        st = route(device, &logits, count, selection_bias, policy, &meta, false, nullptr, nullptr, 0, nullptr, nullptr,
+                   nullptr, routes_inside ? &inside : nullptr);
+        if (st != FH_OK) return st;
         if (folded) {
-            st = shared ? fh_expert_project_with_shared(device, input_experts, shared_input, &x, count, FH_INPUT_GATHER,
-                                                        a, &meta, nullptr, &projected, &sproj)
-                        : fh_expert_project_fused(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected);
+            SharedExpert rider;
+            rider.weight = shared_input;
+            rider.tokens = count;
+            rider.x = nullptr;
+            rider.y = &sproj;
+            st = expert_project(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected,
+                                shared ? &rider : nullptr, routes_inside ? &inside : nullptr);
             if (st != FH_OK) return st;
             Range yr, gr{nullptr, 0};
             st = resolve(device, &y, (uint64_t)count * h, "routed FFN output", &yr);

@@ -32,6 +32,7 @@
 // row tile) adds them in segment order, so results are deterministic.
 #include "device_utils.hpp"
 #include "internal.hpp"
+#include "route_device.hpp"
 
 namespace fh {
 namespace {
@@ -340,9 +341,11 @@ struct Params {
     void* y_shared;
 };
 
-// grid: (row tiles, K segments, m)
-template <uint32_t TYPE, int BS, int IT>
-__global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
+// grid: (row tiles, K segments, m).  ROUTE: the launch's one token has not been routed yet; wave 0
+// of every workgroup routes it (route_token, up to 256 experts) while the token's row, which
+// needs no routing, is already on its way, and the entry's expert comes from that.
+template <uint32_t TYPE, int BS, int IT, bool ROUTE>
+__device__ __forceinline__ void gemv_body(const Params& p, const RouteTokenArgs* route) {
     constexpr int RS = 16 / BS;
     constexpr uint32_t kBlockBytes = block_bytes_of(TYPE);
     extern __shared__ float4 xs[];  // seg_len * kXStride float4, then seg_len * 16 run sums
@@ -362,19 +365,22 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
     const void* xmat = shared && p.x_shared != nullptr ? p.x_shared : p.x;
     void* ymat = shared ? p.y_shared : p.y;
     const uint32_t ym = shared ? m - p.routed : m;  // row of y this entry writes
-    if (p.metadata != nullptr && !shared) {
-        uint32_t expert = __float_as_uint(p.metadata[p.meta_stride * (size_t)m]);
-        live = expert < p.experts;
-        row_base = live ? (size_t)expert * p.n : 0;
+    if constexpr (!ROUTE) {
+        if (p.metadata != nullptr && !shared) {
+            uint32_t expert = __float_as_uint(p.metadata[p.meta_stride * (size_t)m]);
+            live = expert < p.experts;
+            row_base = live ? (size_t)expert * p.n : 0;
+        }
     }
     const uint32_t row = (blockIdx.x * kWaves + wave) * RS + rs;
-    const uint8_t* rp = wmat + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
 
     // 1. activations of this segment (requested first, consumed first)
     // float4 index of the segment start in the row this batch entry reads
     size_t xrow = ym;
     if (shared) {
         // token ym's own row, in either form
+    } else if (ROUTE) {
+        xrow = 0;   // the one token
     } else if (p.x_mode == kXGather) {
         const uint32_t token = __float_as_uint(p.metadata[3 * (size_t)m + 1]);
         xrow = token < p.x_rows ? token : p.x_rows - 1;
@@ -399,6 +405,20 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
         xr[i] = q < xq && early ? load_x4(xmat, p.x_dtype, xbase + q) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     asm volatile("" ::: "memory");
+
+    if constexpr (ROUTE) {
+        __shared__ __attribute__((aligned(16))) float route_scores[256];
+        __shared__ float route_records[3 * kMaxTopK];
+        if (wave == 0)
+            route_token<4>(*route, 0u, lane, route_scores, route_records, blockIdx.x == 0 && blockIdx.y == 0 && m == 0);
+        __syncthreads();
+        if (!shared) {
+            const uint32_t expert = __float_as_uint(route_records[3 * m]);
+            live = expert < p.experts;
+            row_base = live ? (size_t)expert * p.n : 0;
+        }
+    }
+    const uint8_t* rp = wmat + ((row_base + (row < p.n ? row : p.n - 1)) * (size_t)p.nb + b0) * kBlockBytes;
 
     // 2. every weight fragment of this wave
     Frag<TYPE> frag[IT];
@@ -479,6 +499,16 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
             store_from_f32(ymat, (size_t)ym * p.n + r, p.y_dtype, total);
         }
     }
+}
+
+template <uint32_t TYPE, int BS, int IT>
+__global__ __launch_bounds__(kThreads) void gemv_kernel(const Params p) {
+    gemv_body<TYPE, BS, IT, false>(p, nullptr);
+}
+
+template <uint32_t TYPE, int BS, int IT>
+__global__ __launch_bounds__(kThreads) void gemv_route_kernel(const Params p, const RouteTokenArgs route) {
+    gemv_body<TYPE, BS, IT, true>(p, &route);
 }
 
 // The routed FFN's last two stages in one launch for a few tokens: the down projection of
@@ -648,6 +678,22 @@ LaunchFn pick(int bs, int it) {
     return nullptr;
 }
 
+typedef void (*RouteLaunchFn)(dim3, size_t, hipStream_t, const Params&, const RouteTokenArgs&);
+
+template <uint32_t TYPE, int BS, int IT>
+void launch_route_impl(dim3 grid, size_t lds, hipStream_t s, const Params& p, const RouteTokenArgs& r) {
+    hipLaunchKernelGGL((gemv_route_kernel<TYPE, BS, IT>), grid, dim3(kThreads), lds, s, p, r);
+}
+
+template <uint32_t TYPE>
+RouteLaunchFn pick_route(int bs, int it) {
+#define FH_CASE(B, I) \
+    if (bs == B && it == I) return launch_route_impl<TYPE, B, I>;
+    FH_CASE(8, 1) FH_CASE(8, 2) FH_CASE(8, 3) FH_CASE(4, 1) FH_CASE(2, 1) FH_CASE(1, 1)
+#undef FH_CASE
+    return nullptr;
+}
+
 }  // namespace
 
 namespace {
@@ -744,7 +790,16 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
                   : a.ggml_type == kIQ4XS ? pick<kIQ4XS>(plan.bs, plan.it)
                   : a.ggml_type == kQ8_0  ? pick<kQ8_0>(plan.bs, plan.it)
                                           : pick<kQ6K>(plan.bs, plan.it);
-    fn(grid, lds, s, p);
+    if (a.route != nullptr) {
+        RouteLaunchFn rf = a.ggml_type == kQ4K     ? pick_route<kQ4K>(plan.bs, plan.it)
+                           : a.ggml_type == kQ5K   ? pick_route<kQ5K>(plan.bs, plan.it)
+                           : a.ggml_type == kIQ4XS ? pick_route<kIQ4XS>(plan.bs, plan.it)
+                           : a.ggml_type == kQ8_0  ? pick_route<kQ8_0>(plan.bs, plan.it)
+                                                   : pick_route<kQ6K>(plan.bs, plan.it);
+        rf(grid, lds, s, p, *a.route);   // gemv_routes said the pair exists
+    } else {
+        fn(grid, lds, s, p);
+    }
     const int f = a.ggml_type == kQ4K ? 0 : a.ggml_type == kQ5K ? 1 : a.ggml_type == kQ6K ? 2 : a.ggml_type == kIQ4XS ? 3 : 4;
     static const char* const expert_names[5] = {"expert_project_q4_k_factored", "expert_project_q5_k_factored",
                                                 "expert_project_q6_k_factored", "expert_project_iq4_xs_factored",
@@ -753,9 +808,17 @@ const char* launch_gemv(hipStream_t s, const GemvArgs& a) {
                                                 "iq4_xs_gemv_ksplit", "q8_0_gemv_ksplit"};
     static const char* const factored_names[5] = {"q4_k_gemv_factored", "q5_k_gemv_factored", "q6_k_gemv_factored",
                                                   "iq4_xs_gemv_factored", "q8_0_gemv_factored"};
+    if (a.route != nullptr) return a.route->rank_order ? "h_moe_route + expert_project" : "moe_route + expert_project";
     if (a.metadata != nullptr) return expert_names[f];
     if (plan.segments > 1) return ksplit_names[f];
     return factored_names[f];
+}
+
+// Whether the projection of one token's entries can route the token itself: rows of one K
+// segment (up to 24 super-blocks) and a router of up to 256 experts.
+bool gemv_routes(uint32_t n, uint32_t k, uint32_t experts, uint32_t top_k) {
+    const GemvPlan plan = gemv_plan(n, k, 1, 0);
+    return plan.segments == 1 && pick_route<kQ4K>(plan.bs, plan.it) != nullptr && experts <= 256 && top_k <= (uint32_t)kMaxTopK;
 }
 
 bool expert_down_combine_fits(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t top_k, bool shared) {

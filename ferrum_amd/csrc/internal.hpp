@@ -130,6 +130,24 @@ enum : uint32_t {
     kXDivide = 3,   // row m / x_div of x: the hybrid engine's project_id, whose routes share a token's row
 };
 
+// what route_token (route_device.hpp) takes: one token's routing by one wave
+struct RouteTokenArgs {
+    const void* logits;
+    uint32_t logits_dtype;
+    const float* bias;
+    float* metadata;
+    uint32_t experts, top_k, sigmoid, normalize;
+    float eps, scaling;
+    uint32_t rank_order;
+    const void* gate_x;
+    uint32_t gate_x_dtype;
+    const float* gate_w;
+    uint32_t hidden;
+    float* shared_gate;
+    float* ids_out;
+    float* weights_out;
+};
+
 struct GemvArgs {
     uint32_t ggml_type;
     const void* w;        // packed [n, k] (per expert when metadata is set)
@@ -158,6 +176,10 @@ struct GemvArgs {
     int cu_count;
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)
+    // One token whose routing has not run yet: every workgroup routes it first (one wave, the
+    // bits of moe_route), takes its entry's expert from that, and workgroup 0 writes the records
+    // to route->metadata for the launches that follow.  `metadata` is then only a non-null marker.
+    const RouteTokenArgs* route;
 };
 struct GemvPlan {
     int bs, it;           // block slots per wave step, steps
@@ -165,6 +187,8 @@ struct GemvPlan {
 };
 GemvPlan gemv_plan(uint32_t n, uint32_t k, uint32_t m, int forced_segments);
 const char* launch_gemv(hipStream_t s, const GemvArgs& a);
+// whether a launch with GemvArgs::route set exists for these rows and this router
+bool gemv_routes(uint32_t n, uint32_t k, uint32_t experts, uint32_t top_k);
 
 // gemv.hip: the down projection of a token's routed entries (and its shared expert) with
 // expert_combine's weighted sum in the same launch; the bits of the two separate launches

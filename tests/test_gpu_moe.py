@@ -744,6 +744,62 @@ def test_few_tokens_fold_the_weighted_sum_into_the_down_projection(api, d, ggml,
     assert np.array_equal(apart.raw(), want.raw())
 
 
+@pytest.mark.parametrize("ggml,hidden,experts,top_k,shared,dtype,policy", [
+    (Q4_K, 2048, 256, 8, True, "F16", "softmax"), (Q4_K, 512, 24, 4, False, "F32", "softmax"),
+    (Q6_K, 1024, 64, 6, True, "BF16", "sigmoid"), (synth.Q5_K, 256, 130, 2, True, "F16", "bias"),
+    (23, 4096, 100, 8, False, "F16", "ties"), (8, 6144, 40, 16, True, "F16", "scaled"),
+    (Q4_K, 2816, 7, 7, True, "F16", "softmax")])
+def test_one_token_is_routed_by_its_gate_up_launch(api, d, ggml, hidden, experts, top_k, shared, dtype, policy):
+    # fh_moe_ffn with one token: no moe_route launch; every workgroup of the gate|up launch routes
+    # the token itself and workgroup 0 publishes the records the down projection reads.  The bits
+    # of the three launches (tuning moe_fold_route 0) and of the separate calls, for every input
+    # format and lane layout (rows of 1 - 24 super-blocks), routers of 7 - 256 experts, the sigmoid
+    # policy, a selection bias, tied logits, a scaling factor and an epsilon.
+    inter = 256
+    fmt = api.QuantizationFormat(ggml)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(ggml, experts * 2 * inter, hidden, seed=501), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(ggml, experts * hidden, inter, seed=502), fmt,
+                                         experts, hidden, inter)
+    kw = {}
+    if shared:
+        kw = dict(shared_input=api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt,
+                                                              synth.matrix(ggml, 2 * inter, hidden, seed=503)),
+                  shared_output=api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt,
+                                                               synth.matrix(ggml, hidden, inter, seed=504)))
+    routing = api.MoeRoutingPolicy(experts, top_k)
+    logits = synth.rng(506).standard_normal((1, experts)).astype(np.float32)
+    if policy == "sigmoid":
+        routing = api.MoeRoutingPolicy(experts, top_k, api.MoeScoringFunction.Sigmoid, True, 1e-6, 1.0)
+    elif policy == "bias":
+        routing = api.MoeRoutingPolicy(experts, top_k, api.MoeScoringFunction.Softmax, True, 0.0, 1.0, True)
+        kw["selection_bias"] = api.Tensor.from_f32(d, (experts,), api.DType.F32,
+                                                   synth.rng(508).standard_normal(experts).astype(np.float32) * 0.1)
+    elif policy == "ties":
+        logits = np.round(logits * 2) / 2   # many equal logits: the lower expert id wins
+    elif policy == "scaled":
+        routing = api.MoeRoutingPolicy(experts, top_k, api.MoeScoringFunction.Softmax, False, 0.0, 2.5)
+    moe = api.SparseMoe(d, win, wout, routing, **kw)
+    dt = getattr(api.DType, dtype)
+    x = synth.activations(1, hidden, seed=505, f16=True) * np.float32(2.0 ** -5)
+    xt = api.Tensor.from_f32(d, x.shape, dt, x)
+    lt = api.Tensor.from_f32(d, (1, experts), api.DType.F32, logits)
+    gate = api.Tensor.from_f32(d, (1,), api.DType.F32, np.array([0.625], np.float32)) if shared else None
+    want = moe.forward(xt, lt, shared_gate=gate)
+    assert np.abs(want.to_f32()).max() > 1e-5
+    d.set_tuning("moe_fold_route", 1)
+    got = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+    assert np.array_equal(got.raw(), want.raw())
+    again = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+    assert np.array_equal(again.raw(), want.raw())
+    d.set_tuning("moe_fold_route", 0)
+    try:
+        apart = moe.forward_in_one_call(xt, lt, shared_gate=gate)
+    finally:
+        d.set_tuning("moe_fold_route", 1)
+    assert np.array_equal(apart.raw(), want.raw())
+
+
 def test_shared_expert_runs_apart_when_an_experts_rows_do_not_fit_lds(api, d):
     # 32 rows of 2816 halves are more than the grouped kernel's LDS: the routed rows are staged and
     # the shared expert takes the dense kernels, which is what the separate calls do, bit for bit

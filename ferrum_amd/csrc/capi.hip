@@ -257,6 +257,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemm_few_tiles_split"] = 1;  // up to 16 rows and few weight tiles per workgroup: super-blocks dealt over the waves (0 = whole tiles per wave)
     d->tuning["moe_fold_combine"] = 1;      // fh_moe_ffn with few tokens: down projection and weighted sum in one launch (0 = two)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
+    d->tuning["gemv_stream_own_loads"] = 1; // the streamed Q4_K GEMV's waves load the super-blocks they multiply (tiles of up to 14 rows); 0: the tile row by row
     d->tuning["gemv_stream"] = 1;           // dense Q4_K / Q6_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
@@ -357,7 +358,7 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 2;
     } else if (k == "gemm_resident" || k == "moe_fold_combine" || k == "moe_fold_route") {
         ok = value == 0 || value == 1;
-    } else if (k == "gemm_few_tiles_split") {
+    } else if (k == "gemm_few_tiles_split" || k == "gemv_stream_own_loads") {
         ok = value == 0 || value == 1;
     } else if (k == "gemv_stream") {
         ok = value >= 0 && value <= 2;
@@ -679,6 +680,7 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
         a.experts = 1;
         a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
         a.stream = (int)tuning(device, "gemv_stream");
+        a.stream_own = tuning(device, "gemv_stream_own_loads") != 0;
         a.cu_count = device->props.multiProcessorCount;
         a.x_mode = silu_mul ? kXSiluMul : kXPlain;
         a.x_rows = m;
@@ -740,6 +742,7 @@ fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* wei
     a.experts = 1;
     a.ksplit = (int)tuning(device, "k_quant_gemv_ksplit");
     a.stream = (int)tuning(device, "gemv_stream");
+    a.stream_own = tuning(device, "gemv_stream_own_loads") != 0;
     a.cu_count = device->props.multiProcessorCount;
     a.x_mode = kXPlain;
     a.x_rows = m;

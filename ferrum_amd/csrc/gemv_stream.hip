@@ -62,6 +62,7 @@ struct StreamParams {
     uint32_t n, nb;
     uint32_t tile_rows;   // rows per workgroup, 1..16
     uint32_t row_stride;  // bytes between rows of the tile in LDS
+    uint32_t tile_bytes;  // of the tile region in LDS
     uint32_t x_dtype, y_dtype;
     // rows longer than a tile can hold: grid.y K segments of seg_blocks super-blocks each
     uint32_t segments, seg_blocks, m;
@@ -75,12 +76,13 @@ __device__ __forceinline__ void lds_load16(const void* g, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
 }
 
-// s_waitcnt vmcnt(n), n a wave-uniform run-time value up to 15 (0 beyond)
+// s_waitcnt vmcnt(n), n a wave-uniform run-time value up to 20 (0 beyond)
 __device__ __forceinline__ void wait_vmcnt(uint32_t n) {
 #define FH_VM(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
     switch (n) {
         FH_VM(1) FH_VM(2) FH_VM(3) FH_VM(4) FH_VM(5) FH_VM(6) FH_VM(7) FH_VM(8)
         FH_VM(9) FH_VM(10) FH_VM(11) FH_VM(12) FH_VM(13) FH_VM(14) FH_VM(15)
+        FH_VM(16) FH_VM(17) FH_VM(18) FH_VM(19) FH_VM(20)
         default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     }
 #undef FH_VM
@@ -189,7 +191,11 @@ __device__ __forceinline__ uint2 lds_u2_unaligned(const uint8_t* p) {
 // <= WAVES * MAXB * 256).  Three workgroups of eight waves share a compute unit: six waves per
 // SIMD (ten-wave workgroups were tried for 20-block rows, two blocks per wave; only two of them
 // fit a compute unit's wave slots, and the launch took a third longer).
-template <uint32_t TYPE, int DT, int WAVES, int MAXB>
+// OWN: a wave requests exactly the super-blocks it multiplies -- a block of all the tile's
+// rows is tile_rows x 9 pieces of 16 bytes, 64 pieces per instruction -- and waits for its own
+// loads only; the tile in LDS is then [block][row][144 bytes] (rows 36 words apart: sixteen rows
+// read sixteen different groups of four banks).
+template <uint32_t TYPE, int DT, int WAVES, int MAXB, bool OWN = false>
 __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     constexpr uint32_t kSWaves = WAVES;
     constexpr uint32_t kBlock = StreamFormat<TYPE>::kBytes;    // bytes of a super-block
@@ -211,8 +217,8 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     const uint32_t rows = min(p.tile_rows, p.n - row0);
 
     uint8_t* const tile = lds;
-    uint8_t* const slot = tile + p.tile_rows * p.row_stride + wave * kSlotBytes;
-    float* const rsum = reinterpret_cast<float*>(tile + p.tile_rows * p.row_stride + kSWaves * kSlotBytes);
+    uint8_t* const slot = tile + p.tile_bytes + wave * kSlotBytes;
+    float* const rsum = reinterpret_cast<float*>(tile + p.tile_bytes + kSWaves * kSlotBytes);
 
     // 1. this wave's activation blocks are requested first
     const size_t xrow = ((size_t)blockIdx.z * p.nb + first) * 256u;
@@ -237,11 +243,31 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kBlock + lane * 16u;
     const uint32_t tile_addr = (uint32_t)(uintptr_t)tile;
     uint32_t issued = 0;
-    for (uint32_t i = wave; i < total; i += kSWaves) {
-        const uint32_t r = i / per_row, c = i - r * per_row;
-        if (c * 1024u + lane * 16u < row_bytes)
-            lds_load16(wbase + (size_t)r * full_row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
-        ++issued;
+    // OWN: a super-block of the tile is tile_rows x 9 pieces of 16 bytes, piece 64 j + lane by instruction j
+    const uint32_t block_pieces = p.tile_rows * (kBlock / 16u), groups = (block_pieces + 63u) / 64u;
+    const uint32_t block_pitch = block_pieces * 16u;
+    if constexpr (OWN) {
+#pragma unroll
+        for (int i = 0; i < MAXB; ++i) {
+            const uint32_t b = wave + kSWaves * i;
+            if (b < nb) {
+                for (uint32_t j = 0; j < groups; ++j) {
+                    const uint32_t piece = 64u * j + lane, rl = piece / (kBlock / 16u), pc = piece - rl * (kBlock / 16u);
+                    const uint32_t r = min(rl, rows - 1u);
+                    if (piece < block_pieces)
+                        lds_load16(p.w + (size_t)(row0 + r) * full_row_bytes + (size_t)(first + b) * kBlock + 16u * pc,
+                                   tile_addr + b * block_pitch + 1024u * j);
+                    ++issued;
+                }
+            }
+        }
+    } else {
+        for (uint32_t i = wave; i < total; i += kSWaves) {
+            const uint32_t r = i / per_row, c = i - r * per_row;
+            if (c * 1024u + lane * 16u < row_bytes)
+                lds_load16(wbase + (size_t)r * full_row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
+            ++issued;
+        }
     }
     if (lane < 4u) reinterpret_cast<uint32_t*>(slot + 1024u + kAuxBytes)[lane] = 0u;
 
@@ -263,8 +289,10 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
         }
     }
     stage(xv[0], slot, lane);   // the first block while the tile is on its way
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    if constexpr (!OWN) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
 
     // 4. multiply this wave's super-blocks
     const uint32_t n = lane & 15u, g = lane >> 4;
@@ -284,9 +312,13 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
             u32x4 xa[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) xa[u] = *reinterpret_cast<const u32x4*>(xlane + u * xstep);
+            if constexpr (OWN) {
+                // this block's loads have landed when only the later blocks' are outstanding
+                wait_vmcnt(issued - (uint32_t)(i + 1) * groups);
+            }
             if constexpr (TYPE == kQ4K) {
                 const float4 aux = *reinterpret_cast<const float4*>(auxp);
-                const uint8_t* const blk = wrow + b * kBlock;
+                const uint8_t* const blk = OWN ? tile + b * block_pitch + nc * kBlock : wrow + b * kBlock;
                 const uint4 hdr = *reinterpret_cast<const uint4*>(blk);
                 const uint4 qa = *reinterpret_cast<const uint4*>(blk + 16u + 32u * g);
                 const uint4 qb = *reinterpret_cast<const uint4*>(blk + 32u + 32u * g);
@@ -432,6 +464,12 @@ void gemv_stream_q4k(const StreamParams p) {
     gemv_stream_body<kQ4K, DT, WAVES, MAXB>(p);
 }
 
+template <int DT, int WAVES, int MAXB>
+__global__ __launch_bounds__(WAVES * kWave) __attribute__((amdgpu_waves_per_eu(6, 6)))
+void gemv_stream_q4k_own(const StreamParams p) {
+    gemv_stream_body<kQ4K, DT, WAVES, MAXB, true>(p);
+}
+
 // Q6_K rows are 46% longer: two workgroups share a compute unit, four waves per SIMD.
 template <int DT, int WAVES, int MAXB>
 __global__ __launch_bounds__(WAVES * kWave) void gemv_stream_q6k(const StreamParams p) {
@@ -506,6 +544,7 @@ const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPla
     p.nb = a.k / 256u;
     p.tile_rows = plan.tile_rows;
     p.row_stride = plan.row_stride;
+    p.tile_bytes = plan.tile_rows * plan.row_stride;
     p.x_dtype = a.x_dtype;
     p.y_dtype = a.y_dtype;
     p.segments = plan.segments;
@@ -534,6 +573,31 @@ const char* launch_gemv_stream(hipStream_t s, const GemvArgs& a, const StreamPla
     }
     const int shape = plan.seg_blocks <= 16u ? 0 : plan.seg_blocks <= 24u ? 1 : 2;
     const int format = a.ggml_type == kQ6K ? 1 : 0;
+    // Q4_K tiles of up to 14 rows (two load instructions per super-block): every wave loads what it
+    // multiplies and no workgroup barrier stands between the loads and the arithmetic.  Same box,
+    // 17408 x 5120: 12.15 against 13.2 us and 12.3 against 12.4 us on two boxes (f16 activations 12.1
+    // against 12.4); 5120 x 5120 6.5 either way.  Taller tiles need a third, nearly empty instruction
+    // per block and lose (4096 x 4096: 4.54 against 4.40 us, 18992 x 5120: 14.0 against 13.8).
+    const uint32_t own_bytes = plan.seg_blocks * plan.tile_rows * kQ4Bytes;
+    if (a.stream_own && format == 0 && plan.tile_rows * (kQ4Bytes / 16u) <= 128u && own_bytes <= 65536u) {
+        static const Kernel own_kernels[3][3] = {
+            {gemv_stream_q4k_own<FH_F32, 8, 2>, gemv_stream_q4k_own<FH_F32, 8, 3>, gemv_stream_q4k_own<FH_F32, 8, 6>},
+            {gemv_stream_q4k_own<FH_F16, 8, 2>, gemv_stream_q4k_own<FH_F16, 8, 3>, gemv_stream_q4k_own<FH_F16, 8, 6>},
+            {gemv_stream_q4k_own<FH_BF16, 8, 2>, gemv_stream_q4k_own<FH_BF16, 8, 3>, gemv_stream_q4k_own<FH_BF16, 8, 6>},
+        };
+        Kernel kernel = own_kernels[a.x_dtype][shape];
+        static bool once = false;
+        if (!once) {
+            for (const auto& row : own_kernels)
+                for (Kernel k : row)
+                    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            once = true;
+        }
+        p.tile_bytes = own_bytes;
+        const uint32_t lds = own_bytes + plan.waves * kSlotBytes + plan.waves * 64u;
+        hipLaunchKernelGGL(kernel, dim3(plan.tiles, plan.segments, a.m), dim3(plan.waves * kWave), lds, s, p);
+        return plan.segments > 1 ? "q4_k_gemv_ksplit" : "q4_k_gemv_factored";
+    }
     hipLaunchKernelGGL(kernels[format][a.x_dtype][shape], dim3(plan.tiles, plan.segments, a.m), dim3(plan.waves * kWave),
                        plan.lds_bytes, s, p);
     if (format == 1) return plan.segments > 1 ? "q6_k_gemv_ksplit" : "q6_k_gemv_factored";

@@ -173,6 +173,7 @@ struct GemvArgs {
     void* shared_y;
     // the streamed matrix-core kernel may take the launch (dense Q4_K or Q6_K, plain rows, rows that fit LDS)
     int stream;           // 0 never, 1 where it is the faster kernel, 2 wherever it can run
+    bool stream_own;      // the streamed Q4_K kernel's waves load their own super-blocks where tiles are <= 14 rows
     int cu_count;
     float* partials;      // scratch for K segments (gemv_plan says how much)
     uint32_t* counters;   // zeroed scratch, one word per (row tile, m)

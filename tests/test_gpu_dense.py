@@ -333,6 +333,14 @@ def test_streamed_gemv_matches_the_oracle(api, d, ggml, n, k, dtype):
         with fma_gemv(d):
             other = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
         assert rel_l2(out.tensor.to_f32(), other) <= 1e-5 and not np.array_equal(bits(out.tensor.to_f32()), bits(other))
+        # tiles of up to 14 rows are loaded block by block by the waves that multiply them, taller
+        # ones row by row by all waves: the same arithmetic either way
+        d.set_tuning("gemv_stream_own_loads", 0)
+        try:
+            by_rows = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+        finally:
+            d.set_tuning("gemv_stream_own_loads", 1)
+        assert np.array_equal(bits(by_rows), bits(out.tensor.to_f32()))
     d.set_tuning("gemv_stream", 1)
 
 

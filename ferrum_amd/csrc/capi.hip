@@ -365,7 +365,7 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
     } else if (k == "gemm_wide_shape") {
         ok = value >= 0 && value <= 2;
     } else if (k == "gemm_wide32_tile") {
-        ok = value == 0 || value == 12 || value == 14 || value == 15 || value == 24 || value == 25;
+        ok = value == 0 || value == 12 || value == 13 || value == 14 || value == 15 || value == 24 || value == 25;
     } else if (k == "gemm_wide_min_rows") {
         ok = value >= 1;
     } else if (k == "gemm_skinny_max_rows") {

@@ -1102,15 +1102,26 @@ struct Wide32Tile {
     double alone, pair_first, pair_all;
 };
 constexpr Wide32Tile kWide32Tiles[] = {
-    {1, 2, 49.0, 61.0, 71.0}, {1, 4, 64.0, 88.0, 108.0}, {1, 5, 79.0, 0.0, 0.0},
+    {1, 2, 49.0, 61.0, 71.0}, {1, 3, 58.6, 0.0, 0.0}, {1, 4, 64.0, 88.0, 108.0}, {1, 5, 79.0, 0.0, 0.0},
     {2, 4, 90.0, 0.0, 0.0},   {2, 5, 108.0, 0.0, 0.0},
 };
 // an eighth of a tile's time is its prologue and its stores, the rest goes with the length of a row
 inline double wide_row_length_factor(uint32_t k) { return 0.125 + 0.875 * (double)k / 5120.0; }
 
-WidePlan wide32_make(uint32_t m, uint32_t n, int rt, int nt) {
-    const uint32_t rows = 128u * (uint32_t)rt, cols = 32u * (uint32_t)nt;
-    return WidePlan{nt, cols, (m + rows - 1) / rows, (n + cols - 1) / cols, rt};
+// The 128 x 96 tile is there for one case: a few columns more than 64 per workgroup make one
+// workgroup per compute unit where 128 x 64 tiles would number a few more than the compute units and
+// the units with two set the time (17408 columns on 256 units: 68 columns each, 128 rows in 58.6 -
+// 60.9 against 61.1 us, 96 rows in 56.6 - 58.6 against 60.0 on two boxes; the same bits).  Its width is the fewest columns,
+// a multiple of four, that make at most `cus` workgroups; 0 tiles when that is not in 65 .. 96.
+WidePlan wide32_make(uint32_t m, uint32_t n, int rt, int nt, int cus = 256) {
+    const uint32_t rows = 128u * (uint32_t)rt, tiles_m = (m + rows - 1) / rows;
+    uint32_t cols = 32u * (uint32_t)nt;
+    if (nt == 3) {
+        const uint32_t per_row_tile = (uint32_t)cus / tiles_m;
+        cols = per_row_tile == 0 ? 0 : ((n + per_row_tile - 1) / per_row_tile + 3u) & ~3u;
+        if (cols <= 64u || cols > 96u) return WidePlan{3, 96, tiles_m, 0, rt};
+    }
+    return WidePlan{nt, cols, tiles_m, (n + cols - 1) / cols, rt};
 }
 
 double wide32_estimate(const Wide32Tile& t, uint64_t wgs, uint64_t cus) {
@@ -1136,7 +1147,7 @@ WidePlan wide32_plan(uint32_t m, uint32_t n, uint32_t k, int cus, double* estima
     WidePlan best{};
     double best_us = 1e300;
     for (const Wide32Tile& t : kWide32Tiles) {
-        const WidePlan p = wide32_make(m, n, t.rt, t.nt);
+        const WidePlan p = wide32_make(m, n, t.rt, t.nt, cus);
         const uint64_t wgs = (uint64_t)p.tiles_m * p.tiles_n;
         if (wgs * 2 < (uint64_t)cus) continue;
         const double us = wide32_estimate(t, wgs, (uint64_t)cus);
@@ -1203,7 +1214,8 @@ template <uint32_t TYPE, int DT>
 void launch_wide_nt(hipStream_t s, const GemmArgs& a, const WidePlan& plan, const WidePlan& p32) {
     if (p32.nt != 0) {
         if (p32.rt == 1) {
-            if (p32.nt == 2) launch_wide32<TYPE, DT, 2, 1>(s, a, p32);
+            if (p32.nt == 3) launch_wide32<TYPE, DT, 3, 1>(s, a, p32);
+            else if (p32.nt == 2) launch_wide32<TYPE, DT, 2, 1>(s, a, p32);
             else if (p32.nt == 5) launch_wide32<TYPE, DT, 5, 1>(s, a, p32);
             else launch_wide32<TYPE, DT, 4, 1>(s, a, p32);
         } else {
@@ -1241,7 +1253,8 @@ const char* launch_gemm(hipStream_t s, const GemmArgs& a) {
     double us32 = 1e300;
     if (a.wide_shape != 0 && a.m >= (uint32_t)a.wide_min_rows) {
         if (a.wide32_tile != 0) {
-            p32 = wide32_make(a.m, a.n, a.wide32_tile / 10, a.wide32_tile % 10);
+            p32 = wide32_make(a.m, a.n, a.wide32_tile / 10, a.wide32_tile % 10, a.cu_count);
+            if (p32.tiles_n == 0) p32 = wide32_make(a.m, a.n, 1, 4);   // no width of the 96-column tile fits this shape
             us32 = 0.0;
         } else {
             p32 = wide32_plan(a.m, a.n, a.k, a.cu_count, &us32);

@@ -650,8 +650,9 @@ def test_wide_gemm_on_the_32x32x16_instruction(api, d, ggml, dtype):
 
 @pytest.mark.parametrize("m", [80, 128, 200, 330, 512])
 def test_the_tile_picked_by_row_count_gives_the_bits_of_the_largest(api, d, m):
-    # 17000 columns at every row count that changes the tile (128 x 64 up to 128 rows, 128 x 160 up
-    # to 256, 128 x 128 up to 384, 256 x 160 beyond); the pick against the forced 256 x 160 tile.
+    # 17000 columns at every row count that changes the tile (128 x 68 of the 96-column tile up to
+    # 128 rows, 128 x 160 up to 256, 128 x 128 up to 384, 256 x 160 beyond); the pick and the forced
+    # 128 x 64 and 128 x 96 tiles against the forced 256 x 160 tile.
     n, k = 17000, 2816
     w = qm(api, d, Q4_K, n, k, synth.matrix(Q4_K, n, k, seed=173))
     x = synth.activations(m, k, seed=174, f16=True)
@@ -663,6 +664,9 @@ def test_the_tile_picked_by_row_count_gives_the_bits_of_the_largest(api, d, m):
         picked = d.project_quantized(xt, w, out_dtype=api.DType.F32)
         d.set_tuning("gemm_wide32_tile", 25)
         largest = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        for forced in (12, 13):
+            d.set_tuning("gemm_wide32_tile", forced)
+            assert np.array_equal(d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.raw(), largest.tensor.raw())
     finally:
         d.set_tuning("gemm_wide32_tile", tile)
         d.set_tuning("gemm_resident", resident)

@@ -368,20 +368,19 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
         names.append(dev.last_operation())
 
     best = min(run_graph(dev, enqueue, steps, 2)[1] for _ in range(2)) / steps
-    separate = None
-    if tokens == 1:
-        # one token: the same FFN through fh_moe_ffn, which adds the weighted sum inside
-        # the down projection's launch (three launches, the same bits); the four separate calls
-        # of SparseMoe.forward are reported beside it
-        out = api.Tensor.zeros(dev, (tokens, hidden), f16)
+    # The same FFN through fh_moe_ffn (the same bits).  For one token it routes inside the gate|up
+    # launch and adds the weighted sum inside the down projection's (two launches); for many it groups
+    # the records by expert once for both projections.  The separate calls of SparseMoe.forward are
+    # reported beside it.
+    out = api.Tensor.zeros(dev, (tokens, hidden), f16)
 
-        def enqueue_one(i):
-            moe.forward_in_one_call(x, logit_sets[i % variants], out=out)
+    def enqueue_one(i):
+        moe.forward_in_one_call(x, logit_sets[i % variants], out=out)
 
-        enqueue_one(0)
-        dev.synchronize()
-        separate = best
-        best = min(run_graph(dev, enqueue_one, steps, 2)[1] for _ in range(2)) / steps
+    enqueue_one(0)
+    dev.synchronize()
+    separate = best
+    best = min(run_graph(dev, enqueue_one, steps, 2)[1] for _ in range(2)) / steps
     per_expert = (2 * inter * hidden + hidden * inter) // 256 * BLOCK_BYTES[Q4_K]
     mean_hit = float(np.mean(hit))
     act_bytes = tokens * hidden * 2 * 2 + tokens * experts * 4
@@ -419,11 +418,11 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
         "cpu_baseline": cpu_line,
         "workload": f"Q4_K MoE FFN T={tokens} hidden=2048 experts=256 top-8 + shared expert, f16 x",
         "operation": ("fh_moe_ffn: (moe_route + expert_project with the shared expert riding) + (expert_project + combine)"
-                      if separate is not None else
-                      "moe_route + 2 x (expert_project with the shared expert riding) + combine" if tokens * top_k <= 31
-                      else "moe_route + 2 x (expert_project grouped, shared expert pieces inside) + 2 x silu_mul + combine"),
+                      if tokens * top_k <= 31 else
+                      "fh_moe_ffn: moe_route + expert_group + 2 x (expert_project grouped, shared expert pieces inside) "
+                      "+ silu_mul + combine"),
         "us": round(best * 1e6, 2),
-        "us_as_separate_calls": round(separate * 1e6, 2) if separate is not None else None,
+        "us_as_separate_calls": round(separate * 1e6, 2),
         "GB/s": round(nbytes / best / 1e9, 1),
         "frac_hbm": round(nbytes / best / 1e9 / HBM_PEAK_GBS, 4),
         "TFLOP/s": round(flops / best / 1e12, 2),

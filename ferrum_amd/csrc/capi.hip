@@ -1309,7 +1309,10 @@ namespace {
 
 fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_view* x, uint32_t x_rows,
                          uint32_t form, uint32_t assignments, const fh_view* metadata, const fh_view* y,
-                         const SharedExpert* shared = nullptr, const RouteTokenArgs* route = nullptr) {
+                         const SharedExpert* shared = nullptr, const RouteTokenArgs* route = nullptr,
+                         bool grouped_before = false) {
+    // grouped_before: the grouped form finds offsets and order of these very records (all ids valid)
+    // at the head of the scratch, left there by the call before; the scratch must not grow in between
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (form > FH_INPUT_SILU_MUL) return fail(FH_ERR_PARAMETER, "unknown input form %u", form);
     if (shared != nullptr && form == FH_INPUT_ROWS)
@@ -1442,9 +1445,10 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
             }
             tile_x = rows_x;
         }
-        launch_expert_group(device->stream, reinterpret_cast<const float*>(mr.begin), assignments,
-                            (uint32_t)weight->experts, offsets, order, const_cast<uint8_t*>(yr.begin),
-                            (uint32_t)(rows * dtype_bytes(y->dtype)));
+        if (!grouped_before)
+            launch_expert_group(device->stream, reinterpret_cast<const float*>(mr.begin), assignments,
+                                (uint32_t)weight->experts, offsets, order, const_cast<uint8_t*>(yr.begin),
+                                (uint32_t)(rows * dtype_bytes(y->dtype)));
         GemmArgs g{};
         g.ggml_type = weight->ggml_type;
         g.w = weight->ptr;
@@ -1755,18 +1759,38 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
             FH_HIP(hipGetLastError());
             continue;
         }
-        if (shared && rides && fused) {
-            st = fh_expert_project_with_shared(device, input_experts, shared_input, &x, count, FH_INPUT_GATHER, a, &meta,
-                                               nullptr, &projected, &sproj);
+        // Both projections of a chunk group the same records by expert: the second finds the first's
+        // offsets and order at the head of the scratch (the router's ids are all valid, and the scratch
+        // is brought to the larger call's size before the first, so it does not move in between).
+        const int64_t group_from = tuning(device, "expert_grouped_min_assignments");
+        const bool regroup_once = fused && dt != FH_F32 && group_from > 0 && a >= (uint64_t)group_from && e <= 1024 &&
+                                  (!shared || rides);
+        if (regroup_once) {
+            const size_t words = ((size_t)e + 1 + a + 3) & ~(size_t)3;
+            const size_t widest = std::max<size_t>(h, inter);
+            st = ensure_scratch(device, words * sizeof(uint32_t) + ((size_t)a + count) * widest * sizeof(uint16_t));
             if (st != FH_OK) return st;
-            st = fh_expert_project_with_shared(device, output_experts, shared_output, &projected, count,
-                                               FH_INPUT_SILU_MUL, a, &meta, &sproj, &expert_out, &sout);
+        }
+        if (shared && rides && fused) {
+            SharedExpert in_rider, out_rider;
+            in_rider.weight = shared_input;
+            in_rider.tokens = count;
+            in_rider.y = &sproj;
+            out_rider.weight = shared_output;
+            out_rider.tokens = count;
+            out_rider.x = &sproj;
+            out_rider.y = &sout;
+            st = expert_project(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected, &in_rider);
+            if (st != FH_OK) return st;
+            st = expert_project(device, output_experts, &projected, count, FH_INPUT_SILU_MUL, a, &meta, &expert_out,
+                                &out_rider, nullptr, regroup_once);
             if (st != FH_OK) return st;
         } else {
             if (fused) {
-                st = fh_expert_project_fused(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected);
+                st = expert_project(device, input_experts, &x, count, FH_INPUT_GATHER, a, &meta, &projected);
                 if (st != FH_OK) return st;
-                st = fh_expert_project_fused(device, output_experts, &projected, a, FH_INPUT_SILU_MUL, a, &meta, &expert_out);
+                st = expert_project(device, output_experts, &projected, a, FH_INPUT_SILU_MUL, a, &meta, &expert_out,
+                                    nullptr, nullptr, regroup_once);
                 if (st != FH_OK) return st;
             } else {
                 st = fh_expert_assign(device, &x, count, (uint32_t)h, &meta, k, &assigned);

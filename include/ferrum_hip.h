@@ -423,7 +423,8 @@ fh_status fh_expert_combine(fh_device* device, const fh_view* in, const fh_view*
  * expert_silu_mul folded into the projections and the shared expert riding in the routed launches
  * where fh_expert_project_with_shared allows, so the result has their bits (a single token's
  * weighted sum is added inside the down projection's launch, and its routing inside the gate|up
- * launch: the same arithmetic in two launches).  Tokens are taken in
+ * launch: the same arithmetic in two launches; many tokens' records are grouped by expert once for
+ * both projections).  Tokens are taken in
  * chunks whose routing temporaries stay under the tuning value moe_routing_temporary_limit
  * (src/nn/moe.rs:232-256); the temporaries live in a workspace the library keeps per device,
  * which grows outside recordings only (run the call once before recording it). */

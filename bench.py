@@ -102,7 +102,7 @@ class Case:
         self.ggml, self.n, self.k, self.m, self.label = ggml, n, k, m, label
         wbytes = n * (k // 256) * BLOCK_BYTES[ggml]
         if copies is None:
-            copies = max(2, min(24, -(-ROTATE_BYTES // wbytes)))
+            copies = max(2, -(-ROTATE_BYTES // wbytes))
         base = synth.matrix(ggml, n, k, seed=1).reshape(n, -1)
         self.packed = base
         fmt = api.QuantizationFormat.from_ggml_type(ggml)
@@ -177,6 +177,7 @@ def report(case, seconds_per_step):
         "TFLOP/s": round(tf, 2),
         "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
         "weight_copies": len(case.weights),
+        "rotated_bytes": len(case.weights) * case.weight_bytes,
     }
 
 
@@ -353,14 +354,18 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
     moe.workspace(tokens, f16)
     x_host = synth.activations(tokens, hidden, seed=15, f16=True) * np.float32(2.0 ** -6)
     x = api.Tensor.from_f32(dev, (tokens, hidden), f16, x_host)
-    variants = 16
-    logit_sets, hit, first_logits = [], [], None
+    # distinct experts hit over one rotation of the logit sets: all 256 (453 MB) at 512 tokens; for one token
+    # 96 sets reach about 95% of them (~430 MB), more than the 256 MB last-level cache
+    variants = 16 if tokens >= 64 else 96
+    logit_sets, hit, first_logits, touched = [], [], None, set()
     for i in range(variants):
         values = synth.rng(16, i).standard_normal((tokens, experts)).astype(np.float32)
         if first_logits is None:
             first_logits = values
         logit_sets.append(api.Tensor.from_f32(dev, values.shape, f32, values))
-        hit.append(len(np.unique(np.argsort(-values, axis=1)[:, :top_k])))
+        chosen = np.unique(np.argsort(-values, axis=1)[:, :top_k])
+        hit.append(len(chosen))
+        touched.update(int(e) for e in chosen)
     names = []
 
     def enqueue(i):
@@ -429,6 +434,8 @@ def moe_case(api, synth, dev, tokens, steps, cpu=True):
         "frac_mfma_f16": round(flops / best / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
         "experts_hit_mean": mean_hit,
         "algorithmic_bytes": int(nbytes),
+        "rotated_bytes": int((len(touched) + 1) * per_expert),
+        "logit_sets": variants,
     }
 
 
@@ -452,27 +459,44 @@ def copy_calibration(api, dev, rows=65536, width=1024, launches=10):
                       "copied_correctly": bool(same)}), flush=True)
 
 
+READ_FORMS = (0, 25604, 25616, 51204, 51208, 102404, 102408, 1025608, 1025616, 1051208)
+
+
 def read_probe_case(api, synth, dev, steps, warmup):
-    """The headline's rotating matrices read by a kernel that only loads them."""
+    """A kernel that only loads the rotating matrices: (1) every launch shape of the probe on the
+    headline's matrices, the best of which is the ceiling a streaming kernel of that size has;
+    (2) that shape and the GEMV, back to back, on every GEMV shape of the benchmark."""
     head = Case(api, synth, dev, Q4_K, 17408, 5120, 1, api.DType.F32, "plain 128-bit read of the 17408x5120 Q4_K matrices")
     head.enqueue = lambda i: dev.probe_read(head.weights[i % len(head.weights)])
-    _, event = measure(dev, head, steps, warmup)
-    per = event / steps
-    gemv = Case.__new__(Case)
-    gemv.__dict__.update(head.__dict__)
-    gemv.label = "Q4_K GEMV M=1 K=5120 N=17408 f32 x"
-    gemv.enqueue = lambda i: dev.project_quantized(gemv.x, gemv.weights[i % len(gemv.weights)], out=gemv.y)
-    _, gevent = measure(dev, gemv, steps, warmup)
-    gper = gevent / steps
-    print(json.dumps({
-        "read_probe": {"kernel": head.operation, "bytes_per_launch": head.weight_bytes, "us": round(per * 1e6, 3),
-                       "GB/s": round(head.weight_bytes / per / 1e9, 1),
-                       "frac_hbm": round(head.weight_bytes / per / 1e9 / HBM_PEAK_GBS, 4)},
-        "gemv_same_run": {"kernel": gemv.operation, "us": round(gper * 1e6, 3),
-                          "GB/s": round(gemv.bytes / gper / 1e9, 1),
-                          "frac_hbm": round(gemv.bytes / gper / 1e9 / HBM_PEAK_GBS, 4)},
-        "gemv_over_read": round(gper / per, 3),
-        "weight_copies_rotated": len(head.weights), "steps": steps}), flush=True)
+    sweep = {}
+    for form in READ_FORMS:
+        dev.set_tuning("probe_read_form", form)
+        _, event = measure(dev, head, steps, warmup)
+        sweep[head.operation] = round(event / steps * 1e6, 3)
+    best_name = min(sweep, key=sweep.get)
+    best_form = READ_FORMS[list(sweep).index(best_name)]
+    dev.set_tuning("probe_read_form", best_form)
+    rows = []
+    shapes = ((Q4_K, 4096, 4096), (Q4_K, 5120, 5120), (Q4_K, 17408, 5120), (Q4_K, 5120, 17408),
+              (Q6_K, 5120, 17408), (Q6_K, 151936, 5120))
+    for ggml, n, k in shapes:
+        name = "Q4_K" if ggml == Q4_K else "Q6_K"
+        case = head if (ggml, n, k) == (Q4_K, 17408, 5120) else Case(
+            api, synth, dev, ggml, n, k, 1, api.DType.F32, f"{name} GEMV M=1 K={k} N={n} f32 x")
+        case.enqueue = lambda i, c=case: dev.probe_read(c.weights[i % len(c.weights)])
+        _, event = measure(dev, case, steps, warmup)
+        per, probe_kernel = event / steps, case.operation
+        case.enqueue = lambda i, c=case: dev.project_quantized(c.x, c.weights[i % len(c.weights)], out=c.y)
+        _, gevent = measure(dev, case, steps, warmup)
+        gper = gevent / steps
+        rows.append({
+            "shape": f"{name} N={n} K={k}", "weight_bytes": case.weight_bytes, "rotated_bytes": len(case.weights) * case.weight_bytes,
+            "read_probe_us": round(per * 1e6, 3), "read_probe_frac_hbm": round(case.weight_bytes / per / 1e9 / HBM_PEAK_GBS, 4),
+            "gemv_kernel": case.operation, "gemv_us": round(gper * 1e6, 3),
+            "gemv_frac_hbm": round(case.bytes / gper / 1e9 / HBM_PEAK_GBS, 4), "gemv_over_read": round(gper / per, 3)})
+        del case
+    print(json.dumps({"read_probe_forms_on_17408x5120_q4k_us": sweep, "best_form": best_name, "probe_kernel": probe_kernel,
+                      "per_shape": rows, "steps": steps}), flush=True)
 
 
 def mfma_probe_case(dev, steps):
@@ -481,7 +505,8 @@ def mfma_probe_case(dev, steps):
     cus = int(dev.properties().get("compute_units") or 256)
     iterations = 4096
     out = {}
-    for shape, name in ((0, "v_mfma_f32_16x16x32_f16"), (1, "v_mfma_f32_32x32x16_f16")):
+    for shape, name in ((0, "v_mfma_f32_16x16x32_f16"), (1, "v_mfma_f32_32x32x16_f16"),
+                        (2, "v_mfma_f32_32x32x16_f16 on random f16 operands")):
         for waves in (1, 4):
             flops = [0.0]
 

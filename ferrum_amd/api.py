@@ -655,7 +655,8 @@ class Device:
 
     def probe_mfma(self, shape: int, groups: int, iterations: int) -> float:
         """fh_probe_mfma: an MFMA issue loop from registers (shape 0 = 16x16x32 f16,
-        1 = 32x32x16 f16); returns the floating-point operations of the launch."""
+        1 = 32x32x16 f16, 2 = 32x32x16 f16 on pseudo-random operands); returns the
+        floating-point operations of the launch."""
         flops = ctypes.c_double()
         _check(_lib.fh_probe_mfma(self._handle, shape, groups, iterations, ctypes.byref(flops)))
         return float(flops.value)

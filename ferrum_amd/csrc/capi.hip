@@ -261,6 +261,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["gemv_stream"] = 1;           // dense Q4_K / Q6_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
+    d->tuning["probe_read_form"] = 0;       // fh_probe_read: 100 x threads per workgroup + loads per lane (+ 1000000: LDS-direct loads); 0 = 256 x 8
     fh_status st = ensure_scratch(d, 0);
     if (st == FH_OK) {
         // this device's address of the fixed scratch (the device is current), counters at zero
@@ -374,6 +375,9 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 0;
     } else if (k == "gemm_f32_min_rows") {
         ok = value == 0 || value >= 2;
+    } else if (k == "probe_read_form") {
+        ok = value == 0 || value == 25604 || value == 25608 || value == 25616 || value == 51204 || value == 51208 ||
+             value == 102404 || value == 102408 || value == 1025608 || value == 1025616 || value == 1051208;
     } else if (k == "moe_routing_temporary_limit") {
         // set_moe_routing_temporary_limit (src/metal/legacy.rs:523-531): positive, on an idle device
         ok = value > 0 && !device->capturing;
@@ -772,15 +776,15 @@ fh_status fh_probe_read(fh_device* device, const fh_qmatrix* weight) {
     fh_status st = ensure_scratch(device, 0);
     if (st != FH_OK) return st;
     device->last_operation = launch_read_probe(device->stream, weight->ptr, weight->bytes,
-                                               reinterpret_cast<uint32_t*>(scratch_data(device)));
+                                               reinterpret_cast<uint32_t*>(scratch_data(device)), tuning(device, "probe_read_form"));
     FH_HIP(hipGetLastError());
     return FH_OK;
 }
 
 fh_status fh_probe_mfma(fh_device* device, uint32_t shape, uint32_t groups, uint32_t iterations, double* flops) {
     if (device == nullptr || flops == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
-    if (shape > 1 || groups == 0 || groups > 65535 || iterations == 0)
-        return fail(FH_ERR_SHAPE, "mfma probe: shape 0 or 1, 1..65535 workgroups, at least one iteration");
+    if (shape > 2 || groups == 0 || groups > 65535 || iterations == 0)
+        return fail(FH_ERR_SHAPE, "mfma probe: shape 0, 1 or 2, 1..65535 workgroups, at least one iteration");
     fh_status st = ensure_scratch(device, (size_t)groups * 256 * sizeof(float));
     if (st != FH_OK) return st;
     device->last_operation = launch_mfma_probe(device->stream, (int)shape, groups, iterations,

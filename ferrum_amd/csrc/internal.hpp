@@ -12,6 +12,7 @@
 #include <string>
 
 #include "../../include/ferrum_hip.h"
+#include "../../include/ferrum_hip_probe.h"
 
 struct fh_device {
     // The device object lives until fh_device_destroy has been called and the last buffer,
@@ -109,7 +110,7 @@ const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const voi
                                     uint32_t out_dtype);
 
 // probe.hip: measurement kernels (a plain 128-bit read of a buffer; an MFMA issue loop)
-const char* launch_read_probe(hipStream_t s, const void* data, size_t bytes, uint32_t* sink);
+const char* launch_read_probe(hipStream_t s, const void* data, size_t bytes, uint32_t* sink, int64_t form);
 const char* launch_mfma_probe(hipStream_t s, int shape, uint32_t groups, uint32_t iterations, float* sink,
                               double* flops);
 const char* launch_coissue_probe(hipStream_t s, uint32_t groups, uint32_t iterations, uint32_t mfma,

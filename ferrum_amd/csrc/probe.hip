@@ -7,7 +7,9 @@
 //  * mfma_probe: every wave issues `iterations` rounds of eight independent MFMA
 //    chains on register operands and stores one float at the end.  Its rate is what the
 //    matrix cores sustain for one instruction shape, the figure a tile GEMM is read
-//    against.
+//    against.  With RANDOM set the operands are pseudo-random f16 values instead of small
+//    integers: the matrix cores then draw more power and, with every compute unit
+//    multiplying, the chip lowers its clock.
 //  * coissue_probe: workgroups of eight waves, two per SIMD.  Waves 0..3 issue
 //    v_mfma_f32_32x32x16_f16 (when `mfma` is set), waves 4..7 issue rounds of eight
 //    independent v_fma_f32 (when `valu_rounds` is not zero).  Timed alone and
@@ -21,22 +23,40 @@
 namespace fh {
 namespace {
 
-constexpr int kReadUnroll = 8;
-
-__global__ __launch_bounds__(256) void read_probe(const uint4* __restrict__ p, size_t n16,
-                                                  uint32_t* __restrict__ sink) {
-    const size_t base = (size_t)blockIdx.x * 256 * kReadUnroll + threadIdx.x;
-    uint4 v[kReadUnroll];
+// THREADS per workgroup, UNROLL 128-bit loads per lane (a wave's loads of one round are contiguous);
+// DIRECT: the loads go to LDS (LDS-direct, no register written) instead of registers.
+template <int THREADS, int UNROLL, bool DIRECT>
+__global__ __launch_bounds__(THREADS) void read_probe(const uint4* __restrict__ p, size_t n16,
+                                                      uint32_t* __restrict__ sink) {
+    const size_t base = (size_t)blockIdx.x * THREADS * UNROLL + threadIdx.x;
+    if constexpr (DIRECT) {
+        // every wave has UNROLL KB of LDS of its own; lanes past the end re-read the last 16 bytes
+        extern __shared__ __attribute__((aligned(16))) uint8_t probe_lds[];
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
-    for (int i = 0; i < kReadUnroll; ++i) {
-        const size_t idx = base + (size_t)i * 256;
-        v[i] = idx < n16 ? p[idx] : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < UNROLL; ++i) {
+            const size_t idx = base + (size_t)i * THREADS;
+            const uint4* src = p + (idx < n16 ? idx : n16 - 1);
+            const uint32_t at = (wave * UNROLL + i) * 1024u;
+            // M0 carries the LDS address of an LDS-direct load; nothing else in this kernel uses M0
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(at) : "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const uint32_t a = *reinterpret_cast<const uint32_t*>(probe_lds + threadIdx.x * 16u);
+        if (a == 0x9e3779b9u && p[0].x == 0x12345678u) sink[0] = a;
+    } else {
+        uint4 v[UNROLL];
+#pragma unroll
+        for (int i = 0; i < UNROLL; ++i) {
+            const size_t idx = base + (size_t)i * THREADS;
+            v[i] = idx < n16 ? p[idx] : make_uint4(0, 0, 0, 0);
+        }
+        uint32_t a = 0;
+#pragma unroll
+        for (int i = 0; i < UNROLL; ++i) a ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+        // the store keeps the loads alive; one lane in 2^32 takes it on random data, into scratch
+        if (a == 0x9e3779b9u) sink[0] = a;
     }
-    uint32_t a = 0;
-#pragma unroll
-    for (int i = 0; i < kReadUnroll; ++i) a ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
-    // the store keeps the loads alive; one lane in 2^32 takes it on random data, into scratch
-    if (a == 0x9e3779b9u) sink[0] = a;
 }
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -46,13 +66,27 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 constexpr int kChains = 8;
 
 // SHAPE 0: v_mfma_f32_16x16x32_f16 (16384 flop), SHAPE 1: v_mfma_f32_32x32x16_f16 (32768 flop)
-template <int SHAPE>
+template <int SHAPE, bool RANDOM = false>
 __global__ __launch_bounds__(256) void mfma_probe(uint32_t iterations, float seed, float* __restrict__ sink) {
     half8 a, b;
+    if constexpr (RANDOM) {
+        // sign and mantissa from a linear congruential sequence per lane, exponent 0.5 .. 2
+        uint32_t h = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+        uint32_t w[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        a[i] = (_Float16)(seed * (float)((threadIdx.x + i) & 7));
-        b[i] = (_Float16)(seed * (float)((threadIdx.x * 3 + i) & 7));
+        for (int i = 0; i < 8; ++i) {
+            h = h * 1664525u + 1013904223u;
+            w[i] = (h & 0x83ff83ffu) | (((h >> 10) & 1u) ? 0x3c003c00u : 0x38003800u);
+        }
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        a = __builtin_bit_cast(half8, u32x4{w[0], w[1], w[2], w[3]});
+        b = __builtin_bit_cast(half8, u32x4{w[4], w[5], w[6], w[7]});
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = (_Float16)(seed * (float)((threadIdx.x + i) & 7));
+            b[i] = (_Float16)(seed * (float)((threadIdx.x * 3 + i) & 7));
+        }
     }
     float total = 0.0f;
     if constexpr (SHAPE == 0) {
@@ -136,12 +170,29 @@ const char* launch_coissue_probe(hipStream_t stream, uint32_t groups, uint32_t i
     return mfma != 0 && valu_rounds != 0 ? "coissue_probe_mfma_and_valu" : mfma != 0 ? "coissue_probe_mfma" : "coissue_probe_valu";
 }
 
-const char* launch_read_probe(hipStream_t stream, const void* data, size_t bytes, uint32_t* sink) {
-    const size_t n16 = bytes / 16;
-    const size_t per_group = (size_t)256 * kReadUnroll;
+template <int THREADS, int UNROLL, bool DIRECT>
+void launch_read_form(hipStream_t stream, const void* data, size_t n16, uint32_t* sink) {
+    const size_t per_group = (size_t)THREADS * UNROLL;
     const unsigned groups = (unsigned)((n16 + per_group - 1) / per_group);
-    read_probe<<<dim3(groups), dim3(256), 0, stream>>>(static_cast<const uint4*>(data), n16, sink);
-    return "read_probe";
+    const size_t lds = DIRECT ? (size_t)(THREADS / 64) * UNROLL * 1024 : 0;
+    read_probe<THREADS, UNROLL, DIRECT><<<dim3(groups), dim3(THREADS), lds, stream>>>(static_cast<const uint4*>(data), n16, sink);
+}
+
+// form = 100 x threads per workgroup + loads per lane, + 1000000 for LDS-direct loads; 0 = 256 threads x 8 loads
+const char* launch_read_probe(hipStream_t stream, const void* data, size_t bytes, uint32_t* sink, int64_t form) {
+    const size_t n16 = bytes / 16;
+    switch (form) {
+        case 25604: launch_read_form<256, 4, false>(stream, data, n16, sink); return "read_probe_256x4";
+        case 25616: launch_read_form<256, 16, false>(stream, data, n16, sink); return "read_probe_256x16";
+        case 51204: launch_read_form<512, 4, false>(stream, data, n16, sink); return "read_probe_512x4";
+        case 51208: launch_read_form<512, 8, false>(stream, data, n16, sink); return "read_probe_512x8";
+        case 102404: launch_read_form<1024, 4, false>(stream, data, n16, sink); return "read_probe_1024x4";
+        case 102408: launch_read_form<1024, 8, false>(stream, data, n16, sink); return "read_probe_1024x8";
+        case 1025608: launch_read_form<256, 8, true>(stream, data, n16, sink); return "read_probe_256x8_lds_direct";
+        case 1025616: launch_read_form<256, 16, true>(stream, data, n16, sink); return "read_probe_256x16_lds_direct";
+        case 1051208: launch_read_form<512, 8, true>(stream, data, n16, sink); return "read_probe_512x8_lds_direct";
+        default: launch_read_form<256, 8, false>(stream, data, n16, sink); return "read_probe";
+    }
 }
 
 const char* launch_mfma_probe(hipStream_t stream, int shape, uint32_t groups, uint32_t iterations,
@@ -151,6 +202,10 @@ const char* launch_mfma_probe(hipStream_t stream, int shape, uint32_t groups, ui
     if (shape == 0) {
         mfma_probe<0><<<dim3(groups), dim3(256), 0, stream>>>(iterations, 0x1p-10f, sink);
         return "mfma_probe_16x16x32_f16";
+    }
+    if (shape == 2) {
+        mfma_probe<1, true><<<dim3(groups), dim3(256), 0, stream>>>(iterations, 0x1p-10f, sink);
+        return "mfma_probe_32x32x16_f16_random_operands";
     }
     mfma_probe<1><<<dim3(groups), dim3(256), 0, stream>>>(iterations, 0x1p-10f, sink);
     return "mfma_probe_32x32x16_f16";

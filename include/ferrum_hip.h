@@ -186,23 +186,6 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
 fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* weight,
                                         const fh_view* x, uint32_t m, const fh_view* y);
 
-/* Measurement kernels with no counterpart in the reference; the benchmark launches them
- * to show what the device delivers with no operator attached.  fh_probe_read reads every
- * byte of a resident matrix with 128-bit loads and writes nothing: the HBM rate a
- * streaming kernel is compared with.  fh_probe_mfma runs `groups` workgroups of four
- * waves, each wave issuing `iterations` rounds of eight independent
- * v_mfma_f32_16x16x32_f16 (shape 0) or v_mfma_f32_32x32x16_f16 (shape 1) from registers;
- * *flops receives the floating-point operations of the launch.  fh_probe_coissue runs
- * `groups` workgroups of eight waves, two per SIMD: waves 0..3 issue `iterations` x 8
- * v_mfma_f32_32x32x16_f16 when `mfma` is set, waves 4..7 `iterations` x `valu_rounds` x 8
- * v_fma_f32 when `valu_rounds` is not zero; timing the three combinations shows whether the
- * two kinds of arithmetic overlap on a SIMD. */
-fh_status fh_probe_read(fh_device* device, const fh_qmatrix* weight);
-fh_status fh_probe_mfma(fh_device* device, uint32_t shape, uint32_t groups, uint32_t iterations,
-                        double* flops);
-fh_status fh_probe_coissue(fh_device* device, uint32_t groups, uint32_t iterations, uint32_t mfma,
-                           uint32_t valu_rounds);
-
 /* MetalDevice::argmax_rows (src/ops/transformer.rs:768-792, kernel
  * src/metal/shaders/ops.metal:2438-2464): greedy selection over the rows of a
  * logits matrix, the step after the lm_head projection.  out is an f32 carrier

@@ -10,12 +10,19 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "ferrum_hip.h")
+# measurement kernels, declared apart from the operator surface
+PROBE_HEADER = os.path.join(ROOT, "include", "ferrum_hip_probe.h")
 
 
-def declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+def declared_symbols(path=None):
+    texts = [open(p).read() for p in ([path] if path else [HEADER, PROBE_HEADER])]
+    text = re.sub(r"/\*.*?\*/", "", "\n".join(texts), flags=re.S)
     return sorted(set(re.findall(r"\b(fh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_measurement_kernels_stay_out_of_the_operator_header():
+    assert not [n for n in declared_symbols(HEADER) if n.startswith("fh_probe_")]
+    assert declared_symbols(PROBE_HEADER) == ["fh_probe_coissue", "fh_probe_mfma", "fh_probe_read"]
 
 
 def test_library_exports_every_declared_symbol():

@@ -391,6 +391,11 @@ def test_a3b_ffn_as_benchmarked_with_256_distinct_experts(api, d, tokens):
     assert rel_l2(got, want) <= 3e-3
     per_token = np.linalg.norm(got - want, axis=1) / np.linalg.norm(want, axis=1)
     assert per_token.max() <= 1e-2, int(per_token.argmax())
+    # The call bench.py times at both token counts is the single-call form (fh_moe_ffn): the same bits as
+    # the separate calls, and so the same distance to the host statement.
+    fused = moe.forward_in_one_call(xt, api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)).to_f32()
+    assert np.array_equal(fused.view(np.uint32), got.view(np.uint32))
+    assert rel_l2(fused, want) <= 3e-3
 
 
 # ------------------------------------------------------- decode-sized fusions

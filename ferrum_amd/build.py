@@ -11,6 +11,8 @@ import shutil
 import subprocess
 import sys
 
+from . import isa_check
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
@@ -50,12 +52,42 @@ def _compile(src: str, extra: list[str]) -> str:
     return obj
 
 
+def _assembly(src: str, extra: list[str]) -> str:
+    """The device assembly hipcc writes for one of this library's sources, as text."""
+    out = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".s")
+    cmd = [hipcc(), *[f for f in FLAGS if f != "-fPIC"], *extra, "-S", "--offload-device-only",
+           os.path.join(CSRC, src), "-o", out]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed for {src}:\n{proc.stdout}\n{proc.stderr}")
+    with open(out) as f:
+        return f.read()
+
+
+def check_toolchain() -> str:
+    """The hipcc release in use; a release other than the validated one is reported on stderr
+    (the check of the generated code below and the GPU parity tests are then the gate)."""
+    proc = subprocess.run([hipcc(), "--version"], capture_output=True, text=True)
+    release = isa_check.hipcc_release(proc.stdout)
+    if release != isa_check.VALIDATED_HIPCC:
+        sys.stderr.write(f"ferrum_amd.build: hipcc {release or '(unknown)'} is not the release the hand-scheduled kernels "
+                         f"were validated with ({isa_check.VALIDATED_HIPCC}); run the GPU parity tests before use\n")
+    return release
+
+
 def build(extra_flags: list[str] | None = None, jobs: int = 8, output: str | None = None) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     extra = list(extra_flags or [])
+    check_toolchain()
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        # the sources with hand-scheduled loads are also compiled to assembly text, which is checked
+        # for what the compiler must not have done around those loads
+        texts = {s: pool.submit(_assembly, s, extra) for s in isa_check.CHECKED_SOURCES}
         objs = list(pool.map(lambda s: _compile(s, extra), SOURCES))
+        broken = [v for s, t in texts.items() for v in isa_check.violations(t.result(), s)]
+    if broken:
+        raise RuntimeError("the generated code breaks an invariant of the hand-scheduled loads:\n" + "\n".join(broken[:40]))
     target = output or LIB_PATH
     tmp = target + ".tmp"
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

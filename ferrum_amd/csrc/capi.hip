@@ -5,6 +5,7 @@
 // alignment and input/output aliasing are rejected before anything launches.
 #include <cmath>
 #include <cstdarg>
+#include <mutex>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -264,11 +265,21 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["probe_read_form"] = 0;       // fh_probe_read: 100 x threads per workgroup + loads per lane (+ 1000000: LDS-direct loads); 0 = 256 x 8
     fh_status st = ensure_scratch(d, 0);
     if (st == FH_OK) {
-        // this device's address of the fixed scratch (the device is current), counters at zero
+        // This device's address of the fixed scratch (the device is current).  Its counters are set to zero
+        // once per GPU and process: launches leave them at zero, and a second handle on a GPU whose first
+        // handle has a K-split launch in flight must not reset that launch's tickets.
         void* fixed = nullptr;
         e = hipGetSymbolAddress(&fixed, HIP_SYMBOL(scratch));
-        if (e == hipSuccess) e = hipMemsetAsync(fixed, 0, kFixedCounterWords * sizeof(uint32_t), d->stream);
-        if (e == hipSuccess) e = hipStreamSynchronize(d->stream);
+        if (e == hipSuccess) {
+            static std::mutex zero_lock;
+            static bool zeroed[256] = {};
+            std::lock_guard<std::mutex> hold(zero_lock);
+            if (ordinal < 256 && !zeroed[ordinal]) {
+                e = hipMemsetAsync(fixed, 0, kFixedCounterWords * sizeof(uint32_t), d->stream);
+                if (e == hipSuccess) e = hipStreamSynchronize(d->stream);
+                if (e == hipSuccess) zeroed[ordinal] = true;
+            }
+        }
         if (e != hipSuccess) st = hip_fail(e, "fixed scratch");
         d->fixed_scratch = fixed;
     }
@@ -874,7 +885,10 @@ fh_status route(fh_device* device, const fh_view* logits, uint32_t tokens, const
     if (!fits_u32((uint64_t)tokens * p.top_k * 3) || !fits_u32((uint64_t)tokens * p.experts))
         return fail(FH_ERR_SHAPE, "expert assignment count overflow");
     Range lr, mr, br{nullptr, 0};
-    fh_status st = resolve(device, logits, (uint64_t)tokens * p.experts, "router logits", &lr, 4);
+    // the kernel loads logits one element at a time: a chunk of 16-bit logits over an odd number of experts
+    // may start at any element
+    fh_status st = resolve(device, logits, (uint64_t)tokens * p.experts, "router logits", &lr,
+                           logits != nullptr ? dtype_bytes(logits->dtype) : 4);
     if (st != FH_OK) return st == FH_ERR_DEVICE_MISMATCH ? fail(FH_ERR_SHAPE, "invalid sparse routing geometry") : st;
     if (selection_bias != nullptr) {
         if (selection_bias->dtype != FH_F32) return fail(FH_ERR_SHAPE, "invalid sparse routing geometry");
@@ -1767,8 +1781,12 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         // offsets and order at the head of the scratch (the router's ids are all valid, and the scratch
         // is brought to the larger call's size before the first, so it does not move in between).
         const int64_t group_from = tuning(device, "expert_grouped_min_assignments");
+        // (With a shared expert whose rows do not fit LDS a projection runs the shared matrix as a dense call of its
+        // own after the grouping, and that call may put partial sums where the lists lie: both then group for themselves.)
+        const bool shared_stays_inside = !shared || (rides && expert_rows_fit_lds((uint32_t)h, a, (uint32_t)e) &&
+                                                     expert_rows_fit_lds((uint32_t)inter, a, (uint32_t)e));
         const bool regroup_once = fused && dt != FH_F32 && group_from > 0 && a >= (uint64_t)group_from && e <= 1024 &&
-                                  (!shared || rides);
+                                  shared_stays_inside;
         if (regroup_once) {
             const size_t words = ((size_t)e + 1 + a + 3) & ~(size_t)3;
             const size_t widest = std::max<size_t>(h, inter);

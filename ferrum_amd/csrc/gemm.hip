@@ -848,6 +848,12 @@ struct Wide32 {
 };
 
 // LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
+// The statement writes M0 without being able to declare it (M0 is refused in a clobber list):
+// sound while the compiler keeps nothing of its own in M0 in this kernel, which has no other
+// client of it.  The load returns no register and is covered only by the hand-placed
+// `s_waitcnt vmcnt(0)` statements of the main loop; those wait for everything, so loads of the
+// compiler's own in between cannot make them wrong.  The build checks the generated text for
+// the M0 rule and for scratch (ferrum_amd/isa_check.py).
 __device__ __forceinline__ void lds_direct16(const void* g, uint32_t lds_addr) {
     const uint32_t a = __builtin_amdgcn_readfirstlane(lds_addr);
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
@@ -1037,7 +1043,13 @@ __global__ __launch_bounds__(512) void gemm_wide32_kernel(const uint8_t* __restr
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the activations of slab c + 1 have landed
         __syncthreads();           // its weights are visible; slab c is in registers, its buffers are free
         __builtin_amdgcn_sched_barrier(0);
-        // past the end the last slab is loaded once more, into the stage nobody reads
+        // On the last pass (c + 2 == slabs) there is no further slab, and the clamp loads slab
+        // slabs - 1 a second time: into the stage it already occupies, the one this step and the
+        // tail below read.  The bytes written are the bytes already there, so the readers see
+        // the same values whichever copy they meet; the straight-line body stays one code path.
+        // This holds only while the clamp names the slab that stage holds: a deeper ring or
+        // another stage index must peel this pass and drop its loads instead.
+        static_assert(Geo::kRingBytes == 2 * Geo::kStageBytes, "the clamped reload below relies on a two-stage activation ring");
         step(f1, f0, c + 1, 0, yes, yes, c + 2 < slabs ? c + 2 : slabs - 1);
     }
     {

@@ -71,6 +71,15 @@ struct StreamParams {
 };
 
 // LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
+// The statement writes M0 (the instruction's LDS base) and cannot declare it: this target rejects
+// M0 in a clobber list.  It is sound as long as the compiler keeps no value of its own in M0 across
+// the statement, which holds for code that uses none of M0's other clients (s_movrel, GWS and
+// sendmsg operands, ds_*_addtid, lane-indexed v_readlane through M0): these kernels have none.
+// The load is counted in vmcnt like any vector-memory load and returns no register; the only wait
+// that covers it is the author's wait_vmcnt / s_waitcnt vmcnt below, so between such a load and
+// the wait that counts it there must be no vector-memory instruction of the compiler's.  The
+// build compiles this file to assembly text as well and checks all three facts there
+// (ferrum_amd/isa_check.py); it refuses to link a library that breaks one.
 __device__ __forceinline__ void lds_load16(const void* g, uint32_t lds_addr) {
     const uint32_t a = __builtin_amdgcn_readfirstlane(lds_addr);
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
@@ -220,7 +229,14 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     uint8_t* const slot = tile + p.tile_bytes + wave * kSlotBytes;
     float* const rsum = reinterpret_cast<float*>(tile + p.tile_bytes + kSWaves * kSlotBytes);
 
-    // 1. this wave's activation blocks are requested first
+    // 1. this wave's activation blocks are requested first.  These are register loads the
+    // compiler cannot see the latency of: xraw[i] holds the data only after wait_vmcnt(issued)
+    // under 3., which lets exactly the `issued` later LDS-direct loads stay in flight (vmcnt
+    // retires in order, so "at most `issued` outstanding" means every load before them is done).
+    // Until then nothing may read, copy or spill xraw: the empty asm with "+v"(xraw[i]) after the
+    // wait is the first use the compiler is shown, the kernel has no scratch, and the build's
+    // check of the generated text fails if any instruction between a load and the wait names a
+    // destination register.
     const size_t xrow = ((size_t)blockIdx.z * p.nb + first) * 256u;
     typename std::conditional<DT == FH_F32, u32x4, u32x2>::type xraw[MAXB];
 #pragma unroll

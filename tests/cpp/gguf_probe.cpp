@@ -2,12 +2,14 @@
 // line, for the CPU tests to compare with the Python reader; a rejected file
 // prints "error: <message>" and exits with 2.  argv[2], when given, is the
 // array-skipping limit; argv[3] == "untagged" drops the architecture rule.
+// "<file> plan qwen" and "<file> plan lfm2moe [nobias]" print the model-level binding of the
+// file's tensors instead (exit 3 for a rejection that is not of the Gguf kind).
 #include <cinttypes>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
-#include "ferrum_gguf.hpp"
+#include "ferrum_gguf_models.hpp"
 
 using namespace ferrum;
 
@@ -28,9 +30,35 @@ static void print(const gguf::MetadataValue& v) {
     }
 }
 
+static void print_plan(const gguf::models::ModelShape& m, const gguf::models::TensorPlan& plan) {
+    std::printf("shape %s vocab %zu hidden %zu heads %zu kv %zu head_dim %zu layers %zu tied %d bias %d qk_norm %d\n",
+                m.architecture.c_str(), m.vocab_size, m.hidden_size, m.num_attention_heads, m.num_key_value_heads,
+                m.head_dim, m.layers.size(), (int)m.tie_word_embeddings, (int)m.qkv_bias, (int)m.qk_norm);
+    for (const auto& b : plan.bindings) {
+        std::printf("bind %s <-", b.canonical.c_str());
+        for (const auto& source : b.sources) std::printf(" %s", source.c_str());
+        std::printf(" shape");
+        for (size_t d : b.shape) std::printf(" %zu", d);
+        std::printf(" kind %d type %u\n", (int)b.kind, b.type_id);
+    }
+    std::printf("totals %zu tensors %zu bytes %zu parameters redundant %d\n", plan.tensor_count, plan.source_tensor_bytes,
+                plan.parameter_count, (int)plan.redundant_output);
+}
+
 int main(int argc, char** argv) {
     if (argc < 2) return 64;
     try {
+        if (argc >= 4 && !std::strcmp(argv[2], "plan")) {
+            gguf::Reader file = gguf::Reader::open(argv[1]);
+            if (!std::strcmp(argv[3], "qwen")) {
+                const auto [shape, plan] = gguf::models::plan_qwen(file);
+                print_plan(shape, plan);
+            } else {
+                const auto shape = gguf::models::lfm2_moe_shape(file, !(argc > 4 && !std::strcmp(argv[4], "nobias")));
+                print_plan(shape, gguf::models::plan_lfm2_moe(file, shape));
+            }
+            return 0;
+        }
         if (argc == 5 && !std::strcmp(argv[2], "stack")) {   // <file> stack <gate> <up>: FNV-1a of the interleaved rows
             gguf::Reader file = gguf::Reader::open(argv[1]);
             const auto shape = file.tensor(argv[3]).logical_expert_shape();

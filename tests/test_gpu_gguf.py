@@ -112,3 +112,62 @@ def test_other_formats_load_from_a_gguf_file(tmp_path, ggml):
     assert (e.experts(), e.rows_per_expert(), e.columns()) == (experts, rows, k)
     assert np.array_equal(bits(d.dequantize(e.matrix_view()).to_f32()),
                           bits(oracle.dequantize(ggml, ex, experts * rows, k)))
+
+
+def test_a_whole_lfm2_moe_file_binds_by_canonical_name_and_runs_a_sparse_layer(tmp_path):
+    # the model-level adapter (src/model/lfm2_moe/gguf.rs:165-320, 434-574): every quantized tensor
+    # of the file lands on the device under its canonical name, blocks verbatim, gate and up
+    # experts interleaved; a sparse layer built from the bound matrices gives the host answer
+    import test_gguf_models as files
+    from ferrum_amd import api, gguf_models
+    d = api.Device.new()
+    tensors = files.lfm2_tensors()
+    path = tmp_path / "lfm2moe.gguf"
+    path.write_bytes(gf.build([(n, *v) for n, v in tensors.items()], files.lfm2_metadata()))
+    f = gguf.GgufReader.open(str(path))
+    plan = gguf_models.plan_lfm2_moe(f, gguf_models.lfm2_moe_shape(f))
+    weights, quantized_bytes = gguf_models.bind_quantized(d, f, plan)
+    assert sorted(weights) == sorted(b.canonical for b in plan.quantized())
+    assert quantized_bytes == sum(np.asarray(v[2]).nbytes for v in tensors.values() if v[1] != 0)
+    assert 0 < quantized_bytes <= plan.source_tensor_bytes
+    H, I, E = files.H, files.MOE_INTER, files.EXPERTS
+    q = weights["layers.1.q.weight"]
+    assert (q.rows(), q.columns(), q.format().value) == (files.HEADS * files.HD, H, Q4_K)
+    packed_q = np.asarray(tensors["blk.1.attn_q.weight"][2])
+    assert np.array_equal(bits(d.dequantize(q).to_f32()), bits(oracle.dequantize(Q4_K, packed_q, q.rows(), H)))
+    win, wout = weights["layers.2.moe.input.weight"], weights["layers.2.moe.output.weight"]
+    assert (win.experts(), win.rows_per_expert(), win.columns()) == (E, 2 * I, H)
+    assert (wout.experts(), wout.rows_per_expert(), wout.columns(), wout.format().value) == (E, H, I, Q6_K)
+    gate = np.asarray(tensors["blk.2.ffn_gate_exps.weight"][2])
+    up = np.asarray(tensors["blk.2.ffn_up_exps.weight"][2])
+    down = np.asarray(tensors["blk.2.ffn_down_exps.weight"][2])
+    row_bytes = H // 256 * 144
+    stacked = np.concatenate([gate.reshape(E, I, row_bytes), up.reshape(E, I, row_bytes)], axis=1).reshape(-1)
+    assert np.array_equal(bits(d.dequantize(win.matrix_view()).to_f32()), bits(oracle.dequantize(Q4_K, stacked, E * 2 * I, H)))
+    top_k, tokens = 2, 3
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(E, top_k))
+    rng = synth.rng(61)
+    x = (rng.standard_normal((tokens, H)) * 2.0 ** -5).astype(np.float32)
+    logits = rng.standard_normal((tokens, E)).astype(np.float32)
+    got = moe.forward(api.Tensor.from_f32(d, x.shape, api.DType.F32, x),
+                      api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)).to_f32()
+    m = oracle.select_routes(logits, E, top_k)
+    o_up = oracle.expert_project(Q4_K, stacked, E, 2 * I, H, oracle.expert_assign(x, m), m, accumulate="f64")
+    o_down = oracle.expert_project(Q6_K, down, E, H, I, oracle.expert_silu_mul(o_up, I), m, accumulate="f64")
+    want = oracle.expert_combine(o_down, m, tokens, H, top_k)
+    assert np.abs(want).max() > 1e-4
+    assert float(np.linalg.norm(got - want) / np.linalg.norm(want)) <= 2e-5
+    # a Qwen file the same way: only the listed types are uploaded when asked
+    qt = files.qwen_tensors("qwen3", tied=False)
+    path = tmp_path / "qwen3.gguf"
+    path.write_bytes(gf.build([(n, *v) for n, v in qt.items()], files.qwen_metadata("qwen3")))
+    f = gguf.GgufReader.open(str(path))
+    shape, plan = gguf_models.plan_qwen(f)
+    only_q6, _ = gguf_models.bind_quantized(d, f, plan, only=(Q6_K,))
+    assert sorted(only_q6) == sorted(["embedding.weight", "lm_head.weight"] + [f"layers.{l}.{n}.weight"
+                                                                              for l in range(shape.num_layers) for n in ("v", "down")])
+    head = only_q6["lm_head.weight"]
+    xr = synth.activations(1, files.H, seed=62)
+    got = d.project_quantized(api.Tensor.from_f32(d, xr.shape, api.DType.F32, xr), head).tensor.to_f32()
+    assert_matmul_parity(got, oracle.project(Q6_K, np.asarray(qt["output.weight"][2]), files.VOCAB, files.H, xr, accumulate="f64"),
+                         "lm_head bound by canonical name")

@@ -705,6 +705,71 @@ def test_the_ffn_in_one_call_gives_the_bits_of_the_separate_calls(api, d, dtype,
         moe.forward_in_one_call(xt, api.Tensor.zeros(d, (tokens, experts + 1), api.DType.F32))
 
 
+@pytest.mark.parametrize("logit_dtype", ["BF16", "F16"])
+def test_chunks_of_16_bit_logits_over_an_odd_number_of_experts(api, d, logit_dtype):
+    # three tokens a chunk over 7 experts: the second chunk's logits start 42 bytes in, a
+    # 2-byte boundary that is not a 4-byte one.  Both the chunked step-by-step pass and the
+    # chunked single call give the bits of the pass that was not cut.
+    experts, hidden, inter, top_k, tokens = 7, 512, 256, 2, 10
+    fmt = api.QuantizationFormat(Q4_K)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=311), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * hidden, inter, seed=312), fmt,
+                                         experts, hidden, inter)
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k))
+    x = synth.activations(tokens, hidden, seed=313, f16=True) * np.float32(2.0 ** -5)
+    logits = synth.rng(314).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
+    lt = api.Tensor.from_f32(d, logits.shape, getattr(api.DType, logit_dtype), logits)
+    whole = moe.forward(xt, lt)
+    assert np.abs(whole.to_f32()).max() > 1e-3
+    moe.take_stats()
+    before = d.moe_routing_temporary_limit()
+    try:
+        d.set_moe_routing_temporary_limit(3 * moe.temporary_bytes(1, xt.dtype))
+        cut = moe.forward(xt, lt)
+        assert moe.take_stats().peak_temporary_bytes == 3 * moe.temporary_bytes(1, xt.dtype)
+        cut_one_call = moe.forward_in_one_call(xt, lt)
+    finally:
+        d.set_moe_routing_temporary_limit(before)
+    # fewer than 32 assignments either way: every row comes from the per-assignment kernel
+    assert np.array_equal(cut.raw(), whole.raw())
+    assert np.array_equal(cut_one_call.raw(), whole.raw())
+
+
+@pytest.mark.parametrize("min_rows", [2, 1000])
+def test_one_call_ffn_when_the_shared_expert_runs_apart_from_a_grouped_projection(api, d, min_rows):
+    # 32 rows of 2816 halves do not fit the grouped kernel's LDS, so the shared expert's matrices
+    # run as dense calls of their own after each grouped projection (on the tile kernel, or on
+    # the per-row kernel under a high kernel-choice floor).  Those calls may use the scratch the
+    # grouping lists lie in: the second projection groups the records again, and the single call
+    # gives the bits of the separate calls.
+    experts, hidden, inter, top_k, tokens = 4, 2816, 2816, 2, 40
+    fmt = api.QuantizationFormat(Q4_K)
+    win = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * 2 * inter, hidden, seed=321), fmt,
+                                        experts, 2 * inter, hidden)
+    wout = api.QuantizedExpertMatrix.new(d, synth.matrix(Q4_K, experts * hidden, inter, seed=322), fmt,
+                                         experts, hidden, inter)
+    sin = api.QuantizedMatrix.from_bytes(d, 2 * inter, hidden, fmt, synth.matrix(Q4_K, 2 * inter, hidden, seed=323))
+    sout = api.QuantizedMatrix.from_bytes(d, hidden, inter, fmt, synth.matrix(Q4_K, hidden, inter, seed=324))
+    moe = api.SparseMoe(d, win, wout, api.MoeRoutingPolicy(experts, top_k), shared_input=sin, shared_output=sout)
+    x = synth.activations(tokens, hidden, seed=325, f16=True) * np.float32(2.0 ** -5)
+    logits = synth.rng(326).standard_normal((tokens, experts)).astype(np.float32)
+    xt = api.Tensor.from_f32(d, x.shape, api.DType.F16, x)
+    lt = api.Tensor.from_f32(d, logits.shape, api.DType.F32, logits)
+    before = d.get_tuning("gemm_min_rows")
+    d.set_tuning("gemm_min_rows", min_rows)
+    try:
+        want = moe.forward(xt, lt)
+        got = moe.forward_in_one_call(xt, lt)
+        again = moe.forward_in_one_call(xt, lt)
+    finally:
+        d.set_tuning("gemm_min_rows", before)
+    assert np.abs(want.to_f32()).max() > 1e-3
+    assert np.array_equal(got.raw(), want.raw())
+    assert np.array_equal(again.raw(), want.raw())
+
+
 @pytest.mark.parametrize("ggml,inter,top_k,tokens,shared,dtype", [
     (Q4_K, 512, 8, 1, True, "F16"), (Q4_K, 512, 8, 1, True, "BF16"), (Q4_K, 512, 8, 1, False, "F32"),
     (Q6_K, 768, 4, 1, True, "F16"), (Q6_K, 1024, 3, 1, False, "F16"), (synth.Q5_K, 1536, 2, 1, True, "F16"),

@@ -10,7 +10,7 @@
 #include <cstring>
 #include <vector>
 
-#include "ferrum_gguf.hpp"
+#include "ferrum_gguf_models.hpp"
 #include "ferrum_hip.hpp"
 
 extern "C" {
@@ -96,7 +96,8 @@ struct FileTensor {
     uint32_t type;
     const std::vector<uint8_t>* payload;
 };
-static std::string gguf_file(const std::vector<FileTensor>& tensors) {
+static std::string gguf_file(const std::vector<FileTensor>& tensors, const std::string& architecture = "qwen3moe",
+                             const std::vector<std::pair<std::string, uint32_t>>& numbers = {}) {
     std::string out("GGUF");
     auto put = [&out](const void* p, size_t n) { out.append(static_cast<const char*>(p), n); };
     auto u32 = [&](uint32_t v) { put(&v, 4); };
@@ -104,9 +105,10 @@ static std::string gguf_file(const std::vector<FileTensor>& tensors) {
     auto str = [&](const std::string& v) { u64(v.size()); out += v; };
     u32(3);
     u64(tensors.size());
-    u64(2);
-    str("general.architecture"); u32(8); str("qwen3moe");
+    u64(2 + numbers.size());
+    str("general.architecture"); u32(8); str(architecture);
     str("general.quantization_version"); u32(4); u32(2);
+    for (const auto& [key, value] : numbers) { str(key); u32(4); u32(value); }
     uint64_t cursor = 0;
     std::vector<uint64_t> offsets;
     for (const auto& t : tensors) {
@@ -344,6 +346,54 @@ int main() {
             threw = err.kind() == ErrorKind::Gguf;
         }
         report("a rank-3 tensor is not a matrix: Error::Gguf", threw);
+    }
+    {
+        // a whole Qwen3 file bound by canonical name (src/model/qwen_gguf.rs:32-268): the plan names every
+        // tensor, the quantized ones reach the device verbatim under the model's own names
+        const size_t h = 256, heads = 2, kv = 1, hd = 128, inter = 512, vocab = 512;
+        auto dense = [](size_t count) { return std::vector<uint8_t>(count * 4, 0); };
+        const auto embd = blocks(QuantizationFormat::Q6_K, vocab, h, 51), norm = dense(h), head_norm = dense(hd);
+        const auto wq = blocks(QuantizationFormat::Q4_K, heads * hd, h, 52), wk = blocks(QuantizationFormat::Q4_K, kv * hd, h, 53);
+        const auto wv = blocks(QuantizationFormat::Q6_K, kv * hd, h, 54), wo = blocks(QuantizationFormat::Q4_K, h, heads * hd, 55);
+        const auto wg = blocks(QuantizationFormat::Q4_K, inter, h, 56), wu = blocks(QuantizationFormat::Q4_K, inter, h, 57);
+        const auto wd = blocks(QuantizationFormat::Q6_K, h, inter, 58);
+        std::istringstream stream(gguf_file(
+            {{"token_embd.weight", {h, vocab}, FH_GGML_Q6_K, &embd}, {"output_norm.weight", {h}, 0, &norm},
+             {"blk.0.attn_norm.weight", {h}, 0, &norm}, {"blk.0.ffn_norm.weight", {h}, 0, &norm},
+             {"blk.0.attn_q.weight", {h, heads * hd}, FH_GGML_Q4_K, &wq}, {"blk.0.attn_k.weight", {h, kv * hd}, FH_GGML_Q4_K, &wk},
+             {"blk.0.attn_v.weight", {h, kv * hd}, FH_GGML_Q6_K, &wv}, {"blk.0.attn_output.weight", {heads * hd, h}, FH_GGML_Q4_K, &wo},
+             {"blk.0.attn_q_norm.weight", {hd}, 0, &head_norm}, {"blk.0.attn_k_norm.weight", {hd}, 0, &head_norm},
+             {"blk.0.ffn_gate.weight", {h, inter}, FH_GGML_Q4_K, &wg}, {"blk.0.ffn_up.weight", {h, inter}, FH_GGML_Q4_K, &wu},
+             {"blk.0.ffn_down.weight", {inter, h}, FH_GGML_Q6_K, &wd}},
+            "qwen3",
+            {{"qwen3.embedding_length", (uint32_t)h}, {"qwen3.attention.head_count", (uint32_t)heads},
+             {"qwen3.attention.head_count_kv", (uint32_t)kv}, {"qwen3.attention.key_length", (uint32_t)hd},
+             {"qwen3.attention.value_length", (uint32_t)hd}, {"qwen3.feed_forward_length", (uint32_t)inter},
+             {"qwen3.block_count", 1u}}));
+        gguf::Reader file(stream);
+        const auto [shape, plan] = gguf::models::plan_qwen(file);
+        report("the Qwen3 plan reads the model shape and names all thirteen tensors",
+               shape.vocab_size == vocab && shape.hidden_size == h && shape.head_dim == hd && shape.tie_word_embeddings &&
+                   shape.layers.size() == 1 && plan.bindings.size() == 13 && plan.tensor_count == 13 &&
+                   plan.binding("layers.0.down.weight").sources[0] == "blk.0.ffn_down.weight");
+        const gguf::models::BoundWeights bound = gguf::models::bind_quantized(d, file, plan);
+        size_t packed_bytes = embd.size() + wq.size() + wk.size() + wv.size() + wo.size() + wg.size() + wu.size() + wd.size();
+        bool exact = bound.matrices.size() == 8 && bound.experts.empty() && bound.quantized_tensor_bytes == packed_bytes;
+        if (exact) {
+            const QuantizedMatrix& down = bound.matrices.at("layers.0.down.weight");
+            std::vector<float> want(h * inter);
+            fo_dequantize(FH_GGML_Q6_K, wd.data(), h, inter, want.data());
+            const auto got = d.dequantize(down).to_f32();
+            exact = down.rows() == h && down.columns() == inter && std::memcmp(got.data(), want.data(), want.size() * 4) == 0;
+        }
+        report("its quantized tensors are on the device under their canonical names, bit for bit", exact);
+        bool threw = false;
+        try {
+            plan.binding("lm_head.weight");   // tied: the file has no output.weight
+        } catch (const Error& err) {
+            threw = err.kind() == ErrorKind::Weight;
+        }
+        report("a tied model has no lm_head binding: Error::Weight", threw);
     }
     {
         // residual add + RMSNorm (add_rmsnorm, src/ops/mod.rs:762-820): bit-exact residual, normalised

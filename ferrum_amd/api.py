@@ -182,7 +182,7 @@ class DType(enum.IntEnum):
 
 
 class QuantizationFormat(enum.Enum):
-    Q8_0 = 8       # the hybrid engine's Format::Q8_0; rows in runs of eight 34-byte blocks
+    Q8_0 = 8       # the hybrid engine's Format::Q8_0: 34-byte blocks of 32 weights (src/loader/gguf.rs:99)
     Q4_K = 12
     Q5_K = 13
     Q6_K = 14
@@ -199,12 +199,11 @@ class QuantizationFormat(enum.Enum):
         return self.value
 
     def block_elements(self) -> int:
-        """Weights per unit of a row: a super-block, or for Q8_0 eight 32-weight GGML blocks
-        (rows are a multiple of 256 weights long in every format)."""
-        return 256
+        """Weights per block: a row is a whole number of them (256, or 32 for Q8_0)."""
+        return 32 if self.value == 8 else 256
 
     def block_bytes(self) -> int:
-        return {8: 272, 12: 144, 13: 176, 14: 210, 23: 136}[self.value]
+        return {8: 34, 12: 144, 13: 176, 14: 210, 23: 136}[self.value]
 
 
 def _f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:

@@ -102,6 +102,93 @@ fh_status ensure_scratch(fh_device* d, size_t data_bytes) {
     FH_HIP(hipMemsetAsync(d->scratch, 0, counter_bytes, d->stream));
     return FH_OK;
 }
+// A block the library owns for its own temporaries (it holds no count on the device), grown like
+// the scratch: outside recordings only, by at least 2x, old blocks kept for the recorded executions
+// that carry their address.
+fh_status ensure_block(fh_device* d, fh_buffer*& slot, size_t bytes, const char* what) {
+    if (slot != nullptr && slot->bytes >= bytes) return FH_OK;
+    if (d->capturing)
+        return fail(FH_ERR_SYNCHRONIZATION, "%s must grow: run the call once before recording it", what);
+    FH_HIP(hipStreamSynchronize(d->stream));
+    if (slot == nullptr) {
+        slot = new (std::nothrow) fh_buffer();
+        if (slot == nullptr) return fail(FH_ERR_ALLOCATION, "out of host memory");
+        slot->device = d;
+    }
+    if (bytes < 2 * slot->bytes) bytes = 2 * slot->bytes;
+    if (slot->ptr) {
+        if (d->live_graphs > 0) d->retired_scratch.push_back(slot->ptr);
+        else (void)hipFree(slot->ptr);
+    }
+    slot->ptr = nullptr;
+    slot->bytes = 0;
+    hipError_t e = hipMalloc(&slot->ptr, bytes);
+    if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+    slot->bytes = bytes;
+    return FH_OK;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// ---- matrices whose rows are stored padded (Q8_0 rows of 32 n weights, n not a multiple of 8) ----
+// An entry point that meets one runs on the matrix as it is stored (rows of stored_cols weights,
+// the added blocks empty) and on its activations rewritten to that width, zeros in the added
+// columns, in a block of the device's own.  Everything behind that point is the ordinary path.
+fh_qmatrix as_stored(const fh_qmatrix* w) {
+    fh_qmatrix m = *w;
+    m.cols = w->stored_cols;
+    return m;
+}
+
+struct PaddedActivations {
+    struct Item {
+        const fh_view* x;
+        uint64_t pieces;   // rows x parts: runs of `cols` elements
+        const char* what;
+        fh_view* out;
+        Range range;
+    };
+    fh_device* device;
+    uint64_t cols, stored;
+    Item items[2];
+    int count = 0;
+    PaddedActivations(fh_device* d, const fh_qmatrix* w) : device(d), cols(w->cols), stored(w->stored_cols) {}
+    void add(const fh_view* x, uint64_t pieces, const char* what, fh_view* out) {
+        items[count++] = Item{x, pieces, what, out, Range{nullptr, 0}};
+    }
+    // checks the views, then writes the padded copies and points `out` at them
+    fh_status run() {
+        size_t at = 0, offsets[2] = {0, 0};
+        for (int i = 0; i < count; ++i) {
+            Item& it = items[i];
+            if (!fits_u32(it.pieces * stored)) return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
+            fh_status st = resolve(device, it.x, it.pieces * cols, it.what, &it.range);
+            if (st != FH_OK) return st;
+            offsets[i] = at;
+            at += align256((size_t)(it.pieces * stored) * dtype_bytes(it.x->dtype));
+        }
+        fh_status st = ensure_block(device, device->padded_rows, at, "the block for padded activations");
+        if (st != FH_OK) return st;
+        for (int i = 0; i < count; ++i) {
+            const Item& it = items[i];
+            launch_pad_rows(device->stream, it.range.begin, static_cast<uint8_t*>(device->padded_rows->ptr) + offsets[i],
+                            (size_t)it.pieces, (size_t)cols, (size_t)stored, dtype_bytes(it.x->dtype));
+            *it.out = fh_view{device->padded_rows, offsets[i], it.x->dtype};
+        }
+        FH_HIP(hipGetLastError());
+        return FH_OK;
+    }
+    // an output may not alias the activations as the caller passed them
+    fh_status keep_apart(const fh_view* y, uint64_t elements, const char* what, const char* message) const {
+        Range yr;
+        fh_status st = resolve(device, y, elements, what, &yr);
+        if (st != FH_OK) return st;
+        for (int i = 0; i < count; ++i)
+            if (overlaps(items[i].range, yr)) return fail(FH_ERR_RANGE, "%s", message);
+        return FH_OK;
+    }
+};
+
 uint32_t* scratch_counters(fh_device* d) { return static_cast<uint32_t*>(d->scratch); }
 uint8_t* scratch_data(fh_device* d) {
     return static_cast<uint8_t*>(d->scratch) + fh_device::kCounterWords * sizeof(uint32_t);
@@ -316,6 +403,11 @@ void fh_device_destroy(fh_device* device) {
         delete device->workspace;
         device->workspace = nullptr;
     }
+    if (device->padded_rows) {
+        if (device->padded_rows->ptr) (void)hipFree(device->padded_rows->ptr);
+        delete device->padded_rows;
+        device->padded_rows = nullptr;
+    }
     for (void* old : device->retired_scratch) (void)hipFree(old);
     device->retired_scratch.clear();
     device->scratch = nullptr;
@@ -506,40 +598,57 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
                        : ggml_type == kQ6K ? "Q6_K"
                        : ggml_type == kQ8_0 ? "Q8_0"
                                             : "IQ4_XS";
-    if (rows == 0 || cols == 0 || cols % 256 != 0)
-        return fail(FH_ERR_SHAPE, "%s matrix requires nonempty rows and columns divisible by block size 256",
-                    name);
+    // a row is whole blocks: super-blocks of 256 weights, or for Q8_0 the 32-weight blocks of its GGML
+    // geometry (src/loader/gguf.rs:99)
+    const uint64_t unit = ggml_type == kQ8_0 ? 32 : 256;
+    const size_t unit_bytes = ggml_type == kQ8_0 ? 34 : bb;
+    if (rows == 0 || cols == 0 || cols % unit != 0)
+        return fail(FH_ERR_SHAPE, "%s matrix requires nonempty rows and columns divisible by block size %u",
+                    name, (unsigned)unit);
     if (experts == 0) return fail(FH_ERR_SHAPE, "quantized expert matrix row geometry mismatch");
+    const uint64_t stored_cols = (cols + 255) / 256 * 256;
     unsigned __int128 total_rows = (unsigned __int128)rows * experts;
-    unsigned __int128 byte_len = total_rows * (cols / 256) * bb;
-    if (total_rows > 0xffffffffull || byte_len > (unsigned __int128)SIZE_MAX / 2)
+    unsigned __int128 byte_len = total_rows * (cols / unit) * unit_bytes;
+    unsigned __int128 stored_len = total_rows * (stored_cols / 256) * bb;
+    if (total_rows > 0xffffffffull || stored_len > (unsigned __int128)SIZE_MAX / 2)
         return fail(FH_ERR_SHAPE, "packed matrix byte size overflow");
     if (packed == nullptr) return fail(FH_ERR_PARAMETER, "null payload");
-    if (packed_len % bb != 0)
+    if (packed_len % unit_bytes != 0)
         return fail(FH_ERR_GGUF, "tensor %s stream ended inside a block", name);
     if ((unsigned __int128)packed_len != byte_len)
         return fail(FH_ERR_SHAPE, "%s payload is %zu bytes, geometry needs %llu", name, packed_len,
                     (unsigned long long)byte_len);
     const uint8_t* p = static_cast<const uint8_t*>(packed);
-    for (size_t off = 0; off < packed_len; off += bb) {
-        if (ggml_type == kQ8_0) {
-            for (size_t sub = 0; sub < 272; sub += 34)
-                if (!f16_finite(p + off + sub)) return fail(FH_ERR_WEIGHT, "%s scale must be finite", name);
-            continue;
-        }
+    for (size_t off = 0; off < packed_len; off += unit_bytes) {
         bool ok = ggml_type == kQ6K     ? f16_finite(p + off + 208)
-                  : ggml_type == kIQ4XS ? f16_finite(p + off)
+                  : ggml_type == kIQ4XS || ggml_type == kQ8_0 ? f16_finite(p + off)
                                         : (f16_finite(p + off) && f16_finite(p + off + 2));
         if (!ok) return fail(FH_ERR_WEIGHT, "%s scale must be finite", name);
+    }
+    // Q8_0 rows that do not end on a run of eight blocks are stored with the run completed by
+    // empty blocks (scale and quants zero): the kernels then see rows of `stored_cols` weights,
+    // and the entry points bring the activations to that width (pad_activations below)
+    std::vector<uint8_t> staged;
+    const size_t upload_len = (size_t)stored_len;
+    if (stored_cols != cols) {
+        try {
+            staged.assign(upload_len, 0);
+        } catch (const std::bad_alloc&) {
+            return fail(FH_ERR_ALLOCATION, "out of host memory");
+        }
+        const size_t row_bytes = (size_t)(cols / 32) * 34, stored_row_bytes = (size_t)(stored_cols / 32) * 34;
+        for (size_t r = 0; r < (size_t)total_rows; ++r)
+            std::memcpy(staged.data() + r * stored_row_bytes, p + r * row_bytes, row_bytes);
+        p = staged.data();
     }
     FH_HIP(hipSetDevice(device->ordinal));
     void* dptr = nullptr;
     // 16 spare bytes keep vector loads of the last block inside the allocation
-    hipError_t e = hipMalloc(&dptr, packed_len + 16);
+    hipError_t e = hipMalloc(&dptr, upload_len + 16);
     if (e != hipSuccess)
-        return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", packed_len, hipGetErrorString(e));
-    e = hipMemcpyAsync(dptr, packed, packed_len, hipMemcpyHostToDevice, device->stream);
-    if (e == hipSuccess) e = hipMemsetAsync(static_cast<uint8_t*>(dptr) + packed_len, 0, 16, device->stream);
+        return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", upload_len, hipGetErrorString(e));
+    e = hipMemcpyAsync(dptr, p, upload_len, hipMemcpyHostToDevice, device->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(static_cast<uint8_t*>(dptr) + upload_len, 0, 16, device->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(device->stream);
     if (e != hipSuccess) {
         (void)hipFree(dptr);
@@ -557,6 +666,7 @@ fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows
     m->ggml_type = ggml_type;
     m->rows = rows;
     m->cols = cols;
+    m->stored_cols = stored_cols;
     m->experts = experts;
     *out = m;
     return FH_OK;
@@ -583,7 +693,7 @@ fh_status fh_dequantize(fh_device* device, const fh_qmatrix* weight, const fh_vi
     Range o;
     fh_status st = resolve(device, out, rows * weight->cols, "dequantize output", &o);
     if (st != FH_OK) return st;
-    device->last_operation = launch_dequantize(device->stream, weight->ggml_type, weight->ptr, rows,
+    device->last_operation = launch_dequantize(device->stream, weight->ggml_type, weight->ptr, rows, weight->stored_cols,
                                                weight->cols, const_cast<uint8_t*>(o.begin), out->dtype);
     FH_HIP(hipGetLastError());
     return FH_OK;
@@ -612,7 +722,7 @@ fh_status fh_embedding_gather_quantized(fh_device* device, const fh_qmatrix* wei
     FH_HIP(hipMemcpyAsync(scratch_data(device), tokens, need, hipMemcpyHostToDevice, device->stream));
     FH_HIP(hipStreamSynchronize(device->stream));
     device->last_operation =
-        launch_embedding_gather(device->stream, weight->ggml_type, weight->ptr, weight->cols,
+        launch_embedding_gather(device->stream, weight->ggml_type, weight->ptr, weight->stored_cols, weight->cols,
                                 reinterpret_cast<const uint32_t*>(scratch_data(device)), count,
                                 const_cast<uint8_t*>(o.begin), out->dtype);
     FH_HIP(hipGetLastError());
@@ -635,6 +745,16 @@ fh_status project(fh_device* device, const fh_qmatrix* weight, const fh_view* x,
     const uint64_t n = weight->rows * weight->experts, k = weight->cols;
     if (m == 0 || k > 0xffffffffull - 32)
         return fail(FH_ERR_SHAPE, "quantized projection requires [M,K] matching [N,K]");
+    if (weight->padded()) {
+        const fh_qmatrix stored = as_stored(weight);
+        PaddedActivations pad(device, weight);
+        fh_view px{};
+        pad.add(x, (uint64_t)m * (silu_mul ? 2 : 1), "projection input", &px);
+        fh_status pst = pad.run();
+        if (pst == FH_OK) pst = pad.keep_apart(y, (uint64_t)m * n, "projection output", "projection output aliases its input");
+        if (pst != FH_OK) return pst;
+        return project(device, &stored, &px, m, y, silu_mul, f32_tile_from);
+    }
     const uint64_t x_elements = (uint64_t)m * k * (silu_mul ? 2 : 1);
     if (!fits_u32(x_elements) || !fits_u32((uint64_t)m * n) || !fits_u32(n))
         return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
@@ -733,6 +853,9 @@ fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* wei
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device) return fail(FH_ERR_DEVICE_MISMATCH, "weight belongs to another device");
     if (device->fixed_scratch == nullptr) return fail(FH_ERR_DISPATCH, "the fixed scratch is not set up");
+    if (weight->padded())
+        return fail(FH_ERR_SHAPE, "rows of %llu weights are stored padded and need a temporary for the activations: "
+                    "fh_project_quantized takes them", (unsigned long long)weight->cols);
     const uint64_t n = weight->rows * weight->experts, k = weight->cols;
     if (m == 0 || k > 0xffffffffull - 32)
         return fail(FH_ERR_SHAPE, "quantized projection requires [M,K] matching [N,K]");
@@ -1017,12 +1140,52 @@ struct SharedExpert {
     const fh_view* y = nullptr;
 };
 
+// The shared expert of a launch on a padded matrix: its matrix as stored, its own activations padded too.
+// `parts`: runs of `cols` elements per row of the shared expert's input.
+struct PaddedRider {
+    fh_qmatrix stored{};
+    fh_view x{};
+    SharedExpert rider;
+    const SharedExpert* get(const SharedExpert* shared) const { return shared != nullptr ? &rider : nullptr; }
+};
+
+fh_status pad_rider(PaddedActivations& pad, const fh_qmatrix* weight, const SharedExpert* shared, uint32_t parts,
+                    PaddedRider* out) {
+    if (shared == nullptr) return FH_OK;
+    if (shared->weight == nullptr || shared->y == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+    if (shared->weight->cols != weight->cols)
+        return fail(FH_ERR_SHAPE, "the shared expert's matrix must have one expert's shape and format");
+    out->stored = as_stored(shared->weight);
+    out->rider = *shared;
+    out->rider.weight = &out->stored;
+    if (shared->x != nullptr) {
+        pad.add(shared->x, (uint64_t)shared->tokens * parts, "shared expert input", &out->x);
+        out->rider.x = &out->x;
+    }
+    return FH_OK;
+}
+
 fh_status hybrid_project_id(fh_device* device, const fh_qmatrix* weight, const fh_view* x, const fh_view* ids,
                             uint32_t routes, uint32_t x_div, const fh_view* y, const SharedExpert* shared) {
     if (device == nullptr || weight == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
     if (weight->device != device || routes == 0 || x_div == 0 || routes % x_div != 0 || ids == nullptr ||
         ids->dtype != FH_F32)
         return fail(FH_ERR_SHAPE, "expert projection geometry");
+    if (weight->padded()) {
+        const fh_qmatrix stored = as_stored(weight);
+        PaddedActivations pad(device, weight);
+        PaddedRider pr;
+        fh_view px{};
+        pad.add(x, (uint64_t)routes / x_div, "expert input", &px);
+        fh_status pst = pad_rider(pad, weight, shared, 1, &pr);
+        if (pst == FH_OK) pst = pad.run();
+        if (pst == FH_OK) pst = pad.keep_apart(y, (uint64_t)routes * weight->rows, "expert output", "expert output aliases an input");
+        if (pst == FH_OK && shared != nullptr)
+            pst = pad.keep_apart(shared->y, (uint64_t)shared->tokens * weight->rows, "shared expert output",
+                                 "shared expert output aliases another tensor");
+        if (pst != FH_OK) return pst;
+        return hybrid_project_id(device, &stored, &px, ids, routes, x_div, y, pr.get(shared));
+    }
     const uint64_t rows = weight->rows, k = weight->cols;
     if (!fits_u32((uint64_t)routes * rows) || !fits_u32((uint64_t)routes / x_div * k))
         return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
@@ -1166,6 +1329,22 @@ fh_status hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, cons
     if (weight->device != device || routes == 0 || weight->experts > 1024 || offsets == nullptr ||
         offsets->dtype != FH_F32 || x == nullptr || y == nullptr)
         return fail(FH_ERR_SHAPE, "expert projection geometry");
+    if (weight->padded()) {
+        const fh_qmatrix stored = as_stored(weight);
+        PaddedActivations pad(device, weight);
+        PaddedRider pr;
+        fh_view px{};
+        pad.add(x, routes, "expert input", &px);
+        if (shared != nullptr && shared->x == nullptr) return fail(FH_ERR_PARAMETER, "null argument");
+        fh_status pst = pad_rider(pad, weight, shared, 1, &pr);
+        if (pst == FH_OK) pst = pad.run();
+        if (pst == FH_OK) pst = pad.keep_apart(y, (uint64_t)routes * weight->rows, "expert output", "expert output aliases an input");
+        if (pst == FH_OK && shared != nullptr)
+            pst = pad.keep_apart(shared->y, (uint64_t)shared->tokens * weight->rows, "shared expert output",
+                                 "shared expert output aliases another tensor");
+        if (pst != FH_OK) return pst;
+        return hybrid_project_mm_id(device, &stored, &px, offsets, routes, y, pr.get(shared));
+    }
     const uint64_t rows = weight->rows, k = weight->cols;
     if (!fits_u32((uint64_t)routes * rows) || !fits_u32((uint64_t)routes * k))
         return fail(FH_ERR_SHAPE, "index does not fit in 32 bits");
@@ -1341,6 +1520,27 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         metadata->buffer->device != device || x == nullptr || x->buffer == nullptr ||
         x->buffer->device != device)
         return fail(FH_ERR_SHAPE, "quantized expert projection geometry mismatch");
+    if (weight->padded()) {
+        if (route != nullptr || grouped_before)
+            return fail(FH_ERR_DISPATCH, "a matrix whose rows are stored padded takes the separate launches");
+        if (shared != nullptr && (form == FH_INPUT_SILU_MUL) != (shared->x != nullptr))
+            return fail(FH_ERR_PARAMETER, "the shared expert takes its own input in the SiLU form only");
+        const fh_qmatrix stored = as_stored(weight);
+        PaddedActivations pad(device, weight);
+        PaddedRider pr;
+        fh_view px{};
+        const uint32_t parts = form == FH_INPUT_SILU_MUL ? 2 : 1;
+        pad.add(x, form == FH_INPUT_GATHER ? (uint64_t)x_rows : (uint64_t)assignments * parts, "expert input", &px);
+        fh_status pst = pad_rider(pad, weight, shared, parts, &pr);
+        if (pst == FH_OK) pst = pad.run();
+        if (pst == FH_OK)
+            pst = pad.keep_apart(y, (uint64_t)assignments * weight->rows, "expert output", "expert output aliases an input");
+        if (pst == FH_OK && shared != nullptr)
+            pst = pad.keep_apart(shared->y, (uint64_t)shared->tokens * weight->rows, "shared expert output",
+                                 "shared expert output aliases another tensor");
+        if (pst != FH_OK) return pst;
+        return expert_project(device, &stored, &px, x_rows, form, assignments, metadata, y, pr.get(shared));
+    }
     const uint64_t rows = weight->rows, k = weight->cols;
     // elements the input view must hold: [A,K], [tokens,K] or [A,2K]
     const uint64_t x_elements = form == FH_INPUT_GATHER ? (uint64_t)x_rows * k
@@ -1623,33 +1823,9 @@ fh_status fh_expert_combine_shared(fh_device* device, const fh_view* in, const f
 
 namespace {
 
-// The workspace: a buffer object the library owns (it holds no count on the device), grown
-// like the scratch: outside recordings only, by at least 2x, old blocks kept for the recorded
-// executions that carry their address.
 fh_status ensure_workspace(fh_device* d, size_t bytes) {
-    if (d->workspace != nullptr && d->workspace->bytes >= bytes) return FH_OK;
-    if (d->capturing)
-        return fail(FH_ERR_SYNCHRONIZATION, "the routed FFN's workspace must grow: run the call once before recording it");
-    FH_HIP(hipStreamSynchronize(d->stream));
-    if (d->workspace == nullptr) {
-        d->workspace = new (std::nothrow) fh_buffer();
-        if (d->workspace == nullptr) return fail(FH_ERR_ALLOCATION, "out of host memory");
-        d->workspace->device = d;
-    }
-    if (bytes < 2 * d->workspace->bytes) bytes = 2 * d->workspace->bytes;
-    if (d->workspace->ptr) {
-        if (d->live_graphs > 0) d->retired_scratch.push_back(d->workspace->ptr);
-        else (void)hipFree(d->workspace->ptr);
-    }
-    d->workspace->ptr = nullptr;
-    d->workspace->bytes = 0;
-    hipError_t e = hipMalloc(&d->workspace->ptr, bytes);
-    if (e != hipSuccess) return fail(FH_ERR_ALLOCATION, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
-    d->workspace->bytes = bytes;
-    return FH_OK;
+    return ensure_block(d, d->workspace, bytes, "the routed FFN's workspace");
 }
-
-size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
 
@@ -1677,6 +1853,9 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
     if (out->dtype != hidden->dtype) return fail(FH_ERR_DTYPE, "the routed FFN writes the activation dtype");
     const uint32_t k = policy->top_k, dt = hidden->dtype;
     const size_t es = dtype_bytes(dt), inter = (size_t)two_i / 2, si = shared ? (size_t)shared_output->cols : 0;
+    // matrices whose rows are stored padded take the separate launches, each padding its own activations
+    const bool stored_padded = input_experts->padded() || output_experts->padded() ||
+                               (shared && (shared_input->padded() || shared_output->padded()));
     const bool rides = shared && shared_input->rows == two_i && shared_input->ggml_type == input_experts->ggml_type &&
                        shared_output->ggml_type == output_experts->ggml_type;
 
@@ -1728,7 +1907,8 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         // shared expert).  From two tokens on the two launches are the faster way (22.1 against
         // 23.2 us): the projection's launch stages an entry's activations once for 32 rows, this one
         // once for 8.
-        const bool folded = count == 1 && a <= 31 && (!shared || rides) && tuning(device, "moe_fold_combine") != 0 &&
+        const bool folded = count == 1 && a <= 31 && (!shared || rides) && !stored_padded &&
+                            tuning(device, "moe_fold_combine") != 0 &&
                             (!shared_gate || shared_gate->dtype == FH_F32) &&
                             expert_down_combine_fits(output_experts->ggml_type, (uint32_t)h, (uint32_t)inter, k, shared);
         // ... and so does the routing: every workgroup of the gate|up launch routes the token
@@ -1786,7 +1966,7 @@ fh_status fh_moe_ffn(fh_device* device, const fh_view* hidden, const fh_view* ro
         const bool shared_stays_inside = !shared || (rides && expert_rows_fit_lds((uint32_t)h, a, (uint32_t)e) &&
                                                      expert_rows_fit_lds((uint32_t)inter, a, (uint32_t)e));
         const bool regroup_once = fused && dt != FH_F32 && group_from > 0 && a >= (uint64_t)group_from && e <= 1024 &&
-                                  shared_stays_inside;
+                                  shared_stays_inside && !stored_padded;
         if (regroup_once) {
             const size_t words = ((size_t)e + 1 + a + 3) & ~(size_t)3;
             const size_t widest = std::max<size_t>(h, inter);

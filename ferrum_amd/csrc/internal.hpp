@@ -38,6 +38,8 @@ struct fh_device {
     std::vector<void*> retired_scratch;
     // temporaries of fh_moe_ffn: one block, grown like the scratch and retired with it
     fh_buffer* workspace = nullptr;
+    // activations rewritten to the width of a matrix whose rows are stored padded: grown the same way
+    fh_buffer* padded_rows = nullptr;
     int live_graphs = 0;
     std::vector<void*> deferred_frees;
     std::vector<std::pair<hipGraphExec_t, hipGraph_t>> deferred_graphs;
@@ -57,6 +59,11 @@ struct fh_qmatrix {
     uint64_t rows = 0;     // per expert
     uint64_t cols = 0;
     uint64_t experts = 1;
+    // Width of a stored row, a multiple of 256: `cols` except for a Q8_0 matrix whose rows are 32 n
+    // weights with n not a multiple of 8, which is kept with every row padded by empty blocks
+    // (scale and quants zero) so that the kernels see runs of eight blocks.
+    uint64_t stored_cols = 0;
+    bool padded() const { return stored_cols != cols; }
 };
 
 struct fh_graph {
@@ -103,9 +110,13 @@ inline size_t dtype_bytes(uint32_t dtype) { return dtype == FH_F32 ? 4 : 2; }
 const char* launch_argmax_rows(hipStream_t s, const void* logits, uint32_t dtype, uint32_t rows, uint32_t width,
                                uint32_t* out);
 void launch_round_to_f16(hipStream_t s, const float* in, uint16_t* out, size_t count);
+// rows are stored `cols` wide (a multiple of 256) and written `out_cols` wide
 const char* launch_dequantize(hipStream_t s, uint32_t ggml_type, const void* w, size_t rows,
-                              size_t cols, void* out, uint32_t out_dtype);
-const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const void* w, size_t cols,
+                              size_t cols, size_t out_cols, void* out, uint32_t out_dtype);
+// pieces of `cols` elements (a multiple of 32) -> pieces of `padded` elements, zero beyond `cols`
+void launch_pad_rows(hipStream_t s, const void* in, void* out, size_t pieces, size_t cols, size_t padded,
+                     size_t element_bytes);
+const char* launch_embedding_gather(hipStream_t s, uint32_t ggml_type, const void* w, size_t cols, size_t out_cols,
                                     const uint32_t* ids_dev, size_t count, void* out,
                                     uint32_t out_dtype);
 

@@ -128,10 +128,14 @@ def q8_0_blocks(count: int, g: np.random.Generator) -> np.ndarray:
 
 def matrix(ggml_type: int, rows: int, cols: int, seed: int, stream: int = 0) -> np.ndarray:
     """Packed row-major ``[rows, cols]`` matrix as a flat uint8 array."""
-    if cols % 256:
-        raise ValueError("columns must be a multiple of 256")
-    count = rows * (cols // 256)
     g = rng(seed, stream)
+    if ggml_type == Q8_0 and cols % 32 == 0 and cols % 256:
+        # rows of 32 n weights that do not end on a run of eight blocks: whole runs, cut to length
+        blocks = rows * (cols // 32)
+        return q8_0_blocks((blocks + 7) // 8, g).reshape(-1)[:blocks * 34].copy()
+    if cols % 256:
+        raise ValueError("columns must be a multiple of 256 (of 32 for Q8_0)")
+    count = rows * (cols // 256)
     if ggml_type == Q4_K:
         return q4_k_blocks(count, g).reshape(-1)
     if ggml_type == Q5_K:

@@ -57,13 +57,18 @@ enum { FH_F32 = 0, FH_F16 = 1, FH_BF16 = 2 };
 /* GGML type ids of the supported formats (src/quantization.rs:24-49; IQ4_XS
  * and Q8_0 are the hybrid engine's Format::Iq4Xs and Format::Q8_0,
  * src/hybrid/weights.rs:29-60: 136-byte blocks of 256 weights and 34-byte
- * blocks of 32, src/loader/gguf.rs:91-121).  Rows are a multiple of 256
- * weights long in every format; for Q8_0 that is eight blocks, 272 bytes.
- * The reference takes Q8_0 rows of any multiple of 32 weights
- * (src/hybrid/weights.rs:29-51); this library refuses the ones that are not a
- * multiple of 256 long: fh_qmatrix_create returns FH_ERR_SHAPE for them and
- * nothing is uploaded.  Every model dimension the reference's loaders produce
- * is a multiple of 256. */
+ * blocks of 32, src/loader/gguf.rs:91-121).  A row is a whole number of
+ * blocks: a multiple of 256 weights, or of 32 for Q8_0 (src/hybrid/weights.rs:1167).
+ * A Q8_0 matrix whose rows do not end on a run of eight blocks is kept on the
+ * device with every row completed to such a run by empty blocks (scale and
+ * quants zero; fh_qmatrix_device_ptr shows that layout, fh_qmatrix_byte_size and
+ * fh_qmatrix_columns the caller's).  Every entry point that multiplies by such
+ * a matrix first copies its activations to that width, zeros in the added
+ * columns, into a block the device owns (one small launch; the block grows
+ * outside recordings only), and then runs as on any other matrix (the added
+ * terms are exact zeros).  fh_project_quantized_no_alloc has no room for
+ * the copy and returns FH_ERR_SHAPE for such a matrix; fh_moe_ffn takes its
+ * separate launches. */
 enum { FH_GGML_Q8_0 = 8, FH_GGML_Q4_K = 12, FH_GGML_Q5_K = 13, FH_GGML_Q6_K = 14, FH_GGML_IQ4_XS = 23 };
 
 typedef struct fh_device fh_device;
@@ -138,7 +143,7 @@ fh_status fh_buffer_fill_zero(fh_buffer* buffer, size_t offset, size_t bytes);
  * validate_gguf_quantized_payload (:212-261) and, for experts > 1,
  * QuantizedExpertMatrix::new (:147-165): a row-major [experts*rows, cols]
  * matrix of verbatim GGUF super-blocks.  `rows` is rows per expert.
- * Errors: FH_ERR_SHAPE (empty, cols % 256, size overflow, length mismatch),
+ * Errors: FH_ERR_SHAPE (empty, cols % 256 or, for Q8_0, cols % 32; size overflow, length mismatch),
  * FH_ERR_GGUF (unsupported type, payload ends inside a block),
  * FH_ERR_WEIGHT (non-finite block scale). */
 fh_status fh_qmatrix_create(fh_device* device, uint32_t ggml_type, uint64_t rows, uint64_t cols,

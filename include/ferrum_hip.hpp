@@ -102,14 +102,15 @@ inline float f16_bits_to_f32(uint16_t h) {
 }
 
 // IQ4_XS and Q8_0 are the hybrid engine's Format::Iq4Xs / Format::Q8_0 (src/hybrid/weights.rs:29-60).
-// Rows are a multiple of 256 weights long in every format; for Q8_0 a unit is eight 34-byte GGML blocks.
+// A row is a whole number of blocks: 256 weights, or for Q8_0 the 32 weights of a 34-byte GGML block
+// (src/loader/gguf.rs:99).
 enum class QuantizationFormat : uint32_t {
     Q8_0 = FH_GGML_Q8_0, Q4_K = FH_GGML_Q4_K, Q5_K = FH_GGML_Q5_K, Q6_K = FH_GGML_Q6_K, IQ4_XS = FH_GGML_IQ4_XS
 };
-inline size_t block_elements(QuantizationFormat) { return 256; }
+inline size_t block_elements(QuantizationFormat f) { return f == QuantizationFormat::Q8_0 ? 32 : 256; }
 inline size_t block_bytes(QuantizationFormat f) {
     switch (f) {
-        case QuantizationFormat::Q8_0: return 272;
+        case QuantizationFormat::Q8_0: return 34;
         case QuantizationFormat::Q4_K: return 144;
         case QuantizationFormat::Q5_K: return 176;
         case QuantizationFormat::Q6_K: return 210;
@@ -315,7 +316,7 @@ public:
                                      size_t experts = 1) const {
         if (rows == 0 || columns == 0 || columns % block_elements(format) != 0 || experts == 0 || rows % experts)
             throw Error(ErrorKind::Shape, "quantized matrix requires nonempty rows and whole blocks");
-        std::vector<uint8_t> host(rows * (columns / 256) * block_bytes(format));
+        std::vector<uint8_t> host(rows * (columns / block_elements(format)) * block_bytes(format));
         fill(host.data(), host.size());
         QuantizedMatrix m;
         m.handle_ = std::make_shared<detail::MatrixHandle>();

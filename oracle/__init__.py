@@ -47,6 +47,10 @@ def _load() -> ctypes.CDLL:
     lib.fo_round_storage_array.argtypes = [f32p, sz, u32, f32p]
     lib.fo_block_bytes.restype = sz
     lib.fo_block_bytes.argtypes = [u32]
+    lib.fo_row_bytes.restype = sz
+    lib.fo_row_bytes.argtypes = [u32, sz]
+    lib.fo_columns_ok.restype = ctypes.c_int
+    lib.fo_columns_ok.argtypes = [u32, sz]
     lib.fo_q4_k_scale_min.restype = None
     lib.fo_q4_k_scale_min.argtypes = [u8p, u32, c.POINTER(u32), c.POINTER(u32)]
     lib.fo_dequantize.restype = i32
@@ -107,6 +111,13 @@ def block_bytes(ggml_type: int) -> int:
     return int(_lib.fo_block_bytes(ggml_type))
 
 
+def row_bytes(ggml_type: int, cols: int) -> int:
+    """Bytes of one packed row: whole super-blocks, or for Q8_0 whole 34-byte blocks of 32 weights."""
+    if not _lib.fo_columns_ok(ggml_type, cols):
+        raise ValueError("unsupported format or a row that is not whole blocks")
+    return int(_lib.fo_row_bytes(ggml_type, cols))
+
+
 def f16_to_f32(bits: int) -> float:
     return float(_lib.fo_f16_to_f32(bits))
 
@@ -136,11 +147,11 @@ def q4_k_scale_min(scales12, group: int):
 
 def dequantize(ggml_type: int, packed, rows: int, cols: int) -> np.ndarray:
     p = _packed(packed)
-    assert p.size == rows * (cols // 256) * block_bytes(ggml_type), "packed length"
+    assert p.size == rows * row_bytes(ggml_type, cols), "packed length"
     out = np.empty((rows, cols), dtype=np.float32)
     rc = _lib.fo_dequantize(ggml_type, _u8(p), rows, cols, _f32(out))
     if rc:
-        raise ValueError("unsupported format or columns not a multiple of 256")
+        raise ValueError("unsupported format or a row that is not whole blocks")
     return out
 
 
@@ -161,7 +172,7 @@ def project(ggml_type: int, packed, n: int, k: int, x, *, accumulate: str = "f32
     p = _packed(packed)
     xa = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
     m = xa.shape[0]
-    assert p.size == n * (k // 256) * block_bytes(ggml_type), "packed length"
+    assert p.size == n * row_bytes(ggml_type, k), "packed length"
     y = np.empty((m, n), dtype=np.float32)
     if accumulate == "f32":
         rc = _lib.fo_project_f32seq(ggml_type, _u8(p), n, k, _f32(xa), m, _f32(y), weight_round,
@@ -206,7 +217,7 @@ def expert_project(ggml_type: int, packed, experts: int, rows: int, k: int, x, m
     xa = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
     meta = np.ascontiguousarray(metadata, dtype=np.float32)
     assert meta.shape == (xa.shape[0], 3)
-    assert p.size == experts * rows * (k // 256) * block_bytes(ggml_type), "packed length"
+    assert p.size == experts * rows * row_bytes(ggml_type, k), "packed length"
     y = np.empty((xa.shape[0], rows), dtype=np.float32)
     rc = _lib.fo_expert_project(ggml_type, _u8(p), experts, rows, k, _f32(xa), _f32(meta),
                                 xa.shape[0], _f32(y), weight_round, out_round,

@@ -35,6 +35,10 @@
  *   fo_dequantize / fo_weight, Q8_0
  *                          pinned: numpy (int8 view times float16 view) on the
  *       reference's random-block generator; block form = per-element form.
+ *       Rows of 32 n weights with n not a multiple of 8 (cols / 32 * 34 bytes,
+ *       src/hybrid/weights.rs:1167): the same byte stream read as rows of 256
+ *       weights gives the same values in the same order, and projections
+ *       equal the numpy product and the hand-written sequential loop.
  *   fo_project_f32seq / fo_project_f64
  *                          pinned: integer special case (d=1, sc=1, dmin=0)
  *       equals an exact integer dot; all-zero quants equal -dmin*m*sum(x);
@@ -177,6 +181,17 @@ size_t fo_block_bytes(uint32_t ggml_type) {
     return 0;
 }
 
+/* A row is whole blocks of the format's own geometry: 256 weights, or 32 weights in 34 bytes for
+ * Q8_0 (src/loader/gguf.rs:99), whose rows need not end on a run of eight blocks. */
+static size_t row_unit(uint32_t ggml_type) { return ggml_type == FO_Q8_0 ? 32 : 256; }
+static size_t row_unit_bytes(uint32_t ggml_type) { return ggml_type == FO_Q8_0 ? 34 : fo_block_bytes(ggml_type); }
+int fo_columns_ok(uint32_t ggml_type, size_t cols) {
+    return fo_block_bytes(ggml_type) != 0 && cols != 0 && cols % row_unit(ggml_type) == 0;
+}
+size_t fo_row_bytes(uint32_t ggml_type, size_t cols) {
+    return cols / row_unit(ggml_type) * row_unit_bytes(ggml_type);
+}
+
 /* ------------------------------------------------------------ Q4_K / Q6_K */
 
 /* 6-bit scale and minimum of 32-weight group `group` (0..7) from the 12
@@ -303,15 +318,12 @@ static void dequant_iq4_xs_block(const uint8_t* b, float* out) {
     }
 }
 
-/* Q8_0, 256 weights = eight blocks of {f16 d, int8 qs[32]}: value = q * d
+/* Q8_0, one block of 32 weights {f16 d, int8 qs[32]}: value = q * d
  * (src/hybrid/draft/gguf.rs:331-338; dequantize_q8_0,
  * src/metal/shaders/hybrid.metal:499-508). */
-static void dequant_q8_0_run(const uint8_t* b, float* out) {
-    for (int block = 0; block < 8; block++) {
-        const uint8_t* p = b + 34 * block;
-        float d = fo_f16_to_f32(le16(p));
-        for (int j = 0; j < 32; j++) out[32 * block + j] = (float)(int8_t)p[2 + j] * d;
-    }
+static void dequant_q8_0_block(const uint8_t* p, float* out) {
+    float d = fo_f16_to_f32(le16(p));
+    for (int j = 0; j < 32; j++) out[j] = (float)(int8_t)p[2 + j] * d;
 }
 
 static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) {
@@ -322,19 +334,22 @@ static void dequant_block(uint32_t ggml_type, const uint8_t* block, float* out) 
     else if (ggml_type == FO_IQ4_XS)
         dequant_iq4_xs_block(block, out);
     else if (ggml_type == FO_Q8_0)
-        dequant_q8_0_run(block, out);
+        dequant_q8_0_block(block, out);
     else
         dequant_q6_k_block(block, out);
 }
 
+/* One packed row of `cols` weights, block by block. */
+static void dequant_row(uint32_t ggml_type, const uint8_t* src, size_t cols, float* out) {
+    size_t unit = row_unit(ggml_type), bytes = row_unit_bytes(ggml_type);
+    for (size_t b = 0; b < cols / unit; b++) dequant_block(ggml_type, src + b * bytes, out + b * unit);
+}
+
 /* Dequantize a packed row-major [rows, cols] matrix to f32 (block form). */
 int fo_dequantize(uint32_t ggml_type, const uint8_t* packed, size_t rows, size_t cols, float* out) {
-    size_t bb = fo_block_bytes(ggml_type);
-    if (bb == 0 || cols % 256 != 0) return 1;
-    size_t blocks = rows * (cols / 256);
-    for (size_t i = 0; i < blocks; i++) {
-        dequant_block(ggml_type, packed + i * bb, out + i * 256);
-    }
+    if (!fo_columns_ok(ggml_type, cols)) return 1;
+    size_t row_bytes = fo_row_bytes(ggml_type, cols);
+    for (size_t row = 0; row < rows; row++) dequant_row(ggml_type, packed + row * row_bytes, cols, out + row * cols);
     return 0;
 }
 
@@ -379,7 +394,7 @@ float fo_weight(uint32_t ggml_type, const uint8_t* packed, size_t row, size_t co
     }
     if (ggml_type == FO_Q8_0) {
         /* one value of the row's flat run of 34-byte blocks: block column / 32, quant column % 32 */
-        const uint8_t* block = packed + row * (blocks * 272) + (column >> 5) * 34;
+        const uint8_t* block = packed + row * ((cols >> 5) * 34) + (column >> 5) * 34;
         return fo_f16_to_f32(le16(block)) * (float)(int8_t)block[2 + (column & 31)];
     }
     if (ggml_type == FO_IQ4_XS) {
@@ -410,7 +425,7 @@ float fo_weight(uint32_t ggml_type, const uint8_t* packed, size_t row, size_t co
 /* src/quantization.rs:212-261 validate_gguf_quantized_payload for the two
  * K formats: 0 ok, 1 partial block, 2 non-finite scale. */
 int fo_validate_payload(uint32_t ggml_type, const uint8_t* payload, size_t len) {
-    size_t bb = fo_block_bytes(ggml_type);
+    size_t bb = fo_block_bytes(ggml_type) == 0 ? 0 : row_unit_bytes(ggml_type);
     if (bb == 0 || len % bb != 0) return 1;
     for (size_t off = 0; off < len; off += bb) {
         const uint8_t* b = payload + off;
@@ -419,8 +434,7 @@ int fo_validate_payload(uint32_t ggml_type, const uint8_t* payload, size_t len) 
         } else if (ggml_type == FO_IQ4_XS) {
             if (!isfinite(fo_f16_to_f32(le16(b)))) return 2;
         } else if (ggml_type == FO_Q8_0) {
-            for (int block = 0; block < 8; block++)
-                if (!isfinite(fo_f16_to_f32(le16(b + 34 * block)))) return 2;
+            if (!isfinite(fo_f16_to_f32(le16(b)))) return 2;
         } else {
             if (!isfinite(fo_f16_to_f32(le16(b + 208)))) return 2;
         }
@@ -444,14 +458,10 @@ typedef struct {
 
 static void* project_worker(void* arg) {
     project_job* j = (project_job*)arg;
-    size_t bb = fo_block_bytes(j->ggml_type);
-    size_t blocks = j->k / 256;
+    size_t row_bytes = fo_row_bytes(j->ggml_type, j->k);
     float* w = (float*)malloc(j->k * sizeof(float));
     for (size_t row = j->row_begin; row < j->row_end; row++) {
-        const uint8_t* src = j->packed + row * blocks * bb;
-        for (size_t b = 0; b < blocks; b++) {
-            dequant_block(j->ggml_type, src + b * bb, w + b * 256);
-        }
+        dequant_row(j->ggml_type, j->packed + row * row_bytes, j->k, w);
         if (j->weight_round)
             for (size_t c = 0; c < j->k; c++) w[c] = fo_round_storage(w[c], (uint32_t)j->weight_round);
         for (size_t mi = 0; mi < j->m; mi++) {
@@ -479,7 +489,7 @@ static void* project_worker(void* arg) {
 }
 
 static int run_project(project_job base, int threads) {
-    if (fo_block_bytes(base.ggml_type) == 0 || base.k % 256 != 0) return 1;
+    if (!fo_columns_ok(base.ggml_type, base.k)) return 1;
     if (threads < 1) threads = 1;
     if ((size_t)threads > base.n) threads = (int)base.n;
     if (threads == 1) {
@@ -693,19 +703,15 @@ void fo_expert_assign(const float* hidden, const float* metadata, size_t assignm
 int fo_expert_project(uint32_t ggml_type, const uint8_t* packed, size_t experts, size_t rows,
                       size_t k, const float* x, const float* metadata, size_t assignments, float* y,
                       int weight_round, int out_round, int f64) {
-    size_t bb = fo_block_bytes(ggml_type);
-    if (bb == 0 || k % 256 != 0) return 1;
-    size_t blocks = k / 256;
+    if (!fo_columns_ok(ggml_type, k)) return 1;
+    size_t row_bytes = fo_row_bytes(ggml_type, k);
     float* w = (float*)malloc(k * sizeof(float));
     for (size_t a = 0; a < assignments; a++) {
         uint32_t expert = float_to_bits(metadata[a * 3]);
         for (size_t r = 0; r < rows; r++) {
             float result = 0.0f;
             if (expert < experts) {
-                const uint8_t* src = packed + ((size_t)expert * rows + r) * blocks * bb;
-                for (size_t b = 0; b < blocks; b++) {
-                    dequant_block(ggml_type, src + b * bb, w + b * 256);
-                }
+                dequant_row(ggml_type, packed + ((size_t)expert * rows + r) * row_bytes, k, w);
                 if (weight_round)
                     for (size_t c = 0; c < k; c++) w[c] = fo_round_storage(w[c], (uint32_t)weight_round);
                 const float* xi = x + a * k;

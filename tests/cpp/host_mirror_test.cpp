@@ -296,6 +296,29 @@ int main() {
             threw = e.kind() == ErrorKind::DeviceMismatch;
         }
         report("a tensor of another device is Error::DeviceMismatch", threw);
+
+        // Q8_0 rows of 2880 weights: ninety 34-byte blocks, which is not whole runs of eight (src/loader/gguf.rs:99)
+        {
+            const size_t qn = 96, qk = 2880, qblocks = qn * (qk / 32);
+            Rng qr{77};
+            std::vector<uint8_t> q8(qblocks * 34);
+            for (auto& b : q8) b = (uint8_t)qr.next();
+            for (size_t i = 0; i < qblocks; ++i) {
+                const uint16_t scale = f32_to_f16_bits((float)(std::fabs(qr.normal()) * 0.002));
+                std::memcpy(q8.data() + i * 34, &scale, 2);
+            }
+            QuantizedMatrix qw = upload(d, QuantizationFormat::Q8_0, qn, qk, q8);
+            std::vector<float> dense(qn * qk), qx(2 * qk), qref(2 * qn);
+            fo_dequantize(FH_GGML_Q8_0, q8.data(), qn, qk, dense.data());
+            const auto on_device = d.dequantize(qw, DType::F32).to_f32();
+            for (auto& v : qx) v = qr.normal();
+            fo_project_f64(FH_GGML_Q8_0, q8.data(), qn, qk, qx.data(), 2, qref.data(), 0, 1);
+            const auto qy = d.project_quantized(d.from_f32({2, qk}, DType::F32, qx), qw);
+            report("Q8_0 rows of ninety blocks: dequantize bit-exact, projection vs f64 oracle",
+                   qw.byte_size() == q8.size() && std::memcmp(on_device.data(), dense.data(), dense.size() * 4) == 0 &&
+                       rel_l2(qy.tensor.to_f32(), qref) <= 1e-5,
+                   rel_l2(qy.tensor.to_f32(), qref));
+        }
     }
     {
         // an execution records the calls and replays them

@@ -38,8 +38,7 @@ def assert_matmul_parity(got, want, what, max_rel_tol=1e-3, l2_tol=1e-5):
 def oracle_columns(ggml_type, packed, n, k, rows, x, **kw):
     """Oracle projection restricted to the weight rows in `rows` (a sample of
     output columns), for shapes whose full product is too slow on the CPU."""
-    bb = oracle.block_bytes(ggml_type)
-    row_bytes = (k // 256) * bb
+    row_bytes = oracle.row_bytes(ggml_type, k)
     sub = np.ascontiguousarray(packed.reshape(n, row_bytes)[rows]).reshape(-1)
     return oracle.project(ggml_type, sub, len(rows), k, x, **kw)
 

@@ -205,7 +205,7 @@ def test_validation(api, d, ggml):
         bad[34 * 11 + 1] = 0x7e                         # NaN scale in the twelfth 34-byte block
         with pytest.raises(api.WeightError):
             qm(api, d, rows, cols, bad, ggml)
-        with pytest.raises(api.ShapeError):             # rows must be a multiple of 256 weights long
-            qm(api, d, rows, 288, packed[: rows * 9 * 34], ggml)
+        with pytest.raises(api.ShapeError):             # a row is whole 32-weight blocks
+            qm(api, d, rows, 304, packed[: rows * 9 * 34], ggml)
     with pytest.raises(api.Error):
         qm(api, d, rows, cols, packed[:-1], ggml)

@@ -769,6 +769,48 @@ def test_q8_0_decoder_equals_numpy_on_the_reference_generator():
     assert oracle.validate_payload(Q8_0, bad) == 2
 
 
+@pytest.mark.parametrize("rows,cols", [(8, 32), (16, 288), (8, 2880), (24, 224)])
+def test_q8_0_rows_that_end_inside_a_run_of_eight_blocks(rows, cols):
+    # a row is cols / 32 * 34 bytes (src/hybrid/weights.rs:1167): the same byte stream read as rows of
+    # 256 weights must give the same values in the same order, and every row the plain numpy product
+    blocks = rows * cols // 32
+    assert cols % 256 and blocks % 8 == 0
+    packed = fx.hybrid_random_blocks(blocks, 34, 34 + cols)
+    assert oracle.row_bytes(Q8_0, cols) == cols // 32 * 34 and oracle.validate_payload(Q8_0, packed) == 0
+    dense = oracle.dequantize(Q8_0, packed, rows, cols)
+    as_runs = oracle.dequantize(Q8_0, packed, blocks // 8, 256)
+    assert np.array_equal(bits(dense.reshape(-1)), bits(as_runs.reshape(-1)))
+    b = packed.reshape(-1, 34)
+    want = (b[:, 2:].view(np.int8).astype(np.float32)
+            * b[:, 0:2].copy().view(np.float16).astype(np.float32)).reshape(rows, cols)
+    assert np.array_equal(bits(dense), bits(want))
+    rng = np.random.default_rng(cols)
+    for _ in range(500):
+        r, c = int(rng.integers(rows)), int(rng.integers(cols))
+        assert bits(np.float32(oracle.weight(Q8_0, packed, r, c, cols))) == bits(dense[r, c])
+    x = fx.xorshift_uniform(3 * cols, 9).reshape(3, cols)
+    ref = x.astype(np.float64) @ dense.astype(np.float64).T
+    assert np.abs(oracle.project(Q8_0, packed, rows, cols, x, accumulate="f64") - ref).max() <= 1e-6 * np.abs(ref).max()
+    # sequential f32 accumulation, K ascending: the loop itself
+    acc = np.zeros(rows, dtype=np.float32)
+    for c in range(cols):
+        acc = (acc + x[0, c] * dense[:, c]).astype(np.float32)
+    assert np.array_equal(bits(oracle.project(Q8_0, packed, rows, cols, x[:1])[0]), bits(acc))
+    # routed rows: each assignment its own expert's slice
+    experts = 2
+    meta = np.zeros((3, 3), dtype=np.uint32)
+    meta[:, 0] = [1, 0, 1]
+    got = oracle.expert_project(Q8_0, packed, experts, rows // experts, cols, x, meta.view(np.float32), accumulate="f64")
+    per = rows // experts
+    for a, e in enumerate(meta[:, 0]):
+        assert np.abs(got[a] - ref[a, e * per:(e + 1) * per]).max() <= 1e-6 * np.abs(ref).max()
+    with pytest.raises(ValueError):
+        oracle.row_bytes(Q8_0, cols + 16)
+    assert oracle.validate_payload(Q8_0, packed[:-1]) == 1
+    bad = packed.copy(); bad[34 * 3: 34 * 3 + 2] = np.frombuffer(np.float16(np.inf).tobytes(), dtype=np.uint8)
+    assert oracle.validate_payload(Q8_0, bad) == 2
+
+
 # ----------------------------------------------- the hybrid engine's route map and combine
 
 def test_moe_map_is_numpy_stable_argsort():

@@ -306,6 +306,14 @@ __device__ __forceinline__ float dpp_max(float v) {
     return fmaxf(v, __int_as_float(moved));
 }
 
+// The same on unsigned integers (and so on the bit patterns of non-negative floats): lanes the
+// pattern leaves unwritten read 0, the identity, which lets the move fold into v_max_u32_dpp.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_umax(uint32_t v) {
+    const uint32_t moved = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+    return moved > v ? moved : v;
+}
+
 // Maximum over the 64 lanes, returned in all lanes; every lane of the wave must be active.
 __device__ __forceinline__ float wave_max(float v) {
     v = dpp_max<0xB1>(v);   // quad_perm [1,0,3,2]

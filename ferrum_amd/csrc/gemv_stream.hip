@@ -105,35 +105,46 @@ __device__ __forceinline__ uint32_t pack_halves(_Float16 lo, _Float16 hi) {
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
+// f16(a s) and f16(b s) in the two halves of a dword, and f16(a s - hi) and f16(b s - hi) against such
+// a pair: one v_fma_mix per value, written straight into its half (s is a power of two, so a s is
+// exact and the first is the plain rounding of the product).
+__device__ __forceinline__ uint32_t hi_pair(float a, float b, float s) {
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(r) : "v"(a), "v"(s));
+    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(r) : "v"(b), "v"(s));
+    return r;
+}
+__device__ __forceinline__ uint32_t lo_pair(float a, float b, float s, uint32_t hi) {
+    uint32_t r;
+    asm("v_fma_mixlo_f16 %0, %1, %2, -%3 op_sel_hi:[0,0,1]" : "=v"(r) : "v"(a), "v"(s), "v"(hi));
+    asm("v_fma_mixhi_f16 %0, %1, %2, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "+v"(r) : "v"(b), "v"(s), "v"(hi));
+    return r;
+}
+
 // One wave writes a super-block's activations (lane = float4 number inside the block) into its
 // slot in operand order.  The 16 lanes of a DPP row hold one chunk (64 weights), which is what a
 // lane group of the A operand covers, so the power-of-two scale is chosen per chunk and never
 // leaves the row.
 __device__ __forceinline__ void stage_block(float4 v, uint8_t* slot, uint32_t lane) {
-    float top = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    top = dpp_max<0xB1>(top);
-    top = dpp_max<0x4E>(top);
-    top = dpp_max<0x141>(top);
-    top = dpp_max<0x140>(top);
-    uint32_t e = __float_as_uint(top) >> 23;
+    // the largest magnitude's exponent: magnitudes order like their bit patterns, and an unsigned
+    // maximum folds into the DPP instruction itself
+    uint32_t top = __float_as_uint(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    top = dpp_umax<0xB1>(top);
+    top = dpp_umax<0x4E>(top);
+    top = dpp_umax<0x141>(top);
+    top = dpp_umax<0x140>(top);
+    uint32_t e = top >> 23;
     e = e < 15u ? 15u : e > 254u ? 254u : e;
     const float s = __uint_as_float((268u - e) << 23);   // 2^(14 - exponent of the chunk's largest)
     // hi = f16(x s), lo = f16(x s - hi): each one fused multiply-add that rounds to a half
-    half2v h02, h13, l02, l13;
-    h02.x = (_Float16)(v.x * s);
-    h02.y = (_Float16)(v.z * s);
-    h13.x = (_Float16)(v.y * s);
-    h13.y = (_Float16)(v.w * s);
-    l02.x = (_Float16)fmaf(v.x, s, -(float)h02.x);
-    l02.y = (_Float16)fmaf(v.z, s, -(float)h02.y);
-    l13.x = (_Float16)fmaf(v.y, s, -(float)h13.x);
-    l13.y = (_Float16)fmaf(v.w, s, -(float)h13.y);
+    const uint32_t h02 = hi_pair(v.x, v.z, s), h13 = hi_pair(v.y, v.w, s);
+    const uint32_t l02 = lo_pair(v.x, v.z, s, h02), l13 = lo_pair(v.y, v.w, s, h13);
     // chunk g, group parity hbit, step u, half of the step
     const uint32_t g = lane >> 4, hbit = (lane >> 3) & 1u, u = (lane >> 1) & 3u;
     uint8_t* const dst = slot + ((u * 4u + g) * 4u + 2u * hbit) * 16u + 8u * (lane & 1u);
     // k slots of an operand dword pair are weights {0, 2} and {1, 3} of four consecutive ones
-    *reinterpret_cast<uint2*>(dst) = make_uint2(__builtin_bit_cast(uint32_t, h02), __builtin_bit_cast(uint32_t, h13));
-    *reinterpret_cast<uint2*>(dst + 16) = make_uint2(__builtin_bit_cast(uint32_t, l02), __builtin_bit_cast(uint32_t, l13));
+    *reinterpret_cast<uint2*>(dst) = make_uint2(h02, h13);
+    *reinterpret_cast<uint2*>(dst + 16) = make_uint2(l02, l13);
     float sum = (v.x + v.y) + (v.z + v.w);
     sum = dpp_add<0xB1>(sum);
     sum = dpp_add<0x4E>(sum);
@@ -155,26 +166,19 @@ __device__ __forceinline__ void stage_block(float4 v, uint8_t* slot, uint32_t la
 // 4 L .. 4 L + 3, so L = 32 h + 8 s + 4 e + j / 4: a quad of lanes is one scale group, which gets
 // a power-of-two scale of its own.
 __device__ __forceinline__ void stage_block_q6k(float4 v, uint8_t* slot, uint32_t lane) {
-    float top = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    top = dpp_max<0xB1>(top);
-    top = dpp_max<0x4E>(top);
-    uint32_t ex = __float_as_uint(top) >> 23;
+    uint32_t top = __float_as_uint(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    top = dpp_umax<0xB1>(top);
+    top = dpp_umax<0x4E>(top);
+    uint32_t ex = top >> 23;
     ex = ex < 15u ? 15u : ex > 254u ? 254u : ex;
     const float s = __uint_as_float((268u - ex) << 23);
-    half2v h02, h13, l02, l13;
-    h02.x = (_Float16)(v.x * s);
-    h02.y = (_Float16)(v.z * s);
-    h13.x = (_Float16)(v.y * s);
-    h13.y = (_Float16)(v.w * s);
-    l02.x = (_Float16)fmaf(v.x, s, -(float)h02.x);
-    l02.y = (_Float16)fmaf(v.z, s, -(float)h02.y);
-    l13.x = (_Float16)fmaf(v.y, s, -(float)h13.x);
-    l13.y = (_Float16)fmaf(v.w, s, -(float)h13.y);
+    const uint32_t h02 = hi_pair(v.x, v.z, s), h13 = hi_pair(v.y, v.w, s);
+    const uint32_t l02 = lo_pair(v.x, v.z, s, h02), l13 = lo_pair(v.y, v.w, s, h13);
     const uint32_t h = lane >> 5, sl = (lane >> 3) & 3u, e = (lane >> 2) & 1u, up = (lane >> 1) & 1u;
     const uint32_t g = 2u * h + e, u = 2u * (sl & 1u) + up, i = 2u * (sl >> 1);
     uint8_t* const dst = slot + ((u * 4u + g) * 4u + i) * 16u + 8u * (lane & 1u);
-    *reinterpret_cast<uint2*>(dst) = make_uint2(__builtin_bit_cast(uint32_t, h02), __builtin_bit_cast(uint32_t, h13));
-    *reinterpret_cast<uint2*>(dst + 16) = make_uint2(__builtin_bit_cast(uint32_t, l02), __builtin_bit_cast(uint32_t, l13));
+    *reinterpret_cast<uint2*>(dst) = make_uint2(h02, h13);
+    *reinterpret_cast<uint2*>(dst + 16) = make_uint2(l02, l13);
     float sum = (v.x + v.y) + (v.z + v.w);
     sum = dpp_add<0xB1>(sum);
     sum = dpp_add<0x4E>(sum);   // the four lanes of a scale group now all hold its sum

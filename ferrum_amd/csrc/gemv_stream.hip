@@ -70,7 +70,18 @@ struct StreamParams {
     uint32_t* counters;   // one per (row tile, batch row), zero between launches
 };
 
-// LDS-direct load: 16 bytes per lane from `g` to LDS address `lds_addr` + 16 * lane.
+// A wave-uniform pointer as a 64-bit value the compiler keeps in scalar registers.
+__device__ __forceinline__ uint64_t uniform_address(const void* pointer) {
+    const uint64_t b = reinterpret_cast<uint64_t>(pointer);
+    // (the builtin returns a signed int: each half goes through uint32_t before it is widened)
+    const uint32_t low = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint32_t high = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    return ((uint64_t)high << 32) | (uint64_t)low;
+}
+
+// LDS-direct load: 16 bytes per lane from `base` + `offset` to LDS address `lds_addr` + 16 * lane.
+// `base` is the same for the whole wave and travels in scalar registers, `offset` is a lane's own
+// 32-bit byte offset: one vector register and no 64-bit vector arithmetic per load.
 // The statement writes M0 (the instruction's LDS base) and cannot declare it: this target rejects
 // M0 in a clobber list.  It is sound as long as the compiler keeps no value of its own in M0 across
 // the statement, which holds for code that uses none of M0's other clients (s_movrel, GWS and
@@ -80,9 +91,10 @@ struct StreamParams {
 // the wait that counts it there must be no vector-memory instruction of the compiler's.  The
 // build compiles this file to assembly text as well and checks all three facts there
 // (ferrum_amd/isa_check.py); it refuses to link a library that breaks one.
-__device__ __forceinline__ void lds_load16(const void* g, uint32_t lds_addr) {
+__device__ __forceinline__ void lds_load16_at(const void* base, uint32_t offset, uint32_t lds_addr) {
     const uint32_t a = __builtin_amdgcn_readfirstlane(lds_addr);
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(a) : "memory");
+    const uint64_t sb = uniform_address(base);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(sb), "s"(a) : "memory");
 }
 
 // s_waitcnt vmcnt(n), n a wave-uniform run-time value up to 20 (0 beyond)
@@ -248,6 +260,8 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
         // a wave with fewer blocks repeats its last one: the register is then defined by the
         // load alone, and nothing can touch it before the wait below
         const uint32_t b = min(wave + kSWaves * i, nb - 1u);
+        // (with a scalar base and a lane offset instead of these 64-bit addresses the launch measured
+        // 0.3 us slower on the 17408 x 5120 matrix, three rounds in turn on one device)
         if constexpr (DT == FH_F32) {
             const float* src = static_cast<const float*>(p.x) + xrow + b * 256u + lane * 4u;
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xraw[i]) : "v"(src) : "memory");
@@ -260,24 +274,32 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
     // 2. the tile: instruction i covers kilobyte (i % per_row) of row (i / per_row)
     const uint32_t per_row = (row_bytes + 1023u) >> 10;
     const uint32_t total = rows * per_row;
-    const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kBlock + lane * 16u;
+    const uint8_t* const wbase = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kBlock;
     const uint32_t tile_addr = (uint32_t)(uintptr_t)tile;
     uint32_t issued = 0;
     // OWN: a super-block of the tile is tile_rows x 9 pieces of 16 bytes, piece 64 j + lane by instruction j
     const uint32_t block_pieces = p.tile_rows * (kBlock / 16u), groups = (block_pieces + 63u) / 64u;
     const uint32_t block_pitch = block_pieces * 16u;
     if constexpr (OWN) {
+        // where a lane's piece of a block lies from the block's first row on: the same for every block
+        uint32_t lane_offset[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t piece = 64u * j + lane, rl = piece / (kBlock / 16u), pc = piece - rl * (kBlock / 16u);
+            lane_offset[j] = min(rl, rows - 1u) * full_row_bytes + 16u * pc;
+        }
+        const uint8_t* const first_row = p.w + (size_t)row0 * full_row_bytes + (size_t)first * kBlock;
 #pragma unroll
         for (int i = 0; i < MAXB; ++i) {
             const uint32_t b = wave + kSWaves * i;
             if (b < nb) {
-                for (uint32_t j = 0; j < groups; ++j) {
-                    const uint32_t piece = 64u * j + lane, rl = piece / (kBlock / 16u), pc = piece - rl * (kBlock / 16u);
-                    const uint32_t r = min(rl, rows - 1u);
-                    if (piece < block_pieces)
-                        lds_load16(p.w + (size_t)(row0 + r) * full_row_bytes + (size_t)(first + b) * kBlock + 16u * pc,
-                                   tile_addr + b * block_pitch + 1024u * j);
-                    ++issued;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if ((uint32_t)j < groups) {
+                        if (64u * j + lane < block_pieces)
+                            lds_load16_at(first_row + b * kBlock, lane_offset[j], tile_addr + b * block_pitch + 1024u * j);
+                        ++issued;
+                    }
                 }
             }
         }
@@ -285,7 +307,8 @@ __device__ __forceinline__ void gemv_stream_body(const StreamParams& p) {
         for (uint32_t i = wave; i < total; i += kSWaves) {
             const uint32_t r = i / per_row, c = i - r * per_row;
             if (c * 1024u + lane * 16u < row_bytes)
-                lds_load16(wbase + (size_t)r * full_row_bytes + c * 1024u, tile_addr + r * p.row_stride + c * 1024u);
+                lds_load16_at(wbase + (size_t)r * full_row_bytes + c * 1024u, lane * 16u,
+                              tile_addr + r * p.row_stride + c * 1024u);
             ++issued;
         }
     }

@@ -833,8 +833,9 @@ __device__ __forceinline__ float16v mfma32(uint4 a, uint4 b, float16v c) {
 }
 
 // LDS of the 32x32x16 form: four activation rings of 16 KB (one per multiplying wave, two
-// stages of 64 rows x 64 K), then the two weight slabs.  The rings come first: an LDS-direct
-// load takes its LDS address from M0, which holds 16 bits.
+// stages of 64 rows x 64 K), then the two weight slabs.  (The rings come first; M0, which carries an
+// LDS-direct load's LDS address, also reaches the addresses above 64 KB: 69632, 135168 and 150000
+// were written and read back on this device.)
 // (RT = row tiles of 32 per multiplying wave: 2 for the 256-row tile, 1 for a 128-row tile)
 template <int RT>
 struct Wide32 {

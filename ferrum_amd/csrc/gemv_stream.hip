@@ -534,8 +534,10 @@ StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t
     uint32_t h = (n + cus * rounds - 1u) / (cus * rounds);
     if (h > 16u) h = 16u;
     if (h < 1u) h = 1u;
-    // An LDS-direct load names its LDS address in 16 bits of M0, so a tile stays below 64 KB, and
-    // a wave owns at most six super-blocks: longer rows are cut into K segments of equal length.
+    // A tile stays below 64 KB (two or three workgroups then share a compute unit's LDS; the
+    // LDS-direct loads themselves reach every LDS address: M0 values of 69632, 135168 and 150000 were
+    // written to and read back on this device) and a wave owns at most six super-blocks: longer rows
+    // are cut into K segments of equal length.
     auto stride_of = [block](uint32_t blocks) {
         uint32_t units = (block * blocks + 15u) / 16u;   // bytes / 16
         if ((units & 1u) == 0) ++units;    // odd number of 16-byte units: 16 rows start in 16 different bank groups

@@ -534,10 +534,12 @@ StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t
     uint32_t h = (n + cus * rounds - 1u) / (cus * rounds);
     if (h > 16u) h = 16u;
     if (h < 1u) h = 1u;
-    // A tile stays below 64 KB (two or three workgroups then share a compute unit's LDS; the
-    // LDS-direct loads themselves reach every LDS address: M0 values of 69632, 135168 and 150000 were
-    // written to and read back on this device) and a wave owns at most six super-blocks: longer rows
-    // are cut into K segments of equal length.
+    // A tile stays below 64 KB -- 70 KB for Q6_K, whose workgroups share a compute unit in twos and
+    // whose sixteen rows of 5120 weights are 67 KB -- so that two or three workgroups share a compute
+    // unit's LDS (the LDS-direct loads themselves reach every LDS address: M0 values of 69632, 135168
+    // and 150000 were written to and read back on this device), and a wave owns at most six
+    // super-blocks: longer rows are cut into K segments of equal length.
+    const uint32_t tile_cap = q6 ? 70u * 1024u : 65536u;
     auto stride_of = [block](uint32_t blocks) {
         uint32_t units = (block * blocks + 15u) / 16u;   // bytes / 16
         if ((units & 1u) == 0) ++units;    // odd number of 16-byte units: 16 rows start in 16 different bank groups
@@ -549,12 +551,12 @@ StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t
     // (the segments then spread the work, so the tiles are as tall as the matrix instruction)
     // the reference's K-split switch asks for at least that many segments, as far as whole blocks go
     const uint32_t wanted = forced_segments > 1 ? ((uint32_t)forced_segments < nb ? (uint32_t)forced_segments : nb) : 1u;
-    if (wanted > 1u || nb > 48u || h * stride_of(nb) > 65536u) h = n < 16u ? n : 16u;
+    if (wanted > 1u || nb > 48u || h * stride_of(nb) > tile_cap) h = n < 16u ? n : 16u;
     uint32_t segments = wanted, seg = (nb + wanted - 1u) / wanted;
     // LDS-direct loads want dword-aligned addresses: a Q6_K segment starts on an even block
     auto even_up = [q6](uint32_t blocks) { return q6 ? (blocks + 1u) & ~1u : blocks; };
     if (segments > 1u) seg = even_up(seg);
-    while (seg > 48u || h * stride_of(seg) > (segments == 1 ? 65536u : budget)) {
+    while (seg > 48u || h * stride_of(seg) > (segments == 1 ? tile_cap : budget)) {
         ++segments;
         seg = even_up((nb + segments - 1u) / segments);
         if (seg <= (q6 ? 2u : 1u)) break;
@@ -563,7 +565,7 @@ StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t
     plan.segments = segments;
     plan.seg_blocks = seg;
     plan.row_stride = stride_of(seg);
-    if (h * plan.row_stride > 65536u) h = 65536u / plan.row_stride;
+    if (h * plan.row_stride > tile_cap) h = tile_cap / plan.row_stride;
     plan.tile_rows = h;
     plan.tiles = (n + h - 1u) / h;
     plan.waves = 8u;
@@ -573,8 +575,13 @@ StreamPlan gemv_stream_plan(uint32_t ggml_type, uint32_t n, uint32_t k, uint32_t
     // tiles of rows of 5120 do not hide (17408 x 5120 in fourteen-row tiles: 22.6 against 21.3 us on
     // the FMA kernel; 151936 x 5120 in fifteen-row tiles 142 - 147 against 141 - 142 us, in two K
     // segments 168 us); rows that must be cut into segments in any case gain (5120 x 17408: 22.7
-    // against 25.0 us).
-    const bool wins = q6 ? nb > 48u : (uint64_t)n * nb >= 16384u;
+    // against 25.0 us).  Output matrices of a million super-blocks or more whose rows the FMA kernel
+    // cannot cut evenly over its eight block slots gain too, in uncut sixteen-row tiles (us, FMA
+    // against this kernel: 151936 x 5120 139.7 / 134.5, 65536 x 5120 63.2 / 62.2, 262144 x 2560 131.7 /
+    // 116.1; but 151936 x 4096 112.9 / 117.8, 128256 x 4096 95.9 / 100.4, 151936 x 2048 58.8 / 60.2,
+    // 32000 x 5120 33.3 / 33.8).
+    const bool big_head = q6 && segments == 1u && h == 16u && (nb & 7u) != 0 && (uint64_t)n * nb >= 1000000u;
+    const bool wins = q6 ? nb > 48u || big_head : (uint64_t)n * nb >= 16384u;
     plan.ok = nb >= 1 && seg >= 1u && seg <= 48u && segments <= 65535u && h >= 1u && (any_size || wins) &&
               plan.lds_bytes <= 160u * 1024u && m >= 1 && m <= 65535u && (!q6 || (nb & 1u) == 0);
     return plan;

@@ -344,6 +344,29 @@ def test_streamed_gemv_matches_the_oracle(api, d, ggml, n, k, dtype):
     d.set_tuning("gemv_stream", 1)
 
 
+def test_large_q6_k_output_matrix_streams_in_uncut_sixteen_row_tiles(api, d):
+    # a million super-blocks in rows the FMA kernel cannot cut evenly over its block slots (20 per row):
+    # sixteen rows of 5120 Q6_K weights are a 67 KB tile
+    n, k = 52000, 5120
+    base = synth.matrix(Q6_K, 2000, k, seed=97).reshape(2000, -1)
+    packed = np.tile(base, (n // 2000, 1)).reshape(-1)
+    w = qm(api, d, Q6_K, n, k, packed)
+    for dtype, code in (("F32", oracle.F32), ("F16", oracle.F16)):
+        x = oracle.round_storage(synth.activations(1, k, seed=98), code).reshape(1, k)
+        xt = api.Tensor.from_f32(d, (1, k), getattr(api.DType, dtype), x)
+        out = d.project_quantized(xt, w, out_dtype=api.DType.F32)
+        assert out.operation == "q6_k_gemv_factored"
+        got = out.tensor.to_f32()
+        rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), synth.rng(99).integers(0, n, 120)]))
+        want = oracle_columns(Q6_K, packed, n, k, rows, x, accumulate="f64")
+        assert_matmul_parity(got[:, rows], want, f"streamed q6_k {n}x{k} {dtype}")
+        with fma_gemv(d):
+            other = d.project_quantized(xt, w, out_dtype=api.DType.F32).tensor.to_f32()
+        # another kernel, another order of summation: equal to the tolerance and not to the bit
+        assert rel_l2(got, other) <= 1e-5 and not np.array_equal(bits(got), bits(other))
+        assert np.array_equal(bits(got[0, :2000]), bits(got[0, 2000:4000]))   # the rows repeat
+
+
 @pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
 def test_streamed_gemv_scales_every_chunk_by_itself(api, d, ggml):
     # activations whose 64-value chunks differ by dozens of orders of magnitude, zero chunks, one

@@ -186,7 +186,9 @@ fh_status fh_project_quantized(fh_device* device, const fh_qmatrix* weight, cons
  * array inside the library, one copy per GPU, held until the process ends.  The call
  * makes no hipMalloc / hipFree and does not synchronise.  FH_ERR_SHAPE when a launch
  * would need more than 4096 counters (row tiles x m) or 1032192 bytes of partial sums
- * (K segments x m x N x 4); nothing is launched then.  All calls on one GPU share the
+ * (K segments x m x N x 4), or for a Q8_0 matrix whose rows are stored padded (rows of
+ * 32 n weights, n not a multiple of 8: the activations would need a widened copy); nothing
+ * is launched then.  All calls on one GPU share the
  * array: calls that overlap in time on one GPU (two streams, two threads) race. */
 fh_status fh_project_quantized_no_alloc(fh_device* device, const fh_qmatrix* weight,
                                         const fh_view* x, uint32_t m, const fh_view* y);

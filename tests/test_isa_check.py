@@ -59,6 +59,16 @@ def test_each_break_is_named(old, new, message):
         assert all(v.startswith("x.hip:") for v in found)
 
 
+def test_requests_with_a_scalar_base_are_hand_loads_too():
+    # `global_load_lds_dwordx4 vOFFSET, s[BASE]`: one vector register of lane offsets, the base in scalar registers
+    scalar = GOOD.replace("global_load_lds_dwordx4 v[2:3], off", "global_load_lds_dwordx4 v14, s[8:9]", 1)
+    assert scalar != GOOD and isa_check.violations(scalar) == []
+    broken = scalar.replace("s_add_u32 s2, s2, 1", "global_load_dword v11, v[2:3], off", 1)
+    assert any("hand-counted wait" in v for v in isa_check.violations(broken, "x.hip"))
+    broken = scalar.replace("s_add_u32 s2, s2, 1", "s_mov_b32 m0, s9", 1)
+    assert any("M0 is used outside" in v for v in isa_check.violations(broken, "x.hip"))
+
+
 def test_the_release_is_read_from_hipcc_version_text():
     assert isa_check.hipcc_release("HIP version: 7.2.26015-fc0010cf6a\nAMD clang version 22") == "7.2.26015"
     assert isa_check.hipcc_release("nothing") == ""

@@ -47,7 +47,7 @@ BLOCK_BYTES = {Q8_0: 272, Q4_K: 144, Q5_K: 176, Q6_K: 210, IQ4_XS: 136}    # per
 ROTATE_BYTES = 600 << 20     # distinct weight bytes visited before a buffer repeats
 
 CSRC = os.path.join(ROOT, "ferrum_amd", "csrc")
-GEMV_SOURCES = ("gemv_stream.hip", "gemv.hip", "device_utils.hpp")
+GEMV_SOURCES = ("gemv_stream.hip", "gemv.hip", "device_utils.hpp", "lds_direct.hpp")
 GEMM_SOURCES = ("gemm.hip", "tile_decode.hpp", "device_utils.hpp")
 
 

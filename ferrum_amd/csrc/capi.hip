@@ -346,6 +346,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["moe_fold_combine"] = 1;      // fh_moe_ffn with few tokens: down projection and weighted sum in one launch (0 = two)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
     d->tuning["gemv_stream_own_loads"] = 1; // the streamed Q4_K GEMV's waves load the super-blocks they multiply (tiles of up to 14 rows); 0: the tile row by row
+    d->tuning["expert_weight_ring"] = 1;    // grouped Q4_K expert projection with short rows: weights through LDS rings (0 = straight into registers)
     d->tuning["gemv_stream"] = 1;           // dense Q4_K / Q6_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)
@@ -462,7 +463,7 @@ fh_status fh_set_tuning(fh_device* device, const char* key, int64_t value) {
         ok = value >= 2;
     } else if (k == "gemm_resident" || k == "moe_fold_combine" || k == "moe_fold_route") {
         ok = value == 0 || value == 1;
-    } else if (k == "gemm_few_tiles_split" || k == "gemv_stream_own_loads") {
+    } else if (k == "gemm_few_tiles_split" || k == "gemv_stream_own_loads" || k == "expert_weight_ring") {
         ok = value == 0 || value == 1;
     } else if (k == "gemv_stream") {
         ok = value >= 0 && value <= 2;
@@ -1411,6 +1412,7 @@ fh_status hybrid_project_mm_id(fh_device* device, const fh_qmatrix* weight, cons
     g.experts = (uint32_t)weight->experts;
     g.expert_offsets = reinterpret_cast<const uint32_t*>(fr.begin);
     g.expert_order = nullptr;   // rows are already expert-sorted
+    g.weight_ring = tuning(device, "expert_weight_ring") != 0;
     if (shared != nullptr) {
         g.shared_w = shared->weight->ptr;
         g.shared_rows = shared->tokens;
@@ -1683,6 +1685,7 @@ fh_status expert_project(fh_device* device, const fh_qmatrix* weight, const fh_v
         g.expert_order = order;
         g.gather_metadata = gathers ? reinterpret_cast<const float*>(mr.begin) : nullptr;
         g.x_rows = x_rows;
+        g.weight_ring = tuning(device, "expert_weight_ring") != 0;
         if (shared != nullptr) {
             g.shared_w = shared->weight->ptr;
             g.shared_rows = shared->tokens;

@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 
 #include "device_utils.hpp"
+#include "lds_direct.hpp"
 #include "tile_decode.hpp"
 #include "internal.hpp"
 
@@ -448,6 +449,46 @@ struct ResidentShared {
     uint32_t tiles_per_slice;
 };
 
+// Copies `mt` activation rows into LDS for the resident kernels: row `tok` of the item to
+// xs[tok * ld ..], its 16-byte pieces swizzled by the row's low four bits; eight pieces per thread
+// in flight at a time.  The row behind a slot is found through up to two tables (the expert-sorted
+// order, then the assignment's token).  All eight pieces look their rows up together, table by
+// table, before any row is read: a round trip per table and one for the rows, where piece after
+// piece would chain up to twenty-four.
+__device__ __forceinline__ void gather_rows(uint16_t* xs, const uint16_t* __restrict__ xsrc, uint32_t mt,
+                                            uint32_t pieces, uint32_t k, uint32_t ld, uint32_t first_token,
+                                            const uint32_t* __restrict__ order, const float* __restrict__ metadata,
+                                            uint32_t x_rows, uint32_t tid) {
+    const uint32_t total = mt * pieces;
+    for (uint32_t base = 0; base < total; base += 8 * kResThreads) {
+        u32x4 v[8];
+        uint32_t dst[8], row[8], pc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
+            const uint32_t tok = idx / pieces;
+            pc[j] = idx - tok * pieces;
+            dst[j] = tok * ld + 8 * (pc[j] ^ (tok & 15u));
+            row[j] = first_token + tok;  // without tables a slot is its row
+        }
+        if (order != nullptr) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) row[j] = order[row[j]];
+        }
+        if (metadata != nullptr) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t token = __float_as_uint(metadata[3 * (size_t)row[j] + 1]);
+                row[j] = token < x_rows ? token : x_rows - 1;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const u32x4*>(xsrc + (size_t)row[j] * k + 8 * (size_t)pc[j]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
+    }
+}
+
 template <uint32_t TYPE, int DT, int TT>
 __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint8_t* __restrict__ w,
                                                                      const uint16_t* __restrict__ x,
@@ -503,30 +544,8 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
         const uint16_t* xsrc = shared && sh.x != nullptr ? sh.x : x;
         void* ydst = shared ? sh.y : y;
         if (item != 0) __syncthreads();  // the previous item is done with the rows
-        // gather the rows, eight 16-byte pieces per thread in flight at a time
-        const uint32_t total = mt * pieces;
-        for (uint32_t base = 0; base < total; base += 8 * kResThreads) {
-            u32x4 v[8];
-            uint32_t dst[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const uint32_t idx = min(base + j * kResThreads + tid, total - 1);
-                const uint32_t tok = idx / pieces, pc = idx - tok * pieces;
-                dst[j] = tok * ld + 8 * (pc ^ (tok & 15u));
-                const uint32_t slot = first_token + tok;
-                uint32_t row = slot;  // a shared group's slots are its tokens
-                if (!shared) {
-                    row = order != nullptr ? order[slot] : slot;
-                    if (metadata != nullptr) {
-                        const uint32_t token = __float_as_uint(metadata[3 * (size_t)row + 1]);
-                        row = token < x_rows ? token : x_rows - 1;
-                    }
-                }
-                v[j] = *reinterpret_cast<const u32x4*>(xsrc + (size_t)row * k + 8 * pc);
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) *reinterpret_cast<u32x4*>(xs + dst[j]) = v[j];
-        }
+        gather_rows(xs, xsrc, mt, pieces, k, ld, first_token, shared ? nullptr : order, shared ? nullptr : metadata,
+                    x_rows, tid);
         __syncthreads();
         if (tile_begin >= tile_end) continue;  // uniform per wave; no barrier follows in this item
 
@@ -625,6 +644,188 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
 #pragma unroll
         for (int i = 0; i < kResRing - 1; ++i)
             if (u + i < units) consume(ring[i]);
+    }
+}
+
+// expert_resident_kernel with the weights going through LDS.  Loading weights straight into the
+// MFMA operand layout puts sixteen different rows under sixteen neighbouring lanes, and the vector
+// L1 then looks up one line per lane: the weight stream of that kernel stops at 3.4 TB/s.  A 16-row
+// tile of weights is one contiguous run of 16 x nb x 144 bytes, so here every wave copies its tiles
+// into a ring of LDS slots of its own with LDS-direct loads -- whole kilobytes per instruction, the
+// next tiles on their way while this one is multiplied -- and the lanes pick their header and their
+// chunk's quants out of LDS.  It needs room for the rings beside the token rows (rows of up to
+// ~1024 weights for 32 tokens), and n a multiple of 16 (a tile is read whole).  Q4_K.
+template <int DT, int TT, int NB>
+__global__ __launch_bounds__(kResThreads) void expert_ring_kernel(const uint8_t* __restrict__ w,
+                                                                 const uint16_t* __restrict__ x,
+                                                                 void* __restrict__ y, uint32_t n,
+                                                                 uint32_t nb, uint32_t y_dtype,
+                                                                 const uint32_t* __restrict__ offsets,
+                                                                 const uint32_t* __restrict__ order,
+                                                                 uint32_t tiles_per_wg,
+                                                                 const float* __restrict__ metadata,
+                                                                 uint32_t x_rows, uint32_t routes,
+                                                                 const ResidentShared sh, uint32_t ring_tiles) {
+    constexpr uint32_t kBB = 144;
+    constexpr int kTokens = 16 * TT;
+    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t k = nb * 256, ld = k;
+    const uint32_t expert_first = offsets != nullptr ? min(offsets[blockIdx.y], routes) : 0;
+    const uint32_t expert_upto = offsets != nullptr ? min(offsets[blockIdx.y + 1], routes) : 0;
+    const uint32_t count = expert_upto > expert_first ? expert_upto - expert_first : 0;
+    const uint32_t tiles = n / 16;
+    const uint32_t pieces = k / 8;  // 16-byte pieces per activation row
+    // a tile of weights: 16 rows x nb super-blocks, contiguous; its ring slot, in whole kilobytes of requests
+    const uint32_t tile_bytes = 16u * nb * kBB, per_tile = (tile_bytes + 1023u) >> 10;
+    uint8_t* const ring = reinterpret_cast<uint8_t*>(xs) + (size_t)kTokens * k * 2 + (size_t)wave * ring_tiles * tile_bytes;
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)ring;
+
+    const uint32_t passes = (count + kTokens - 1) / kTokens;
+    const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, wgs = gridDim.x * gridDim.y;
+    const uint32_t shared_pieces = sh.w != nullptr ? (sh.tokens + kTokens - 1) / kTokens * sh.slices : 0;
+    const uint32_t my_pieces = shared_pieces > wg ? (shared_pieces - wg + wgs - 1) / wgs : 0;
+    for (uint32_t item = 0; item < passes + my_pieces; ++item) {
+        const bool shared = item >= passes;  // uniform over the workgroup
+        uint32_t first_token, mt, tile_begin, tile_end;
+        if (!shared) {
+            first_token = expert_first + item * kTokens;
+            mt = min((uint32_t)kTokens, count - item * kTokens);
+            tile_begin = blockIdx.x * tiles_per_wg + wave;
+            tile_end = min(tiles, (blockIdx.x + 1) * tiles_per_wg);
+        } else {
+            const uint32_t piece = wg + (item - passes) * wgs;
+            const uint32_t group = piece / sh.slices, slice = piece - group * sh.slices;
+            first_token = group * kTokens;
+            mt = min((uint32_t)kTokens, sh.tokens - first_token);
+            tile_begin = slice * sh.tiles_per_slice + wave;
+            tile_end = min(tiles, (slice + 1) * sh.tiles_per_slice);
+        }
+        const uint8_t* wexpert = shared ? sh.w : w + (size_t)blockIdx.y * n * nb * kBB;
+        const uint16_t* xsrc = shared && sh.x != nullptr ? sh.x : x;
+        void* ydst = shared ? sh.y : y;
+        if (item != 0) __syncthreads();  // the previous item is done with the rows
+        // this wave's tiles: tile_begin, tile_begin + 8, ..; the first ones are requested once the rows are
+        // in LDS (the gather's own loads are the compiler's, and nothing of its may stand between a
+        // request and the wait that counts it)
+        const uint32_t my_tiles = tile_begin < tile_end ? (tile_end - tile_begin + kResWaves - 1) / kResWaves : 0;
+        uint32_t requested = 0;
+        auto request_tile = [&]() {
+            const uint8_t* const base = wexpert + (size_t)(tile_begin + requested * kResWaves) * tile_bytes;
+            const uint32_t slot_addr = ring_addr + (requested % ring_tiles) * tile_bytes;
+            for (uint32_t c = 0; c < per_tile; ++c) {
+                if (c * 1024u + lane * 16u < tile_bytes) lds_load16_at(base + c * 1024u, lane * 16u, slot_addr + c * 1024u);
+            }
+            ++requested;
+        };
+        gather_rows(xs, xsrc, mt, pieces, k, ld, first_token, shared ? nullptr : order, shared ? nullptr : metadata,
+                    x_rows, tid);
+        __syncthreads();
+        if (my_tiles == 0) continue;  // uniform per wave; no barrier follows in this item
+
+        // B operand rows: token 16t + r, clamped (columns past mt are never stored)
+        uint32_t boff[TT];
+        uint32_t out_token[TT];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+            const uint32_t tok = min(16u * t + r, mt - 1);
+            boff[t] = tok * ld;
+            out_token[t] = order != nullptr && !shared ? order[first_token + tok] : first_token + tok;
+        }
+        // (the loads above are the last of the compiler's before the requests: it waits for them here,
+        // where nothing of this wave's is in flight)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int t = 0; t < TT; ++t) asm volatile("" : "+v"(out_token[t]));
+        while (requested < my_tiles && requested < ring_tiles) request_tile();
+        uint32_t kl[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) kl[s] = (((Quarter<kQ4K>::klocal(g, s) >> 3) ^ r) << 3);  // row 16t + r: swizzle r
+
+        // Every tile multiplies the same token rows.  Where they fit the wave's registers (two waves a
+        // SIMD leave each 256) the B operands are read out of LDS once per item and not once per tile:
+        // read per tile they are 16 KB per wave and super-block, more LDS traffic than the weights
+        // (32 registers per super-block and 16 tokens)
+        constexpr bool kRowsInRegisters = NB * TT <= 4;
+        uint4 brow[kRowsInRegisters ? NB * 8 * TT : 1];
+        if constexpr (kRowsInRegisters) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+#pragma unroll
+                    for (int t = 0; t < TT; ++t)
+                        brow[(b * 8 + s) * TT + t] = *reinterpret_cast<const uint4*>(xs + 256 * b + boff[t] + kl[s]);
+        }
+
+        float4v acc[TT];
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+        // lane (r, g) finds row r of a slot at r x nb x 144
+        const uint32_t lane_row = r * nb * kBB;
+        for (uint32_t i = 0; i < my_tiles; ++i) {
+            const uint32_t tile = tile_begin + i * kResWaves;
+            // requests retire in issue order: behind tile i's stand those of the tiles asked for since
+            wait_vmcnt((requested - 1u - i) * per_tile);
+            const uint8_t* const slot = ring + (i % ring_tiles) * tile_bytes + lane_row;
+            // the whole tile (NB super-blocks of the lane's row) leaves its slot at once, and the slot
+            // is asked for the tile `ring_tiles` places ahead before anything is multiplied: a slot is
+            // out of flight for one LDS round trip, not for a tile's arithmetic.  (Reading tile i + 1
+            // out of LDS while tile i is multiplied takes that round trip out of the wave's way too and
+            // changes nothing: the kernel is bound by its decode arithmetic.)
+            Quarter<kQ4K> q[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) q[b].load(slot + b * kBB, g);
+            if (requested < my_tiles) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                request_tile();
+            }
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                uint4 a[8];
+                q[b].template decode<DT>(g, a);
+                const uint16_t* xb = xs + 256 * b;
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+#pragma unroll
+                    for (int t = 0; t < TT; ++t) {
+                        uint4 bfrag;
+                        if constexpr (kRowsInRegisters) bfrag = brow[(b * 8 + s) * TT + t];
+                        else bfrag = *reinterpret_cast<const uint4*>(xb + boff[t] + kl[s]);
+                        acc[t] = mfma16<DT>(a[s], bfrag, acc[t]);
+                    }
+                }
+            }
+            // C layout of 16x16x32: acc[t][v] = (weight row 4g + v, token 16t + r)
+            const uint32_t out_row = tile * 16 + 4 * g;
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+                if (16u * t + r < mt) {
+                    const size_t base = (size_t)out_token[t] * n + out_row;
+                    if (y_dtype == FH_F32) {
+                        *reinterpret_cast<float4*>(static_cast<float*>(ydst) + base) =
+                            make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+                    } else {
+                        uint2 packed;
+                        if (y_dtype == FH_F16) {
+                            packed.x = f32_to_f16_bits(acc[t][0]) | (f32_to_f16_bits(acc[t][1]) << 16);
+                            packed.y = f32_to_f16_bits(acc[t][2]) | (f32_to_f16_bits(acc[t][3]) << 16);
+                        } else {
+                            packed.x = f32_to_bf16_bits(acc[t][0]) | (f32_to_bf16_bits(acc[t][1]) << 16);
+                            packed.y = f32_to_bf16_bits(acc[t][2]) | (f32_to_bf16_bits(acc[t][3]) << 16);
+                        }
+                        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(ydst) + base) = packed;
+                    }
+                }
+                acc[t] = float4v{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+        // (the last tile's wait left none of this wave's requests in flight; said where the next
+        // item's loads can see it)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 }
 
@@ -854,6 +1055,30 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                 const uint32_t want = rgrid.x * rgrid.y / groups > 0 ? rgrid.x * rgrid.y / groups : 1;
                 sh.tiles_per_slice = (tiles + want - 1) / want;
                 sh.slices = (tiles + sh.tiles_per_slice - 1) / sh.tiles_per_slice;
+            }
+            // weights through rings in LDS where those fit beside the rows (short rows: the down projections)
+            if constexpr (TYPE == kQ4K) {
+                const size_t tile_bytes = (size_t)16 * nb * 144;
+                const size_t room = kResLdsBytes > lds ? (kResLdsBytes - lds) / (kResWaves * tile_bytes) : 0;
+                const uint32_t ring_tiles = room >= 3 ? 3u : (uint32_t)room;
+                if (a.weight_ring && a.n % 16 == 0 && nb <= 4 && ring_tiles >= 2) {
+                    const size_t ring_lds = lds + kResWaves * ring_tiles * tile_bytes;
+                    typedef void (*Ring)(const uint8_t*, const uint16_t*, void*, uint32_t, uint32_t, uint32_t, const uint32_t*,
+                                         const uint32_t*, uint32_t, const float*, uint32_t, uint32_t, const ResidentShared,
+                                         uint32_t);
+                    static const Ring rings[2][4] = {
+                        {expert_ring_kernel<DT, 1, 1>, expert_ring_kernel<DT, 1, 2>, expert_ring_kernel<DT, 1, 3>,
+                         expert_ring_kernel<DT, 1, 4>},
+                        {expert_ring_kernel<DT, 2, 1>, expert_ring_kernel<DT, 2, 2>, expert_ring_kernel<DT, 2, 3>,
+                         expert_ring_kernel<DT, 2, 4>}};
+                    const Ring kernel = rings[wide ? 1 : 0][nb - 1];
+                    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)ring_lds);
+                    hipLaunchKernelGGL(kernel, rgrid, dim3(kResThreads), ring_lds, s, w, x, a.y, a.n, nb, a.y_dtype,
+                                       a.expert_offsets, a.expert_order, tiles_per_wg, a.gather_metadata, a.x_rows, a.m, sh,
+                                       ring_tiles);
+                    return;
+                }
             }
             if (wide) {
                 auto kernel = expert_resident_kernel<TYPE, DT, 2>;

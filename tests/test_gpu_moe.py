@@ -247,6 +247,42 @@ def test_grouped_expert_projection_matches_the_oracle_and_the_direct_form(api, d
     assert np.array_equal(bits(half), bits(oracle.round_storage(got, code)))
 
 
+@pytest.mark.parametrize("dtype", ["F16", "BF16"])
+@pytest.mark.parametrize("cols,crowd", [(256, 37), (512, 37), (512, 11), (768, 37), (1024, 11), (1024, 37)])
+def test_grouped_q4_k_projection_with_short_rows_streams_weights_through_lds(api, d, cols, crowd, dtype):
+    # Rows of one to four super-blocks and a whole number of 16-row tiles: every wave copies its
+    # weight tiles into a ring in LDS.  The same call with the ring switched off loads them straight
+    # into registers and multiplies in the same order, so the bits agree.  `crowd` assignments
+    # for expert 1: 37 take two passes of 32 tokens, 11 fit one 16-token tile.
+    experts, rows = 5, 80
+    rng = synth.rng(61)
+    ids = np.concatenate([np.full(crowd, 1), np.full(9, 0), np.full(13, 2), [4], [9, 77]])
+    rng.shuffle(ids)
+    packed = synth.matrix(Q4_K, experts * rows, cols, seed=62)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(Q4_K), experts, rows, cols)
+    dt = getattr(api.DType, dtype)
+    code = oracle.F16 if dtype == "F16" else oracle.BF16
+    x = api.Tensor.from_f32(d, (len(ids), cols), dt, synth.activations(len(ids), cols, seed=63))
+    meta = api.Tensor.from_bits(d, (len(ids), 3), _routing_rows(ids))
+    valid = ids < experts
+
+    got = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32)
+    assert d.last_operation() == "expert_project_q4_k_grouped_mfma"
+    got = got.to_f32()
+    d.set_tuning("expert_weight_ring", 0)
+    try:
+        registers = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32).to_f32()
+    finally:
+        d.set_tuning("expert_weight_ring", 1)
+    assert np.array_equal(bits(got), bits(registers))
+    safe = _routing_rows(np.where(valid, ids, 0)).view(np.float32)
+    tile = oracle.expert_project(Q4_K, packed, experts, rows, cols, x.to_f32(), safe, weight_round=code, accumulate="f64")
+    assert np.all(got[~valid] == 0), "rows of unknown experts are zero"
+    assert_matmul_parity(got[valid], tile[valid], "grouped expert projection, weights through LDS")
+    half = d.expert_project_quantized(x, meta, w, cols, experts).to_f32()   # output in the input dtype
+    assert np.array_equal(bits(half), bits(oracle.round_storage(got, code)))
+
+
 @pytest.mark.parametrize("tokens", [1, 512])
 def test_a3b_style_ffn_with_shared_expert(api, d, tokens):
     # hidden 2048, 256 experts of intermediate 512, top-8 after softmax with

@@ -69,6 +69,20 @@ def test_requests_with_a_scalar_base_are_hand_loads_too():
     assert any("M0 is used outside" in v for v in isa_check.violations(broken, "x.hip"))
 
 
+def test_a_store_may_stand_behind_a_request_into_lds_but_not_behind_a_register_load():
+    # vmcnt counts stores too and everything retires in order: a store among the later operations only
+    # lengthens the wait for a request into LDS.  Behind a load into registers it stays a break (the
+    # scan cannot tell which of the two waits the author counted).
+    store = "global_store_dwordx4 v[20:21], v[22:25], off"
+    lds_only = GOOD.replace("global_load_dwordx2 v[4:5], v[2:3], off", "s_nop 0", 1)
+    assert isa_check.violations(lds_only.replace("s_add_u32 s2, s2, 1", store, 1)) == []
+    both = isa_check.violations(GOOD.replace("s_add_u32 s2, s2, 1", store, 1), "x.hip")
+    assert any("hand-counted wait" in v for v in both), both
+    # a load of the compiler's behind the same request is still named
+    load = lds_only.replace("s_add_u32 s2, s2, 1", "global_load_dword v11, v[2:3], off", 1)
+    assert any("hand-counted wait" in v for v in isa_check.violations(load, "x.hip"))
+
+
 def test_the_release_is_read_from_hipcc_version_text():
     assert isa_check.hipcc_release("HIP version: 7.2.26015-fc0010cf6a\nAMD clang version 22") == "7.2.26015"
     assert isa_check.hipcc_release("nothing") == ""

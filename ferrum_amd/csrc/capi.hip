@@ -346,7 +346,7 @@ fh_status fh_device_create(int32_t ordinal, fh_device** out) {
     d->tuning["moe_fold_combine"] = 1;      // fh_moe_ffn with few tokens: down projection and weighted sum in one launch (0 = two)
     d->tuning["gemm_resident"] = 1;         // rows that fit LDS whole take the rows-resident kernel (0 = square tiles)
     d->tuning["gemv_stream_own_loads"] = 1; // the streamed Q4_K GEMV's waves load the super-blocks they multiply (tiles of up to 14 rows); 0: the tile row by row
-    d->tuning["expert_weight_ring"] = 1;    // grouped Q4_K expert projection with short rows: weights through LDS rings (0 = straight into registers)
+    d->tuning["expert_weight_ring"] = 1;    // grouped Q4_K / Q6_K expert projection with short rows: weights through LDS rings (0 = straight into registers)
     d->tuning["gemv_stream"] = 1;           // dense Q4_K / Q6_K GEMV on the streamed matrix-core kernel: 0 never, 1 where it wins, 2 wherever it runs
     d->tuning["moe_routing_temporary_limit"] = 128ll << 20;  // bytes of routing temporaries per SparseMoe chunk (src/metal/legacy.rs:95)
     d->tuning["gemm_f32_min_rows"] = 0;     // f32 activations take the f16 tile kernels from this many rows (0 = never)

@@ -654,8 +654,9 @@ __global__ __launch_bounds__(kResThreads) void expert_resident_kernel(const uint
 // into a ring of LDS slots of its own with LDS-direct loads -- whole kilobytes per instruction, the
 // next tiles on their way while this one is multiplied -- and the lanes pick their header and their
 // chunk's quants out of LDS.  It needs room for the rings beside the token rows (rows of up to
-// ~1024 weights for 32 tokens), and n a multiple of 16 (a tile is read whole).  Q4_K.
-template <int DT, int TT, int NB>
+// ~1024 weights for 32 tokens), and n a multiple of 16 (a tile is read whole).  Q4_K and Q6_K (a
+// tile of either is a whole number of 16-byte pieces at a 16-byte aligned address).
+template <uint32_t TYPE, int DT, int TT, int NB>
 __global__ __launch_bounds__(kResThreads) void expert_ring_kernel(const uint8_t* __restrict__ w,
                                                                  const uint16_t* __restrict__ x,
                                                                  void* __restrict__ y, uint32_t n,
@@ -666,7 +667,7 @@ __global__ __launch_bounds__(kResThreads) void expert_ring_kernel(const uint8_t*
                                                                  const float* __restrict__ metadata,
                                                                  uint32_t x_rows, uint32_t routes,
                                                                  const ResidentShared sh, uint32_t ring_tiles) {
-    constexpr uint32_t kBB = 144;
+    constexpr uint32_t kBB = Quarter<TYPE>::kBlockBytes;
     constexpr int kTokens = 16 * TT;
     extern __shared__ __attribute__((aligned(16))) uint16_t xs[];
 
@@ -743,13 +744,13 @@ __global__ __launch_bounds__(kResThreads) void expert_ring_kernel(const uint8_t*
         while (requested < my_tiles && requested < ring_tiles) request_tile();
         uint32_t kl[8];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) kl[s] = (((Quarter<kQ4K>::klocal(g, s) >> 3) ^ r) << 3);  // row 16t + r: swizzle r
+        for (int s = 0; s < 8; ++s) kl[s] = (((Quarter<TYPE>::klocal(g, s) >> 3) ^ r) << 3);  // row 16t + r: swizzle r
 
         // Every tile multiplies the same token rows.  Where they fit the wave's registers (two waves a
         // SIMD leave each 256) the B operands are read out of LDS once per item and not once per tile:
         // read per tile they are 16 KB per wave and super-block, more LDS traffic than the weights
         // (32 registers per super-block and 16 tokens)
-        constexpr bool kRowsInRegisters = NB * TT <= 4;
+        constexpr bool kRowsInRegisters = NB * TT <= 4 && TYPE == kQ4K;
         uint4 brow[kRowsInRegisters ? NB * 8 * TT : 1];
         if constexpr (kRowsInRegisters) {
 #pragma unroll
@@ -776,7 +777,7 @@ __global__ __launch_bounds__(kResThreads) void expert_ring_kernel(const uint8_t*
             // out of flight for one LDS round trip, not for a tile's arithmetic.  (Reading tile i + 1
             // out of LDS while tile i is multiplied takes that round trip out of the wave's way too and
             // changes nothing: the kernel is bound by its decode arithmetic.)
-            Quarter<kQ4K> q[NB];
+            Quarter<TYPE> q[NB];
 #pragma unroll
             for (int b = 0; b < NB; ++b) q[b].load(slot + b * kBB, g);
             if (requested < my_tiles) {
@@ -1057,8 +1058,10 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                 sh.slices = (tiles + sh.tiles_per_slice - 1) / sh.tiles_per_slice;
             }
             // weights through rings in LDS where those fit beside the rows (short rows: the down projections)
-            if constexpr (TYPE == kQ4K) {
-                const size_t tile_bytes = (size_t)16 * nb * 144;
+            // (Q4_K 49 against 55 us and Q6_K 74 against 77 for 256 experts x 2048 x 512 over 4096 rows; IQ4_XS,
+            // whose rows' operands do not fit the registers beside its decode, 62 either way: it stays)
+            if constexpr (TYPE == kQ4K || TYPE == kQ6K) {
+                const size_t tile_bytes = (size_t)16 * nb * Quarter<TYPE>::kBlockBytes;
                 const size_t room = kResLdsBytes > lds ? (kResLdsBytes - lds) / (kResWaves * tile_bytes) : 0;
                 const uint32_t ring_tiles = room >= 3 ? 3u : (uint32_t)room;
                 if (a.weight_ring && a.n % 16 == 0 && nb <= 4 && ring_tiles >= 2) {
@@ -1067,10 +1070,10 @@ void launch_tt(hipStream_t s, const GemmArgs& a) {
                                          const uint32_t*, uint32_t, const float*, uint32_t, uint32_t, const ResidentShared,
                                          uint32_t);
                     static const Ring rings[2][4] = {
-                        {expert_ring_kernel<DT, 1, 1>, expert_ring_kernel<DT, 1, 2>, expert_ring_kernel<DT, 1, 3>,
-                         expert_ring_kernel<DT, 1, 4>},
-                        {expert_ring_kernel<DT, 2, 1>, expert_ring_kernel<DT, 2, 2>, expert_ring_kernel<DT, 2, 3>,
-                         expert_ring_kernel<DT, 2, 4>}};
+                        {expert_ring_kernel<TYPE, DT, 1, 1>, expert_ring_kernel<TYPE, DT, 1, 2>, expert_ring_kernel<TYPE, DT, 1, 3>,
+                         expert_ring_kernel<TYPE, DT, 1, 4>},
+                        {expert_ring_kernel<TYPE, DT, 2, 1>, expert_ring_kernel<TYPE, DT, 2, 2>, expert_ring_kernel<TYPE, DT, 2, 3>,
+                         expert_ring_kernel<TYPE, DT, 2, 4>}};
                     const Ring kernel = rings[wide ? 1 : 0][nb - 1];
                     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)ring_lds);

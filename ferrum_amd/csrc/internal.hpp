@@ -279,7 +279,7 @@ struct GemmArgs {
     bool rows_resident;
     bool use_resident;    // set by launch_gemm_resident only
     bool few_tiles_split; // up to 16 rows, few weight tiles per workgroup: the tiles' super-blocks are dealt over the waves
-    bool weight_ring;     // routed form, rows resident: Q4_K weights through LDS rings where they fit beside the rows
+    bool weight_ring;     // routed form, rows resident: Q4_K and Q6_K weights through LDS rings where they fit beside the rows
 };
 const char* launch_gemm(hipStream_t s, const GemmArgs& a);
 

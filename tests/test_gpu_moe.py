@@ -249,7 +249,8 @@ def test_grouped_expert_projection_matches_the_oracle_and_the_direct_form(api, d
 
 @pytest.mark.parametrize("dtype", ["F16", "BF16"])
 @pytest.mark.parametrize("cols,crowd", [(256, 37), (512, 37), (512, 11), (768, 37), (1024, 11), (1024, 37)])
-def test_grouped_q4_k_projection_with_short_rows_streams_weights_through_lds(api, d, cols, crowd, dtype):
+@pytest.mark.parametrize("ggml", [Q4_K, Q6_K])
+def test_grouped_projection_with_short_rows_streams_weights_through_lds(api, d, ggml, cols, crowd, dtype):
     # Rows of one to four super-blocks and a whole number of 16-row tiles: every wave copies its
     # weight tiles into a ring in LDS.  The same call with the ring switched off loads them straight
     # into registers and multiplies in the same order, so the bits agree.  `crowd` assignments
@@ -258,8 +259,8 @@ def test_grouped_q4_k_projection_with_short_rows_streams_weights_through_lds(api
     rng = synth.rng(61)
     ids = np.concatenate([np.full(crowd, 1), np.full(9, 0), np.full(13, 2), [4], [9, 77]])
     rng.shuffle(ids)
-    packed = synth.matrix(Q4_K, experts * rows, cols, seed=62)
-    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(Q4_K), experts, rows, cols)
+    packed = synth.matrix(ggml, experts * rows, cols, seed=62)
+    w = api.QuantizedExpertMatrix.new(d, packed, api.QuantizationFormat(ggml), experts, rows, cols)
     dt = getattr(api.DType, dtype)
     code = oracle.F16 if dtype == "F16" else oracle.BF16
     x = api.Tensor.from_f32(d, (len(ids), cols), dt, synth.activations(len(ids), cols, seed=63))
@@ -267,7 +268,7 @@ def test_grouped_q4_k_projection_with_short_rows_streams_weights_through_lds(api
     valid = ids < experts
 
     got = d.expert_project_quantized(x, meta, w, cols, experts, out_dtype=api.DType.F32)
-    assert d.last_operation() == "expert_project_q4_k_grouped_mfma"
+    assert d.last_operation() == {Q4_K: "expert_project_q4_k_grouped_mfma", Q6_K: "expert_project_q6_k_grouped_mfma"}[ggml]
     got = got.to_f32()
     d.set_tuning("expert_weight_ring", 0)
     try:
@@ -276,7 +277,7 @@ def test_grouped_q4_k_projection_with_short_rows_streams_weights_through_lds(api
         d.set_tuning("expert_weight_ring", 1)
     assert np.array_equal(bits(got), bits(registers))
     safe = _routing_rows(np.where(valid, ids, 0)).view(np.float32)
-    tile = oracle.expert_project(Q4_K, packed, experts, rows, cols, x.to_f32(), safe, weight_round=code, accumulate="f64")
+    tile = oracle.expert_project(ggml, packed, experts, rows, cols, x.to_f32(), safe, weight_round=code, accumulate="f64")
     assert np.all(got[~valid] == 0), "rows of unknown experts are zero"
     assert_matmul_parity(got[valid], tile[valid], "grouped expert projection, weights through LDS")
     half = d.expert_project_quantized(x, meta, w, cols, experts).to_f32()   # output in the input dtype
